@@ -1,0 +1,268 @@
+// extern "C" entry points of libfastlstm_hip.so (declared in include/fastlstm_hip.h).
+// Every function validates its arguments before the first HIP call.
+#include <atomic>
+
+#include "gemm.hpp"
+#include "internal.hpp"
+#include "recurrent_bwd.hpp"
+#include "recurrent_fwd.hpp"
+
+using namespace fastlstm;
+
+namespace fastlstm {
+
+static std::atomic<long long> g_spin_limit{400000000ll};  // 4 s of the 100 MHz clock
+long long spin_limit_ticks() { return g_spin_limit.load(); }
+
+namespace {
+
+int check_dims(int T, int B, int I, int H) {
+    if (T <= 0 || B <= 0 || I <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    const long long lim = (1ll << 31) - 1;
+    if ((long long)T * B > lim || (long long)B * 4 * H > lim || 4ll * H * std::max(I, H) > lim) return FASTLSTM_ERR_DIM;
+    return FASTLSTM_OK;
+}
+
+struct DeviceInfo {
+    int num_cus = 0, lds = 0;
+};
+
+int device_info(int device, DeviceInfo *out) {
+    static DeviceInfo cache[64];
+    if (device < 0) {
+        if (hipGetDevice(&device) != hipSuccess) return FASTLSTM_ERR_HIP;
+    }
+    if (device >= 64) return FASTLSTM_ERR_HIP;
+    if (cache[device].num_cus == 0) {
+        int cus = 0, lds = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess)
+            return FASTLSTM_ERR_HIP;
+        cache[device].lds = lds;
+        cache[device].num_cus = cus;
+    }
+    *out = cache[device];
+    return FASTLSTM_OK;
+}
+
+typedef hipError_t (*FwdLauncher)(const FwdParams &, int, int, int, int, int, hipStream_t, int *);
+typedef hipError_t (*BwdLauncher)(const BwdParams &, int, int, int, int, int, hipStream_t, int *);
+FwdLauncher fwd_launcher(int dtype) {
+    return dtype == FASTLSTM_FP32 ? launch_fwd_f32 : (dtype == FASTLSTM_FP16 ? launch_fwd_f16 : launch_fwd_bf16);
+}
+BwdLauncher bwd_launcher(int dtype) {
+    return dtype == FASTLSTM_FP32 ? launch_bwd_f32 : (dtype == FASTLSTM_FP16 ? launch_bwd_f16 : launch_bwd_bf16);
+}
+
+}  // namespace
+}  // namespace fastlstm
+
+extern "C" {
+
+int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan) {
+    if (!plan) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    DeviceInfo di;
+    int rc = device_info(device, &di);
+    if (rc) return rc;
+    return fastlstm_plan_for(di.num_cus, di.lds, B, H, dtype, backward, plan);
+}
+
+int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int T,
+                       int B, int I, int H, int dtype, void *stream) {
+    if (!x || !Wx || !bx || !bh || !ifgo) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(x) || !aligned16(Wx) || !aligned16(ifgo)) return FASTLSTM_ERR_ALIGN;
+    GemmParams p{};
+    p.A = x; p.B = Wx; p.C = ifgo; p.bias0 = bx; p.bias1 = bh;
+    p.M = T * B; p.N = 4 * H; p.K = I;
+    p.lda = I; p.ldb = I; p.ldc = 4 * H;
+    p.splits = 1; p.k_per_split = I;
+    return launch_gemm(dtype, p, false, false, static_cast<hipStream_t>(stream)) == hipSuccess ? FASTLSTM_OK
+                                                                                               : FASTLSTM_ERR_HIP;
+}
+
+int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
+                     void *stream) {
+    if (!d_ifgo || !Wx || !dx) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(d_ifgo) || !aligned16(Wx) || !aligned16(dx)) return FASTLSTM_ERR_ALIGN;
+    GemmParams p{};
+    p.A = d_ifgo; p.B = Wx; p.C = dx;
+    p.M = T * B; p.N = I; p.K = 4 * H;
+    p.lda = 4 * H; p.ldb = I; p.ldc = I;
+    p.splits = 1; p.k_per_split = 4 * H;
+    return launch_gemm(dtype, p, false, true, static_cast<hipStream_t>(stream)) == hipSuccess ? FASTLSTM_OK
+                                                                                              : FASTLSTM_ERR_HIP;
+}
+
+// split-K factor of a weight-gradient product C[M,N] with reduction length K
+static int wgrad_splits(int M, int N, int K, int dtype) {
+    const int tiles = cdiv(M, kBM) * cdiv(N, kBN);
+    if (tiles >= 128) return 1;
+    const int bk = gemm_bk(dtype);
+    int s = std::min(cdiv(512, tiles), std::max(1, K / (4 * bk)));
+    return std::max(1, std::min(s, 1024));
+}
+static int colsum_chunks(int R) { return std::max(1, std::min(256, R / 64)); }
+
+size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
+    if (!dtype_ok(dtype) || check_dims(T, B, I, H)) return 0;
+    const int K = T * B, M = 4 * H;
+    const int sx = wgrad_splits(M, I, K, dtype), sh = wgrad_splits(M, H, K, dtype);
+    size_t part = std::max(sx > 1 ? (size_t)sx * M * I : 0, sh > 1 ? (size_t)sh * M * H : 0) * sizeof(float);
+    size_t cs = (size_t)colsum_chunks(K) * M * sizeof(float);
+    return align_up(cs, 256) + align_up(part, 256) + 256;
+}
+
+int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
+                        void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype, void *stream) {
+    if (!d_ifgo || !x || !h || !dWx || !dWh || !db || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(d_ifgo) || !aligned16(x) || !aligned16(h) || !aligned16(dWx) || !aligned16(dWh) ||
+        !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    if (ws_bytes < fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype)) return FASTLSTM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int K = T * B, M = 4 * H;
+    const int chunks = colsum_chunks(K);
+    float *cs_part = static_cast<float *>(ws);
+    float *gemm_part = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) +
+                                                 align_up((size_t)chunks * M * sizeof(float), 256));
+    if (launch_colsum(dtype, d_ifgo, db, cs_part, K, M, chunks, s) != hipSuccess) return FASTLSTM_ERR_HIP;
+    for (int which = 0; which < 2; ++which) {
+        const int N = which == 0 ? I : H;
+        GemmParams p{};
+        p.A = d_ifgo; p.B = which == 0 ? x : h; p.C = which == 0 ? dWx : dWh;
+        p.Cpart = gemm_part;
+        p.M = M; p.N = N; p.K = K;
+        p.lda = M; p.ldb = N; p.ldc = N;
+        p.splits = wgrad_splits(M, N, K, dtype);
+        const int bk = gemm_bk(dtype);
+        p.k_per_split = cdiv(cdiv(K, p.splits), bk) * bk;
+        p.splits = cdiv(K, p.k_per_split);
+        if (launch_gemm(dtype, p, true, true, s) != hipSuccess) return FASTLSTM_ERR_HIP;
+    }
+    return FASTLSTM_OK;
+}
+
+int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes,
+                            int T, int B, int H, int dtype, void *stream) {
+    if (!ifgo || !out || !cell || !Wh || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    if (!aligned16(ifgo) || !aligned16(out) || !aligned16(cell) || !aligned16(Wh) || !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    fastlstm_plan pl;
+    if (int rc = fastlstm_plan_device(-1, B, H, dtype, 0, &pl)) return rc;
+    if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+    const bool sync = pl.wave_split != 2;
+    const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    unsigned char *wsb = static_cast<unsigned char *>(ws);
+    FwdParams p{};
+    p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = pl.n_htiles;
+    p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
+    p.KS = cdiv(H, kstep);
+    p.spin_limit = spin_limit_ticks();
+    const int n_bt_total = cdiv(B, pl.bt);
+    const size_t launch_ws = sync ? recurrent_ws_launch_bytes(H, dtype, pl.bt, pl.n_btiles, pl.n_htiles, false) : 0;
+    FwdLauncher launch = fwd_launcher(dtype);
+    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
+        const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+        unsigned char *base = wsb + 1024 + (size_t)c * launch_ws;
+        p.flags = reinterpret_cast<int *>(base);
+        p.xbuf = base + align_up((size_t)pl.n_btiles * p.flag_stride * sizeof(int), 1024);
+        p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
+        p.b_base = bt0 * pl.bt;
+        const int grid = n_bt * pl.n_htiles;
+        int occ = 0;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, pl.lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
+            hipSuccess)
+            return FASTLSTM_ERR_HIP;
+    }
+    return FASTLSTM_OK;
+}
+
+int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
+                            void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
+                            int dtype, void *stream) {
+    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    if (!aligned16(dout) || !aligned16(dh) || !aligned16(dc) || !aligned16(ifgo) || !aligned16(cell) ||
+        !aligned16(d_ifgo) || !aligned16(Wh) || !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    fastlstm_plan pl;
+    if (int rc = fastlstm_plan_device(-1, B, H, dtype, 1, &pl)) return rc;
+    if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+    const bool sync = pl.wave_split != 2;
+    const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    unsigned char *wsb = static_cast<unsigned char *>(ws);
+    BwdParams p{};
+    p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = pl.n_htiles;
+    p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
+    p.KSB = cdiv(4 * H, kstep);
+    p.ht = pl.ht;
+    p.spin_limit = spin_limit_ticks();
+    const int n_bt_total = cdiv(B, pl.bt);
+    const size_t launch_ws = sync ? recurrent_ws_launch_bytes(H, dtype, pl.bt, pl.n_btiles, pl.n_htiles, true) : 0;
+    BwdLauncher launch = bwd_launcher(dtype);
+    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
+        const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+        unsigned char *base = wsb + 1024 + (size_t)c * launch_ws;
+        p.flags = reinterpret_cast<int *>(base);
+        p.xbuf = base + align_up((size_t)pl.n_btiles * p.flag_stride * sizeof(int), 1024);
+        p.n_bt = pl.n_btiles;
+        p.b_base = bt0 * pl.bt;
+        const int grid = n_bt * pl.n_htiles;
+        int occ = 0;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, pl.lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
+            hipSuccess)
+            return FASTLSTM_ERR_HIP;
+    }
+    return FASTLSTM_OK;
+}
+
+int fastlstm_ws_status(const void *ws_head) {
+    if (!ws_head) return FASTLSTM_ERR_NULL;
+    const WsHeader *h = static_cast<const WsHeader *>(ws_head);
+    return h->abort_flag ? FASTLSTM_ERR_TIMEOUT : FASTLSTM_OK;
+}
+
+void fastlstm_set_spin_limit(long long ticks) {
+    if (ticks > 0) fastlstm::g_spin_limit.store(ticks);
+}
+
+const char *fastlstm_strerror(int status) {
+    switch (status) {
+        case FASTLSTM_OK: return "ok";
+        case FASTLSTM_ERR_NULL: return "a required pointer is NULL";
+        case FASTLSTM_ERR_DIM: return "a dimension is non-positive or too large";
+        case FASTLSTM_ERR_DTYPE: return "unsupported dtype (0 = fp32, 1 = fp16, 2 = bf16)";
+        case FASTLSTM_ERR_ALIGN: return "a pointer is not 16-byte aligned";
+        case FASTLSTM_ERR_RESIDENCY:
+            return "the W_h slice does not fit in LDS or the barrier group cannot be co-resident";
+        case FASTLSTM_ERR_WORKSPACE: return "workspace is smaller than required";
+        case FASTLSTM_ERR_HIP: return "a HIP runtime call failed";
+        case FASTLSTM_ERR_TIMEOUT: return "a barrier wait timed out (results are invalid)";
+        default: return "unknown status";
+    }
+}
+
+const char *fastlstm_version(void) { return "fastlstm_hip 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,113 @@
+// Shared device/host helpers for the gfx950 LSTM kernels: element-type traits,
+// MFMA wrappers with one fragment convention for all three dtypes, fast gate
+// non-linearities and the host-side launch plumbing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fastlstm_hip.h"
+
+namespace fastlstm {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kThreads = 256;  // 4 waves, one per SIMD
+constexpr int kFragBytes = 1024;  // one MFMA operand block: 64 lanes x 16 bytes
+
+// ---------------------------------------------------------------------------
+// Element traits.  A "fragment" is 16 bytes per lane: EPL elements of K for the
+// matrix row (lane % 16), K-group (lane / 16).  One "k-step" contracts
+// KSTEP = 4 * EPL elements of K:
+//   16-bit: one v_mfma_f32_16x16x32 (lane holds 8 consecutive k),
+//   fp32  : four v_mfma_f32_16x16x4 (MFMA e contracts element e of all 4 lane
+//           groups; the K order inside a k-step is permuted identically for
+//           both operands, which leaves the product unchanged).
+// Logical k of (kstep, lanegroup q, element e) = kstep*KSTEP + q*EPL + e.
+// ---------------------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int EPL = 4, KSTEP = 16, BYTES = 4;
+    static constexpr int DT = FASTLSTM_FP32;
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+template <> struct Elem<_Float16> {
+    static constexpr int EPL = 8, KSTEP = 32, BYTES = 2;
+    static constexpr int DT = FASTLSTM_FP16;
+    static __device__ __forceinline__ float to_f32(_Float16 v) { return (float)v; }
+    static __device__ __forceinline__ _Float16 from_f32(float v) { return (_Float16)v; }
+};
+template <> struct Elem<__bf16> {
+    static constexpr int EPL = 8, KSTEP = 32, BYTES = 2;
+    static constexpr int DT = FASTLSTM_BF16;
+    static __device__ __forceinline__ float to_f32(__bf16 v) { return (float)v; }
+    static __device__ __forceinline__ __bf16 from_f32(float v) { return (__bf16)v; }
+};
+
+// D(16x16) += A(16 x KSTEP) . B(KSTEP x 16); a/b are the 16-byte fragments.
+// Result layout: lane holds D[4*(lane/16) + e][lane % 16], e = 0..3.
+template <typename T>
+__device__ __forceinline__ f32x4 mfma_kstep(const u32x4 a, const u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma_kstep<_Float16>(const u32x4 a, const u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma_kstep<__bf16>(const u32x4 a, const u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma_kstep<float>(const u32x4 a, const u32x4 b, f32x4 c) {
+    const f32x4 af = __builtin_bit_cast(f32x4, a), bf = __builtin_bit_cast(f32x4, b);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[0], bf[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[1], bf[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[2], bf[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[3], bf[3], c, 0, 0, 0);
+    return c;
+}
+
+// Gate non-linearities in fp32.  The fp32 element type uses the full-accuracy
+// library exp and IEEE division (parity bar 1e-4 against nn.LSTM over 100+
+// steps); the 16-bit types use the hardware exp2/rcp approximations, whose
+// error (~1e-7 absolute) is far below the 16-bit rounding of every stored value.
+template <bool ACCURATE> __device__ __forceinline__ float sigmoidf_(float x) {
+    if constexpr (ACCURATE) {
+        return 1.0f / (1.0f + expf(-x));
+    } else {
+        return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+    }
+}
+template <bool ACCURATE> __device__ __forceinline__ float tanhf_(float x) {
+    if constexpr (ACCURATE) {
+        return tanhf(x);
+    } else {
+        // 1 - 2/(1+e^{2x}); saturates correctly at +-inf of the exponential
+        return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * x));
+    }
+}
+
+__host__ __device__ inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline int elem_bytes(int dtype) { return dtype == FASTLSTM_FP32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype >= FASTLSTM_FP32 && dtype <= FASTLSTM_BF16; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Workspace header shared by the two recurrent kernels (first 256 bytes).
+struct WsHeader {
+    int abort_flag;  // set to 1 by the first barrier wait that times out
+    int timeout_group, timeout_step, timeout_seen;
+    int reserved[60];
+};
+static_assert(sizeof(WsHeader) == 256, "workspace header is 256 bytes");
+
+long long spin_limit_ticks();
+
+}  // namespace fastlstm

@@ -1,0 +1,34 @@
+// Declarations shared between the translation units of libfastlstm_hip.so.
+#pragma once
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace fastlstm {
+
+struct GemmParams;
+struct FwdParams;
+struct BwdParams;
+
+hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hipStream_t s);
+hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
+                         hipStream_t s);
+int gemm_bk(int dtype);
+
+// one function per element type (separate translation units, compiled in parallel)
+#define FASTLSTM_DECL_REC(SUF)                                                                       \
+    hipError_t launch_fwd_##SUF(const FwdParams &p, int ht, int bt, int split, int grid, int lds,   \
+                                hipStream_t s, int *max_blocks_per_cu);                              \
+    hipError_t launch_bwd_##SUF(const BwdParams &p, int ht, int bt, int split, int grid, int lds,   \
+                                hipStream_t s, int *max_blocks_per_cu);
+FASTLSTM_DECL_REC(f32)
+FASTLSTM_DECL_REC(f16)
+FASTLSTM_DECL_REC(bf16)
+#undef FASTLSTM_DECL_REC
+
+int fwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
+int bwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
+size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync);
+size_t recurrent_ws_launch_bytes(int H, int dtype, int bt, int n_bt, int n_ht, bool backward);
+
+}  // namespace fastlstm

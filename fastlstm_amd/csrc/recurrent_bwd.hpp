@@ -1,0 +1,285 @@
+// Persistent reverse-time kernel: d_ifgo[t], dh_0, dc_0 for one LSTM layer in one launch.
+//
+// Replaces lstm_persistent_seq_bwd (fastlstm/kernels.py:1201-1409).  Per step
+// t = T-1 .. 0, for the workgroup's tile of bt batch rows x ht hidden units:
+//     dh  = dh_rec + dout[t]
+//     dc += dh * sigmoid(o) * (1 - tanh(c_t)^2)
+//     d_o = dh * tanh(c_t) * sigmoid(o) * (1 - sigmoid(o))
+//     d_f = dc * c_{t-1} * sigmoid(f) * (1 - sigmoid(f))
+//     d_i = dc * tanh(g) * sigmoid(i) * (1 - sigmoid(i))
+//     d_g = dc * sigmoid(i) * (1 - tanh(g)^2)
+//     dc  = dc * sigmoid(f)                                   (kernels.py:1301-1316)
+//     d_ifgo[t] <- (d_i, d_f, d_g, d_o);  barrier over the hidden tiles of the batch tile
+//     dh_rec = d_ifgo[t][rows, 0:4H] . Wh[0:4H, units]        (kernels.py:1362-1383)
+// The gates are re-evaluated from the stored (rounded) pre-activations and cell
+// states, as the reference does.  Unlike the reference (kernels.py:1286-1291,
+// 1337-1342, 1388-1390) dc and dh_rec never leave fp32 registers: both are local
+// to the (unit, batch row) a thread owns.
+//
+// MI355X mapping: the column slice Wh[:, units] is transposed ONCE into LDS in MFMA
+// operand order (K = (unit', gate) pairs, 4H long) and stays resident; d_ifgo[t]
+// travels between workgroups through a double-buffered exchange buffer in operand
+// order, so the K = 4H contraction reads fully coalesced 1 KiB blocks.
+#pragma once
+#include "recurrent_common.hpp"
+
+namespace fastlstm {
+
+struct BwdParams {
+    const void *dout;   // [T,B,H]
+    void *dh, *dc;      // [B,H] in: grads of h_T, c_T; out: grads of h_0, c_0
+    const void *ifgo;   // [T,B,4H]
+    const void *cell;   // [T+1,B,H]
+    void *d_ifgo;       // [T,B,4H]
+    const void *Wh;     // [4H,H]
+    WsHeader *hdr;
+    int *flags;
+    unsigned char *xbuf;   // [2][n_bt][NT][KSB] fragment blocks
+    int T, B, H;
+    int b_base;
+    int n_bt, n_ht, flag_stride;
+    int KSB;            // k-steps covering 4H
+    int ht;             // hidden units per workgroup (SPLIT 0/1: 4, 8 or 16)
+    long long spin_limit;
+};
+
+// SPLIT 0: waves split K (NTW n-tiles per WG); SPLIT 1: waves split N (NTW n-tiles per wave);
+// SPLIT 2: barrier-free small-H form, wave w owns unit tile w (up to 64 units), one n-tile.
+template <typename T, int NTW, int SPLIT>
+__global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    constexpr bool SYNC = SPLIT != 2;
+    constexpr bool ACC = (E::DT == FASTLSTM_FP32);
+    constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;
+    constexpr int P = SPLIT == 0 ? 4 : 1;
+    constexpr int MTB = SPLIT == 2 ? 4 : 1;          // unit tiles (16 rows each) per workgroup
+    constexpr int IPT = SPLIT == 2 ? 4 : NT;         // (unit, batch row) items per thread, upper bound
+    constexpr int BT = 16 * NT;
+    constexpr int CH = 8 / NTW;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int KSB = p.KSB, H = p.H, B = p.B, T_ = p.T;
+    const int HT = SYNC ? p.ht : 16 * MTB;           // unit slots per workgroup
+    const int RPT = SYNC ? p.ht : 16;                // weight rows stored per unit tile
+    const int n_utiles = SYNC ? 1 : cdiv(H, 16);     // unit tiles actually used
+
+    int g, j;
+    if constexpr (SYNC) {
+        const int lin = xcd_major_id(blockIdx.x, gridDim.x);
+        g = lin / p.n_ht;
+        j = lin % p.n_ht;
+    } else {
+        g = blockIdx.x;
+        j = 0;
+    }
+    const int u0 = j * HT;
+    const int b0 = p.b_base + g * BT;
+
+    const size_t wbytes = (size_t)MTB * KSB * 4 * RPT * 16;
+    unsigned char *Wl = smem;
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem + wbytes);                   // [P][MTB][NT][64]
+    unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * MTB * NT * kWave);  // SPLIT 2
+
+    const T *dout = static_cast<const T *>(p.dout);
+    const T *ifgo = static_cast<const T *>(p.ifgo);
+    const T *cell = static_cast<const T *>(p.cell);
+    T *d_ifgo = static_cast<T *>(p.d_ifgo);
+    const T *Wh = static_cast<const T *>(p.Wh);
+
+    // ---- prologue: Wh[:, units] -> LDS, transposed into operand order ------------------
+    {
+        const int Kpad = KSB * E::KSTEP;
+        const int total = Kpad * HT;
+        for (int idx = tid; idx < total; idx += kThreads) {
+            const int ul = idx % HT, k = idx / HT;
+            const int uk = k >> 2, gate = k & 3;
+            T v = E::from_f32(0.f);
+            if (uk < H && u0 + ul < H) v = Wh[((size_t)gate * H + uk) * H + u0 + ul];
+            const int mtile = SYNC ? 0 : (ul >> 4);
+            const int r = SYNC ? ul : (ul & 15);
+            const int ks = k / E::KSTEP, kk = k % E::KSTEP;
+            const size_t off = ((((size_t)mtile * KSB + ks) * 4 + kk / E::EPL) * RPT + r) * 16 +
+                               (kk % E::EPL) * E::BYTES;
+            *reinterpret_cast<T *>(Wl + off) = v;
+        }
+        if constexpr (!SYNC) {
+            for (int idx = tid; idx < 2 * KSB * kWave; idx += kThreads)
+                reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    __syncthreads();
+
+    // ---- per-thread items: it = tid + 256 m -> (row n, unit ul, n-tile nt) --------------
+    float dc_state[IPT], dh_rec[IPT], c1v[IPT];
+    size_t off_h[IPT], off_p[IPT];
+    int xoff[IPT], roff[IPT];
+    bool valid[IPT];
+    const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
+#pragma unroll
+    for (int m = 0; m < IPT; ++m) {
+        const int it = tid + kThreads * m;
+        const int n = it & 15, rest = it >> 4;
+        const int ul = rest % HT, nt = rest / HT;
+        const int unit = u0 + ul, b = b0 + nt * 16 + n;
+        valid[m] = nt < NT && unit < H && b < B;
+        off_h[m] = (size_t)b * H + unit;
+        off_p[m] = (size_t)b * 4 * H + unit;
+        xoff[m] = nt * KSB * kFragBytes + frag_offset<T>(n, unit * 4);
+        const int mtile = ul >> 4, ur = ul & 15;
+        roff[m] = ((mtile * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
+        dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
+        dc_state[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dc)[off_h[m]]) : 0.f;
+        c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
+    }
+
+    const size_t slot_bytes = (size_t)p.n_bt * NT * KSB * kFragBytes;
+    unsigned char *xg = SYNC ? p.xbuf + (size_t)g * NT * KSB * kFragBytes : xl;
+    const size_t xslot = SYNC ? slot_bytes : (size_t)KSB * kFragBytes;
+    int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
+    const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
+
+    // operands of the first step
+    T pre[IPT][4], c0r[IPT], dor[IPT];
+    auto fetch = [&](int t) {
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            const T zero = E::from_f32(0.f);
+            const T *src = ifgo + (size_t)t * B4H + off_p[m];
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) pre[m][gt] = valid[m] ? src[(size_t)gt * H] : zero;
+            c0r[m] = valid[m] ? cell[(size_t)t * BH + off_h[m]] : zero;
+            dor[m] = valid[m] ? dout[(size_t)t * BH + off_h[m]] : zero;
+        }
+    };
+    fetch(T_ - 1);
+
+    for (int s = 0; s < T_; ++s) {
+        const int t = T_ - 1 - s;
+        unsigned char *xw = xg + (size_t)(s & 1) * xslot;
+
+        // ---- point-wise gate backward for this thread's items --------------------------
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            if (valid[m]) {
+                const float si = sigmoidf_<ACC>(E::to_f32(pre[m][0]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(pre[m][1]));
+                const float tg = tanhf_<ACC>(E::to_f32(pre[m][2]));
+                const float so = sigmoidf_<ACC>(E::to_f32(pre[m][3]));
+                const float tc = tanhf_<ACC>(c1v[m]);
+                const float c0 = E::to_f32(c0r[m]);
+                const float dh = dh_rec[m] + E::to_f32(dor[m]);
+                const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
+                const float d_o = dh * tc * so * (1.f - so);
+                const float d_f = dc1 * c0 * sf * (1.f - sf);
+                const float d_i = dc1 * tg * si * (1.f - si);
+                const float d_g = dc1 * si * (1.f - tg * tg);
+                dc_state[m] = dc1 * sf;
+                c1v[m] = c0;  // c_{t-1} is the next step's c_t
+                const T ti = E::from_f32(d_i), tf = E::from_f32(d_f), tgg = E::from_f32(d_g),
+                        to = E::from_f32(d_o);
+                // exchange copy first (critical path): 4 consecutive k = (unit, gate 0..3)
+                T *xd = reinterpret_cast<T *>(xw + xoff[m]);
+                if constexpr (E::BYTES == 2) {
+                    T pk[4] = {ti, tf, tgg, to};
+                    *reinterpret_cast<u32x2 *>(xd) = *reinterpret_cast<u32x2 *>(pk);
+                } else {
+                    T pk[4] = {ti, tf, tgg, to};
+                    *reinterpret_cast<u32x4 *>(xd) = *reinterpret_cast<u32x4 *>(pk);
+                }
+                T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
+                dst[0] = ti;
+                dst[(size_t)H] = tf;
+                dst[(size_t)2 * H] = tgg;
+                dst[(size_t)3 * H] = to;
+            }
+        }
+        if constexpr (SYNC) publish_version(my_flag, s + 1);
+        else __syncthreads();
+
+        // next step's recurrence-independent operands: issue before waiting
+        if (s + 1 < T_) fetch(t - 1);
+
+        if constexpr (SYNC) {
+            if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, g, s);
+            __syncthreads();
+        }
+
+        // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over K = 4H ----
+        f32x4 acc[NTW];
+#pragma unroll
+        for (int i = 0; i < NTW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int kfirst = SPLIT == 0 ? wave : 0, kstride = SPLIT == 0 ? 4 : 1;
+        const int nk = (SPLIT == 2 && wave >= n_utiles) ? 0 : (SPLIT == 0 ? (KSB - wave + 3) / 4 : KSB);
+        const int nt_base = SPLIT == 1 ? wave * NTW : 0;
+        const int mtile = SPLIT == 2 ? wave : 0;
+        const int q = lane >> 4, r = lane & 15;
+        const unsigned char *wrow = Wl + (((size_t)mtile * KSB * 4 + q) * RPT + (r % RPT)) * 16;
+        const unsigned char *xb = xw;
+
+        auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
+#pragma unroll
+            for (int cc = 0; cc < CH; ++cc) {
+                const int ki = ki0 + cc;
+                if (ki < nk) {
+                    const int ks = kfirst + ki * kstride;
+#pragma unroll
+                    for (int i = 0; i < NTW; ++i)
+                        bq[cc][i] = *reinterpret_cast<const u32x4 *>(
+                            xb + ((size_t)((nt_base + i) * KSB + ks) * kWave + lane) * 16);
+                }
+            }
+        };
+        auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
+#pragma unroll
+            for (int cc = 0; cc < CH; ++cc) {
+                const int ki = ki0 + cc;
+                if (ki < nk) {
+                    const int ks = kfirst + ki * kstride;
+                    const u32x4 af = *reinterpret_cast<const u32x4 *>(wrow + (size_t)ks * 4 * RPT * 16);
+#pragma unroll
+                    for (int i = 0; i < NTW; ++i) acc[i] = mfma_kstep<T>(af, bq[cc][i], acc[i]);
+                }
+            }
+        };
+        {
+            u32x4 bqA[CH][NTW], bqB[CH][NTW];
+            const int nchunks = (nk + CH - 1) / CH;
+            if (nchunks > 0) load_b(bqA, 0);
+            for (int ci = 0; ci < nchunks; ci += 2) {
+                if (ci + 1 < nchunks) load_b(bqB, (ci + 1) * CH);
+                compute(bqA, ci * CH);
+                if (ci + 1 < nchunks) {
+                    if (ci + 2 < nchunks) load_b(bqA, (ci + 2) * CH);
+                    compute(bqB, (ci + 1) * CH);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NTW; ++i) {
+            const int pp = SPLIT == 0 ? wave : 0;
+            red[((pp * MTB + mtile) * NT + nt_base + i) * kWave + lane] = acc[i];
+        }
+        __syncthreads();
+        const float *redf = reinterpret_cast<const float *>(red);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            float v = redf[roff[m]];
+#pragma unroll
+            for (int pp = 1; pp < P; ++pp) v += redf[roff[m] + pp * MTB * NT * kWave * 4];
+            dh_rec[m] = v;
+        }
+        // the next iteration's publish (or block barrier) orders these reads before the
+        // next writes to `red`
+    }
+
+    T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
+#pragma unroll
+    for (int m = 0; m < IPT; ++m)
+        if (valid[m]) {
+            dh_out[off_h[m]] = E::from_f32(dh_rec[m]);
+            dc_out[off_h[m]] = E::from_f32(dc_state[m]);
+        }
+}
+
+}  // namespace fastlstm

@@ -1,0 +1,4 @@
+// Persistent forward / reverse kernels, element type _Float16.
+#define REC_T _Float16
+#define REC_SUF f16
+#include "recurrent_inst.inc"

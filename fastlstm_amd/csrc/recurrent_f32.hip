@@ -1,0 +1,4 @@
+// Persistent forward / reverse kernels, element type float.
+#define REC_T float
+#define REC_SUF f32
+#include "recurrent_inst.inc"

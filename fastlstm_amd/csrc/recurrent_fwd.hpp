@@ -1,0 +1,268 @@
+// Persistent forward kernel: the whole time loop of one LSTM layer in one launch.
+//
+// Replaces persistent_fwd_kernel (fastlstm/kernels.py:414-663) and, for H <= 64,
+// fully_fused_persistent_fwd_kernel's barrier-free single-tile form
+// (fastlstm/kernels.py:672-819).  Per step t, for the workgroup's tile of
+// bt batch rows x ht hidden units:
+//     p      = ifgo[t] (holds x_t.Wx^T + b) + h_{t-1} . Wh_slice^T      fp32 accumulate
+//     ifgo[t] <- p rounded to T (kept for the backward pass, kernels.py:631-640)
+//     c      = sigmoid(p_f)*c + sigmoid(p_i)*tanh(p_g)                   c stays in fp32 registers
+//     h      = sigmoid(p_o)*tanh(c);  cell[t+1] <- c, out[t+1] <- h      (kernels.py:647-657)
+//
+// MI355X mapping
+//  * The workgroup's slice of W_h (4*ht rows x H) is copied ONCE into LDS, already in
+//    MFMA operand order, and stays there for all T steps (the reference re-reads it from
+//    L2 every step when H > 128, kernels.py:550-578).
+//  * Rows of an M tile are ordered (unit, gate) so that the 4 accumulator registers of a
+//    lane are exactly i,f,g,o of one (unit, batch row): the gate maths needs no shuffles.
+//  * h_t travels between workgroups through a small double-buffered exchange buffer that
+//    is laid out in MFMA operand order too: a consumer wave fetches a whole 16 x KSTEP
+//    operand block with one fully coalesced 1 KiB load, straight into registers.
+//  * The 4 waves split K (small batch tiles), the batch tiles (large ones) or the W rows
+//    (barrier-free small-H form); partial sums meet in LDS.
+#pragma once
+#include "recurrent_common.hpp"
+
+namespace fastlstm {
+
+struct FwdParams {
+    void *ifgo;        // [T,B,4H]
+    void *out;         // [T+1,B,H]
+    void *cell;        // [T+1,B,H]
+    const void *Wh;    // [4H,H]
+    WsHeader *hdr;
+    int *flags;        // [n_bt][flag_stride]
+    unsigned char *xbuf;  // [2][n_bt][NT][KS] fragment blocks
+    int T, B, H;
+    int b_base;        // first batch row covered by this launch
+    int n_bt, n_ht, flag_stride;
+    int KS;            // k-steps covering H
+    long long spin_limit;
+};
+
+// SPLIT 0: waves split K   (MT m-tiles, NTW n-tiles per WG, 4 partial sums)
+// SPLIT 1: waves split N   (MT m-tiles per WG, NTW n-tiles per wave, 4*NTW per WG)
+// SPLIT 2: waves split M   (MT m-tiles per wave, 4*MT per WG, one n-tile; no cross-WG sync)
+template <typename T, int MT, int NTW, int SPLIT>
+__global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const FwdParams p) {
+    using E = Elem<T>;
+    constexpr bool SYNC = SPLIT != 2;
+    constexpr bool ACC = (E::DT == FASTLSTM_FP32);
+    constexpr int MTT = SPLIT == 2 ? 4 * MT : MT;    // m-tiles per workgroup
+    constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;   // n-tiles per workgroup
+    constexpr int P = SPLIT == 0 ? 4 : 1;            // partial sums per output tile
+    constexpr int TILES = MTT * NT;
+    constexpr int IPT = (TILES + 3) / 4;             // (tile, lane) items per thread
+    constexpr int HT = 4 * MTT, BT = 16 * NT;
+    constexpr int CH = 8 / NTW;                      // k-steps fetched per batch of loads
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, n = lane & 15;
+    const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+
+    int g, j;
+    if constexpr (SYNC) {
+        const int lin = xcd_major_id(blockIdx.x, gridDim.x);
+        g = lin / p.n_ht;
+        j = lin % p.n_ht;
+    } else {
+        g = blockIdx.x;
+        j = 0;
+    }
+    const int u0 = j * HT;                  // first hidden unit of this workgroup
+    const int b0 = p.b_base + g * BT;       // first batch row
+
+    unsigned char *Wl = smem;                                  // [MTT][KS] blocks
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem + (size_t)MTT * KS * kFragBytes);  // [P][TILES][64]
+    unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * TILES * kWave);  // SPLIT 2: [2][KS] blocks
+
+    T *ifgo = static_cast<T *>(p.ifgo);
+    T *out = static_cast<T *>(p.out);
+    T *cell = static_cast<T *>(p.cell);
+    const T *Wh = static_cast<const T *>(p.Wh);
+
+    // ---- prologue 1: W_h slice -> LDS in operand order (zero padded) ----------------
+    {
+        const int chunks_per_row = KS * 4;  // 16-byte chunks along K
+        const int total = MTT * 16 * chunks_per_row;
+        const bool vec = (H % E::EPL) == 0;
+        for (int idx = tid; idx < total; idx += kThreads) {
+            const int row = idx / chunks_per_row, kc = idx % chunks_per_row;
+            const int mt = row >> 4, r = row & 15;
+            const int unit = u0 + mt * 4 + (r >> 2), gate = r & 3;
+            const int k0 = kc * E::EPL;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (unit < H && k0 < H) {
+                const T *src = Wh + ((size_t)gate * H + unit) * H + k0;
+                if (vec) {
+                    v = *reinterpret_cast<const u32x4 *>(src);
+                } else {
+                    T tmp[E::EPL];
+#pragma unroll
+                    for (int e = 0; e < E::EPL; ++e) tmp[e] = (k0 + e < H) ? src[e] : E::from_f32(0.f);
+                    v = *reinterpret_cast<u32x4 *>(tmp);
+                }
+            }
+            const int ks = kc >> 2, qq = kc & 3;
+            *reinterpret_cast<u32x4 *>(Wl + ((size_t)(mt * KS + ks) * kWave + qq * 16 + r) * 16) = v;
+        }
+        if constexpr (!SYNC) {
+            for (int idx = tid; idx < 2 * KS * kWave; idx += kThreads)
+                reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    __syncthreads();
+
+    // ---- per-thread items: (tile = wave + 4m, lane) -> (unit, batch row) -------------
+    float c_state[IPT];
+    size_t off_h[IPT];    // b*H + unit
+    size_t off_p[IPT];    // b*4H + unit
+    int xoff[IPT];        // byte offset of (unit, row) inside one exchange slot of this group
+    bool valid[IPT];
+#pragma unroll
+    for (int m = 0; m < IPT; ++m) {
+        const int tl = wave + 4 * m;
+        const int mt = tl / NT, nt = tl % NT;
+        const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
+        valid[m] = (tl < TILES) && unit < H && b < B;
+        off_h[m] = (size_t)b * H + unit;
+        off_p[m] = (size_t)b * 4 * H + unit;
+        xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
+        c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
+    }
+
+    const size_t slot_bytes = (size_t)p.n_bt * NT * KS * kFragBytes;
+    unsigned char *xg = SYNC ? p.xbuf + (size_t)g * NT * KS * kFragBytes : xl;
+    const size_t xslot = SYNC ? slot_bytes : (size_t)KS * kFragBytes;
+    int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
+    const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
+
+    // ---- prologue 2: publish h_0 (version 1) ------------------------------------------
+#pragma unroll
+    for (int m = 0; m < IPT; ++m)
+        if (valid[m]) *reinterpret_cast<T *>(xg + xoff[m]) = out[off_h[m]];
+    if constexpr (SYNC) publish_version(my_flag, 1);
+    else __syncthreads();
+
+    const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
+
+    for (int t = 0; t < T_; ++t) {
+        // operands that do not depend on the recurrence: fetch before waiting
+        T pre[IPT][4];
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            const T *src = ifgo + (size_t)t * B4H + off_p[m];
+#pragma unroll
+            for (int gt = 0; gt < 4; ++gt) pre[m][gt] = valid[m] ? src[(size_t)gt * H] : E::from_f32(0.f);
+        }
+
+        if constexpr (SYNC) {
+            if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
+            __syncthreads();
+        }
+
+        // ---- acc[mt][i] += Wslice(mt) . h_{t-1}(nt)^T over this wave's k-steps ----------
+        const unsigned char *xb = xg + (size_t)(t & 1) * xslot;
+        f32x4 acc[MT][NTW];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        const int kfirst = SPLIT == 0 ? wave : 0, kstride = SPLIT == 0 ? 4 : 1;
+        const int nk = SPLIT == 0 ? (KS - wave + 3) / 4 : KS;  // k-steps of this wave
+        const int nt_base = SPLIT == 1 ? wave * NTW : 0;
+        const int mt_base = SPLIT == 2 ? wave * MT : 0;
+
+        auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
+#pragma unroll
+            for (int cc = 0; cc < CH; ++cc) {
+                const int ki = ki0 + cc;
+                if (ki < nk) {
+                    const int ks = kfirst + ki * kstride;
+#pragma unroll
+                    for (int i = 0; i < NTW; ++i)
+                        bq[cc][i] = *reinterpret_cast<const u32x4 *>(
+                            xb + ((size_t)((nt_base + i) * KS + ks) * kWave + lane) * 16);
+                }
+            }
+        };
+        auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
+#pragma unroll
+            for (int cc = 0; cc < CH; ++cc) {
+                const int ki = ki0 + cc;
+                if (ki < nk) {
+                    const int ks = kfirst + ki * kstride;
+#pragma unroll
+                    for (int a = 0; a < MT; ++a) {
+                        const u32x4 af = *reinterpret_cast<const u32x4 *>(
+                            Wl + ((size_t)((mt_base + a) * KS + ks) * kWave + lane) * 16);
+#pragma unroll
+                        for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(af, bq[cc][i], acc[a][i]);
+                    }
+                }
+            }
+        };
+        {
+            u32x4 bqA[CH][NTW], bqB[CH][NTW];
+            const int nchunks = (nk + CH - 1) / CH;
+            if (nchunks > 0) load_b(bqA, 0);
+            for (int ci = 0; ci < nchunks; ci += 2) {
+                if (ci + 1 < nchunks) load_b(bqB, (ci + 1) * CH);
+                compute(bqA, ci * CH);
+                if (ci + 1 < nchunks) {
+                    if (ci + 2 < nchunks) load_b(bqA, (ci + 2) * CH);
+                    compute(bqB, (ci + 1) * CH);
+                }
+            }
+        }
+
+        // ---- partial sums -> LDS, then every (tile, lane) item sums its P partials ------
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) {
+                const int tl = (mt_base + a) * NT + nt_base + i;
+                const int pp = SPLIT == 0 ? wave : 0;
+                red[(pp * TILES + tl) * kWave + lane] = acc[a][i];
+            }
+        __syncthreads();
+
+        unsigned char *xn = xg + (size_t)((t + 1) & 1) * xslot;
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            const int tl = wave + 4 * m;
+            if (tl < TILES) {
+                f32x4 s = red[tl * kWave + lane];
+#pragma unroll
+                for (int pp = 1; pp < P; ++pp) s += red[(pp * TILES + tl) * kWave + lane];
+                if (valid[m]) {
+                    const float pi = E::to_f32(pre[m][0]) + s[0];
+                    const float pf = E::to_f32(pre[m][1]) + s[1];
+                    const float pg = E::to_f32(pre[m][2]) + s[2];
+                    const float po = E::to_f32(pre[m][3]) + s[3];
+                    const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
+                    const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
+                    c_state[m] = c1;
+                    const T hT = E::from_f32(h1);
+                    *reinterpret_cast<T *>(xn + xoff[m]) = hT;   // first: it is on the critical path
+                    T *dst = ifgo + (size_t)t * B4H + off_p[m];
+                    dst[0] = E::from_f32(pi);
+                    dst[(size_t)H] = E::from_f32(pf);
+                    dst[(size_t)2 * H] = E::from_f32(pg);
+                    dst[(size_t)3 * H] = E::from_f32(po);
+                    out[(size_t)(t + 1) * BH + off_h[m]] = hT;
+                    cell[(size_t)(t + 1) * BH + off_h[m]] = E::from_f32(c1);
+                }
+            }
+        }
+        if constexpr (SYNC) {
+            if (t + 1 < T_) publish_version(my_flag, t + 2);
+        } else {
+            __syncthreads();
+        }
+    }
+}
+
+}  // namespace fastlstm

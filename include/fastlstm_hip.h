@@ -1,0 +1,132 @@
+/*
+ * libfastlstm_hip.so -- C ABI of the MI355X (gfx950) LSTM forward/backward path.
+ *
+ * The reference (oleicht/FastLSTM) is pure Python and has no FFI of its own:
+ * its boundary for this path is the set of host functions in fastlstm/lstm.py
+ * that launch Triton kernels and cuBLAS GEMMs.  Each entry point below replaces
+ * one of those launch sites; the Python wrappers in fastlstm_amd/lstm.py bind
+ * them with ctypes and keep the reference's Python signatures.
+ *
+ * Conventions
+ *  - every data pointer is a DEVICE pointer owned by the caller, 16-byte
+ *    aligned, densely packed row-major with the shapes given below;
+ *  - `stream` is a hipStream_t passed as void*; every launch is asynchronous
+ *    on it and nothing here synchronises the host;
+ *  - the library never allocates device memory: scratch comes in through the
+ *    `ws` arguments, sized by the *_workspace_bytes / plan calls, and the
+ *    recurrence workspaces must be ZERO-FILLED by the caller before each call
+ *    (the same contract as the reference's zero-initialised sync buffer,
+ *    fastlstm/lstm.py:96-100, 249);
+ *  - return value: 0 on success, a negative fastlstm_status otherwise; argument
+ *    validation happens before the first HIP call, so the error paths can be
+ *    exercised on a machine without a GPU;
+ *  - dtype: element type of all activations/weights (fastlstm_dtype); all
+ *    accumulation is fp32.
+ */
+#ifndef FASTLSTM_HIP_H
+#define FASTLSTM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { FASTLSTM_FP32 = 0, FASTLSTM_FP16 = 1, FASTLSTM_BF16 = 2 } fastlstm_dtype;
+
+typedef enum {
+    FASTLSTM_OK = 0,
+    FASTLSTM_ERR_NULL = -1,      /* a required pointer is NULL */
+    FASTLSTM_ERR_DIM = -2,       /* non-positive or overflowing dimension */
+    FASTLSTM_ERR_DTYPE = -3,     /* dtype not in fastlstm_dtype */
+    FASTLSTM_ERR_ALIGN = -4,     /* pointer not 16-byte aligned */
+    FASTLSTM_ERR_RESIDENCY = -5, /* W_h slice does not fit on chip / grid cannot be co-resident */
+    FASTLSTM_ERR_WORKSPACE = -6, /* workspace smaller than required */
+    FASTLSTM_ERR_HIP = -7,       /* a HIP runtime call failed (no device, launch error) */
+    FASTLSTM_ERR_TIMEOUT = -8    /* a workspace status word reports a barrier time-out */
+} fastlstm_status;
+
+/* Tiling of one recurrent launch.  A workgroup owns `bt` batch rows x `ht`
+ * hidden units (x 4 gates); the `n_htiles` workgroups of one batch tile
+ * exchange h_t (forward) / d_ifgo_t (backward) every timestep and never talk
+ * to other batch tiles.  n_btiles * n_htiles <= num_cus so that every
+ * workgroup is resident while its peers spin (the rule of
+ * fastlstm/configs.py:29-58); a batch that does not fit is processed in
+ * `batch_chunks` sequential launches (fastlstm/kernels.py:514, 663). */
+typedef struct {
+    int num_cus;      /* compute units used for planning */
+    int lds_limit;    /* bytes of LDS one workgroup may use */
+    int bt, ht;       /* batch rows / hidden units per workgroup */
+    int n_btiles;     /* batch tiles per launch */
+    int n_htiles;     /* hidden tiles (= barrier group size); 1 => no cross-CU sync */
+    int batch_chunks; /* sequential launches needed to cover B */
+    int wave_split;   /* 0: waves split K, 1: waves split batch tiles, 2: waves split W rows */
+    int lds_bytes;    /* LDS the kernel will request */
+    size_t ws_bytes;  /* workspace the caller must pass (zero-filled) */
+} fastlstm_plan;
+
+/* Pure host function (no HIP call): the tiling rule for a device with
+ * `num_cus` compute units and `lds_limit` bytes of LDS per workgroup.
+ * backward = 0 plans fastlstm_fwd_persistent, 1 plans fastlstm_bwd_persistent.
+ * Replaces fastlstm/configs.py:29-58, 146-276 (grid sizing + tile pruning). */
+int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int dtype, int backward,
+                      fastlstm_plan *plan);
+
+/* Same, for the current HIP device `device` (queries CU count and LDS size). */
+int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan);
+
+/* K1 -- ifgo[T*B,4H] = x[T*B,I] . Wx[4H,I]^T + (bx + bh).
+ * Replaces torch.addmm(bx + bh, x.view(T*B,-1), Wx.T) at fastlstm/lstm.py:66-68. */
+int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo,
+                       int T, int B, int I, int H, int dtype, void *stream);
+
+/* K2/K3 -- the time loop.  In: ifgo[T,B,4H] holds x.Wx^T+b, out[0]=h_0, cell[0]=c_0.
+ * Out: ifgo overwritten with the full pre-activations, out[1..T]=h_t, cell[1..T]=c_t.
+ * out, cell: [T+1,B,H]; Wh: [4H,H]; ws: zero-filled, plan.ws_bytes (forward plan).
+ * Replaces the persistent_fwd_kernel launch at fastlstm/lstm.py:131-142
+ * (kernel: fastlstm/kernels.py:414-663; H <= 64 takes the single-tile,
+ * barrier-free form of fastlstm/kernels.py:672-819). */
+int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws,
+                            size_t ws_bytes, int T, int B, int H, int dtype, void *stream);
+
+/* K4 -- the reverse time loop.  In: dout[T,B,H]; dh,dc [B,H] hold the gradients
+ * flowing into h_T, c_T; ifgo, cell as written by the forward.  Out: d_ifgo[T,B,4H];
+ * dh, dc overwritten with the gradients of h_0, c_0.  ws: zero-filled,
+ * plan.ws_bytes (backward plan).
+ * Replaces the lstm_persistent_seq_bwd launch at fastlstm/lstm.py:277-290
+ * (kernel: fastlstm/kernels.py:1201-1409). */
+int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo,
+                            const void *cell, void *d_ifgo, const void *Wh, void *ws,
+                            size_t ws_bytes, int T, int B, int H, int dtype, void *stream);
+
+/* K5 -- dx[T*B,I] = d_ifgo[T*B,4H] . Wx[4H,I].   Replaces fastlstm/lstm.py:294. */
+int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H,
+                     int dtype, void *stream);
+
+/* K6-K9 -- dWx[4H,I] = d_ifgo^T . x,  dWh[4H,H] = d_ifgo^T . h[0..T-1],
+ * db[4H] = column sums of d_ifgo; no transposed copy of d_ifgo is made.
+ * h: [T+1,B,H] (only slots 0..T-1 are read).  ws: fastlstm_wgrad_workspace_bytes.
+ * Replaces Wgrad at fastlstm/lstm.py:494-501. */
+int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh,
+                        void *db, void *ws, size_t ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream);
+size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
+
+/* Reads the status word the recurrent kernels leave at the start of their
+ * workspace; `ws_head` points to a HOST copy of the first 64 bytes.
+ * 0 = ok, FASTLSTM_ERR_TIMEOUT = a barrier wait gave up (the kernel still ran
+ * to completion, its results are invalid). */
+int fastlstm_ws_status(const void *ws_head);
+
+/* Upper bound, in 100 MHz ticks, a barrier wait may spin before it gives up
+ * (default 4e8 = 4 s).  Tests lower it to force the time-out path from the host. */
+void fastlstm_set_spin_limit(long long ticks);
+
+const char *fastlstm_strerror(int status);
+const char *fastlstm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTLSTM_HIP_H */
