@@ -1,0 +1,296 @@
+#!/usr/bin/env python3
+"""Benchmark of the LSTM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload B|A|C|D|E] [--no-cpu] [--no-miopen]
+
+A "step" is one pass of the workload's hot path over one batch of synthetic input
+(already resident in HBM).  The default workload is BASELINE.json's headline
+configuration B: single-layer fp16 FORWARD, batch 64, seq_len 512, input = hidden =
+1024 (x ~ N(0,1), h0,c0 ~ N(0,0.1), weights U(+-1/32), seeded).  Prints ONE JSON
+line: metric/value = batch*timesteps per second of that step, plus
+  roofline      for the dominant kernel (the persistent recurrence), measured with HIP
+                events on the launch stream,
+  kernels       per-stage timings (input-projection GEMM, recurrence, and for the
+                forward+backward pass: reverse recurrence, dx GEMM, weight-gradient GEMMs),
+  fwd_bwd       the same workload timed forward+backward (loss = sum(out)),
+  nn_lstm_rocm  torch.nn.LSTM (MIOpen) on the same GPU, same shapes and dtype,
+  cpu_baseline  the CPU oracle (C, OpenMP) on a bounded sample of the same workload,
+  nn_lstm_cpu   torch.nn.LSTM on the host CPU cores on the same sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: dtype, mode, B, T, I, H, layers
+    "A": ("fp32", "fwd_bwd", 16, 128, 256, 256, 1),
+    "B": ("fp16", "fwd", 64, 512, 1024, 1024, 1),
+    "C": ("bf16", "fwd_bwd", 128, 256, 2048, 2048, 1),
+    "D": ("fp16", "fwd_bwd", 256, 1024, 64, 64, 1),
+    "E": ("fp16", "fwd_bwd", 32, 2048, 1024, 1024, 2),
+}
+PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MFMA, published
+HBM_PEAK_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="B", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-miopen", action="store_true", help="skip the nn.LSTM-on-ROCm leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the LSTM recurrence is not sharded across "
+              "GPUs; see DESIGN.md 'How it would shard'); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    import fastlstm_amd.lstm as L
+    from fastlstm_amd import FastLSTM, _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    dname, mode, B, T, I, H, layers = WORKLOADS[args.workload]
+    dt = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}[dname]
+    code = {"fp32": 0, "fp16": 1, "bf16": 2}[dname]
+
+    # ---- synthetic inputs (seeded, generated on the CPU in fp32, then cast) -------------
+    g = torch.Generator().manual_seed(1234 + ord(args.workload) - ord("A"))
+    torch.manual_seed(1234)
+    model = FastLSTM(I, H, num_layers=layers)  # U(+-1/sqrt(H)) init, nn.LSTM order
+    x_cpu = torch.randn(T, B, I, generator=g)
+    if args.workload == "D":
+        x_cpu = torch.rand(T, B, I, generator=g) * 2 - 1
+    h0_cpu = torch.randn(layers, B, H, generator=g) * 0.1 if args.workload == "B" else torch.zeros(layers, B, H)
+    c0_cpu = torch.randn(layers, B, H, generator=g) * 0.1 if args.workload == "B" else torch.zeros(layers, B, H)
+    model = model.to(dev, dt)
+    x = x_cpu.to(dev, dt)
+    h0, c0 = h0_cpu.to(dev, dt), c0_cpu.to(dev, dt)
+
+    def step_fwd():
+        return model(x, (h0, c0))
+
+    def step_fwd_bwd():
+        for p in model.parameters():
+            p.grad = None
+        out, _ = model(x, (h0, c0))
+        out.sum().backward()
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def ev_time(fn, reps=10, warmup=2):
+        """average device time of fn (ms), HIP events on the current (launch) stream"""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / reps
+
+    headline = step_fwd if mode == "fwd" else step_fwd_bwd
+    with torch.enable_grad():
+        ms = timed(headline, args.steps, args.warmup)
+        ms_fwd = ms if mode == "fwd" else timed(step_fwd, args.steps, args.warmup)
+        ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), 2)
+    value = B * T / (ms * 1e-3)
+
+    # ---- per-stage device times through the C ABI (layer-0 shapes) -----------------------
+    stream = torch.cuda.current_stream().cuda_stream
+    Wx, Wh = model.weight_ih_l0.detach(), model.weight_hh_l0.detach()
+    bx, bh = model.bias_ih_l0.detach(), model.bias_hh_l0.detach()
+    ifgo0 = torch.empty(T, B, 4 * H, device=dev, dtype=dt)
+    ifgo = torch.empty_like(ifgo0)
+    out = torch.empty(T + 1, B, H, device=dev, dtype=dt)
+    cell = torch.empty(T + 1, B, H, device=dev, dtype=dt)
+    out[0], cell[0] = h0[0], c0[0]
+    plan_f, plan_b = _lib.Plan(), _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
+    ws_f = torch.zeros(plan_f.ws_bytes, dtype=torch.uint8, device=dev)
+    ws_b = torch.zeros(plan_b.ws_bytes, dtype=torch.uint8, device=dev)
+
+    def k1():
+        _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
+                                          ifgo0.data_ptr(), T, B, I, H, code, stream), "k1")
+
+    def rec_fwd():
+        ifgo.copy_(ifgo0)
+        ws_f.zero_()
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
+                                               ws_f.data_ptr(), ws_f.numel(), T, B, H, code, stream), "fwd")
+
+    def rec_fwd_overhead():
+        ifgo.copy_(ifgo0)
+        ws_f.zero_()
+
+    t_k1 = ev_time(k1)
+    t_rec = ev_time(rec_fwd) - ev_time(rec_fwd_overhead)
+    kernels = {"gemm_ifgo_ms": round(t_k1, 4), "recurrent_fwd_ms": round(t_rec, 4),
+               "recurrent_fwd_us_per_step": round(t_rec * 1e3 / T, 3),
+               "gemm_ifgo_tflops": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12, 2),
+               "gemm_ifgo_frac_of_mfma_peak": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
+               "plan_fwd": plan_f.as_dict(), "plan_bwd": plan_b.as_dict()}
+    torch.cuda.synchronize()
+    _lib.check(lib.fastlstm_ws_status(ws_f[:64].cpu().numpy().tobytes()), "forward barrier status")
+
+    # backward stages
+    dout = torch.ones(T, B, H, device=dev, dtype=dt)
+    d_ifgo = torch.empty_like(ifgo)
+    dh_n = torch.zeros(B, H, device=dev, dtype=dt)
+    dc_n = torch.zeros(B, H, device=dev, dtype=dt)
+    dx = torch.empty(T, B, I, device=dev, dtype=dt)
+    dWx, dWh_, db = torch.empty_like(Wx), torch.empty_like(Wh), torch.empty_like(bx)
+    ws_w = torch.empty(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code), dtype=torch.uint8, device=dev)
+
+    def rec_bwd():
+        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
+        _lib.check(lib.fastlstm_bwd_persistent(dout.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
+                                               cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), ws_b.data_ptr(),
+                                               ws_b.numel(), T, B, H, code, stream), "bwd")
+
+    def rec_bwd_overhead():
+        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
+
+    def k5():
+        _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, stream), "k5")
+
+    def k89():
+        _lib.check(lib.fastlstm_gemm_wgrad(d_ifgo.data_ptr(), x.data_ptr(), out.data_ptr(), dWx.data_ptr(),
+                                           dWh_.data_ptr(), db.data_ptr(), ws_w.data_ptr(), ws_w.numel(), T, B, I, H,
+                                           code, stream), "wgrad")
+
+    t_rb = ev_time(rec_bwd, reps=5) - ev_time(rec_bwd_overhead, reps=5)
+    t_k5 = ev_time(k5, reps=5)
+    t_k89 = ev_time(k89, reps=5)
+    torch.cuda.synchronize()
+    _lib.check(lib.fastlstm_ws_status(ws_b[:64].cpu().numpy().tobytes()), "backward barrier status")
+    kernels.update({
+        "recurrent_bwd_ms": round(t_rb, 4), "recurrent_bwd_us_per_step": round(t_rb * 1e3 / T, 3),
+        "gemm_dx_ms": round(t_k5, 4),
+        "gemm_dx_tflops": round(2.0 * T * B * I * 4 * H / (t_k5 * 1e-3) / 1e12, 2),
+        "gemm_wgrad_ms": round(t_k89, 4),
+        "gemm_wgrad_tflops": round(2.0 * T * B * 4 * H * (I + H) / (t_k89 * 1e-3) / 1e12, 2),
+    })
+
+    # ---- roofline of the dominant kernel: the persistent forward recurrence -------------
+    rec_flops = 2.0 * B * H * 4 * H * T          # algorithmic flops of one launch
+    ach = rec_flops / (t_rec * 1e-3) / 1e12
+    roofline = {"kernel": "lstm_fwd_persistent_kernel", "bound": "mfma", "achieved": round(ach, 2),
+                "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dname], 4),
+                "traffic": None,
+                "note": "latency-bound: T sequential steps, each ends in a cross-CU barrier; see "
+                        "kernels.recurrent_fwd_us_per_step"}
+
+    res = {
+        "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dname, "data": "synthetic",
+        "config": {"workload": "%s: %d-layer LSTM %s %s, B=%d T=%d I=%d H=%d" % (args.workload, layers, dname, mode, B, T, I, H)},
+        "fwd": {"ms": round(ms_fwd, 4), "bt_per_s": round(B * T / (ms_fwd * 1e-3), 1)},
+        "fwd_bwd": {"ms": round(ms_full, 4), "bt_per_s": round(B * T / (ms_full * 1e-3), 1)},
+        "roofline": roofline, "kernels": kernels,
+    }
+
+    # ---- torch.nn.LSTM on the same GPU (MIOpen): the 1.5x target's denominator -----------
+    if not args.no_miopen:
+        try:
+            ref = torch.nn.LSTM(I, H, num_layers=layers).to(dev, dt)
+            with torch.no_grad():
+                for n, p in model.named_parameters():
+                    getattr(ref, n).copy_(p)
+
+            def ref_fwd():
+                return ref(x, (h0, c0))
+
+            def ref_full():
+                for p in ref.parameters():
+                    p.grad = None
+                o, _ = ref(x, (h0, c0))
+                o.sum().backward()
+
+            r_f = timed(ref_fwd, max(3, args.steps // 2), 2)
+            r_b = timed(ref_full, max(3, args.steps // 2), 2)
+            res["nn_lstm_rocm"] = {"fwd_ms": round(r_f, 4), "fwd_bwd_ms": round(r_b, 4),
+                                   "speedup_fwd": round(r_f / ms_fwd, 3), "speedup_fwd_bwd": round(r_b / ms_full, 3)}
+        except Exception as exc:  # MIOpen may not support a configuration
+            res["nn_lstm_rocm"] = {"error": str(exc)[:200]}
+
+    # ---- CPU baselines on a bounded sample (same B, I, H; fewer timesteps) ---------------
+    if not args.no_cpu:
+        from oracle import lstm_oracle as orc
+        import numpy as np
+
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        torch.set_num_threads(cores)
+        Wx_c, Wh_c = model.weight_ih_l0.detach().float().cpu(), model.weight_hh_l0.detach().float().cpu()
+        bx_c, bh_c = model.bias_ih_l0.detach().float().cpu(), model.bias_hh_l0.detach().float().cpu()
+        a = [t.numpy() for t in (Wx_c, bx_c, Wh_c, bh_c)]
+
+        def oracle_run(ts):
+            t0 = time.perf_counter()
+            o, c, p = orc.forward(x_cpu[:ts].numpy(), h0_cpu[0].numpy(), c0_cpu[0].numpy(), a[0], a[1], a[2], a[3],
+                                  dtype=np.float32)
+            if mode == "fwd_bwd":
+                orc.backward(np.ones((ts, B, H), np.float32), None, None, x_cpu[:ts].numpy(), o, c, p, a[0], a[2],
+                             dtype=np.float32)
+            return time.perf_counter() - t0
+
+        probe = min(T, 4)
+        per_step = oracle_run(probe) / probe
+        ts = int(max(probe, min(T, 12.0 / max(per_step, 1e-9))))
+        el = oracle_run(ts)
+        res["cpu_baseline"] = {"value": round(B * ts / el, 1), "unit": "batch*timesteps/s", "cores": cores,
+                               "kind": "port",
+                               "sample": "C/OpenMP fp32 oracle, layer 0, same B/I/H, first %d of %d timesteps, %s (%.1f s)"
+                                         % (ts, T, mode, el)}
+        ref_c = torch.nn.LSTM(I, H)
+        with torch.no_grad():
+            ref_c.weight_ih_l0.copy_(Wx_c); ref_c.weight_hh_l0.copy_(Wh_c)
+            ref_c.bias_ih_l0.copy_(bx_c); ref_c.bias_hh_l0.copy_(bh_c)
+        xs = x_cpu[:ts]
+
+        def cpu_ref():
+            t0 = time.perf_counter()
+            if mode == "fwd":
+                with torch.no_grad():
+                    ref_c(xs, (h0_cpu[:1], c0_cpu[:1]))
+            else:
+                o, _ = ref_c(xs, (h0_cpu[:1], c0_cpu[:1]))
+                o.sum().backward()
+            return time.perf_counter() - t0
+
+        cpu_ref()
+        el2 = min(cpu_ref() for _ in range(2))
+        res["nn_lstm_cpu"] = {"value": round(B * ts / el2, 1), "unit": "batch*timesteps/s", "cores": cores,
+                              "sample": "torch.nn.LSTM fp32 on the host, same sample (%d timesteps, %s)" % (ts, mode)}
+
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -40,11 +40,12 @@ __device__ __forceinline__ void wait_versions(const int *flags, int n, int targe
             ok &= (__hip_atomic_load(flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target);
         if (__all(ok)) break;
         __builtin_amdgcn_s_sleep(1);
-        if (++polls >= 32) {
+        // a spin limit <= 1 means "give up at the first failed poll" (host-forced failure path)
+        if (++polls >= 32 || spin_limit <= 1) {
             polls = 0;
             if (__hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
             const long long now = (long long)wall_clock64();
-            if (t0 == 0) {
+            if (t0 == 0 && spin_limit > 1) {
                 t0 = now;
             } else if (now - t0 > spin_limit) {
                 if (lane == 0) {

@@ -89,8 +89,10 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
     lib = _lib.load()
     with torch.cuda.device(x.device):
         ifgo = torch.empty((seq_len, batch_size, 4 * hidden_size), device=x.device, dtype=x.dtype)
-        out, cell = torch.empty((2, seq_len + 1, batch_size, hidden_size), device=x.device,
-                                dtype=x.dtype).unbind(0)
+        # two allocations (the reference slices one, lstm.py:84-86): each base pointer must
+        # be 16-byte aligned for the vector loads of the weight-gradient GEMM
+        out = torch.empty((seq_len + 1, batch_size, hidden_size), device=x.device, dtype=x.dtype)
+        cell = torch.empty_like(out)
         if h0 is not None:  # fastlstm/lstm.py:88-90
             out[0] = h0
             cell[0] = c0
@@ -193,7 +195,7 @@ class PersistentLSTMfn(torch.autograd.Function):
     def backward(ctx, dh, d_out_cell):
         x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
         if d_out_cell is None:
-            dc_n, dh_n = torch.zeros_like(cell[:2]).unbind(0)
+            dc_n, dh_n = torch.zeros_like(cell[0]), torch.zeros_like(cell[0])
         else:
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
         d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(

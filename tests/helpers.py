@@ -52,6 +52,13 @@ def to_np(p, keys):
     return [None if p[k] is None else p[k].detach().cpu().double().numpy() for k in keys]
 
 
+def _np64(a):
+    if torch.is_tensor(a):
+        a = a.detach().double().cpu().numpy()
+    return np.asarray(a, np.float64)
+
+
 def rel_err(a, b):
-    a = np.asarray(a, np.float64); b = np.asarray(b, np.float64)
+    """max |a - b| / max |b| (error max-norm relative to the reference's max-norm)"""
+    a = _np64(a); b = _np64(b)
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))

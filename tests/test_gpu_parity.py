@@ -1,0 +1,414 @@
+"""GPU parity tests (run with -m gpu on an MI355X).  Everything goes through the C ABI
+of libfastlstm_hip.so via the Python mirror of the reference's interface.
+
+Tolerances (north star): fp32 rtol = atol = 1e-4 against torch.nn.LSTM with identical
+weights; fp16/bf16 <= 2e-2 relative (error max-norm / reference max-norm) against an
+fp32/fp64 evaluation with the same 16-bit-rounded weights and inputs.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import fastlstm_amd.lstm as L
+from fastlstm_amd import FastLSTM, PersistentLSTMfn, _lib
+from helpers import make_problem, nn_lstm_reference, rel_err, to_np
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FP32_TOL = 1e-4
+HALF_TOL = 2e-2
+RM = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+FWD_KEYS = ["x", "h0", "c0", "Wx", "bx", "Wh", "bh"]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu_setup():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    old = L.CHECK_STATUS
+    L.CHECK_STATUS = True  # every recurrent launch is checked for barrier time-outs
+    yield
+    L.CHECK_STATUS = old
+
+
+def npy(t):
+    return t.detach().double().cpu().numpy()
+
+
+def dev(t, dt=None):
+    return None if t is None else (t.to(dt) if dt else t).cuda()
+
+
+def assert_close32(got, want, scale_atol=1.0):
+    want = torch.as_tensor(np.asarray(want)) if not torch.is_tensor(want) else want
+    torch.testing.assert_close(got.detach().cpu().double(), want.double(), rtol=FP32_TOL,
+                               atol=FP32_TOL * scale_atol)
+
+
+# --------------------------------------------------------------------------------------
+# 1. the reference's own integration grid (tests/test_lstm.py:160-220): 2 layers, I = 123,
+#    ragged B and H, fp32, module outputs and every parameter gradient vs nn.LSTM
+# --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("seq_size", [10, 100])
+@pytest.mark.parametrize("batch_size", [4, 44, 100])
+@pytest.mark.parametrize("hidden_size", [16, 65, 257])
+def test_fastlstm_module_vs_nn_lstm(seq_size, batch_size, hidden_size):
+    input_size, num_layers = 123, 2
+    torch.manual_seed(123)
+    m1 = FastLSTM(input_size, hidden_size, num_layers=num_layers, version="persistent").cuda()
+    torch.manual_seed(123)
+    m2 = torch.nn.LSTM(input_size, hidden_size, num_layers=num_layers)  # CPU fp32 oracle
+    x = torch.randn(seq_size, batch_size, input_size)
+    y1, (hn1, cn1) = m1(x.cuda())
+    y2, (hn2, cn2) = m2(x)
+    assert_close32(y1, y2)
+    assert_close32(hn1, hn2)
+    assert_close32(cn1, cn2)
+    assert not hn1.requires_grad and not cn1.requires_grad  # nested tuple => no grad (lstm.py:522)
+    y1.sum().backward()
+    y2.sum().backward()
+    for n, p in m1.named_parameters():
+        ref = getattr(m2, n).grad
+        # gradients are sums over T*B terms: atol scales with their magnitude
+        assert_close32(p.grad, ref, scale_atol=max(1.0, float(ref.abs().max())))
+
+
+# --------------------------------------------------------------------------------------
+# 2. every stage through the C ABI against the CPU oracle, all dtypes, ragged shapes
+# --------------------------------------------------------------------------------------
+STAGE_CASES = [
+    # T, B, I, H, dtype
+    (7, 5, 11, 13, torch.float32),        # tiny, everything ragged, barrier-free form
+    (9, 12, 128, 213, torch.float32),     # the reference's unit-test shape (test_lstm.py:46-69)
+    (5, 33, 70, 300, torch.float32),
+    (6, 20, 64, 64, torch.float16),       # config D's hidden size
+    (6, 20, 40, 72, torch.float16),       # H % 8 == 0 but not a tile multiple
+    (5, 7, 30, 100, torch.bfloat16),      # H % 8 != 0: unaligned rows in every kernel
+    (4, 64, 256, 1024, torch.float16),    # config B tiles
+    (3, 128, 128, 2048, torch.bfloat16),  # config C tiles (waves split the batch)
+    (3, 300, 64, 1024, torch.float16),    # large batch: 64-row tiles, waves split the batch
+    (3, 40, 64, 512, torch.float32),
+]
+
+
+@pytest.mark.parametrize("T,B,I,H,dt", STAGE_CASES)
+def test_stages_vs_oracle(oracle, T, B, I, H, dt):
+    p = make_problem(T, B, I, H, seed=T * 1000 + H)
+    pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}  # rounded inputs
+    g = {k: dev(v, dt) for k, v in p.items()}
+    rm = RM[dt]
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    o_out, o_cell, o_ifgo = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=rm)
+    out, cell, ifgo = L.lstm_persistent_fwd(g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"])
+    assert out.shape == (T + 1, B, H) and cell.shape == (T + 1, B, H) and ifgo.shape == (T, B, 4 * H)
+    assert torch.equal(out[0], g["h0"]) and torch.equal(cell[0], g["c0"])
+    for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
+        assert rel_err(got, want) < tol, name
+    # backward, fed with the GPU's own stored activations so that the stage is isolated
+    dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
+    r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
+    dh_buf, dc_buf = g["dh_n"].clone(), g["dc_n"].clone()
+    d_x, dh0, dc0, dWx, dbx, dWh, dbh = L.lstm_persistent_bwd(g["dout"], dc_buf, dh_buf, g["x"], out, cell, ifgo,
+                                                             g["Wx"], g["Wh"])
+    assert dh0 is dh_buf and dc0 is dc_buf and dbx is dbh  # in-place state grads, shared db (lstm.py:334, 501)
+    for name, got, want in (("dx", d_x, r["dx"]), ("dh0", dh0, r["dh0"]), ("dc0", dc0, r["dc0"]),
+                            ("dWx", dWx, r["dWx"]), ("dWh", dWh, r["dWh"]), ("db", dbx, r["db"])):
+        assert rel_err(got, want) < tol, name
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 4, 3), (130, 260, 70), (257, 123, 515), (512, 1024, 256)])
+def test_gemm_stages_vs_matmul(dt, M, N, K):
+    """K1 (x.Wx^T + b), K5 (d.Wx) and K8/K9 (d^T.x) against float64 matmul; shapes chosen
+    so that T*B = M, 4H = N (K1) etc. hit ragged tiles, unaligned rows and split-K."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(M + N + K)
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    H = max(1, N // 4)
+    T, B, I = 1, M, K
+    x = torch.randn(T, B, I, generator=g).to(dt).cuda()
+    Wx = (torch.randn(4 * H, I, generator=g) * 0.1).to(dt).cuda()
+    bx = torch.randn(4 * H, generator=g).to(dt).cuda()
+    bh = torch.randn(4 * H, generator=g).to(dt).cuda()
+    code = RM[dt]
+    st = torch.cuda.current_stream().cuda_stream
+    ifgo = torch.empty(T, B, 4 * H, dtype=dt, device="cuda")
+    _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), ifgo.data_ptr(),
+                                      T, B, I, H, code, st), "k1")
+    want = x.double().view(B, I) @ Wx.double().T + bx.double() + bh.double()
+    assert rel_err(ifgo.reshape(B, -1), want) < tol
+    d = torch.randn(T, B, 4 * H, generator=g).to(dt).cuda()
+    dx = torch.empty(T, B, I, dtype=dt, device="cuda")
+    _lib.check(lib.fastlstm_gemm_dx(d.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, st), "k5")
+    want = d.double().view(B, -1) @ Wx.double()
+    assert rel_err(dx.reshape(B, I), want) < tol
+    h = torch.randn(T + 1, B, H, generator=g).to(dt).cuda()
+    dbx, dbh, dWx, dWh = L.Wgrad(d, x, h)
+    assert dbx is dbh
+    d2 = d.double().view(B, -1)
+    assert rel_err(dWx, (d2.T @ x.double().view(B, I))) < tol
+    assert rel_err(dWh, (d2.T @ h[:-1].double().view(B, H))) < tol
+    assert rel_err(dbx, d2.sum(0)) < tol
+
+
+def test_gpu_matches_golden_vectors():
+    z = np.load(os.path.join(ROOT, "tests", "golden", "lstm_golden.npz"))
+    for name in ("tiny", "ragged", "nostate", "onestep"):
+        t = lambda k: torch.from_numpy(z["%s/in/%s" % (name, k)]).cuda() if "%s/in/%s" % (name, k) in z.files else None
+        x, h0, c0 = t("x").requires_grad_(True), t("h0"), t("c0")
+        ws = [t(k).requires_grad_(True) for k in ("Wx", "bx", "Wh", "bh")]
+        if h0 is not None:
+            h0.requires_grad_(True); c0.requires_grad_(True)
+        out, (hn, cn) = PersistentLSTMfn.apply(x, h0, c0, *ws)
+        assert_close32(out, z[name + "/out/out"])
+        assert_close32(hn, z[name + "/out/h_n"])
+        assert_close32(cn, z[name + "/out/c_n"])
+
+
+# --------------------------------------------------------------------------------------
+# 3. autograd boundary semantics (fastlstm/lstm.py:504-538)
+# --------------------------------------------------------------------------------------
+def test_autograd_function_contract():
+    T, B, I, H = 6, 5, 9, 20
+    p = make_problem(T, B, I, H, seed=3, dtype=torch.float32)
+    ref = nn_lstm_reference(p, with_state_grads=False, dtype=torch.float32)
+    x = p["x"].cuda().requires_grad_(True)
+    h0, c0 = p["h0"].cuda().requires_grad_(True), p["c0"].cuda().requires_grad_(True)
+    Wx, bx, Wh, bh = (p[k].cuda().requires_grad_(True) for k in ("Wx", "bx", "Wh", "bh"))
+    out, (hn, cn) = PersistentLSTMfn.apply(x, h0, c0, Wx, bx, Wh, bh)
+    assert out.shape == (T, B, H) and hn.shape == (B, H) and cn.shape == (B, H)
+    (out * p["dout"].cuda()).sum().backward()
+    for got, key in ((x.grad, "dx"), (h0.grad, "dh0"), (c0.grad, "dc0"), (Wx.grad, "dWx"), (Wh.grad, "dWh"),
+                     (bx.grad, "dbx"), (bh.grad, "dbh")):
+        assert_close32(got, ref[key], scale_atol=max(1.0, float(ref[key].abs().max())))
+    # h_0 = None: no state gradients, zeros initial state (lstm.py:535-537)
+    x2 = p["x"].cuda().requires_grad_(True)
+    out2, _ = PersistentLSTMfn.apply(x2, None, None, Wx, bx, Wh, bh)
+    out0, _ = PersistentLSTMfn.apply(x2, torch.zeros(B, H).cuda(), torch.zeros(B, H).cuda(), Wx, bx, Wh, bh)
+    assert torch.equal(out2, out0)
+    # 2-D input is one timestep (lstm.py:33-34) == nn.LSTMCell
+    o1, (h1, c1) = PersistentLSTMfn.apply(p["x"][0].cuda(), h0, c0, Wx, bx, Wh, bh)
+    cellm = torch.nn.LSTMCell(I, H)
+    with torch.no_grad():
+        cellm.weight_ih.copy_(p["Wx"]); cellm.weight_hh.copy_(p["Wh"]); cellm.bias_ih.copy_(p["bx"]); cellm.bias_hh.copy_(p["bh"])
+        hr, cr = cellm(p["x"][0], (p["h0"], p["c0"]))
+    assert o1.shape == (1, B, H)
+    assert_close32(h1, hr); assert_close32(c1, cr)
+
+
+def test_recurrence_vanishes_with_zero_wh(oracle):
+    T, B, I, H = 5, 20, 32, 96
+    p = make_problem(T, B, I, H, seed=5, dtype=torch.float32)
+    p["Wh"] = torch.zeros_like(p["Wh"])
+    out, cell, ifgo = L.lstm_persistent_fwd(*(dev(p[k]) for k in FWD_KEYS))
+    pre = torch.nn.functional.linear(p["x"].double(), p["Wx"].double(), (p["bx"] + p["bh"]).double())
+    assert_close32(ifgo, pre)
+
+
+def test_runs_are_bit_reproducible():
+    T, B, I, H = 12, 48, 64, 320
+    p = make_problem(T, B, I, H, seed=8, dtype=torch.float16)
+    g = {k: dev(v) for k, v in p.items()}
+    res = []
+    for _ in range(2):
+        out, cell, ifgo = L.lstm_persistent_fwd(*(g[k] for k in FWD_KEYS))
+        r = L.lstm_persistent_bwd(g["dout"], g["dc_n"].clone(), g["dh_n"].clone(), g["x"], out, cell, ifgo, g["Wx"], g["Wh"])
+        res.append([out, cell, ifgo, *r])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+
+
+def test_backward_is_linear_in_upstream_gradient():
+    T, B, I, H = 10, 16, 48, 128
+    p = make_problem(T, B, I, H, seed=9, dtype=torch.float32)
+    g = {k: dev(v) for k, v in p.items()}
+    out, cell, ifgo = L.lstm_persistent_fwd(*(g[k] for k in FWD_KEYS))
+    z = lambda: torch.zeros(B, H, device="cuda")
+    a = L.lstm_persistent_bwd(g["dout"], z(), z(), g["x"], out, cell, ifgo, g["Wx"], g["Wh"])
+    b = L.lstm_persistent_bwd(g["dout"] * 2, z(), z(), g["x"], out, cell, ifgo, g["Wx"], g["Wh"])
+    for u, v in zip(a, b):
+        torch.testing.assert_close(v, 2 * u, rtol=1e-5, atol=1e-6)
+
+
+def test_batch_larger_than_one_launch(oracle):
+    """B = 1100 with H = 1024 needs more than one launch of the barrier groups
+    (batch_chunks > 1, kernels.py:514/663 of the reference)."""
+    T, B, I, H = 2, 1100, 16, 1024
+    plan = _lib.Plan()
+    _lib.check(_lib.load().fastlstm_plan_device(0, B, H, 1, 0, plan), "plan")
+    assert plan.batch_chunks > 1
+    p = make_problem(T, B, I, H, seed=12)
+    dt = torch.float16
+    pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}
+    g = {k: dev(v, dt) for k, v in p.items()}
+    o_out, o_cell, _ = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=1)
+    out, cell, ifgo = L.lstm_persistent_fwd(*(g[k] for k in FWD_KEYS))
+    assert rel_err(out, o_out) < HALF_TOL
+    r = oracle.backward(*to_np(pr, ["dout", "dh_n", "dc_n", "x"]), npy(out), npy(cell), npy(ifgo),
+                        *to_np(pr, ["Wx", "Wh"]), round_mode=1)
+    res = L.lstm_persistent_bwd(g["dout"], g["dc_n"].clone(), g["dh_n"].clone(), g["x"], out, cell, ifgo, g["Wx"], g["Wh"])
+    assert rel_err(res[1], r["dh0"]) < HALF_TOL
+    assert rel_err(res[5], r["dWh"]) < HALF_TOL
+
+
+def test_autocast_and_training_step():
+    """Mixed precision as scripts/overfit.py of the reference uses it: fp32 parameters,
+    autocast to bf16 inside the Function (lstm.py:509-515), fp32 gradients back."""
+    torch.manual_seed(0)
+    m = FastLSTM(24, 96).cuda()
+    head = torch.nn.Linear(96, 1).cuda()
+    opt = torch.optim.Adam(list(m.parameters()) + list(head.parameters()), lr=1e-2)
+    x = torch.randn(20, 8, 24).cuda()
+    y = torch.randn(20, 8, 1).cuda()
+    losses = []
+    for _ in range(30):
+        opt.zero_grad()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, (hn, cn) = m(x)
+            assert out.dtype == torch.bfloat16
+            loss = torch.nn.functional.mse_loss(head(out).float(), y)
+        loss.backward()
+        assert m.weight_hh_l0.grad.dtype == torch.float32
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < 0.7 * losses[0], losses
+
+
+def test_barrier_timeout_is_reported_not_hung():
+    """Failure path forced from the host: with a spin limit of one tick a wait that is not
+    satisfied at its first poll gives up, raises the abort flag (which ends every other
+    wait too) and the grid drains; the status word reports it.  The kernel exits normally."""
+    lib = _lib.load()
+    T, B, H, code = 64, 16, 512, 1
+    plan = _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan), "plan")
+    assert plan.n_htiles > 1
+    ifgo = torch.randn(T, B, 4 * H, device="cuda").half()
+    out = torch.zeros(T + 1, B, H, device="cuda").half()
+    cell = torch.zeros(T + 1, B, H, device="cuda").half()
+    Wh = (torch.randn(4 * H, H, device="cuda") * 0.03).half()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        ws = torch.zeros(plan.ws_bytes, dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.clone().data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
+                                               ws.data_ptr(), ws.numel(), T, B, H, code, st), "fwd")
+        torch.cuda.synchronize()  # returns: the grid drained
+        return lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes())
+
+    try:
+        lib.fastlstm_set_spin_limit(1)
+        assert launch() == _lib.ERR_TIMEOUT
+    finally:
+        lib.fastlstm_set_spin_limit(400000000)
+    assert launch() == _lib.OK  # and the next launch is healthy
+    assert torch.isfinite(out.float()).all()
+
+
+# --------------------------------------------------------------------------------------
+# 4. BASELINE.json configurations at their real shapes
+# --------------------------------------------------------------------------------------
+def _module_pair(I, H, layers, dt, seed):
+    torch.manual_seed(seed)
+    m = FastLSTM(I, H, num_layers=layers)
+    ref = torch.nn.LSTM(I, H, num_layers=layers)
+    with torch.no_grad():
+        for n, prm in m.named_parameters():
+            prm.copy_(prm.to(dt).float())        # weights representable in dt
+            getattr(ref, n).copy_(prm)
+    return m.to("cuda", dt), ref
+
+
+def test_config_A_fp32_fwd_bwd_full_size():
+    T, B, I, H = 128, 16, 256, 256
+    m, ref = _module_pair(I, H, 1, torch.float32, 1234)
+    x = torch.randn(T, B, I, generator=torch.Generator().manual_seed(1))
+    xg = x.cuda().requires_grad_(True)
+    xr = x.clone().requires_grad_(True)
+    y, (hn, cn) = m(xg)
+    yr, (hr, cr) = ref(xr)
+    assert_close32(y, yr); assert_close32(hn, hr); assert_close32(cn, cr)
+    y.sum().backward(); yr.sum().backward()
+    assert_close32(xg.grad, xr.grad, scale_atol=max(1.0, float(xr.grad.abs().max())))
+    for n, prm in m.named_parameters():
+        rg = getattr(ref, n).grad
+        assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
+
+
+def test_config_B_fp16_forward_full_size():
+    T, B, I, H = 512, 64, 1024, 1024
+    m, ref = _module_pair(I, H, 1, torch.float16, 1235)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, B, I, generator=g).half().float()
+    h0 = (torch.randn(1, B, H, generator=g) * 0.1).half().float()
+    c0 = (torch.randn(1, B, H, generator=g) * 0.1).half().float()
+    with torch.no_grad():
+        y, (hn, cn) = m(x.cuda().half(), (h0.cuda().half(), c0.cuda().half()))
+        yr, (hr, cr) = ref(x, (h0, c0))
+    assert rel_err(y, yr) < HALF_TOL
+    assert rel_err(hn, hr) < HALF_TOL
+    assert rel_err(cn, cr) < HALF_TOL
+
+
+def test_config_C_bf16_tiles_fwd_bwd():
+    """Config C's tiling (B=128, I=H=2048, bf16) with T cut to 24 so the CPU reference
+    finishes in seconds; the per-step work and every kernel shape are the real ones."""
+    T, B, I, H = 24, 128, 2048, 2048
+    m, ref = _module_pair(I, H, 1, torch.bfloat16, 1236)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, B, I, generator=g).bfloat16().float()
+    dout = torch.randn(T, B, H, generator=g).bfloat16().float()
+    h0 = torch.zeros(1, B, H); c0 = torch.zeros(1, B, H)
+    xg = x.cuda().bfloat16().requires_grad_(True)
+    h0g, c0g = h0.cuda().bfloat16().requires_grad_(True), c0.cuda().bfloat16().requires_grad_(True)
+    y, _ = m(xg, (h0g, c0g))
+    (y.float() * dout.cuda()).sum().backward()
+    xr = x.clone().requires_grad_(True)
+    h0r, c0r = h0.clone().requires_grad_(True), c0.clone().requires_grad_(True)
+    yr, _ = ref(xr, (h0r, c0r))
+    (yr * dout).sum().backward()
+    assert rel_err(y, yr) < HALF_TOL
+    assert rel_err(xg.grad, xr.grad) < HALF_TOL
+    assert rel_err(h0g.grad, h0r.grad) < HALF_TOL
+    assert rel_err(c0g.grad, c0r.grad) < HALF_TOL
+    for n, prm in m.named_parameters():
+        assert rel_err(prm.grad, getattr(ref, n).grad) < HALF_TOL, n
+    assert torch.equal(m.bias_ih_l0.grad, m.bias_hh_l0.grad)
+
+
+def test_config_D_small_hidden_fp16_full_size():
+    """loss = mean(out^2) over 16.7 M elements: the upstream gradient 2*out/N is ~1e-7 and
+    underflows fp16 (any fp16 backward would lose it), so the loss is scaled by 2^20 the
+    way AMP loss scaling does and the fp32 reference's gradients are scaled alike."""
+    T, B, I, H = 1024, 256, 64, 64
+    scale = 2.0 ** 20
+    m, ref = _module_pair(I, H, 1, torch.float16, 1237)
+    x = (torch.rand(T, B, I, generator=torch.Generator().manual_seed(4)) * 2 - 1).half().float()
+    y, _ = m(x.cuda().half())
+    ((y.float() ** 2).mean() * scale).backward()
+    yr, _ = ref(x)
+    ((yr ** 2).mean() * scale).backward()
+    assert rel_err(y, yr) < HALF_TOL
+    for n, prm in m.named_parameters():
+        assert rel_err(prm.grad, getattr(ref, n).grad) < HALF_TOL, n
+
+
+def test_config_E_two_layers_fp16():
+    """Config E (2 stacked layers, B=32, I=H=1024) with T = 256 of its 2048 steps for the
+    CPU reference's sake; 16-bit error growth over the full length is covered by config D."""
+    T, B, I, H = 256, 32, 1024, 1024
+    m, ref = _module_pair(I, H, 2, torch.float16, 1238)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, B, I, generator=g).half().float()
+    dout = torch.randn(T, B, H, generator=g).half().float()
+    y, (hn, cn) = m(x.cuda().half())
+    (y.float() * dout.cuda()).sum().backward()
+    yr, (hr, cr) = ref(x)
+    (yr * dout).sum().backward()
+    assert hn.shape == (2, B, H)
+    assert rel_err(y, yr) < HALF_TOL
+    assert rel_err(cn, cr) < HALF_TOL
+    for n, prm in m.named_parameters():
+        assert rel_err(prm.grad, getattr(ref, n).grad) < HALF_TOL, n
