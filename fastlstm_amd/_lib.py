@@ -39,6 +39,7 @@ SIGNATURES = {
     "fastlstm_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "fastlstm_ws_status": (_i, [_vp]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
+    "fastlstm_set_gemm_trace": (None, [_vp]),
     "fastlstm_strerror": (ctypes.c_char_p, [_i]),
     "fastlstm_version": (ctypes.c_char_p, []),
 }

@@ -80,8 +80,11 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
     p.M = T * B; p.N = 4 * H; p.K = I;
     p.lda = I; p.ldb = I; p.ldc = 4 * H;
     p.splits = 1; p.k_per_split = I;
-    return launch_gemm(dtype, p, false, false, static_cast<hipStream_t>(stream)) == hipSuccess ? FASTLSTM_OK
-                                                                                               : FASTLSTM_ERR_HIP;
+    int tile, splits;
+    gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, false, false, &tile, &splits);
+    return launch_gemm_tiled(dtype, p, false, false, tile, static_cast<hipStream_t>(stream)) == hipSuccess
+               ? FASTLSTM_OK
+               : FASTLSTM_ERR_HIP;
 }
 
 int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
@@ -95,24 +98,28 @@ int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B,
     p.M = T * B; p.N = I; p.K = 4 * H;
     p.lda = 4 * H; p.ldb = I; p.ldc = I;
     p.splits = 1; p.k_per_split = 4 * H;
-    return launch_gemm(dtype, p, false, true, static_cast<hipStream_t>(stream)) == hipSuccess ? FASTLSTM_OK
-                                                                                              : FASTLSTM_ERR_HIP;
+    int tile, splits;
+    gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, true, false, &tile, &splits);
+    return launch_gemm_tiled(dtype, p, false, true, tile, static_cast<hipStream_t>(stream)) == hipSuccess
+               ? FASTLSTM_OK
+               : FASTLSTM_ERR_HIP;
 }
 
-// split-K factor of a weight-gradient product C[M,N] with reduction length K
-static int wgrad_splits(int M, int N, int K, int dtype) {
-    const int tiles = cdiv(M, kBM) * cdiv(N, kBN);
-    if (tiles >= 128) return 1;
-    const int bk = gemm_bk(dtype);
-    int s = std::min(cdiv(512, tiles), std::max(1, K / (4 * bk)));
-    return std::max(1, std::min(s, 1024));
+// tile and split-K factor of a weight-gradient product C[M,N] = A^T.B with reduction length K
+static void wgrad_plan(int M, int N, int K, int dtype, int *tile, int *splits, int *k_per_split) {
+    gemm_plan(dtype, M, N, K, M, N, true, true, true, tile, splits);
+    const int bk = *tile ? 64 : gemm_bk(dtype);
+    *k_per_split = cdiv(cdiv(K, *splits), bk) * bk;
+    *splits = cdiv(K, *k_per_split);
 }
 static int colsum_chunks(int R) { return std::max(1, std::min(256, R / 64)); }
 
 size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
     if (!dtype_ok(dtype) || check_dims(T, B, I, H)) return 0;
     const int K = T * B, M = 4 * H;
-    const int sx = wgrad_splits(M, I, K, dtype), sh = wgrad_splits(M, H, K, dtype);
+    int tile, sx, sh, kps;
+    wgrad_plan(M, I, K, dtype, &tile, &sx, &kps);
+    wgrad_plan(M, H, K, dtype, &tile, &sh, &kps);
     size_t part = std::max(sx > 1 ? (size_t)sx * M * I : 0, sh > 1 ? (size_t)sh * M * H : 0) * sizeof(float);
     size_t cs = (size_t)colsum_chunks(K) * M * sizeof(float);
     return align_up(cs, 256) + align_up(part, 256) + 256;
@@ -141,11 +148,9 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
         p.Cpart = gemm_part;
         p.M = M; p.N = N; p.K = K;
         p.lda = M; p.ldb = N; p.ldc = N;
-        p.splits = wgrad_splits(M, N, K, dtype);
-        const int bk = gemm_bk(dtype);
-        p.k_per_split = cdiv(cdiv(K, p.splits), bk) * bk;
-        p.splits = cdiv(K, p.k_per_split);
-        if (launch_gemm(dtype, p, true, true, s) != hipSuccess) return FASTLSTM_ERR_HIP;
+        int tile;
+        wgrad_plan(M, N, K, dtype, &tile, &p.splits, &p.k_per_split);
+        if (launch_gemm_tiled(dtype, p, true, true, tile, s) != hipSuccess) return FASTLSTM_ERR_HIP;
     }
     return FASTLSTM_OK;
 }
@@ -262,6 +267,8 @@ const char *fastlstm_strerror(int status) {
         default: return "unknown status";
     }
 }
+
+void fastlstm_set_gemm_trace(void *buf) { set_gemm_trace(static_cast<long long *>(buf)); }
 
 const char *fastlstm_version(void) { return "fastlstm_hip 0.1 (gfx950)"; }
 

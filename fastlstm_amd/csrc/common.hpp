@@ -93,6 +93,18 @@ template <bool ACCURATE> __device__ __forceinline__ float tanhf_(float x) {
     }
 }
 
+constexpr int kNumXcd = 8;
+
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by id.  Numbering
+// them XCD-major gives every XCD a contiguous range of logical ids, so that neighbours in
+// the logical order -- the hidden tiles of one batch tile, adjacent C tiles of a GEMM --
+// share an L2.
+__device__ __forceinline__ int xcd_major_id(int bid, int nwg) {
+    const int xcd = bid % kNumXcd, slot = bid / kNumXcd;
+    const int base = nwg / kNumXcd, rem = nwg % kNumXcd;
+    return xcd * base + (xcd < rem ? xcd : rem) + slot;
+}
+
 __host__ __device__ inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 __host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

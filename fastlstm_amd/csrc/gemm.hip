@@ -1,5 +1,6 @@
 // Host launchers for the MFMA GEMM stages (K1, K5, K8, K9) and the db column sum.
 #include "gemm.hpp"
+#include "gemm16.hpp"
 #include "internal.hpp"
 
 namespace fastlstm {
@@ -31,6 +32,39 @@ hipError_t launch_gemm_t(const GemmParams &p, hipStream_t stream) {
     return e;
 }
 
+template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
+    using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
+    static bool attr_set = false;
+    auto kern = gemm16_kernel<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int grid = cdiv(p.M, BM) * cdiv(p.N, BN) * p.splits;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (p.splits > 1) {
+        const size_t total = (size_t)p.M * p.N;
+        const int blocks = (int)std::min<size_t>((total + 255) / 256, 4096);
+        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, p.Cpart,
+                           static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+template <typename T, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+hipError_t launch_gemm16_dt(const GemmParams &p, bool a_km, bool b_km, hipStream_t s) {
+    if (!a_km && !b_km) return launch_gemm16_t<T, false, false, BM, BN, NS, WVM, WVN, KSPT>(p, s);
+    if (!a_km && b_km) return launch_gemm16_t<T, false, true, BM, BN, NS, WVM, WVN, KSPT>(p, s);
+    if (a_km && b_km) return launch_gemm16_t<T, true, true, BM, BN, NS, WVM, WVN, KSPT>(p, s);
+    return hipErrorInvalidValue;
+}
+
 template <typename T> hipError_t launch_gemm_dt(const GemmParams &p, bool a_km, bool b_km, hipStream_t s) {
     if (!a_km && !b_km) return launch_gemm_t<T, false, false>(p, s);
     if (!a_km && b_km) return launch_gemm_t<T, false, true>(p, s);
@@ -59,6 +93,58 @@ hipError_t launch_colsum_t(const void *in, void *out, float *part, int R, int C,
 }
 
 }  // namespace
+
+// The 16-bit fast kernel needs: K range of every split a multiple of 64, 16-byte aligned
+// rows, operands addressable with 32-bit byte offsets.
+bool gemm16_eligible(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km) {
+    if (dtype == FASTLSTM_FP32) return false;
+    if (K % 64 != 0 || lda % 8 != 0 || ldb % 8 != 0) return false;
+    // 32-bit byte offsets, with room for the rows a partial tile reaches past the operand
+    const size_t a_bytes = (size_t)((a_km ? K : M) + 256) * lda * 2, b_bytes = (size_t)((b_km ? K : N) + 256) * ldb * 2;
+    return a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
+}
+
+// Tile edge (256 or 128; 0 = generic kernel) and split-K factor for a product.
+void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km, bool allow_split,
+               int *tile, int *splits) {
+    *splits = 1;
+    if (!gemm16_eligible(dtype, M, N, K, lda, ldb, a_km, b_km)) {
+        *tile = 0;
+        const int tiles = cdiv(M, kBM) * cdiv(N, kBN);
+        if (allow_split && tiles < 128) {
+            const int bk = gemm_bk(dtype);
+            *splits = std::max(1, std::min(std::min(cdiv(512, tiles), std::max(1, K / (4 * bk))), 1024));
+        }
+        return;
+    }
+    const int t256 = cdiv(M, 256) * cdiv(N, 256), t128 = cdiv(M, 128) * cdiv(N, 128);
+    const int max_split = allow_split ? std::max(1, K / 512) : 1;  // >= 8 k-tiles per split
+    if (t256 >= 192) {
+        *tile = 256;
+    } else if (std::min(cdiv(256, t256), max_split) * t256 >= 192) {
+        *tile = 256;
+        *splits = std::min(cdiv(256, t256), max_split);
+    } else {
+        *tile = 128;
+        if (t128 < 192) *splits = std::max(1, std::min(cdiv(512, t128), max_split));
+    }
+}
+
+static long long *g_trace = nullptr;
+void set_gemm_trace(long long *buf) { g_trace = buf; }
+
+hipError_t launch_gemm_tiled(int dtype, const GemmParams &p_in, bool a_km, bool b_km, int tile, hipStream_t s) {
+    GemmParams p = p_in;
+    p.trace = g_trace;
+#define FASTLSTM_TILE_CASE(ID, BM, BN, NS, WVM, WVN, KSPT)                                                  \
+    if (tile == ID)                                                                                         \
+        return dtype == FASTLSTM_FP16 ? launch_gemm16_dt<_Float16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s) \
+                                      : launch_gemm16_dt<__bf16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s);
+    FASTLSTM_TILE_CASE(128, 128, 128, 2, 2, 2, 2)   // 2 workgroups per CU
+    FASTLSTM_TILE_CASE(256, 256, 256, 2, 4, 2, 2)   // 8 waves, 64 x 128 per wave, 2 x 64 KiB stages
+#undef FASTLSTM_TILE_CASE
+    return launch_gemm(dtype, p, a_km, b_km, s);
+}
 
 hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hipStream_t s) {
     switch (dtype) {

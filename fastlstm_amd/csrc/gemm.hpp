@@ -25,6 +25,7 @@ struct GemmParams {
     int M, N, K;
     int lda, ldb, ldc;
     int splits, k_per_split;
+    long long *trace;     // optional: 4 clock stamps per workgroup (diagnostics), else nullptr
 };
 
 constexpr int kBM = 128, kBN = 128;

@@ -14,6 +14,10 @@ hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hip
 hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
                          hipStream_t s);
 int gemm_bk(int dtype);
+void set_gemm_trace(long long *buf);
+void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km, bool allow_split,
+               int *tile, int *splits);
+hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_km, int tile, hipStream_t s);
 
 // one function per element type (separate translation units, compiled in parallel)
 #define FASTLSTM_DECL_REC(SUF)                                                                       \

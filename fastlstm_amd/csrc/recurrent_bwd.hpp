@@ -21,6 +21,8 @@
 // travels between workgroups through a double-buffered exchange buffer in operand
 // order, so the K = 4H contraction reads fully coalesced 1 KiB blocks.
 #pragma once
+#include <type_traits>
+
 #include "recurrent_common.hpp"
 
 namespace fastlstm {
@@ -133,42 +135,52 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
     }
 
-    const size_t slot_bytes = (size_t)p.n_bt * NT * KSB * kFragBytes;
-    unsigned char *xg = SYNC ? p.xbuf + (size_t)g * NT * KSB * kFragBytes : xl;
-    const size_t xslot = SYNC ? slot_bytes : (size_t)KSB * kFragBytes;
+    using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
+    const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KSB * kFragBytes : (unsigned)KSB * kFragBytes;
+    const unsigned xgrp = SYNC ? (unsigned)g * NT * KSB * kFragBytes : 0u;
+    const Xchg xch(SYNC ? p.xbuf : xl, 2 * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
 
-    // operands of the first step
-    T pre[IPT][4], c0r[IPT], dor[IPT];
-    auto fetch = [&](int t) {
+    // Stored activations and dout do not depend on the recurrence.  With a barrier per step
+    // the next step's operands are requested right before the wait; the barrier-free form
+    // keeps PD steps in flight (nothing else in its short step hides an HBM round trip).
+    constexpr int PD = SYNC ? 1 : 4;
+    T pre[PD][IPT][4], c0r[PD][IPT], dor[PD][IPT];
+    auto fetch = [&](int t, T(&dp)[IPT][4], T(&dc0)[IPT], T(&dd)[IPT]) {
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const T zero = E::from_f32(0.f);
             const T *src = ifgo + (size_t)t * B4H + off_p[m];
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) pre[m][gt] = valid[m] ? src[(size_t)gt * H] : zero;
-            c0r[m] = valid[m] ? cell[(size_t)t * BH + off_h[m]] : zero;
-            dor[m] = valid[m] ? dout[(size_t)t * BH + off_h[m]] : zero;
+            for (int gt = 0; gt < 4; ++gt) dp[m][gt] = valid[m] ? src[(size_t)gt * H] : zero;
+            dc0[m] = valid[m] ? cell[(size_t)t * BH + off_h[m]] : zero;
+            dd[m] = valid[m] ? dout[(size_t)t * BH + off_h[m]] : zero;
         }
     };
-    fetch(T_ - 1);
+#pragma unroll
+    for (int u = 0; u < PD; ++u)
+        if (u < T_) fetch(T_ - 1 - u, pre[u], c0r[u], dor[u]);
 
-    for (int s = 0; s < T_; ++s) {
+    for (int s0 = 0; s0 < T_; s0 += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {
+        const int s = s0 + u;
+        if (s >= T_) break;
         const int t = T_ - 1 - s;
-        unsigned char *xw = xg + (size_t)(s & 1) * xslot;
+        const unsigned xw = xgrp + (unsigned)(s & 1) * xslot;
 
         // ---- point-wise gate backward for this thread's items --------------------------
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             if (valid[m]) {
-                const float si = sigmoidf_<ACC>(E::to_f32(pre[m][0]));
-                const float sf = sigmoidf_<ACC>(E::to_f32(pre[m][1]));
-                const float tg = tanhf_<ACC>(E::to_f32(pre[m][2]));
-                const float so = sigmoidf_<ACC>(E::to_f32(pre[m][3]));
+                const float si = sigmoidf_<ACC>(E::to_f32(pre[u][m][0]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(pre[u][m][1]));
+                const float tg = tanhf_<ACC>(E::to_f32(pre[u][m][2]));
+                const float so = sigmoidf_<ACC>(E::to_f32(pre[u][m][3]));
                 const float tc = tanhf_<ACC>(c1v[m]);
-                const float c0 = E::to_f32(c0r[m]);
-                const float dh = dh_rec[m] + E::to_f32(dor[m]);
+                const float c0 = E::to_f32(c0r[u][m]);
+                const float dh = dh_rec[m] + E::to_f32(dor[u][m]);
                 const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
                 const float d_o = dh * tc * so * (1.f - so);
                 const float d_f = dc1 * c0 * sf * (1.f - sf);
@@ -179,14 +191,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 const T ti = E::from_f32(d_i), tf = E::from_f32(d_f), tgg = E::from_f32(d_g),
                         to = E::from_f32(d_o);
                 // exchange copy first (critical path): 4 consecutive k = (unit, gate 0..3)
-                T *xd = reinterpret_cast<T *>(xw + xoff[m]);
-                if constexpr (E::BYTES == 2) {
-                    T pk[4] = {ti, tf, tgg, to};
-                    *reinterpret_cast<u32x2 *>(xd) = *reinterpret_cast<u32x2 *>(pk);
-                } else {
-                    T pk[4] = {ti, tf, tgg, to};
-                    *reinterpret_cast<u32x4 *>(xd) = *reinterpret_cast<u32x4 *>(pk);
-                }
+                T pk[4] = {ti, tf, tgg, to};
+                if constexpr (E::BYTES == 2) xch.store8(xw + xoff[m], *reinterpret_cast<u32x2 *>(pk));
+                else xch.store16(xw + xoff[m], *reinterpret_cast<u32x4 *>(pk));
                 T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
                 dst[0] = ti;
                 dst[(size_t)H] = tf;
@@ -197,8 +204,8 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         if constexpr (SYNC) publish_version(my_flag, s + 1);
         else __syncthreads();
 
-        // next step's recurrence-independent operands: issue before waiting
-        if (s + 1 < T_) fetch(t - 1);
+        // recurrence-independent operands of a later step: issue before waiting
+        if (s + PD < T_) fetch(t - PD, pre[u], c0r[u], dor[u]);
 
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, g, s);
@@ -215,7 +222,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         const int mtile = SPLIT == 2 ? wave : 0;
         const int q = lane >> 4, r = lane & 15;
         const unsigned char *wrow = Wl + (((size_t)mtile * KSB * 4 + q) * RPT + (r % RPT)) * 16;
-        const unsigned char *xb = xw;
+        const unsigned xb = xw;
 
         auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
 #pragma unroll
@@ -225,8 +232,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                     const int ks = kfirst + ki * kstride;
 #pragma unroll
                     for (int i = 0; i < NTW; ++i)
-                        bq[cc][i] = *reinterpret_cast<const u32x4 *>(
-                            xb + ((size_t)((nt_base + i) * KSB + ks) * kWave + lane) * 16);
+                        bq[cc][i] = xch.load16(xb + (unsigned)(((nt_base + i) * KSB + ks) * kWave + lane) * 16u);
                 }
             }
         };
@@ -271,6 +277,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         }
         // the next iteration's publish (or block barrier) orders these reads before the
         // next writes to `red`
+    }
     }
 
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);

@@ -7,26 +7,67 @@
 // with the number of data versions it has published so far (no read-modify-write,
 // no contention on a shared counter); a consumer polls the n_htiles flags of its
 // group with one coalesced load per poll until all of them reached the version it
-// needs.  Publishing is a device-scope release (L2 write-back), waiting ends in a
-// device-scope acquire (L1/L2 invalidate), because the 8 XCDs of an MI355X have
-// separate L2s.  Every wait is bounded: after `spin_limit` ticks of the 100 MHz
-// clock it raises an abort flag in the workspace header that ends every other
-// wait as well, so the grid always drains.
+// needs.  The 8 XCDs of an MI355X have separate L2s, so everything that crosses
+// workgroups -- the exchange data and the flags -- is written and read with
+// DEVICE-SCOPE accesses (sc1: stores write through to memory, loads miss the
+// non-coherent cache levels).  That keeps the per-step critical path free of whole-L2
+// write-backs and invalidates: a producer drains its own exchange stores
+// (s_waitcnt vmcnt(0)), the workgroup meets at a barrier, one thread raises the flag.
+// Setting kDeviceScopeExchange to false selects plain accesses bracketed by a
+// device-scope release/acquire fence pair instead (L2 write-back + invalidate per step).
+// Every wait is bounded: after `spin_limit` ticks of the 100 MHz clock it raises an
+// abort flag in the workspace header that ends every other wait as well, so the grid
+// always drains.
 #pragma once
 #include "common.hpp"
 
 namespace fastlstm {
 
-constexpr int kNumXcd = 8;
+constexpr bool kDeviceScopeExchange = true;
+constexpr int kAuxDevice = 16;  // buffer-instruction cache policy: sc1 = device scope
 
-// Workgroups are handed to the XCDs round-robin by id.  Number the workgroups
-// XCD-major so that consecutive logical ids -- the hidden tiles of one batch
-// tile -- sit on as few XCDs (L2s) as possible.
-__device__ __forceinline__ int xcd_major_id(int bid, int nwg) {
-    const int xcd = bid % kNumXcd, slot = bid / kNumXcd;
-    const int base = nwg / kNumXcd, rem = nwg % kNumXcd;
-    return xcd * base + (xcd < rem ? xcd : rem) + slot;
-}
+// Exchange buffer in global memory, addressed through a buffer resource so that the
+// 16-byte operand loads can carry the device-scope cache policy.
+struct XchgGlobal {
+    __amdgpu_buffer_rsrc_t rsrc;
+    unsigned char *base;
+    __device__ __forceinline__ XchgGlobal(unsigned char *b, unsigned bytes)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(b, 0, bytes, 0x00020000)), base(b) {}
+    __device__ __forceinline__ u32x4 load16(unsigned off) const {
+        if constexpr (kDeviceScopeExchange) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAuxDevice);
+        else return *reinterpret_cast<const u32x4 *>(base + off);
+    }
+    template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
+        if constexpr (!kDeviceScopeExchange) {
+            *reinterpret_cast<T *>(base + off) = v;
+        } else if constexpr (sizeof(T) == 2) {
+            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rsrc, off, 0, kAuxDevice);
+        } else {
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc, off, 0, kAuxDevice);
+        }
+    }
+    __device__ __forceinline__ void store8(unsigned off, u32x2 v) const {
+        if constexpr (kDeviceScopeExchange) __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, off, 0, kAuxDevice);
+        else *reinterpret_cast<u32x2 *>(base + off) = v;
+    }
+    __device__ __forceinline__ void store16(unsigned off, u32x4 v) const {
+        if constexpr (kDeviceScopeExchange) __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, 0, kAuxDevice);
+        else *reinterpret_cast<u32x4 *>(base + off) = v;
+    }
+};
+
+// Same interface over LDS (barrier-free small-H kernels: the exchange never leaves the CU).
+struct XchgLds {
+    unsigned char *base;
+    __device__ __forceinline__ XchgLds(unsigned char *b, unsigned) : base(b) {}
+    __device__ __forceinline__ u32x4 load16(unsigned off) const { return *reinterpret_cast<const u32x4 *>(base + off); }
+    template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
+        *reinterpret_cast<T *>(base + off) = v;
+    }
+    __device__ __forceinline__ void store8(unsigned off, u32x2 v) const { *reinterpret_cast<u32x2 *>(base + off) = v; }
+    __device__ __forceinline__ void store16(unsigned off, u32x4 v) const { *reinterpret_cast<u32x4 *>(base + off) = v; }
+};
+
 
 // Called by wave 0 of a workgroup.  flags: the n flags of this barrier group.
 __device__ __forceinline__ void wait_versions(const int *flags, int n, int target, WsHeader *hdr,
@@ -57,17 +98,20 @@ __device__ __forceinline__ void wait_versions(const int *flags, int n, int targe
             }
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if constexpr (kDeviceScopeExchange) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only
+    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
 // Called by all threads of the workgroup after they stored the data of `version`.
 __device__ __forceinline__ void publish_version(int *flag, int version) {
-    // every wave drains its own stores to L2 before the workgroup barrier, then
-    // one thread writes L2 back to memory and raises the flag
+    // every wave drains its own (write-through) exchange stores before the workgroup
+    // barrier, then one thread raises the flag
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0)
-        __hip_atomic_store(flag, version, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) {
+        if constexpr (kDeviceScopeExchange) __hip_atomic_store(flag, version, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else __hip_atomic_store(flag, version, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 // Byte offset of element k of matrix row r inside a run of fragment blocks

@@ -21,6 +21,8 @@
 //  * The 4 waves split K (small batch tiles), the batch tiles (large ones) or the W rows
 //    (barrier-free small-H form); partial sums meet in LDS.
 #pragma once
+#include <type_traits>
+
 #include "recurrent_common.hpp"
 
 namespace fastlstm {
@@ -132,30 +134,48 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
     }
 
-    const size_t slot_bytes = (size_t)p.n_bt * NT * KS * kFragBytes;
-    unsigned char *xg = SYNC ? p.xbuf + (size_t)g * NT * KS * kFragBytes : xl;
-    const size_t xslot = SYNC ? slot_bytes : (size_t)KS * kFragBytes;
+    // exchange buffer: [2 slots][batch tile][NT][KS] operand blocks (global) or [2][KS] (LDS)
+    using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
+    const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KS * kFragBytes : (unsigned)KS * kFragBytes;
+    const unsigned xgrp = SYNC ? (unsigned)g * NT * KS * kFragBytes : 0u;
+    const Xchg xch(SYNC ? p.xbuf : xl, 2 * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
 
     // ---- prologue 2: publish h_0 (version 1) ------------------------------------------
 #pragma unroll
     for (int m = 0; m < IPT; ++m)
-        if (valid[m]) *reinterpret_cast<T *>(xg + xoff[m]) = out[off_h[m]];
+        if (valid[m]) xch.store_elem(xgrp + xoff[m], out[off_h[m]]);
     if constexpr (SYNC) publish_version(my_flag, 1);
     else __syncthreads();
 
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 
-    for (int t = 0; t < T_; ++t) {
-        // operands that do not depend on the recurrence: fetch before waiting
-        T pre[IPT][4];
+    // x_t.Wx^T + b does not depend on the recurrence.  With a barrier per step it is fetched
+    // right before the wait (which hides the latency); the barrier-free form keeps PD steps
+    // of it in flight, because nothing else in its ~0.5 us step can hide an HBM round trip.
+    constexpr int PD = SYNC ? 1 : 4;
+    T pre[PD][IPT][4];
+    auto fetch_pre = [&](int t, T(&dst)[IPT][4]) {
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const T *src = ifgo + (size_t)t * B4H + off_p[m];
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) pre[m][gt] = valid[m] ? src[(size_t)gt * H] : E::from_f32(0.f);
+            for (int gt = 0; gt < 4; ++gt) dst[m][gt] = valid[m] ? src[(size_t)gt * H] : E::from_f32(0.f);
         }
+    };
+    if constexpr (!SYNC) {
+#pragma unroll
+        for (int u = 0; u < PD; ++u)
+            if (u < T_) fetch_pre(u, pre[u]);
+    }
+
+    for (int t0 = 0; t0 < T_; t0 += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {
+        const int t = t0 + u;
+        if (t >= T_) break;
+        if constexpr (SYNC) fetch_pre(t, pre[0]);
 
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
@@ -163,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         }
 
         // ---- acc[mt][i] += Wslice(mt) . h_{t-1}(nt)^T over this wave's k-steps ----------
-        const unsigned char *xb = xg + (size_t)(t & 1) * xslot;
+        const unsigned xb = xgrp + (unsigned)(t & 1) * xslot;
         f32x4 acc[MT][NTW];
 #pragma unroll
         for (int a = 0; a < MT; ++a)
@@ -183,8 +203,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                     const int ks = kfirst + ki * kstride;
 #pragma unroll
                     for (int i = 0; i < NTW; ++i)
-                        bq[cc][i] = *reinterpret_cast<const u32x4 *>(
-                            xb + ((size_t)((nt_base + i) * KS + ks) * kWave + lane) * 16);
+                        bq[cc][i] = xch.load16(xb + (unsigned)(((nt_base + i) * KS + ks) * kWave + lane) * 16u);
                 }
             }
         };
@@ -229,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         __syncthreads();
 
-        unsigned char *xn = xg + (size_t)((t + 1) & 1) * xslot;
+        const unsigned xn = xgrp + (unsigned)((t + 1) & 1) * xslot;
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const int tl = wave + 4 * m;
@@ -238,15 +257,15 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
                 for (int pp = 1; pp < P; ++pp) s += red[(pp * TILES + tl) * kWave + lane];
                 if (valid[m]) {
-                    const float pi = E::to_f32(pre[m][0]) + s[0];
-                    const float pf = E::to_f32(pre[m][1]) + s[1];
-                    const float pg = E::to_f32(pre[m][2]) + s[2];
-                    const float po = E::to_f32(pre[m][3]) + s[3];
+                    const float pi = E::to_f32(pre[u][m][0]) + s[0];
+                    const float pf = E::to_f32(pre[u][m][1]) + s[1];
+                    const float pg = E::to_f32(pre[u][m][2]) + s[2];
+                    const float po = E::to_f32(pre[u][m][3]) + s[3];
                     const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
                     const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
                     c_state[m] = c1;
                     const T hT = E::from_f32(h1);
-                    *reinterpret_cast<T *>(xn + xoff[m]) = hT;   // first: it is on the critical path
+                    xch.store_elem(xn + xoff[m], hT);   // first: it is on the critical path
                     T *dst = ifgo + (size_t)t * B4H + off_p[m];
                     dst[0] = E::from_f32(pi);
                     dst[(size_t)H] = E::from_f32(pf);
@@ -260,8 +279,10 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         if constexpr (SYNC) {
             if (t + 1 < T_) publish_version(my_flag, t + 2);
         } else {
+            if (t + PD < T_) fetch_pre(t + PD, pre[u]);
             __syncthreads();
         }
+    }
     }
 }
 

@@ -123,6 +123,11 @@ int fastlstm_ws_status(const void *ws_head);
  * (default 4e8 = 4 s).  Tests lower it to force the time-out path from the host. */
 void fastlstm_set_spin_limit(long long ticks);
 
+/* Diagnostics: when `buf` (device memory, 32 bytes per workgroup of the largest GEMM grid)
+ * is non-NULL the 16-bit GEMM kernels record 4 stamps of the 100 MHz clock per workgroup
+ * (start, main loop entered, main loop left, done).  NULL switches it off (default). */
+void fastlstm_set_gemm_trace(void *buf);
+
 const char *fastlstm_strerror(int status);
 const char *fastlstm_version(void);
 
