@@ -131,8 +131,10 @@ def main():
     plan_f, plan_b = _lib.Plan(), _lib.Plan()
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
-    ws_f = torch.zeros(plan_f.ws_bytes, dtype=torch.uint8, device=dev)
-    ws_b = torch.zeros(plan_b.ws_bytes, dtype=torch.uint8, device=dev)
+    ws_f = torch.zeros(lib.fastlstm_recurrent_workspace_bytes(plan_f, T, H, code, 0), dtype=torch.uint8, device=dev)
+    ws_b = torch.zeros(lib.fastlstm_recurrent_workspace_bytes(plan_b, T, H, code, 1), dtype=torch.uint8, device=dev)
+    zero_f = ws_f if plan_f.ring_needs_zero else ws_f[:plan_f.ws_zero_bytes]   # the part a call needs zeroed
+    zero_b = ws_b if plan_b.ring_needs_zero else ws_b[:plan_b.ws_zero_bytes]
 
     def k1():
         _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
@@ -140,13 +142,13 @@ def main():
 
     def rec_fwd():
         ifgo.copy_(ifgo0)
-        ws_f.zero_()
+        zero_f.zero_()
         _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
                                                ws_f.data_ptr(), ws_f.numel(), T, B, H, code, stream), "fwd")
 
     def rec_fwd_overhead():
         ifgo.copy_(ifgo0)
-        ws_f.zero_()
+        zero_f.zero_()
 
     t_k1 = ev_time(k1)
     t_rec = ev_time(rec_fwd) - ev_time(rec_fwd_overhead)
@@ -168,13 +170,13 @@ def main():
     ws_w = torch.empty(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code), dtype=torch.uint8, device=dev)
 
     def rec_bwd():
-        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
+        zero_b.zero_(); dh_n.zero_(); dc_n.zero_()
         _lib.check(lib.fastlstm_bwd_persistent(dout.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
                                                cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), ws_b.data_ptr(),
                                                ws_b.numel(), T, B, H, code, stream), "bwd")
 
     def rec_bwd_overhead():
-        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
+        zero_b.zero_(); dh_n.zero_(); dc_n.zero_()
 
     def k5():
         _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, stream), "k5")

@@ -21,7 +21,8 @@ class Plan(ctypes.Structure):
     _fields_ = [("num_cus", ctypes.c_int), ("lds_limit", ctypes.c_int), ("bt", ctypes.c_int),
                 ("ht", ctypes.c_int), ("n_btiles", ctypes.c_int), ("n_htiles", ctypes.c_int),
                 ("batch_chunks", ctypes.c_int), ("wave_split", ctypes.c_int),
-                ("lds_bytes", ctypes.c_int), ("ws_bytes", ctypes.c_size_t)]
+                ("lds_bytes", ctypes.c_int), ("ws_bytes", ctypes.c_size_t),
+                ("ws_zero_bytes", ctypes.c_size_t), ("ring_needs_zero", ctypes.c_int)]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}
@@ -31,6 +32,7 @@ _vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 SIGNATURES = {
     "fastlstm_plan_for": (_i, [_i, _i, _i, _i, _i, _i, ctypes.POINTER(Plan)]),
     "fastlstm_plan_device": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(Plan)]),
+    "fastlstm_recurrent_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i, _i]),
     "fastlstm_gemm_ifgo": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
@@ -40,6 +42,7 @@ SIGNATURES = {
     "fastlstm_ws_status": (_i, [_vp]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
     "fastlstm_set_gemm_trace": (None, [_vp]),
+    "fastlstm_set_recurrent_trace": (None, [_vp]),
     "fastlstm_strerror": (ctypes.c_char_p, [_i]),
     "fastlstm_version": (ctypes.c_char_p, []),
 }

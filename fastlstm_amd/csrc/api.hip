@@ -11,6 +11,7 @@ using namespace fastlstm;
 
 namespace fastlstm {
 
+static long long *g_rec_trace = nullptr;
 static std::atomic<long long> g_spin_limit{400000000ll};  // 4 s of the 100 MHz clock
 long long spin_limit_ticks() { return g_spin_limit.load(); }
 
@@ -176,14 +177,23 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
     p.KS = cdiv(H, kstep);
     p.spin_limit = spin_limit_ticks();
+    p.trace = g_rec_trace;
     const int n_bt_total = cdiv(B, pl.bt);
-    const size_t launch_ws = sync ? recurrent_ws_launch_bytes(H, dtype, pl.bt, pl.n_btiles, pl.n_htiles, false) : 0;
+    const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
+    const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, false);
+    if (sync) {  // as many ring slots as the workspace holds, up to one per version
+        const int full = recurrent_full_slots(T, slot_bytes, false);
+        const size_t avail = (ws_bytes - pl.ws_zero_bytes) / pl.batch_chunks / slot_bytes;
+        p.n_slots = (int)std::min<size_t>(full, avail);
+        // cached loads need a never-reused slot per version and 128-byte lines written by one
+        // workgroup only (16-bit tiles of 4 units share their lines with the neighbour tile)
+        p.coherent_loads = (p.n_slots < T + 1 || (dtype != FASTLSTM_FP32 && pl.ht == 4)) ? 1 : 0;
+    }
     FwdLauncher launch = fwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
-        unsigned char *base = wsb + 1024 + (size_t)c * launch_ws;
-        p.flags = reinterpret_cast<int *>(base);
-        p.xbuf = base + align_up((size_t)pl.n_btiles * p.flag_stride * sizeof(int), 1024);
+        p.flags = reinterpret_cast<int *>(wsb + 1024 + (size_t)c * flags_bytes);
+        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
         p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
@@ -222,13 +232,19 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     p.ht = pl.ht;
     p.spin_limit = spin_limit_ticks();
     const int n_bt_total = cdiv(B, pl.bt);
-    const size_t launch_ws = sync ? recurrent_ws_launch_bytes(H, dtype, pl.bt, pl.n_btiles, pl.n_htiles, true) : 0;
+    const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
+    const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, true);
+    if (sync) {
+        const int full = recurrent_full_slots(T, slot_bytes, true);
+        const size_t avail = (ws_bytes - pl.ws_zero_bytes) / pl.batch_chunks / slot_bytes;
+        p.n_slots = (int)std::min<size_t>(full, avail);
+        p.coherent_loads = p.n_slots < T ? 1 : 0;
+    }
     BwdLauncher launch = bwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
-        unsigned char *base = wsb + 1024 + (size_t)c * launch_ws;
-        p.flags = reinterpret_cast<int *>(base);
-        p.xbuf = base + align_up((size_t)pl.n_btiles * p.flag_stride * sizeof(int), 1024);
+        p.flags = reinterpret_cast<int *>(wsb + 1024 + (size_t)c * flags_bytes);
+        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
         p.n_bt = pl.n_btiles;
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
@@ -269,6 +285,7 @@ const char *fastlstm_strerror(int status) {
 }
 
 void fastlstm_set_gemm_trace(void *buf) { set_gemm_trace(static_cast<long long *>(buf)); }
+void fastlstm_set_recurrent_trace(void *buf) { fastlstm::g_rec_trace = static_cast<long long *>(buf); }
 
 const char *fastlstm_version(void) { return "fastlstm_hip 0.1 (gfx950)"; }
 

@@ -32,7 +32,10 @@ FASTLSTM_DECL_REC(bf16)
 
 int fwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
 int bwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
-size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync);
-size_t recurrent_ws_launch_bytes(int H, int dtype, int bt, int n_bt, int n_ht, bool backward);
+size_t recurrent_flags_bytes(int n_bt, int n_ht);
+size_t recurrent_slot_bytes(int H, int dtype, int bt, int n_bt, bool backward);
+size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync,
+                          int slots);
+int recurrent_full_slots(int T, size_t slot_bytes, bool backward);
 
 }  // namespace fastlstm

@@ -39,7 +39,7 @@ int fwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync) {
     const int KS = cdiv(H, kstep_of(dtype));
     const int MT = cdiv(ht, 4), NT = bt / 16;
     const int P = (split == 0) ? 4 : 1;
-    int lds = MT * KS * kFragBytes;        // resident W_h slice
+    int lds = MT * KS * kFragBytes + kFragBytes;  // resident W_h slice + one all-zero operand block
     lds += P * MT * NT * kFragBytes;       // cross-wave reduction / re-layout buffer
     if (!sync) lds += 2 * NT * KS * kFragBytes;  // h exchange stays in LDS
     return lds;
@@ -52,27 +52,38 @@ int bwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync) {
     const int P = (split == 0) ? 4 : 1;
     int lds;
     if (sync) {
-        lds = KSB * ht * 64;  // [kstep][lane group][ht rows][16 B]
+        lds = KSB * ht * 64 + kFragBytes;  // [kstep][lane group][ht rows][16 B] + all-zero block
         lds += P * NT * kFragBytes;
     } else {
         (void)ht;  // the barrier-free kernel always reserves 4 unit tiles (64 units)
-        lds = 4 * KSB * kFragBytes + 4 * NT * kFragBytes + 2 * NT * KSB * kFragBytes;
+        lds = 4 * KSB * kFragBytes + kFragBytes + 4 * NT * kFragBytes + 2 * NT * KSB * kFragBytes;
     }
     return lds;
 }
 
-// Workspace of ONE launch (after the header): flags, then the 2-slot exchange buffer.
-size_t recurrent_ws_launch_bytes(int H, int dtype, int bt, int n_bt, int n_ht, bool backward) {
-    const int KS = backward ? cdiv(4 * H, kstep_of(dtype)) : cdiv(H, kstep_of(dtype));
-    size_t ws = align_up((size_t)n_bt * align_up((size_t)n_ht, 64) * sizeof(int), 1024);  // flags
-    ws += (size_t)2 * n_bt * (bt / 16) * KS * kFragBytes;                                  // exchange
-    return ws;
+// Workspace layout: header (1 KiB) | flags of every batch chunk | exchange ring of every chunk.
+size_t recurrent_flags_bytes(int n_bt, int n_ht) {
+    return align_up((size_t)n_bt * align_up((size_t)n_ht, 64) * sizeof(int), 1024);
 }
-
-size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync) {
+// One ring slot = the exchange data of one timestep of one launch.
+size_t recurrent_slot_bytes(int H, int dtype, int bt, int n_bt, bool backward) {
+    const int KS = backward ? cdiv(4 * H, kstep_of(dtype)) : cdiv(H, kstep_of(dtype));
+    return (size_t)n_bt * (bt / 16) * KS * kFragBytes;
+}
+size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync,
+                          int slots) {
     size_t ws = 1024;  // header (256 B used)
     if (!sync) return ws;
-    return ws + (size_t)chunks * recurrent_ws_launch_bytes(H, dtype, bt, n_bt, n_ht, backward);
+    return ws + (size_t)chunks * (recurrent_flags_bytes(n_bt, n_ht) +
+                                  (size_t)slots * recurrent_slot_bytes(H, dtype, bt, n_bt, backward));
+}
+// Slots of a full history ring (one per exchanged version), capped so that one launch's ring
+// stays addressable with 32-bit offsets and the workspace stays modest.
+int recurrent_full_slots(int T, size_t slot_bytes, bool backward) {
+    const size_t cap = (size_t)1 << 30;
+    const long long want = backward ? T : (long long)T + 1;
+    const long long fit = (long long)(cap / std::max<size_t>(slot_bytes, 1));
+    return (int)std::max<long long>(2, std::min(want, fit));
 }
 
 }  // namespace fastlstm
@@ -113,7 +124,9 @@ extern "C" int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int d
         plan->batch_chunks = 1;
         plan->wave_split = 2;
         plan->lds_bytes = lds;
-        plan->ws_bytes = recurrent_ws_bytes(H, dtype, 16, plan->n_btiles, 1, 1, backward != 0, false);
+        plan->ws_bytes = recurrent_ws_bytes(H, dtype, 16, plan->n_btiles, 1, 1, backward != 0, false, 2);
+        plan->ws_zero_bytes = plan->ws_bytes;
+        plan->ring_needs_zero = 0;
         return FASTLSTM_OK;
     }
 
@@ -166,6 +179,16 @@ extern "C" int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int d
     plan->batch_chunks = best.chunks;
     plan->wave_split = best.split;
     plan->lds_bytes = best.lds;
-    plan->ws_bytes = recurrent_ws_bytes(H, dtype, best.bt, best.n_bt, best.n_ht, best.chunks, backward != 0, true);
+    plan->ws_bytes = recurrent_ws_bytes(H, dtype, best.bt, best.n_bt, best.n_ht, best.chunks, backward != 0, true, 2);
+    plan->ws_zero_bytes = 1024 + (size_t)best.chunks * recurrent_flags_bytes(best.n_bt, best.n_ht);
+    plan->ring_needs_zero = (B % 16 != 0 || K % KSTEP != 0) ? 1 : 0;
     return FASTLSTM_OK;
+}
+
+extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype, int backward) {
+    if (!plan || T <= 0 || H <= 0 || !dtype_ok(dtype)) return 0;
+    if (plan->wave_split == 2) return plan->ws_bytes;
+    const size_t slot = recurrent_slot_bytes(H, dtype, plan->bt, plan->n_btiles, backward != 0);
+    return recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks, backward != 0,
+                              true, recurrent_full_slots(T, slot, backward != 0));
 }

@@ -36,12 +36,14 @@ struct BwdParams {
     const void *Wh;     // [4H,H]
     WsHeader *hdr;
     int *flags;
-    unsigned char *xbuf;   // [2][n_bt][NT][KSB] fragment blocks
+    unsigned char *xbuf;   // [n_slots][n_bt][NT][KSB] operand blocks
     int T, B, H;
     int b_base;
     int n_bt, n_ht, flag_stride;
     int KSB;            // k-steps covering 4H
     int ht;             // hidden units per workgroup (SPLIT 0/1: 4, 8 or 16)
+    int n_slots;        // exchange ring length (T: every step has its own slot)
+    int coherent_loads; // 1: read the exchange data with device-scope loads
     long long spin_limit;
 };
 
@@ -79,8 +81,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     const int b0 = p.b_base + g * BT;
 
     const size_t wbytes = (size_t)MTB * KSB * 4 * RPT * 16;
-    unsigned char *Wl = smem;
-    f32x4 *red = reinterpret_cast<f32x4 *>(smem + wbytes);                   // [P][MTB][NT][64]
+    unsigned char *Wl = smem;                                                // + one all-zero operand block
+    const size_t zero_off = wbytes;
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem + wbytes + kFragBytes);      // [P][MTB][NT][64]
     unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * MTB * NT * kWave);  // SPLIT 2
 
     const T *dout = static_cast<const T *>(p.dout);
@@ -105,6 +108,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                                (kk % E::EPL) * E::BYTES;
             *reinterpret_cast<T *>(Wl + off) = v;
         }
+        if (tid < kWave) reinterpret_cast<u32x4 *>(Wl + zero_off)[tid] = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!SYNC) {
             for (int idx = tid; idx < 2 * KSB * kWave; idx += kThreads)
                 reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
@@ -138,7 +142,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
     const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KSB * kFragBytes : (unsigned)KSB * kFragBytes;
     const unsigned xgrp = SYNC ? (unsigned)g * NT * KSB * kFragBytes : 0u;
-    const Xchg xch(SYNC ? p.xbuf : xl, 2 * xslot);
+    const int n_slots = SYNC ? p.n_slots : 2;
+    const bool coherent = SYNC && p.coherent_loads;
+    const Xchg xch(SYNC ? p.xbuf : xl, (unsigned)n_slots * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
 
@@ -162,15 +168,18 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     for (int u = 0; u < PD; ++u)
         if (u < T_) fetch(T_ - 1 - u, pre[u], c0r[u], dor[u]);
 
+    int slot = 0;  // ring slot of this step's d_ifgo
     for (int s0 = 0; s0 < T_; s0 += PD) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {
         const int s = s0 + u;
         if (s >= T_) break;
         const int t = T_ - 1 - s;
-        const unsigned xw = xgrp + (unsigned)(s & 1) * xslot;
+        const unsigned xw = xgrp + (unsigned)slot * xslot;
+        slot = (slot + 1 == n_slots) ? 0 : slot + 1;
 
         // ---- point-wise gate backward for this thread's items --------------------------
+        T st_d[IPT][4];
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             if (valid[m]) {
@@ -188,21 +197,35 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 const float d_g = dc1 * si * (1.f - tg * tg);
                 dc_state[m] = dc1 * sf;
                 c1v[m] = c0;  // c_{t-1} is the next step's c_t
-                const T ti = E::from_f32(d_i), tf = E::from_f32(d_f), tgg = E::from_f32(d_g),
-                        to = E::from_f32(d_o);
-                // exchange copy first (critical path): 4 consecutive k = (unit, gate 0..3)
-                T pk[4] = {ti, tf, tgg, to};
-                if constexpr (E::BYTES == 2) xch.store8(xw + xoff[m], *reinterpret_cast<u32x2 *>(pk));
-                else xch.store16(xw + xoff[m], *reinterpret_cast<u32x4 *>(pk));
-                T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
-                dst[0] = ti;
-                dst[(size_t)H] = tf;
-                dst[(size_t)2 * H] = tgg;
-                dst[(size_t)3 * H] = to;
+                // exchange copy now (critical path): 4 consecutive k = (unit, gate 0..3); the
+                // copy for the GEMMs is stored after the flag has been raised
+                st_d[m][0] = E::from_f32(d_i);
+                st_d[m][1] = E::from_f32(d_f);
+                st_d[m][2] = E::from_f32(d_g);
+                st_d[m][3] = E::from_f32(d_o);
+                if constexpr (E::BYTES == 2) xch.store8(xw + xoff[m], *reinterpret_cast<u32x2 *>(st_d[m]));
+                else xch.store16(xw + xoff[m], *reinterpret_cast<u32x4 *>(st_d[m]));
             }
         }
-        if constexpr (SYNC) publish_version(my_flag, s + 1);
-        else __syncthreads();
+        auto bulk_store = [&]() {
+#pragma unroll
+            for (int m = 0; m < IPT; ++m) {
+                if (valid[m]) {
+                    T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
+                    dst[0] = st_d[m][0];
+                    dst[(size_t)H] = st_d[m][1];
+                    dst[(size_t)2 * H] = st_d[m][2];
+                    dst[(size_t)3 * H] = st_d[m][3];
+                }
+            }
+        };
+        if constexpr (SYNC) {
+            publish_version(my_flag, s + 1);
+            bulk_store();
+        } else {
+            bulk_store();
+            __syncthreads();
+        }
 
         // recurrence-independent operands of a later step: issue before waiting
         if (s + PD < T_) fetch(t - PD, pre[u], c0r[u], dor[u]);
@@ -224,31 +247,31 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         const unsigned char *wrow = Wl + (((size_t)mtile * KSB * 4 + q) * RPT + (r % RPT)) * 16;
         const unsigned xb = xw;
 
-        auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
+        // straight-line chunks of CH k-steps, no branch inside (see the forward kernel)
+        auto kloop = [&](auto coh) {
+            constexpr bool COH = decltype(coh)::value;
+            auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
 #pragma unroll
-            for (int cc = 0; cc < CH; ++cc) {
-                const int ki = ki0 + cc;
-                if (ki < nk) {
+                for (int cc = 0; cc < CH; ++cc) {
+                    const int ki = min(ki0 + cc, nk - 1);
                     const int ks = kfirst + ki * kstride;
 #pragma unroll
                     for (int i = 0; i < NTW; ++i)
-                        bq[cc][i] = xch.load16(xb + (unsigned)(((nt_base + i) * KSB + ks) * kWave + lane) * 16u);
+                        bq[cc][i] = xch.template load16<COH>(
+                            xb + (unsigned)(((nt_base + i) * KSB + ks) * kWave + lane) * 16u);
                 }
-            }
-        };
-        auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
+            };
+            auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
 #pragma unroll
-            for (int cc = 0; cc < CH; ++cc) {
-                const int ki = ki0 + cc;
-                if (ki < nk) {
+                for (int cc = 0; cc < CH; ++cc) {
+                    const int ki = ki0 + cc;
                     const int ks = kfirst + ki * kstride;
-                    const u32x4 af = *reinterpret_cast<const u32x4 *>(wrow + (size_t)ks * 4 * RPT * 16);
+                    const unsigned char *wp = ki < nk ? wrow + (size_t)ks * 4 * RPT * 16 : Wl + zero_off + lane * 16;
+                    const u32x4 af = *reinterpret_cast<const u32x4 *>(wp);
 #pragma unroll
                     for (int i = 0; i < NTW; ++i) acc[i] = mfma_kstep<T>(af, bq[cc][i], acc[i]);
                 }
-            }
-        };
-        {
+            };
             u32x4 bqA[CH][NTW], bqB[CH][NTW];
             const int nchunks = (nk + CH - 1) / CH;
             if (nchunks > 0) load_b(bqA, 0);
@@ -260,7 +283,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                     compute(bqB, (ci + 1) * CH);
                 }
             }
-        }
+        };
+        if (coherent) kloop(std::true_type{});
+        else kloop(std::false_type{});
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {
             const int pp = SPLIT == 0 ? wave : 0;

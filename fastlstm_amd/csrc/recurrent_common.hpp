@@ -7,12 +7,18 @@
 // with the number of data versions it has published so far (no read-modify-write,
 // no contention on a shared counter); a consumer polls the n_htiles flags of its
 // group with one coalesced load per poll until all of them reached the version it
-// needs.  The 8 XCDs of an MI355X have separate L2s, so everything that crosses
-// workgroups -- the exchange data and the flags -- is written and read with
-// DEVICE-SCOPE accesses (sc1: stores write through to memory, loads miss the
-// non-coherent cache levels).  That keeps the per-step critical path free of whole-L2
-// write-backs and invalidates: a producer drains its own exchange stores
+// needs.  The 8 XCDs of an MI355X have separate L2s, so the exchange data and the
+// flags are WRITTEN with device-scope stores (sc1: write through to memory) and the
+// flags are polled with device-scope loads.  That keeps the per-step critical path free
+// of whole-L2 write-backs and invalidates: a producer drains its own exchange stores
 // (s_waitcnt vmcnt(0)), the workgroup meets at a barrier, one thread raises the flag.
+// The exchange DATA is read in one of two ways:
+//  * history ring (default): every timestep writes a fresh slot of the exchange buffer, so
+//    no cache can hold a stale copy of an address before its only write; consumers use
+//    ordinary cached loads and the 32 CUs of an XCD share one fetch through their L2
+//    (the data crosses the fabric once per XCD instead of once per CU);
+//  * coherent loads (sc1, miss the non-coherent cache levels): used when the workspace is
+//    too small for T+1 slots, or when two workgroups write parts of the same 128-byte line.
 // Setting kDeviceScopeExchange to false selects plain accesses bracketed by a
 // device-scope release/acquire fence pair instead (L2 write-back + invalidate per step).
 // Every wait is bounded: after `spin_limit` ticks of the 100 MHz clock it raises an
@@ -33,9 +39,11 @@ struct XchgGlobal {
     unsigned char *base;
     __device__ __forceinline__ XchgGlobal(unsigned char *b, unsigned bytes)
         : rsrc(__builtin_amdgcn_make_buffer_rsrc(b, 0, bytes, 0x00020000)), base(b) {}
-    __device__ __forceinline__ u32x4 load16(unsigned off) const {
-        if constexpr (kDeviceScopeExchange) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAuxDevice);
-        else return *reinterpret_cast<const u32x4 *>(base + off);
+    // COHERENT: device-scope load (sc1); otherwise an ordinary cached load
+    template <bool COHERENT> __device__ __forceinline__ u32x4 load16(unsigned off) const {
+        if constexpr (!kDeviceScopeExchange) return *reinterpret_cast<const u32x4 *>(base + off);
+        else if constexpr (COHERENT) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAuxDevice);
+        else return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
     }
     template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
         if constexpr (!kDeviceScopeExchange) {
@@ -60,7 +68,9 @@ struct XchgGlobal {
 struct XchgLds {
     unsigned char *base;
     __device__ __forceinline__ XchgLds(unsigned char *b, unsigned) : base(b) {}
-    __device__ __forceinline__ u32x4 load16(unsigned off) const { return *reinterpret_cast<const u32x4 *>(base + off); }
+    template <bool COHERENT> __device__ __forceinline__ u32x4 load16(unsigned off) const {
+        return *reinterpret_cast<const u32x4 *>(base + off);
+    }
     template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
         *reinterpret_cast<T *>(base + off) = v;
     }

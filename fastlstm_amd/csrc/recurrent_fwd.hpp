@@ -34,12 +34,15 @@ struct FwdParams {
     const void *Wh;    // [4H,H]
     WsHeader *hdr;
     int *flags;        // [n_bt][flag_stride]
-    unsigned char *xbuf;  // [2][n_bt][NT][KS] fragment blocks
+    unsigned char *xbuf;  // [n_slots][n_bt][NT][KS] operand blocks
     int T, B, H;
     int b_base;        // first batch row covered by this launch
     int n_bt, n_ht, flag_stride;
     int KS;            // k-steps covering H
+    int n_slots;       // exchange ring length (T+1: every step has its own slot)
+    int coherent_loads;  // 1: read the exchange data with device-scope loads
     long long spin_limit;
+    long long *trace;  // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
 
 // SPLIT 0: waves split K   (MT m-tiles, NTW n-tiles per WG, 4 partial sums)
@@ -75,8 +78,9 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     const int u0 = j * HT;                  // first hidden unit of this workgroup
     const int b0 = p.b_base + g * BT;       // first batch row
 
-    unsigned char *Wl = smem;                                  // [MTT][KS] blocks
-    f32x4 *red = reinterpret_cast<f32x4 *>(smem + (size_t)MTT * KS * kFragBytes);  // [P][TILES][64]
+    unsigned char *Wl = smem;                                  // [MTT][KS] blocks + one all-zero block
+    const unsigned zero_off = (unsigned)MTT * KS * kFragBytes;
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem + zero_off + kFragBytes);  // [P][TILES][64]
     unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * TILES * kWave);  // SPLIT 2: [2][KS] blocks
 
     T *ifgo = static_cast<T *>(p.ifgo);
@@ -109,6 +113,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             const int ks = kc >> 2, qq = kc & 3;
             *reinterpret_cast<u32x4 *>(Wl + ((size_t)(mt * KS + ks) * kWave + qq * 16 + r) * 16) = v;
         }
+        if (tid < kWave) reinterpret_cast<u32x4 *>(Wl + zero_off)[tid] = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!SYNC) {
             for (int idx = tid; idx < 2 * KS * kWave; idx += kThreads)
                 reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
@@ -138,7 +143,9 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
     const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KS * kFragBytes : (unsigned)KS * kFragBytes;
     const unsigned xgrp = SYNC ? (unsigned)g * NT * KS * kFragBytes : 0u;
-    const Xchg xch(SYNC ? p.xbuf : xl, 2 * xslot);
+    const int n_slots = SYNC ? p.n_slots : 2;
+    const bool coherent = SYNC && p.coherent_loads;
+    const Xchg xch(SYNC ? p.xbuf : xl, (unsigned)n_slots * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
 
@@ -170,20 +177,25 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             if (u < T_) fetch_pre(u, pre[u]);
     }
 
+    int slot_r = 0;  // ring slot that holds h_{t-1}
     for (int t0 = 0; t0 < T_; t0 += PD) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {
         const int t = t0 + u;
         if (t >= T_) break;
+        const int slot_w = (slot_r + 1 == n_slots) ? 0 : slot_r + 1;
         if constexpr (SYNC) fetch_pre(t, pre[0]);
+        long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
+        if (p.trace) tr0 = (long long)wall_clock64();
 
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
             __syncthreads();
         }
+        if (p.trace) tr1 = (long long)wall_clock64();
 
         // ---- acc[mt][i] += Wslice(mt) . h_{t-1}(nt)^T over this wave's k-steps ----------
-        const unsigned xb = xgrp + (unsigned)(t & 1) * xslot;
+        const unsigned xb = xgrp + (unsigned)slot_r * xslot;
         f32x4 acc[MT][NTW];
 #pragma unroll
         for (int a = 0; a < MT; ++a)
@@ -195,35 +207,38 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         const int nt_base = SPLIT == 1 ? wave * NTW : 0;
         const int mt_base = SPLIT == 2 ? wave * MT : 0;
 
-        auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
+        // Straight-line chunks of CH k-steps: the operand loads of a chunk are issued back to
+        // back (one round trip for all of them) and there is not a single branch inside: a k-step
+        // past the end of this wave's share re-reads the last valid block and multiplies it with
+        // the all-zero weight block instead.
+        auto kloop = [&](auto coh) {
+            constexpr bool COH = decltype(coh)::value;
+            auto load_b = [&](u32x4(&bq)[CH][NTW], int ki0) {
 #pragma unroll
-            for (int cc = 0; cc < CH; ++cc) {
-                const int ki = ki0 + cc;
-                if (ki < nk) {
+                for (int cc = 0; cc < CH; ++cc) {
+                    const int ki = min(ki0 + cc, nk - 1);
                     const int ks = kfirst + ki * kstride;
 #pragma unroll
                     for (int i = 0; i < NTW; ++i)
-                        bq[cc][i] = xch.load16(xb + (unsigned)(((nt_base + i) * KS + ks) * kWave + lane) * 16u);
+                        bq[cc][i] = xch.template load16<COH>(
+                            xb + (unsigned)(((nt_base + i) * KS + ks) * kWave + lane) * 16u);
                 }
-            }
-        };
-        auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
+            };
+            auto compute = [&](const u32x4(&bq)[CH][NTW], int ki0) {
 #pragma unroll
-            for (int cc = 0; cc < CH; ++cc) {
-                const int ki = ki0 + cc;
-                if (ki < nk) {
+                for (int cc = 0; cc < CH; ++cc) {
+                    const int ki = ki0 + cc;
                     const int ks = kfirst + ki * kstride;
 #pragma unroll
                     for (int a = 0; a < MT; ++a) {
-                        const u32x4 af = *reinterpret_cast<const u32x4 *>(
-                            Wl + ((size_t)((mt_base + a) * KS + ks) * kWave + lane) * 16);
+                        const unsigned woff = ki < nk ? (unsigned)(((mt_base + a) * KS + ks) * kWave + lane) * 16u
+                                                      : zero_off + lane * 16u;
+                        const u32x4 af = *reinterpret_cast<const u32x4 *>(Wl + woff);
 #pragma unroll
                         for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(af, bq[cc][i], acc[a][i]);
                     }
                 }
-            }
-        };
-        {
+            };
             u32x4 bqA[CH][NTW], bqB[CH][NTW];
             const int nchunks = (nk + CH - 1) / CH;
             if (nchunks > 0) load_b(bqA, 0);
@@ -235,8 +250,14 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                     compute(bqB, (ci + 1) * CH);
                 }
             }
-        }
+        };
+        if (coherent) kloop(std::true_type{});
+        else kloop(std::false_type{});
 
+        if (p.trace) {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // attribute the operand fetch to this phase
+            tr2 = (long long)wall_clock64();
+        }
         // ---- partial sums -> LDS, then every (tile, lane) item sums its P partials ------
 #pragma unroll
         for (int a = 0; a < MT; ++a)
@@ -248,7 +269,11 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         __syncthreads();
 
-        const unsigned xn = xgrp + (unsigned)((t + 1) & 1) * xslot;
+        const unsigned xn = xgrp + (unsigned)slot_w * xslot;
+        // Results of this step.  Only the exchange copy of h_t is on the critical path: it is
+        // stored first and alone, the workgroup publishes, and the bulk stores (pre-activations,
+        // c_t, h_t for the caller) are issued after the flag so that nobody waits for them.
+        T st_p[IPT][4], st_h[IPT], st_c[IPT];
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const int tl = wave + 4 * m;
@@ -264,23 +289,46 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                     const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
                     const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
                     c_state[m] = c1;
-                    const T hT = E::from_f32(h1);
-                    xch.store_elem(xn + xoff[m], hT);   // first: it is on the critical path
-                    T *dst = ifgo + (size_t)t * B4H + off_p[m];
-                    dst[0] = E::from_f32(pi);
-                    dst[(size_t)H] = E::from_f32(pf);
-                    dst[(size_t)2 * H] = E::from_f32(pg);
-                    dst[(size_t)3 * H] = E::from_f32(po);
-                    out[(size_t)(t + 1) * BH + off_h[m]] = hT;
-                    cell[(size_t)(t + 1) * BH + off_h[m]] = E::from_f32(c1);
+                    st_h[m] = E::from_f32(h1);
+                    xch.store_elem(xn + xoff[m], st_h[m]);
+                    st_p[m][0] = E::from_f32(pi);
+                    st_p[m][1] = E::from_f32(pf);
+                    st_p[m][2] = E::from_f32(pg);
+                    st_p[m][3] = E::from_f32(po);
+                    st_c[m] = E::from_f32(c1);
                 }
             }
         }
+        if (p.trace) tr3 = (long long)wall_clock64();
+        auto bulk_store = [&]() {
+#pragma unroll
+            for (int m = 0; m < IPT; ++m) {
+                if (valid[m]) {
+                    T *dst = ifgo + (size_t)t * B4H + off_p[m];
+                    dst[0] = st_p[m][0];
+                    dst[(size_t)H] = st_p[m][1];
+                    dst[(size_t)2 * H] = st_p[m][2];
+                    dst[(size_t)3 * H] = st_p[m][3];
+                    out[(size_t)(t + 1) * BH + off_h[m]] = st_h[m];
+                    cell[(size_t)(t + 1) * BH + off_h[m]] = st_c[m];
+                }
+            }
+        };
         if constexpr (SYNC) {
             if (t + 1 < T_) publish_version(my_flag, t + 2);
+            bulk_store();
         } else {
+            bulk_store();
             if (t + PD < T_) fetch_pre(t + PD, pre[u]);
             __syncthreads();
+        }
+        slot_r = slot_w;
+        if (p.trace && tid == 0) {  // accumulated wait / fetch+mfma / reduce+gates / publish times
+            long long *tr = p.trace + (size_t)blockIdx.x * 4;
+            tr[0] += tr1 - tr0;
+            tr[1] += tr2 - tr1;
+            tr[2] += tr3 - tr2;
+            tr[3] += (long long)wall_clock64() - tr3;
         }
     }
     }

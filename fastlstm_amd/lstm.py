@@ -60,6 +60,14 @@ def _plan(device, B, H, code, backward):
     return plan
 
 
+def _workspace(plan, T, H, code, backward, device):
+    """Recurrence workspace: flags + a two-slot exchange buffer, zero-filled (a few hundred KiB).
+    fastlstm_recurrent_workspace_bytes() sizes a one-slot-per-timestep ring instead, which lets
+    the kernels read the exchange data through the caches; on MI355X it measured no faster, so
+    the small workspace is the default."""
+    return torch.zeros(plan.ws_bytes, dtype=torch.uint8, device=device)
+
+
 def _check_ws(ws, what):
     if CHECK_STATUS:
         head = ws[:64].cpu().numpy().tobytes()  # synchronises
@@ -100,7 +108,7 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
             out[0].zero_()
             cell[0].zero_()
         plan = _plan(x.device, batch_size, hidden_size, code, False)
-        ws = torch.zeros(plan.ws_bytes, dtype=torch.uint8, device=x.device)
+        ws = _workspace(plan, seq_len, hidden_size, code, False, x.device)
         stream = _stream()
         _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
                                           ifgo.data_ptr(), seq_len, batch_size, input_size, hidden_size,
@@ -151,7 +159,7 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
         assert dc_n.is_contiguous() and dh_n.is_contiguous()
         d_ifgo = torch.empty_like(ifgo)
         plan = _plan(x.device, batch_size, hidden_size, code, True)
-        ws = torch.zeros(plan.ws_bytes, dtype=torch.uint8, device=x.device)
+        ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
         _lib.check(lib.fastlstm_bwd_persistent(dh.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(),
                                                ifgo.data_ptr(), cell.data_ptr(), d_ifgo.data_ptr(),

@@ -13,10 +13,10 @@
  *  - `stream` is a hipStream_t passed as void*; every launch is asynchronous
  *    on it and nothing here synchronises the host;
  *  - the library never allocates device memory: scratch comes in through the
- *    `ws` arguments, sized by the *_workspace_bytes / plan calls, and the
- *    recurrence workspaces must be ZERO-FILLED by the caller before each call
- *    (the same contract as the reference's zero-initialised sync buffer,
- *    fastlstm/lstm.py:96-100, 249);
+ *    `ws` arguments, sized by the *_workspace_bytes / plan calls; the flag part of a
+ *    recurrence workspace must be ZERO-FILLED by the caller before each call (the same
+ *    contract as the reference's zero-initialised sync buffer, fastlstm/lstm.py:96-100,
+ *    249) -- see fastlstm_recurrent_workspace_bytes;
  *  - return value: 0 on success, a negative fastlstm_status otherwise; argument
  *    validation happens before the first HIP call, so the error paths can be
  *    exercised on a machine without a GPU;
@@ -63,7 +63,9 @@ typedef struct {
     int batch_chunks; /* sequential launches needed to cover B */
     int wave_split;   /* 0: waves split K, 1: waves split batch tiles, 2: waves split W rows */
     int lds_bytes;    /* LDS the kernel will request */
-    size_t ws_bytes;  /* workspace the caller must pass (zero-filled) */
+    size_t ws_bytes;  /* smallest workspace the recurrent call accepts (2 exchange slots) */
+    size_t ws_zero_bytes; /* leading bytes of the workspace that must be zero (header + flags) */
+    int ring_needs_zero;  /* 1: B or H leave padding in the exchange blocks -> zero the whole workspace */
 } fastlstm_plan;
 
 /* Pure host function (no HIP call): the tiling rule for a device with
@@ -76,6 +78,13 @@ int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int dtype, int b
 /* Same, for the current HIP device `device` (queries CU count and LDS size). */
 int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan);
 
+/* Workspace that gives every timestep its own exchange slot (a "history ring" of T+1 forward /
+ * T backward slots, capped at 1 GiB per launch).  With it the exchange data is read through
+ * the caches (one fetch per XCD); with less, down to plan->ws_bytes, the kernels fall back to
+ * cache-bypassing loads.  The first plan->ws_zero_bytes bytes must be zero; the rest only if
+ * plan->ring_needs_zero. */
+size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype, int backward);
+
 /* K1 -- ifgo[T*B,4H] = x[T*B,I] . Wx[4H,I]^T + (bx + bh).
  * Replaces torch.addmm(bx + bh, x.view(T*B,-1), Wx.T) at fastlstm/lstm.py:66-68. */
 int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo,
@@ -83,7 +92,7 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
 
 /* K2/K3 -- the time loop.  In: ifgo[T,B,4H] holds x.Wx^T+b, out[0]=h_0, cell[0]=c_0.
  * Out: ifgo overwritten with the full pre-activations, out[1..T]=h_t, cell[1..T]=c_t.
- * out, cell: [T+1,B,H]; Wh: [4H,H]; ws: zero-filled, plan.ws_bytes (forward plan).
+ * out, cell: [T+1,B,H]; Wh: [4H,H]; ws: see fastlstm_recurrent_workspace_bytes (forward plan).
  * Replaces the persistent_fwd_kernel launch at fastlstm/lstm.py:131-142
  * (kernel: fastlstm/kernels.py:414-663; H <= 64 takes the single-tile,
  * barrier-free form of fastlstm/kernels.py:672-819). */
@@ -92,8 +101,8 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
 
 /* K4 -- the reverse time loop.  In: dout[T,B,H]; dh,dc [B,H] hold the gradients
  * flowing into h_T, c_T; ifgo, cell as written by the forward.  Out: d_ifgo[T,B,4H];
- * dh, dc overwritten with the gradients of h_0, c_0.  ws: zero-filled,
- * plan.ws_bytes (backward plan).
+ * dh, dc overwritten with the gradients of h_0, c_0.  ws: see
+ * fastlstm_recurrent_workspace_bytes (backward plan).
  * Replaces the lstm_persistent_seq_bwd launch at fastlstm/lstm.py:277-290
  * (kernel: fastlstm/kernels.py:1201-1409). */
 int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo,
@@ -127,6 +136,11 @@ void fastlstm_set_spin_limit(long long ticks);
  * is non-NULL the 16-bit GEMM kernels record 4 stamps of the 100 MHz clock per workgroup
  * (start, main loop entered, main loop left, done).  NULL switches it off (default). */
 void fastlstm_set_gemm_trace(void *buf);
+
+/* Diagnostics: when `buf` (zero-filled device memory, 32 bytes per workgroup) is non-NULL the
+ * forward recurrence accumulates, per workgroup and in 100 MHz ticks, the time spent waiting
+ * for its peers, fetching operands + MFMA, reducing + gate maths, and publishing. */
+void fastlstm_set_recurrent_trace(void *buf);
 
 const char *fastlstm_strerror(int status);
 const char *fastlstm_version(void);
