@@ -36,6 +36,9 @@ WORKLOADS = {
 }
 PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the forward recurrence from rocprofv3 FETCH_SIZE + WRITE_SIZE,
+# scaled by a plain copy of known size (profiles/fwd_recurrence_B_pmc.md); None = not measured
+TRAFFIC_BYTES = {"B": 982.0e6}
 
 
 def main():
@@ -46,6 +49,8 @@ def main():
     ap.add_argument("--workload", default="B", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-miopen", action="store_true", help="skip the nn.LSTM-on-ROCm leg")
+    ap.add_argument("--stage", default="all", choices=["all", "fwd_recurrence"],
+                    help="fwd_recurrence: launch only the dominant kernel and a calibration copy (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the LSTM recurrence is not sharded across "
@@ -99,18 +104,22 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / steps
 
-    def ev_time(fn, reps=10, warmup=2):
-        """average device time of fn (ms), HIP events on the current (launch) stream"""
-        for _ in range(warmup):
+    def ev_time(fn, reps=10, warmup=2, pre=None):
+        """average device time (ms) of the launches fn() makes: one HIP event pair per repetition,
+        recorded on the stream the kernels are launched on (torch's current stream); pre() runs
+        outside the timed region."""
+        total = 0.0
+        for i in range(warmup + reps):
+            if pre:
+                pre()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
             fn()
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(reps):
-            fn()
-        e.record()
-        torch.cuda.synchronize()
-        return s.elapsed_time(e) / reps
+            e.record()
+            torch.cuda.synchronize()
+            if i >= warmup:
+                total += s.elapsed_time(e)
+        return total / reps
 
     headline = step_fwd if mode == "fwd" else step_fwd_bwd
     with torch.enable_grad():
@@ -131,27 +140,36 @@ def main():
     plan_f, plan_b = _lib.Plan(), _lib.Plan()
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
-    ws_f = torch.zeros(lib.fastlstm_recurrent_workspace_bytes(plan_f, T, H, code, 0), dtype=torch.uint8, device=dev)
-    ws_b = torch.zeros(lib.fastlstm_recurrent_workspace_bytes(plan_b, T, H, code, 1), dtype=torch.uint8, device=dev)
-    zero_f = ws_f if plan_f.ring_needs_zero else ws_f[:plan_f.ws_zero_bytes]   # the part a call needs zeroed
-    zero_b = ws_b if plan_b.ring_needs_zero else ws_b[:plan_b.ws_zero_bytes]
+    ws_f = torch.zeros(plan_f.ws_bytes, dtype=torch.uint8, device=dev)   # what lstm.py allocates per call
+    ws_b = torch.zeros(plan_b.ws_bytes, dtype=torch.uint8, device=dev)
 
     def k1():
         _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
                                           ifgo0.data_ptr(), T, B, I, H, code, stream), "k1")
 
     def rec_fwd():
-        ifgo.copy_(ifgo0)
-        zero_f.zero_()
         _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
                                                ws_f.data_ptr(), ws_f.numel(), T, B, H, code, stream), "fwd")
 
-    def rec_fwd_overhead():
+    def rec_fwd_pre():  # the kernel overwrites ifgo in place and needs zeroed flags
         ifgo.copy_(ifgo0)
-        zero_f.zero_()
+        ws_f.zero_()
+
+    if args.stage == "fwd_recurrence":
+        # counter runs (rocprofv3 --pmc): the dominant kernel plus a plain copy of known size
+        # (2 x 256 MiB of traffic) that calibrates FETCH_SIZE / WRITE_SIZE
+        k1()
+        cal_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        cal_dst = torch.empty_like(cal_src)
+        for _ in range(3):
+            rec_fwd_pre()
+            rec_fwd()
+            cal_dst.copy_(cal_src)
+        torch.cuda.synchronize()
+        return
 
     t_k1 = ev_time(k1)
-    t_rec = ev_time(rec_fwd) - ev_time(rec_fwd_overhead)
+    t_rec = ev_time(rec_fwd, pre=rec_fwd_pre)
     kernels = {"gemm_ifgo_ms": round(t_k1, 4), "recurrent_fwd_ms": round(t_rec, 4),
                "recurrent_fwd_us_per_step": round(t_rec * 1e3 / T, 3),
                "gemm_ifgo_tflops": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12, 2),
@@ -170,13 +188,12 @@ def main():
     ws_w = torch.empty(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code), dtype=torch.uint8, device=dev)
 
     def rec_bwd():
-        zero_b.zero_(); dh_n.zero_(); dc_n.zero_()
         _lib.check(lib.fastlstm_bwd_persistent(dout.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
                                                cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), ws_b.data_ptr(),
                                                ws_b.numel(), T, B, H, code, stream), "bwd")
 
-    def rec_bwd_overhead():
-        zero_b.zero_(); dh_n.zero_(); dc_n.zero_()
+    def rec_bwd_pre():
+        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
 
     def k5():
         _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, stream), "k5")
@@ -186,7 +203,7 @@ def main():
                                            dWh_.data_ptr(), db.data_ptr(), ws_w.data_ptr(), ws_w.numel(), T, B, I, H,
                                            code, stream), "wgrad")
 
-    t_rb = ev_time(rec_bwd, reps=5) - ev_time(rec_bwd_overhead, reps=5)
+    t_rb = ev_time(rec_bwd, reps=5, pre=rec_bwd_pre)
     t_k5 = ev_time(k5, reps=5)
     t_k89 = ev_time(k89, reps=5)
     torch.cuda.synchronize()
@@ -204,9 +221,11 @@ def main():
     ach = rec_flops / (t_rec * 1e-3) / 1e12
     roofline = {"kernel": "lstm_fwd_persistent_kernel", "bound": "mfma", "achieved": round(ach, 2),
                 "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dname], 4),
-                "traffic": None,
-                "note": "latency-bound: T sequential steps, each ends in a cross-CU barrier; see "
-                        "kernels.recurrent_fwd_us_per_step"}
+                "traffic": TRAFFIC_BYTES.get(args.workload),
+                "algorithmic": "2*B*H*4H*T flop per launch = %.1f GFLOP" % (rec_flops / 1e9),
+                "launch_ms": round(t_rec, 4),
+                "note": "latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange; "
+                        "us/step is in kernels.recurrent_fwd_us_per_step"}
 
     res = {
         "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
@@ -265,11 +284,12 @@ def main():
         probe = min(T, 4)
         per_step = oracle_run(probe) / probe
         ts = int(max(probe, min(T, 12.0 / max(per_step, 1e-9))))
-        el = oracle_run(ts)
+        passes = int(max(1, min(20, 10.0 / max(per_step * ts, 1e-9))))   # ~10 s of CPU work
+        el = sum(oracle_run(ts) for _ in range(passes)) / passes
         res["cpu_baseline"] = {"value": round(B * ts / el, 1), "unit": "batch*timesteps/s", "cores": cores,
                                "kind": "port",
-                               "sample": "C/OpenMP fp32 oracle, layer 0, same B/I/H, first %d of %d timesteps, %s (%.1f s)"
-                                         % (ts, T, mode, el)}
+                               "sample": "C/OpenMP fp32 oracle, layer 0, same B/I/H, first %d of %d timesteps, %s; "
+                                         "mean of %d passes of %.1f s" % (ts, T, mode, passes, el)}
         ref_c = torch.nn.LSTM(I, H)
         with torch.no_grad():
             ref_c.weight_ih_l0.copy_(Wx_c); ref_c.weight_hh_l0.copy_(Wh_c)
