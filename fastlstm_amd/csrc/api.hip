@@ -189,6 +189,14 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         // workgroup only (16-bit tiles of 4 units share their lines with the neighbour tile)
         p.coherent_loads = (p.n_slots < T + 1 || (dtype != FASTLSTM_FP32 && pl.ht == 4)) ? 1 : 0;
     }
+    // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
+    int lds_bytes = pl.lds_bytes;
+    {
+        const int s = elem_bytes(dtype), gseg = pl.ht * s;
+        const int tile_bytes = (pl.bt * (4 * gseg + 16) + 2 * pl.bt * (gseg + 16)) * (sync ? 1 : 2);
+        p.vec_io = (gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && lds_bytes + tile_bytes <= pl.lds_limit) ? 1 : 0;
+        if (p.vec_io) lds_bytes += tile_bytes;
+    }
     FwdLauncher launch = fwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
@@ -198,9 +206,9 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
         int occ = 0;
-        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
-        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, pl.lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
             hipSuccess)
             return FASTLSTM_ERR_HIP;
     }
@@ -231,6 +239,7 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     p.KSB = cdiv(4 * H, kstep);
     p.ht = pl.ht;
     p.spin_limit = spin_limit_ticks();
+    p.trace = g_rec_trace;
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, true);

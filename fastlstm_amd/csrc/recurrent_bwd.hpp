@@ -45,6 +45,7 @@ struct BwdParams {
     int n_slots;        // exchange ring length (T: every step has its own slot)
     int coherent_loads; // 1: read the exchange data with device-scope loads
     long long spin_limit;
+    long long *trace;   // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
 
 // SPLIT 0: waves split K (NTW n-tiles per WG); SPLIT 1: waves split N (NTW n-tiles per wave);
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     constexpr int MTB = SPLIT == 2 ? 4 : 1;          // unit tiles (16 rows each) per workgroup
     constexpr int IPT = SPLIT == 2 ? 4 : NT;         // (unit, batch row) items per thread, upper bound
     constexpr int BT = 16 * NT;
-    constexpr int CH = 8 / NTW;
+    constexpr int CH = 16 / NTW;                     // k-steps fetched per batch of loads (2 batches in flight)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     float dc_state[IPT], dh_rec[IPT], c1v[IPT];
     size_t off_h[IPT], off_p[IPT];
     int xoff[IPT], roff[IPT];
-    bool valid[IPT];
+    bool valid[IPT], pair_lead[IPT];
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 #pragma unroll
     for (int m = 0; m < IPT; ++m) {
@@ -132,6 +133,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         off_h[m] = (size_t)b * H + unit;
         off_p[m] = (size_t)b * 4 * H + unit;
         xoff[m] = nt * KSB * kFragBytes + frag_offset<T>(n, unit * 4);
+        pair_lead[m] = valid[m] && ((ul & 1) == 0);  // u0 is a multiple of 4: even ul <=> low half of a slot
         const int mtile = ul >> 4, ur = ul & 15;
         roff[m] = ((mtile * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
         dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
@@ -178,6 +180,8 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         const unsigned xw = xgrp + (unsigned)slot * xslot;
         slot = (slot + 1 == n_slots) ? 0 : slot + 1;
 
+        long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
+        if (p.trace) tr0 = (long long)wall_clock64();
         // ---- point-wise gate backward for this thread's items --------------------------
         T st_d[IPT][4];
 #pragma unroll
@@ -197,14 +201,27 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 const float d_g = dc1 * si * (1.f - tg * tg);
                 dc_state[m] = dc1 * sf;
                 c1v[m] = c0;  // c_{t-1} is the next step's c_t
-                // exchange copy now (critical path): 4 consecutive k = (unit, gate 0..3); the
-                // copy for the GEMMs is stored after the flag has been raised
                 st_d[m][0] = E::from_f32(d_i);
                 st_d[m][1] = E::from_f32(d_f);
                 st_d[m][2] = E::from_f32(d_g);
                 st_d[m][3] = E::from_f32(d_o);
-                if constexpr (E::BYTES == 2) xch.store8(xw + xoff[m], *reinterpret_cast<u32x2 *>(st_d[m]));
-                else xch.store16(xw + xoff[m], *reinterpret_cast<u32x4 *>(st_d[m]));
+            } else {
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) st_d[m][gt] = E::from_f32(0.f);
+            }
+            // Exchange copy now (critical path): 4 consecutive k = (unit, gate 0..3); the copy for
+            // the GEMMs is stored after the flag has been raised.  A 16-byte operand slot holds two
+            // units of the 16-bit types: lanes l and l+16 own units u and u+1 of the same batch row,
+            // so the even-unit lane fetches its neighbour's half and writes the whole slot -- the
+            // write-through stores then cover full 32-byte sectors instead of halves.
+            if constexpr (E::BYTES == 2) {
+                const u32x2 mine = *reinterpret_cast<u32x2 *>(st_d[m]);
+                u32x2 other;
+                other[0] = (unsigned)__shfl_down((int)mine[0], 16);
+                other[1] = (unsigned)__shfl_down((int)mine[1], 16);
+                if (pair_lead[m]) xch.store16(xw + xoff[m], u32x4{mine[0], mine[1], other[0], other[1]});
+            } else {
+                if (valid[m]) xch.store16(xw + xoff[m], *reinterpret_cast<u32x4 *>(st_d[m]));
             }
         }
         auto bulk_store = [&]() {
@@ -221,6 +238,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         };
         if constexpr (SYNC) {
             publish_version(my_flag, s + 1);
+            if (p.trace) tr1 = (long long)wall_clock64();
             bulk_store();
         } else {
             bulk_store();
@@ -230,10 +248,12 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         // recurrence-independent operands of a later step: issue before waiting
         if (s + PD < T_) fetch(t - PD, pre[u], c0r[u], dor[u]);
 
+        if (p.trace) tr2 = (long long)wall_clock64();
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, g, s);
             __syncthreads();
         }
+        if (p.trace) tr3 = (long long)wall_clock64();
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over K = 4H ----
         f32x4 acc[NTW];
@@ -299,6 +319,13 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
 #pragma unroll
             for (int pp = 1; pp < P; ++pp) v += redf[roff[m] + pp * MTB * NT * kWave * 4];
             dh_rec[m] = v;
+        }
+        if (p.trace && tid == 0) {  // accumulated gate maths / publish+stores / wait / fetch+mfma+reduce
+            long long *tr = p.trace + (size_t)blockIdx.x * 4;
+            tr[0] += tr1 - tr0;
+            tr[1] += tr2 - tr1;
+            tr[2] += tr3 - tr2;
+            tr[3] += (long long)wall_clock64() - tr3;
         }
         // the next iteration's publish (or block barrier) orders these reads before the
         // next writes to `red`

@@ -41,6 +41,7 @@ struct FwdParams {
     int KS;            // k-steps covering H
     int n_slots;       // exchange ring length (T+1: every step has its own slot)
     int coherent_loads;  // 1: read the exchange data with device-scope loads
+    int vec_io;        // 1: move the ifgo / out / cell tiles through LDS with 16-byte accesses
     long long spin_limit;
     long long *trace;  // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
@@ -82,6 +83,25 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     const unsigned zero_off = (unsigned)MTT * KS * kFragBytes;
     f32x4 *red = reinterpret_cast<f32x4 *>(smem + zero_off + kFragBytes);  // [P][TILES][64]
     unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * TILES * kWave);  // SPLIT 2: [2][KS] blocks
+
+    // Coalesced tile I/O: the workgroup's tile of ifgo[t] (bt rows x 4 gates x ht units) and of
+    // out / cell (bt x ht) lies in global memory as row segments of ht elements.  Moving them
+    // element by element costs one scattered 2-byte access per gate and item; instead the tile
+    // is moved with 16-byte pieces between global memory and padded LDS tiles, and the items
+    // work on LDS.  Needs 16-byte aligned, complete segments (host decides: p.vec_io).
+    constexpr int GSEG = HT * E::BYTES;                 // bytes of one gate segment of a row
+    constexpr bool VEC_OK = GSEG >= 16;
+    constexpr int GROW = 4 * GSEG + 16, SROW = GSEG + 16;   // padded LDS rows (bank spread)
+    constexpr int PPSEG = VEC_OK ? GSEG / 16 : 1;       // 16-byte pieces per segment
+    constexpr int GPIECES = BT * 4 * PPSEG, SPIECES = BT * PPSEG;
+    // wave 0 polls the flags and must not queue its polls behind bulk loads/stores of its own:
+    // the tiles are moved by waves 1..3 only
+    constexpr int IOT = kThreads - kWave;
+    constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
+    const int io_tid = tid - kWave;   // < 0: not an I/O thread
+    constexpr int TILE_BYTES = BT * GROW + 2 * BT * SROW;   // gates tile + h tile + c tile
+    const bool vio = VEC_OK && p.vec_io;
+    unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KS * kFragBytes);  // SYNC: 1 set, else 2 (step parity)
 
     T *ifgo = static_cast<T *>(p.ifgo);
     T *out = static_cast<T *>(p.out);
@@ -126,6 +146,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     size_t off_h[IPT];    // b*H + unit
     size_t off_p[IPT];    // b*4H + unit
     int xoff[IPT];        // byte offset of (unit, row) inside one exchange slot of this group
+    int goff[IPT], soff[IPT];  // byte offsets of the item inside the LDS gates / state tiles
     bool valid[IPT];
 #pragma unroll
     for (int m = 0; m < IPT; ++m) {
@@ -136,6 +157,8 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         off_h[m] = (size_t)b * H + unit;
         off_p[m] = (size_t)b * 4 * H + unit;
         xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
+        goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
+        soff[m] = (nt * 16 + n) * SROW + (mt * 4 + q) * E::BYTES;
         c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
     }
 
@@ -158,10 +181,10 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 
-    // x_t.Wx^T + b does not depend on the recurrence.  With a barrier per step it is fetched
-    // right before the wait (which hides the latency); the barrier-free form keeps PD steps
-    // of it in flight, because nothing else in its ~0.5 us step can hide an HBM round trip.
-    constexpr int PD = SYNC ? 1 : 4;
+    // x_t.Wx^T + b does not depend on the recurrence: it is requested PD steps ahead (an HBM round
+    // trip is ~2 us; loads return in order, so a late one would also hold back the exchange
+    // loads issued after it).  The barrier-free form has ~1 us steps and needs a deeper ring.
+    constexpr int PD = SYNC ? 2 : 4;
     T pre[PD][IPT][4];
     auto fetch_pre = [&](int t, T(&dst)[IPT][4]) {
 #pragma unroll
@@ -171,11 +194,58 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             for (int gt = 0; gt < 4; ++gt) dst[m][gt] = valid[m] ? src[(size_t)gt * H] : E::from_f32(0.f);
         }
     };
-    if constexpr (!SYNC) {
+    u32x4 gpre[PD][GPT];  // vec_io: 16-byte pieces of the gates tile, in flight
+    auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
 #pragma unroll
-        for (int u = 0; u < PD; ++u)
-            if (u < T_) fetch_pre(u, pre[u]);
-    }
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            dst[i] = u32x4{0u, 0u, 0u, 0u};
+            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+                dst[i] = *reinterpret_cast<const u32x4 *>(
+                    ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 + k * (16 / E::BYTES));
+        }
+    };
+    auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            if (io_tid >= 0 && pc < GPIECES)
+                *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
+        }
+    };
+    // LDS tiles -> ifgo[t], out[t+1], cell[t+1] with 16-byte row-contiguous stores
+    auto tiles_to_global = [&](int t, const unsigned char *gt) {
+        const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+                *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
+                                           k * (16 / E::BYTES)) =
+                    *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / PPSEG, k = pc % PPSEG;
+            if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
+                const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
+                *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+            }
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < PD; ++u)
+        if (u < T_) {
+            if (vio) fetch_tile(u, gpre[u]);
+            else fetch_pre(u, pre[u]);
+        }
 
     int slot_r = 0;  // ring slot that holds h_{t-1}
     for (int t0 = 0; t0 < T_; t0 += PD) {
@@ -184,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         const int t = t0 + u;
         if (t >= T_) break;
         const int slot_w = (slot_r + 1 == n_slots) ? 0 : slot_r + 1;
-        if constexpr (SYNC) fetch_pre(t, pre[0]);
+        unsigned char *gt = tiles + (SYNC ? 0 : (t & 1) * TILE_BYTES);
         long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
         if (p.trace) tr0 = (long long)wall_clock64();
 
@@ -267,6 +337,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 const int pp = SPLIT == 0 ? wave : 0;
                 red[(pp * TILES + tl) * kWave + lane] = acc[a][i];
             }
+        if (vio) tile_to_lds(gpre[u], gt);
         __syncthreads();
 
         const unsigned xn = xgrp + (unsigned)slot_w * xslot;
@@ -282,6 +353,11 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
                 for (int pp = 1; pp < P; ++pp) s += red[(pp * TILES + tl) * kWave + lane];
                 if (valid[m]) {
+                    T *gl = reinterpret_cast<T *>(gt + goff[m]);   // the item's 4 gates in the LDS tile
+                    if (vio) {
+#pragma unroll
+                        for (int gg = 0; gg < 4; ++gg) pre[u][m][gg] = gl[gg * HT];
+                    }
                     const float pi = E::to_f32(pre[u][m][0]) + s[0];
                     const float pf = E::to_f32(pre[u][m][1]) + s[1];
                     const float pg = E::to_f32(pre[u][m][2]) + s[2];
@@ -296,6 +372,12 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                     st_p[m][2] = E::from_f32(pg);
                     st_p[m][3] = E::from_f32(po);
                     st_c[m] = E::from_f32(c1);
+                    if (vio) {
+#pragma unroll
+                        for (int gg = 0; gg < 4; ++gg) gl[gg * HT] = st_p[m][gg];
+                        *reinterpret_cast<T *>(gt + BT * GROW + soff[m]) = st_h[m];
+                        *reinterpret_cast<T *>(gt + BT * GROW + BT * SROW + soff[m]) = st_c[m];
+                    }
                 }
             }
         }
@@ -316,11 +398,23 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         };
         if constexpr (SYNC) {
             if (t + 1 < T_) publish_version(my_flag, t + 2);
-            bulk_store();
+            else if (vio) __syncthreads();   // last step: the tiles still have to be complete
+            if (vio) tiles_to_global(t, gt);
+            else bulk_store();
+            if (t + PD < T_) {
+                if (vio) fetch_tile(t + PD, gpre[u]);
+                else fetch_pre(t + PD, pre[u]);
+            }
         } else {
-            bulk_store();
-            if (t + PD < T_) fetch_pre(t + PD, pre[u]);
-            __syncthreads();
+            if (vio) {
+                __syncthreads();
+                tiles_to_global(t, gt);
+                if (t + PD < T_) fetch_tile(t + PD, gpre[u]);
+            } else {
+                bulk_store();
+                if (t + PD < T_) fetch_pre(t + PD, pre[u]);
+                __syncthreads();
+            }
         }
         slot_r = slot_w;
         if (p.trace && tid == 0) {  // accumulated wait / fetch+mfma / reduce+gates / publish times

@@ -138,8 +138,9 @@ void fastlstm_set_spin_limit(long long ticks);
 void fastlstm_set_gemm_trace(void *buf);
 
 /* Diagnostics: when `buf` (zero-filled device memory, 32 bytes per workgroup) is non-NULL the
- * forward recurrence accumulates, per workgroup and in 100 MHz ticks, the time spent waiting
- * for its peers, fetching operands + MFMA, reducing + gate maths, and publishing. */
+ * recurrent kernels accumulate, per workgroup and in 100 MHz ticks, four phase times: forward =
+ * waiting for peers, operand fetch + MFMA, reduce + gate maths, publish; backward = gate maths,
+ * publish + stores, waiting for peers, operand fetch + MFMA + reduce. */
 void fastlstm_set_recurrent_trace(void *buf);
 
 const char *fastlstm_strerror(int status);
