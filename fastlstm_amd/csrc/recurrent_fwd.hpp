@@ -49,7 +49,7 @@ struct FwdParams {
 // SPLIT 0: waves split K   (MT m-tiles, NTW n-tiles per WG, 4 partial sums)
 // SPLIT 1: waves split N   (MT m-tiles per WG, NTW n-tiles per wave, 4*NTW per WG)
 // SPLIT 2: waves split M   (MT m-tiles per wave, 4*MT per WG, one n-tile; no cross-WG sync)
-template <typename T, int MT, int NTW, int SPLIT>
+template <typename T, int MT, int NTW, int SPLIT, bool VIO>
 __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const FwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
     const int io_tid = tid - kWave;   // < 0: not an I/O thread
     constexpr int TILE_BYTES = BT * GROW + 2 * BT * SROW;   // gates tile + h tile + c tile
-    const bool vio = VEC_OK && p.vec_io;
+    static_assert(!VIO || VEC_OK, "tile I/O needs 16-byte gate segments");
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KS * kFragBytes);  // SYNC: 1 set, else 2 (step parity)
 
     T *ifgo = static_cast<T *>(p.ifgo);
@@ -154,8 +154,9 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         const int mt = tl / NT, nt = tl % NT;
         const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
         valid[m] = (tl < TILES) && unit < H && b < B;
-        off_h[m] = (size_t)b * H + unit;
-        off_p[m] = (size_t)b * 4 * H + unit;
+        // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
+        off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
+        off_p[m] = valid[m] ? (size_t)b * 4 * H + unit : (size_t)b0 * 4 * H + u0;
         xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
         goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
         soff[m] = (nt * 16 + n) * SROW + (mt * 4 + q) * E::BYTES;
@@ -182,29 +183,32 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 
     // x_t.Wx^T + b does not depend on the recurrence: it is requested PD steps ahead (an HBM round
-    // trip is ~2 us; loads return in order, so a late one would also hold back the exchange
-    // loads issued after it).  The barrier-free form has ~1 us steps and needs a deeper ring.
+    // trip is ~2 us).  The loads are unconditional -- invalid items / pieces read a valid dummy
+    // address -- so that their results stay in the registers they were loaded into: a
+    // conditional load ends in a register copy, and the copy in a wait for the load.
     constexpr int PD = SYNC ? 2 : 4;
-    T pre[PD][IPT][4];
+    constexpr int PRE_N = VIO ? 1 : PD, GPRE_N = VIO ? PD : 1;
+    T pre[PRE_N][IPT][4];
     auto fetch_pre = [&](int t, T(&dst)[IPT][4]) {
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const T *src = ifgo + (size_t)t * B4H + off_p[m];
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) dst[m][gt] = valid[m] ? src[(size_t)gt * H] : E::from_f32(0.f);
+            for (int gt = 0; gt < 4; ++gt) dst[m][gt] = src[(size_t)gt * H];
         }
     };
-    u32x4 gpre[PD][GPT];  // vec_io: 16-byte pieces of the gates tile, in flight
+    u32x4 gpre[GPRE_N][GPT];  // VIO: 16-byte pieces of the gates tile, in flight
+    const size_t tile_org = (size_t)b0 * 4 * H + u0;   // first element of the tile inside ifgo[t]
     auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
+        if (io_tid < 0) return;
 #pragma unroll
         for (int i = 0; i < GPT; ++i) {
             const int pc = io_tid + IOT * i;
             const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
             const int seg = rem / PPSEG, k = rem % PPSEG;
-            dst[i] = u32x4{0u, 0u, 0u, 0u};
-            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
-                dst[i] = *reinterpret_cast<const u32x4 *>(
-                    ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 + k * (16 / E::BYTES));
+            const bool ok = pc < GPIECES && b0 + row < B;
+            const size_t off = ok ? (size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES) : 0;
+            dst[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + tile_org + off);
         }
     };
     auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
@@ -240,19 +244,24 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         }
     };
-#pragma unroll
-    for (int u = 0; u < PD; ++u)
-        if (u < T_) {
-            if (vio) fetch_tile(u, gpre[u]);
-            else fetch_pre(u, pre[u]);
+    auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (t < T_) {
+            if constexpr (VIO) fetch_tile(t, gpre[u]);
+            else fetch_pre(t, pre[u]);
         }
+    };
+    prefetch(0, std::integral_constant<int, 0>{});
+    prefetch(1, std::integral_constant<int, 1>{});
+    if constexpr (PD > 2) {
+        prefetch(2, std::integral_constant<int, 2>{});
+        prefetch(3, std::integral_constant<int, 3>{});
+    }
 
     int slot_r = 0;  // ring slot that holds h_{t-1}
-    for (int t0 = 0; t0 < T_; t0 += PD) {
-#pragma unroll
-    for (int u = 0; u < PD; ++u) {
-        const int t = t0 + u;
-        if (t >= T_) break;
+    // One timestep; u = t % PD selects the prefetch ring entry at compile time.
+    auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
         const int slot_w = (slot_r + 1 == n_slots) ? 0 : slot_r + 1;
         unsigned char *gt = tiles + (SYNC ? 0 : (t & 1) * TILE_BYTES);
         long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
@@ -337,7 +346,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 const int pp = SPLIT == 0 ? wave : 0;
                 red[(pp * TILES + tl) * kWave + lane] = acc[a][i];
             }
-        if (vio) tile_to_lds(gpre[u], gt);
+        if constexpr (VIO) tile_to_lds(gpre[u], gt);
         __syncthreads();
 
         const unsigned xn = xgrp + (unsigned)slot_w * xslot;
@@ -354,14 +363,16 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 for (int pp = 1; pp < P; ++pp) s += red[(pp * TILES + tl) * kWave + lane];
                 if (valid[m]) {
                     T *gl = reinterpret_cast<T *>(gt + goff[m]);   // the item's 4 gates in the LDS tile
-                    if (vio) {
+                    T x4[4];
 #pragma unroll
-                        for (int gg = 0; gg < 4; ++gg) pre[u][m][gg] = gl[gg * HT];
+                    for (int gg = 0; gg < 4; ++gg) {
+                        if constexpr (VIO) x4[gg] = gl[gg * HT];
+                        else x4[gg] = pre[u][m][gg];
                     }
-                    const float pi = E::to_f32(pre[u][m][0]) + s[0];
-                    const float pf = E::to_f32(pre[u][m][1]) + s[1];
-                    const float pg = E::to_f32(pre[u][m][2]) + s[2];
-                    const float po = E::to_f32(pre[u][m][3]) + s[3];
+                    const float pi = E::to_f32(x4[0]) + s[0];
+                    const float pf = E::to_f32(x4[1]) + s[1];
+                    const float pg = E::to_f32(x4[2]) + s[2];
+                    const float po = E::to_f32(x4[3]) + s[3];
                     const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
                     const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
                     c_state[m] = c1;
@@ -372,7 +383,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                     st_p[m][2] = E::from_f32(pg);
                     st_p[m][3] = E::from_f32(po);
                     st_c[m] = E::from_f32(c1);
-                    if (vio) {
+                    if constexpr (VIO) {
 #pragma unroll
                         for (int gg = 0; gg < 4; ++gg) gl[gg * HT] = st_p[m][gg];
                         *reinterpret_cast<T *>(gt + BT * GROW + soff[m]) = st_h[m];
@@ -398,24 +409,19 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         };
         if constexpr (SYNC) {
             if (t + 1 < T_) publish_version(my_flag, t + 2);
-            else if (vio) __syncthreads();   // last step: the tiles still have to be complete
-            if (vio) tiles_to_global(t, gt);
+            else if constexpr (VIO) __syncthreads();   // last step: the tiles still have to be complete
+            if constexpr (VIO) tiles_to_global(t, gt);
             else bulk_store();
-            if (t + PD < T_) {
-                if (vio) fetch_tile(t + PD, gpre[u]);
-                else fetch_pre(t + PD, pre[u]);
-            }
         } else {
-            if (vio) {
+            if constexpr (VIO) {
                 __syncthreads();
                 tiles_to_global(t, gt);
-                if (t + PD < T_) fetch_tile(t + PD, gpre[u]);
             } else {
                 bulk_store();
-                if (t + PD < T_) fetch_pre(t + PD, pre[u]);
                 __syncthreads();
             }
         }
+        prefetch(t + PD, uc);
         slot_r = slot_w;
         if (p.trace && tid == 0) {  // accumulated wait / fetch+mfma / reduce+gates / publish times
             long long *tr = p.trace + (size_t)blockIdx.x * 4;
@@ -424,7 +430,14 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             tr[2] += tr3 - tr2;
             tr[3] += (long long)wall_clock64() - tr3;
         }
-    }
+    };
+    for (int t0 = 0; t0 < T_; t0 += PD) {
+        step(t0, std::integral_constant<int, 0>{});
+        if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
+        if constexpr (PD > 2) {
+            if (t0 + 2 < T_) step(t0 + 2, std::integral_constant<int, 2>{});
+            if (t0 + 3 < T_) step(t0 + 3, std::integral_constant<int, 3>{});
+        }
     }
 }
 
