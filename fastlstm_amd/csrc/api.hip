@@ -196,6 +196,9 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         const int tile_bytes = (pl.bt * (4 * gseg + 16) + 2 * pl.bt * (gseg + 16)) * (sync ? 1 : 2);
         p.vec_io = (gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && lds_bytes + tile_bytes <= pl.lds_limit) ? 1 : 0;
         if (p.vec_io) lds_bytes += tile_bytes;
+#ifdef FASTLSTM_TIMELINE
+        lds_bytes += 4096;   // room for the diagnostic time stamps of the kernel
+#endif
     }
     FwdLauncher launch = fwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {

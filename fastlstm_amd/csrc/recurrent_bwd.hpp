@@ -130,8 +130,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         const int ul = rest % HT, nt = rest / HT;
         const int unit = u0 + ul, b = b0 + nt * 16 + n;
         valid[m] = nt < NT && unit < H && b < B;
-        off_h[m] = (size_t)b * H + unit;
-        off_p[m] = (size_t)b * 4 * H + unit;
+        // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
+        off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
+        off_p[m] = valid[m] ? (size_t)b * 4 * H + unit : (size_t)b0 * 4 * H + u0;
         xoff[m] = nt * KSB * kFragBytes + frag_offset<T>(n, unit * 4);
         pair_lead[m] = valid[m] && ((ul & 1) == 0);  // u0 is a multiple of 4: even ul <=> low half of a slot
         const int mtile = ul >> 4, ur = ul & 15;
@@ -150,32 +151,38 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
 
-    // Stored activations and dout do not depend on the recurrence.  With a barrier per step
-    // the next step's operands are requested right before the wait; the barrier-free form
-    // keeps PD steps in flight (nothing else in its short step hides an HBM round trip).
-    constexpr int PD = SYNC ? 1 : 4;
+    // Stored activations and dout do not depend on the recurrence: they are requested PD steps
+    // ahead (an HBM round trip is ~2 us).  The loads are unconditional -- invalid items read a valid
+    // dummy address -- so that their results stay in the registers they were loaded into: a
+    // conditional load ends in a register copy, and the copy in a wait for the load.
+    constexpr int PD = SYNC ? 2 : 4;
     T pre[PD][IPT][4], c0r[PD][IPT], dor[PD][IPT];
     auto fetch = [&](int t, T(&dp)[IPT][4], T(&dc0)[IPT], T(&dd)[IPT]) {
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
-            const T zero = E::from_f32(0.f);
             const T *src = ifgo + (size_t)t * B4H + off_p[m];
 #pragma unroll
-            for (int gt = 0; gt < 4; ++gt) dp[m][gt] = valid[m] ? src[(size_t)gt * H] : zero;
-            dc0[m] = valid[m] ? cell[(size_t)t * BH + off_h[m]] : zero;
-            dd[m] = valid[m] ? dout[(size_t)t * BH + off_h[m]] : zero;
+            for (int gt = 0; gt < 4; ++gt) dp[m][gt] = src[(size_t)gt * H];
+            dc0[m] = cell[(size_t)t * BH + off_h[m]];
+            dd[m] = dout[(size_t)t * BH + off_h[m]];
         }
     };
-#pragma unroll
-    for (int u = 0; u < PD; ++u)
-        if (u < T_) fetch(T_ - 1 - u, pre[u], c0r[u], dor[u]);
+    // inputs of reverse step s (timestep T-1-s) into ring entry s % PD
+    auto prefetch = [&](int s, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (s < T_) fetch(T_ - 1 - s, pre[u], c0r[u], dor[u]);
+    };
+    prefetch(0, std::integral_constant<int, 0>{});
+    prefetch(1, std::integral_constant<int, 1>{});
+    if constexpr (PD > 2) {
+        prefetch(2, std::integral_constant<int, 2>{});
+        prefetch(3, std::integral_constant<int, 3>{});
+    }
 
     int slot = 0;  // ring slot of this step's d_ifgo
-    for (int s0 = 0; s0 < T_; s0 += PD) {
-#pragma unroll
-    for (int u = 0; u < PD; ++u) {
-        const int s = s0 + u;
-        if (s >= T_) break;
+    // One reverse step; u = s % PD selects the prefetch ring entry at compile time.
+    auto step = [&](const int s, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
         const int t = T_ - 1 - s;
         const unsigned xw = xgrp + (unsigned)slot * xslot;
         slot = (slot + 1 == n_slots) ? 0 : slot + 1;
@@ -246,7 +253,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         }
 
         // recurrence-independent operands of a later step: issue before waiting
-        if (s + PD < T_) fetch(t - PD, pre[u], c0r[u], dor[u]);
+        prefetch(s + PD, uc);
 
         if (p.trace) tr2 = (long long)wall_clock64();
         if constexpr (SYNC) {
@@ -329,7 +336,14 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         }
         // the next iteration's publish (or block barrier) orders these reads before the
         // next writes to `red`
-    }
+    };
+    for (int s0 = 0; s0 < T_; s0 += PD) {
+        step(s0, std::integral_constant<int, 0>{});
+        if (s0 + 1 < T_) step(s0 + 1, std::integral_constant<int, 1>{});
+        if constexpr (PD > 2) {
+            if (s0 + 2 < T_) step(s0 + 2, std::integral_constant<int, 2>{});
+            if (s0 + 3 < T_) step(s0 + 3, std::integral_constant<int, 3>{});
+        }
     }
 
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);

@@ -103,6 +103,19 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     static_assert(!VIO || VEC_OK, "tile I/O needs 16-byte gate segments");
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KS * kFragBytes);  // SYNC: 1 set, else 2 (step parity)
 
+    // Diagnostic build (-DFASTLSTM_TIMELINE): lane 0 of every wave stamps the 100 MHz clock at fixed
+    // points of timesteps 200..203 into LDS; the stamps go to p.trace (256 words per workgroup:
+    // [step][wave][16 events]) when the kernel ends.  The host adds 4 KiB of LDS for it.
+#ifdef FASTLSTM_TIMELINE
+    long long *tl = reinterpret_cast<long long *>(tiles + (SYNC ? 1 : 2) * TILE_BYTES + 64);
+    for (int idx = tid; idx < 256; idx += kThreads) tl[idx] = 0;
+#define FASTLSTM_TP(ev)                                                                              \
+    do {                                                                                             \
+        if (lane == 0 && t >= 200 && t < 204) tl[((t - 200) * 4 + wave) * 16 + (ev)] = (long long)wall_clock64(); \
+    } while (0)
+#else
+#define FASTLSTM_TP(ev) do {} while (0)
+#endif
     T *ifgo = static_cast<T *>(p.ifgo);
     T *out = static_cast<T *>(p.out);
     T *cell = static_cast<T *>(p.cell);
@@ -266,11 +279,13 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         unsigned char *gt = tiles + (SYNC ? 0 : (t & 1) * TILE_BYTES);
         long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
         if (p.trace) tr0 = (long long)wall_clock64();
-
+        FASTLSTM_TP(0);
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
+            FASTLSTM_TP(1);
             __syncthreads();
         }
+        FASTLSTM_TP(2);
         if (p.trace) tr1 = (long long)wall_clock64();
 
         // ---- acc[mt][i] += Wslice(mt) . h_{t-1}(nt)^T over this wave's k-steps ----------
@@ -332,7 +347,10 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         };
         if (coherent) kloop(std::true_type{});
         else kloop(std::false_type{});
-
+#ifdef FASTLSTM_TIMELINE
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#endif
+        FASTLSTM_TP(3);
         if (p.trace) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // attribute the operand fetch to this phase
             tr2 = (long long)wall_clock64();
@@ -347,7 +365,9 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 red[(pp * TILES + tl) * kWave + lane] = acc[a][i];
             }
         if constexpr (VIO) tile_to_lds(gpre[u], gt);
+        FASTLSTM_TP(4);
         __syncthreads();
+        FASTLSTM_TP(5);
 
         const unsigned xn = xgrp + (unsigned)slot_w * xslot;
         // Results of this step.  Only the exchange copy of h_t is on the critical path: it is
@@ -393,6 +413,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         }
         if (p.trace) tr3 = (long long)wall_clock64();
+        FASTLSTM_TP(6);
         auto bulk_store = [&]() {
 #pragma unroll
             for (int m = 0; m < IPT; ++m) {
@@ -408,8 +429,13 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         };
         if constexpr (SYNC) {
+#ifdef FASTLSTM_TIMELINE
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            FASTLSTM_TP(7);
+#endif
             if (t + 1 < T_) publish_version(my_flag, t + 2);
             else if constexpr (VIO) __syncthreads();   // last step: the tiles still have to be complete
+            FASTLSTM_TP(8);
             if constexpr (VIO) tiles_to_global(t, gt);
             else bulk_store();
         } else {
@@ -422,7 +448,9 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             }
         }
         prefetch(t + PD, uc);
+        FASTLSTM_TP(9);
         slot_r = slot_w;
+#ifndef FASTLSTM_TIMELINE
         if (p.trace && tid == 0) {  // accumulated wait / fetch+mfma / reduce+gates / publish times
             long long *tr = p.trace + (size_t)blockIdx.x * 4;
             tr[0] += tr1 - tr0;
@@ -430,6 +458,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             tr[2] += tr3 - tr2;
             tr[3] += (long long)wall_clock64() - tr3;
         }
+#endif
     };
     for (int t0 = 0; t0 < T_; t0 += PD) {
         step(t0, std::integral_constant<int, 0>{});
@@ -439,6 +468,12 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             if (t0 + 3 < T_) step(t0 + 3, std::integral_constant<int, 3>{});
         }
     }
+#ifdef FASTLSTM_TIMELINE
+    __syncthreads();
+    if (p.trace)
+        for (int idx = tid; idx < 256; idx += kThreads) p.trace[(size_t)blockIdx.x * 256 + idx] = tl[idx];
+#endif
+#undef FASTLSTM_TP
 }
 
 }  // namespace fastlstm
