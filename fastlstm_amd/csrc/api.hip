@@ -252,6 +252,14 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
         p.n_slots = (int)std::min<size_t>(full, avail);
         p.coherent_loads = p.n_slots < T ? 1 : 0;
     }
+    // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
+    int lds_bytes = pl.lds_bytes;
+    {
+        const int s = elem_bytes(dtype), gseg = pl.ht * s;
+        const int tile_bytes = (pl.bt * (4 * gseg + 16) + 2 * pl.bt * (gseg + 16)) * (sync ? 1 : 2);
+        p.vec_io = (gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && lds_bytes + tile_bytes <= pl.lds_limit) ? 1 : 0;
+        if (p.vec_io) lds_bytes += tile_bytes;
+    }
     BwdLauncher launch = bwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
@@ -261,9 +269,9 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
         int occ = 0;
-        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
-        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, pl.lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
+        if (launch(p, pl.ht, pl.bt, pl.wave_split, grid, lds_bytes, static_cast<hipStream_t>(stream), nullptr) !=
             hipSuccess)
             return FASTLSTM_ERR_HIP;
     }

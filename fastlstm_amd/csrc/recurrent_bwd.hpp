@@ -45,12 +45,15 @@ struct BwdParams {
     int n_slots;        // exchange ring length (T: every step has its own slot)
     int coherent_loads; // 1: read the exchange data with device-scope loads
     long long spin_limit;
+    int vec_io;         // 1: the VIO instantiation is launched (complete, 16-byte aligned tile segments)
     long long *trace;   // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
 
 // SPLIT 0: waves split K (NTW n-tiles per WG); SPLIT 1: waves split N (NTW n-tiles per wave);
 // SPLIT 2: barrier-free small-H form, wave w owns unit tile w (up to 64 units), one n-tile.
-template <typename T, int NTW, int SPLIT>
+// VIO: the workgroup's tiles of ifgo[t], cell[t], dout[t] and d_ifgo[t] move between global memory
+// and LDS in 16-byte pieces (waves 1..3) instead of element by element; see the forward kernel.
+template <typename T, int NTW, int SPLIT, bool VIO>
 __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const BwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
@@ -87,6 +90,19 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     f32x4 *red = reinterpret_cast<f32x4 *>(smem + wbytes + kFragBytes);      // [P][MTB][NT][64]
     unsigned char *xl = reinterpret_cast<unsigned char *>(red + P * MTB * NT * kWave);  // SPLIT 2
 
+    // ---- tile I/O geometry (VIO) ---------------------------------------------------------
+    // gates tile [BT][4 gates][HT] with rows padded to GROW bytes, then two state tiles
+    // [BT][HT] (c_{t-1} and dout[t]) with rows of SROW bytes.  HT is a run-time value here.
+    constexpr int HTMAX = SYNC ? 16 : 64;
+    constexpr int PPSEG_MAX = HTMAX * E::BYTES / 16 > 0 ? HTMAX * E::BYTES / 16 : 1;
+    constexpr int IOT = kThreads - kWave;   // wave 0 polls the flags and moves nothing
+    constexpr int GPT = (BT * 4 * PPSEG_MAX + IOT - 1) / IOT, SPT = (BT * PPSEG_MAX + IOT - 1) / IOT;
+    const int GSEG = HT * E::BYTES, GROW = 4 * GSEG + 16, SROW = GSEG + 16;
+    const int PPSEG = GSEG / 16;            // 16-byte pieces per segment (>= 1 when VIO)
+    const int TILE_BYTES = BT * GROW + 2 * BT * SROW;
+    unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KSB * kFragBytes);   // SYNC: 1 set, else 2 (step parity)
+    const int io_tid = tid - kWave;         // < 0: not an I/O thread
+
     const T *dout = static_cast<const T *>(p.dout);
     const T *ifgo = static_cast<const T *>(p.ifgo);
     const T *cell = static_cast<const T *>(p.cell);
@@ -121,6 +137,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     float dc_state[IPT], dh_rec[IPT], c1v[IPT];
     size_t off_h[IPT], off_p[IPT];
     int xoff[IPT], roff[IPT];
+    int goff[IPT], soff[IPT];   // VIO: byte offsets of the item inside the LDS gates / state tiles
     bool valid[IPT], pair_lead[IPT];
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 #pragma unroll
@@ -135,6 +152,8 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         off_p[m] = valid[m] ? (size_t)b * 4 * H + unit : (size_t)b0 * 4 * H + u0;
         xoff[m] = nt * KSB * kFragBytes + frag_offset<T>(n, unit * 4);
         pair_lead[m] = valid[m] && ((ul & 1) == 0);  // u0 is a multiple of 4: even ul <=> low half of a slot
+        goff[m] = (nt * 16 + n) * GROW + ul * E::BYTES;
+        soff[m] = (nt * 16 + n) * SROW + ul * E::BYTES;
         const int mtile = ul >> 4, ur = ul & 15;
         roff[m] = ((mtile * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
         dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
@@ -156,7 +175,8 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     // dummy address -- so that their results stay in the registers they were loaded into: a
     // conditional load ends in a register copy, and the copy in a wait for the load.
     constexpr int PD = SYNC ? 2 : 4;
-    T pre[PD][IPT][4], c0r[PD][IPT], dor[PD][IPT];
+    constexpr int PRE_N = VIO ? 1 : PD, GPRE_N = VIO ? PD : 1;
+    T pre[PRE_N][IPT][4], c0r[PRE_N][IPT], dor[PRE_N][IPT];
     auto fetch = [&](int t, T(&dp)[IPT][4], T(&dc0)[IPT], T(&dd)[IPT]) {
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
@@ -167,12 +187,76 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
             dd[m] = dout[(size_t)t * BH + off_h[m]];
         }
     };
+    // VIO: the 16-byte pieces this thread moves.  Piece pc of the gates tile = (row, gate, k-th
+    // piece of the segment); pieces that do not exist or lie past the batch read the tile origin.
+    unsigned g_glb[GPT], s_glb[SPT];   // element offsets inside ifgo[t] / cell[t]
+    int g_lds[GPT], s_lds[SPT];        // byte offsets inside the LDS tiles
+    bool g_ok[GPT], s_ok[SPT];
+    u32x4 gpre[GPRE_N][GPT], cpre[GPRE_N][SPT], dpre[GPRE_N][SPT];
+    if constexpr (VIO) {
+        const int gpieces = BT * 4 * PPSEG, spieces = BT * PPSEG;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            g_ok[i] = io_tid >= 0 && pc < gpieces && b0 + row < B;
+            g_lds[i] = g_ok[i] ? row * GROW + seg * GSEG + k * 16 : 0;
+            g_glb[i] = (unsigned)((size_t)b0 * 4 * H + u0) +
+                       (g_ok[i] ? (unsigned)(row * 4 * H + seg * H + k * (16 / E::BYTES)) : 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / PPSEG, k = pc % PPSEG;
+            s_ok[i] = io_tid >= 0 && pc < spieces && b0 + row < B;
+            s_lds[i] = s_ok[i] ? row * SROW + k * 16 : 0;
+            s_glb[i] = (unsigned)((size_t)b0 * H + u0) + (s_ok[i] ? (unsigned)(row * H + k * (16 / E::BYTES)) : 0u);
+        }
+    }
+    auto fetch_tiles = [&](int t, u32x4(&gp)[GPT], u32x4(&cp)[SPT], u32x4(&dp)[SPT]) {
+        if (io_tid < 0) return;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) gp[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + g_glb[i]);
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            cp[i] = *reinterpret_cast<const u32x4 *>(cell + (size_t)t * BH + s_glb[i]);
+            dp[i] = *reinterpret_cast<const u32x4 *>(dout + (size_t)t * BH + s_glb[i]);
+        }
+    };
+    auto tiles_to_lds = [&](const u32x4(&gp)[GPT], const u32x4(&cp)[SPT], const u32x4(&dp)[SPT], unsigned char *gt) {
+        unsigned char *stc = gt + BT * GROW, *std_ = stc + BT * SROW;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i)
+            if (g_ok[i]) *reinterpret_cast<u32x4 *>(gt + g_lds[i]) = gp[i];
+#pragma unroll
+        for (int i = 0; i < SPT; ++i)
+            if (s_ok[i]) {
+                *reinterpret_cast<u32x4 *>(stc + s_lds[i]) = cp[i];
+                *reinterpret_cast<u32x4 *>(std_ + s_lds[i]) = dp[i];
+            }
+    };
+    // LDS gates tile (now d_i, d_f, d_g, d_o) -> d_ifgo[t]
+    auto tile_to_global = [&](int t, const unsigned char *gt) {
+#pragma unroll
+        for (int i = 0; i < GPT; ++i)
+            if (g_ok[i])
+                *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
+                    *reinterpret_cast<const u32x4 *>(gt + g_lds[i]);
+    };
     // inputs of reverse step s (timestep T-1-s) into ring entry s % PD
     auto prefetch = [&](int s, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
-        if (s < T_) fetch(T_ - 1 - s, pre[u], c0r[u], dor[u]);
+        if (s < T_) {
+            if constexpr (VIO) fetch_tiles(T_ - 1 - s, gpre[u], cpre[u], dpre[u]);
+            else fetch(T_ - 1 - s, pre[u], c0r[u], dor[u]);
+        }
     };
     prefetch(0, std::integral_constant<int, 0>{});
+    if constexpr (VIO) {   // step 0 works on the LDS tiles right away; its ring entry is refilled in step 0
+        tiles_to_lds(gpre[0], cpre[0], dpre[0], tiles);
+        __syncthreads();
+    }
     prefetch(1, std::integral_constant<int, 1>{});
     if constexpr (PD > 2) {
         prefetch(2, std::integral_constant<int, 2>{});
@@ -189,18 +273,33 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
 
         long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
         if (p.trace) tr0 = (long long)wall_clock64();
+        unsigned char *gt = tiles + (SYNC ? 0 : (s & 1) * TILE_BYTES);         // VIO: this step's tiles
+        unsigned char *gt_next = tiles + (SYNC ? 0 : ((s + 1) & 1) * TILE_BYTES);
         // ---- point-wise gate backward for this thread's items --------------------------
         T st_d[IPT][4];
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             if (valid[m]) {
-                const float si = sigmoidf_<ACC>(E::to_f32(pre[u][m][0]));
-                const float sf = sigmoidf_<ACC>(E::to_f32(pre[u][m][1]));
-                const float tg = tanhf_<ACC>(E::to_f32(pre[u][m][2]));
-                const float so = sigmoidf_<ACC>(E::to_f32(pre[u][m][3]));
+                T x4[4], xc, xd;
+                T *gl = reinterpret_cast<T *>(gt + goff[m]);   // VIO: the item's 4 gates in the LDS tile
+                if constexpr (VIO) {
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) x4[gg] = gl[gg * HT];
+                    xc = *reinterpret_cast<const T *>(gt + BT * GROW + soff[m]);
+                    xd = *reinterpret_cast<const T *>(gt + BT * GROW + BT * SROW + soff[m]);
+                } else {
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) x4[gg] = pre[u][m][gg];
+                    xc = c0r[u][m];
+                    xd = dor[u][m];
+                }
+                const float si = sigmoidf_<ACC>(E::to_f32(x4[0]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(x4[1]));
+                const float tg = tanhf_<ACC>(E::to_f32(x4[2]));
+                const float so = sigmoidf_<ACC>(E::to_f32(x4[3]));
                 const float tc = tanhf_<ACC>(c1v[m]);
-                const float c0 = E::to_f32(c0r[u][m]);
-                const float dh = dh_rec[m] + E::to_f32(dor[u][m]);
+                const float c0 = E::to_f32(xc);
+                const float dh = dh_rec[m] + E::to_f32(xd);
                 const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
                 const float d_o = dh * tc * so * (1.f - so);
                 const float d_f = dc1 * c0 * sf * (1.f - sf);
@@ -212,6 +311,10 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 st_d[m][1] = E::from_f32(d_f);
                 st_d[m][2] = E::from_f32(d_g);
                 st_d[m][3] = E::from_f32(d_o);
+                if constexpr (VIO) {
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) gl[gg * HT] = st_d[m][gg];
+                }
             } else {
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) st_d[m][gt] = E::from_f32(0.f);
@@ -243,13 +346,21 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 }
             }
         };
+        constexpr int un = (u + 1) % PD;   // ring entry of the next step's inputs
         if constexpr (SYNC) {
             publish_version(my_flag, s + 1);
             if (p.trace) tr1 = (long long)wall_clock64();
-            bulk_store();
+            if constexpr (VIO) tile_to_global(t, gt);
+            else bulk_store();
         } else {
-            bulk_store();
-            __syncthreads();
+            if constexpr (VIO) {
+                __syncthreads();
+                tile_to_global(t, gt);
+                if (s + 1 < T_) tiles_to_lds(gpre[un], cpre[un], dpre[un], gt_next);
+            } else {
+                bulk_store();
+                __syncthreads();
+            }
         }
 
         // recurrence-independent operands of a later step: issue before waiting
@@ -259,6 +370,10 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         if constexpr (SYNC) {
             if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, g, s);
             __syncthreads();
+            // the tile has been drained: the next step's inputs may take its place
+            if constexpr (VIO) {
+                if (s + 1 < T_) tiles_to_lds(gpre[un], cpre[un], dpre[un], gt_next);
+            }
         }
         if (p.trace) tr3 = (long long)wall_clock64();
 
