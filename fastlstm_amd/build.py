@@ -16,7 +16,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(LIBDIR, "libfastlstm_hip.so")
-SOURCES = ["api.hip", "gemm.hip", "plan.cpp", "recurrent_f32.hip", "recurrent_f16.hip", "recurrent_bf16.hip"]
+SOURCES = ["api.hip", "gemm.hip", "plan.cpp", "recurrent_f32.hip", "recurrent_f16.hip", "recurrent_bf16.hip",
+           "recurrent_wreg_f32.hip", "recurrent_wreg_f16.hip", "recurrent_wreg_bf16.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -44,7 +45,7 @@ def build(force=False, verbose=False):
     if not force and os.path.exists(LIB):
         if os.path.getmtime(LIB) >= max(os.path.getmtime(d) for d in _deps()):
             return LIB
-    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
         results = list(ex.map(_compile, SOURCES))
     if verbose:
         for _, err in results:

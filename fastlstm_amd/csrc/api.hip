@@ -200,6 +200,11 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         lds_bytes += 4096;   // room for the diagnostic time stamps of the kernel
 #endif
     }
+    // K-split kernels keep the slice in registers when a wave's share is at most 32 fragments
+    if (pl.wave_split == 0) {
+        const int nkw = cdiv(p.KS, 4) <= 4 ? 4 : (cdiv(p.KS, 4) <= 8 ? 8 : 0);
+        if (nkw && (pl.ht / 4) * nkw <= 32) p.w_regs = nkw;
+    }
     FwdLauncher launch = fwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);

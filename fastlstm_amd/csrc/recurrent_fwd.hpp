@@ -42,6 +42,7 @@ struct FwdParams {
     int n_slots;       // exchange ring length (T+1: every step has its own slot)
     int coherent_loads;  // 1: read the exchange data with device-scope loads
     int vec_io;        // 1: move the ifgo / out / cell tiles through LDS with 16-byte accesses
+    int w_regs;        // > 0: k-steps per wave of the W_h slice held in registers (NKW instantiation)
     long long spin_limit;
     long long *trace;  // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
@@ -49,7 +50,10 @@ struct FwdParams {
 // SPLIT 0: waves split K   (MT m-tiles, NTW n-tiles per WG, 4 partial sums)
 // SPLIT 1: waves split N   (MT m-tiles per WG, NTW n-tiles per wave, 4*NTW per WG)
 // SPLIT 2: waves split M   (MT m-tiles per wave, 4*MT per WG, one n-tile; no cross-WG sync)
-template <typename T, int MT, int NTW, int SPLIT, bool VIO>
+// NKW > 0 (SPLIT 0 only): every wave keeps its share of the W_h slice -- MT x NKW operand
+// fragments, k-steps wave, wave+4, ... -- in registers instead of re-reading it from LDS every
+// timestep (the LDS reads of a 128 KiB slice alone take ~0.4 us per step).  Needs KS <= 4*NKW.
+template <typename T, int MT, int NTW, int SPLIT, bool VIO, int NKW = 0>
 __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const FwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
@@ -61,6 +65,8 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     constexpr int IPT = (TILES + 3) / 4;             // (tile, lane) items per thread
     constexpr int HT = 4 * MTT, BT = 16 * NT;
     constexpr int CH = 8 / NTW;                      // k-steps fetched per batch of loads
+    constexpr bool WREG = NKW > 0;
+    static_assert(!WREG || SPLIT == 0, "register-resident weights: K-split kernels only");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -109,6 +115,12 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #ifdef FASTLSTM_TIMELINE
     long long *tl = reinterpret_cast<long long *>(tiles + (SYNC ? 1 : 2) * TILE_BYTES + 64);
     for (int idx = tid; idx < 256; idx += kThreads) tl[idx] = 0;
+    __syncthreads();
+    if (tid == 0) {   // event 15 of (step 200, wave 0): the XCD this workgroup runs on
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        tl[15] = (long long)(xcc & 15u);
+    }
 #define FASTLSTM_TP(ev)                                                                              \
     do {                                                                                             \
         if (lane == 0 && t >= 200 && t < 204) tl[((t - 200) * 4 + wave) * 16 + (ev)] = (long long)wall_clock64(); \
@@ -153,6 +165,17 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         }
     }
     __syncthreads();
+    u32x4 wreg[WREG ? MT : 1][WREG ? NKW : 1];   // this wave's fragments of the slice (zero past KS)
+    if constexpr (WREG) {
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int ki = 0; ki < NKW; ++ki) {
+                const int ks = wave + 4 * ki;
+                const unsigned woff = ks < KS ? (unsigned)((a * KS + ks) * kWave + lane) * 16u : zero_off + lane * 16u;
+                wreg[a][ki] = *reinterpret_cast<const u32x4 *>(Wl + woff);
+            }
+    }
 
     // ---- per-thread items: (tile = wave + 4m, lane) -> (unit, batch row) -------------
     float c_state[IPT];
@@ -345,8 +368,31 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 }
             }
         };
-        if (coherent) kloop(std::true_type{});
-        else kloop(std::false_type{});
+        // register-resident weights: all NKW operand blocks of this wave are requested at once
+        auto kloop_wreg = [&](auto coh) {
+            constexpr bool COH = decltype(coh)::value;
+            u32x4 bq[WREG ? NKW : 1][NTW];
+#pragma unroll
+            for (int ki = 0; ki < (WREG ? NKW : 0); ++ki) {
+                const int ks = min(wave + 4 * ki, KS - 1);   // past the end: any valid block (its weights are zero)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i)
+                    bq[ki][i] = xch.template load16<COH>(xb + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
+            }
+#pragma unroll
+            for (int ki = 0; ki < (WREG ? NKW : 0); ++ki)
+#pragma unroll
+                for (int a = 0; a < MT; ++a)
+#pragma unroll
+                    for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
+        };
+        if constexpr (WREG) {
+            if (coherent) kloop_wreg(std::true_type{});
+            else kloop_wreg(std::false_type{});
+        } else {
+            if (coherent) kloop(std::true_type{});
+            else kloop(std::false_type{});
+        }
 #ifdef FASTLSTM_TIMELINE
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 #endif
