@@ -1,11 +1,13 @@
 // extern "C" entry points of libfastlstm_hip.so (declared in include/fastlstm_hip.h).
 // Every function validates its arguments before the first HIP call.
 #include <atomic>
+#include <mutex>
 
 #include "gemm.hpp"
 #include "internal.hpp"
 #include "recurrent_bwd.hpp"
 #include "recurrent_fwd.hpp"
+#include "recurrent_fwd_xcd.hpp"
 
 using namespace fastlstm;
 
@@ -26,10 +28,47 @@ int check_dims(int T, int B, int I, int H) {
 
 struct DeviceInfo {
     int num_cus = 0, lds = 0;
+    int xcd_round_robin = 0;   // 1: workgroup i of a launch runs on XCD i % 8 (probed once)
 };
 
+// Every workgroup reports the XCD it runs on (hardware register XCC_ID).
+__global__ void xcc_probe_kernel(int *out) {
+    if (threadIdx.x == 0) {
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        out[blockIdx.x] = (int)(xcc & 15u);
+    }
+}
+
+// 1 when the device has 8 XCDs x 32 CUs and deals the workgroups of a launch to the XCDs in turn.
+// Uses pinned host memory the kernel writes directly: no device allocation.
+int probe_xcd_round_robin(int num_cus) {
+    if (num_cus != kNumXcd * 32) return 0;
+    const int n = 4 * num_cus;
+    int *buf = nullptr;
+    if (hipHostMalloc(reinterpret_cast<void **>(&buf), n * sizeof(int), hipHostMallocMapped) != hipSuccess) return 0;
+    for (int i = 0; i < n; ++i) buf[i] = -1;
+    int ok = 0;
+    int *dptr = nullptr;
+    if (hipHostGetDevicePointer(reinterpret_cast<void **>(&dptr), buf, 0) == hipSuccess) {
+        hipLaunchKernelGGL(xcc_probe_kernel, dim3(n), dim3(64), 0, nullptr, dptr);
+        if (hipGetLastError() == hipSuccess && hipDeviceSynchronize() == hipSuccess) {
+            ok = 1;
+            for (int i = 0; i < n; ++i)
+                if (buf[i] != i % kNumXcd) ok = 0;
+        }
+    }
+    (void)hipHostFree(buf);
+    return ok;
+}
+
+DeviceInfo g_device_cache[64];
+void device_info_set_xcd(int device, int rr) {
+    if (device >= 0 && device < 64) g_device_cache[device].xcd_round_robin = rr;
+}
+
 int device_info(int device, DeviceInfo *out) {
-    static DeviceInfo cache[64];
+    DeviceInfo *cache = g_device_cache;
     if (device < 0) {
         if (hipGetDevice(&device) != hipSuccess) return FASTLSTM_ERR_HIP;
     }
@@ -40,10 +79,27 @@ int device_info(int device, DeviceInfo *out) {
             hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess)
             return FASTLSTM_ERR_HIP;
         cache[device].lds = lds;
+        cache[device].xcd_round_robin = -1;   // probed on first use by a planning call (synchronises once)
         cache[device].num_cus = cus;
     }
     *out = cache[device];
     return FASTLSTM_OK;
+}
+
+// The probe synchronises the device, so it runs from fastlstm_plan_device (a host-side planning
+// call) and never from a launch call, which may be under stream capture.
+void probe_device(int device) {
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    DeviceInfo di;
+    if (device_info(device, &di) != FASTLSTM_OK || di.xcd_round_robin >= 0) return;
+    int cur = 0;
+    if (hipGetDevice(&cur) != hipSuccess) return;
+    if (device < 0) device = cur;
+    if (device != cur && hipSetDevice(device) != hipSuccess) return;
+    const int rr = probe_xcd_round_robin(di.num_cus);
+    if (device != cur) (void)hipSetDevice(cur);
+    device_info_set_xcd(device, rr);
 }
 
 typedef hipError_t (*FwdLauncher)(const FwdParams &, int, int, int, int, int, hipStream_t, int *);
@@ -55,19 +111,78 @@ BwdLauncher bwd_launcher(int dtype) {
     return dtype == FASTLSTM_FP32 ? launch_bwd_f32 : (dtype == FASTLSTM_FP16 ? launch_bwd_f16 : launch_bwd_bf16);
 }
 
+typedef hipError_t (*FwdXcdLauncher)(const FwdXcdParams &, int, int, int, int, int, int, hipStream_t, int *);
+
+// The XCD-local forward kernel, when the device deals workgroups to XCDs in turn, the shape fits
+// (see recurrent_fwd_xcd.hpp) and the workspace holds a ring of T+1 slots.  Returns 1 when it
+// does not apply, else a fastlstm_status.
+int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
+                int H, int dtype, hipStream_t stream) {
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return 1;
+    const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    if (H % kstep) return 1;
+    const int KS = H / kstep;
+    int nkw = cdiv(KS, 4) <= 4 ? 4 : (cdiv(KS, 4) <= 8 ? 8 : 0);   // k-steps per wave with 4 waves
+    if (!nkw) return 1;
+    int ht = 0, ntw = 0;
+    const int hts[3] = {8, 16, 32};
+    for (int hi = 0; hi < 3 && !ht; ++hi) {
+        const int c = hts[hi];
+        if (H % c || H / c > 32 || (c / 4) * nkw > 64 || c * s < 16) continue;
+        const int groups_max = kNumXcd * (32 / (H / c));
+        if (cdiv(B, 16) <= groups_max) { ht = c; ntw = 1; }
+        else if (cdiv(B, 32) <= groups_max) { ht = c; ntw = 2; }
+    }
+    if (!ht) return 1;
+    const int mt = ht / 4, n_ht = H / ht, bt = 16 * ntw, n_groups = cdiv(B, bt);
+    // more than 32 fragments per wave: 8 waves share the slice, so that registers remain for the operand loads
+    int nwv = 4;
+    if (mt * nkw > 32) { nwv = 8; nkw /= 2; }
+    const size_t xslot = (size_t)n_groups * ntw * KS * kFragBytes;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)(T + 1) * xslot) return 1;
+    const int gseg = ht * s;
+    int lds = nwv * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
+#ifdef FASTLSTM_TIMELINE
+    lds += 4096;
+#endif
+    FwdXcdParams p{};
+    p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);
+    p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = n_ht; p.gpx = 32 / n_ht; p.n_groups = n_groups; p.KS = KS;
+    p.spin_limit = spin_limit_ticks();
+    p.trace = g_rec_trace;
+    FwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_fwd_xcd_f32
+                                                   : (dtype == FASTLSTM_FP16 ? launch_fwd_xcd_f16 : launch_fwd_xcd_bf16);
+    int occ = 0;
+    if (launch(p, mt, nkw, ntw, nwv, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (occ < 1) return 1;
+    // every CU gets one workgroup (a workgroup takes the whole register file); those without a role return at once
+    if (launch(p, mt, nkw, ntw, nwv, di.num_cus, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    return FASTLSTM_OK;
+}
+
 }  // namespace
 }  // namespace fastlstm
 
 extern "C" {
 
-int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan) {
+static int plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan, bool may_probe) {
     if (!plan) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
     DeviceInfo di;
     int rc = device_info(device, &di);
     if (rc) return rc;
+    if (may_probe && di.xcd_round_robin < 0) probe_device(device);
     return fastlstm_plan_for(di.num_cus, di.lds, B, H, dtype, backward, plan);
+}
+
+int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan) {
+    return plan_device(device, B, H, dtype, backward, plan, true);
 }
 
 int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int T,
@@ -164,11 +279,15 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     if (!aligned16(ifgo) || !aligned16(out) || !aligned16(cell) || !aligned16(Wh) || !aligned16(ws))
         return FASTLSTM_ERR_ALIGN;
     fastlstm_plan pl;
-    if (int rc = fastlstm_plan_device(-1, B, H, dtype, 0, &pl)) return rc;
+    if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     const bool sync = pl.wave_split != 2;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
+    if (sync) {
+        const int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+        if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
+    }
     FwdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -208,7 +327,7 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     FwdLauncher launch = fwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
-        p.flags = reinterpret_cast<int *>(wsb + 1024 + (size_t)c * flags_bytes);
+        p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
         p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
         p.b_base = bt0 * pl.bt;
@@ -233,7 +352,7 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
         !aligned16(d_ifgo) || !aligned16(Wh) || !aligned16(ws))
         return FASTLSTM_ERR_ALIGN;
     fastlstm_plan pl;
-    if (int rc = fastlstm_plan_device(-1, B, H, dtype, 1, &pl)) return rc;
+    if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     const bool sync = pl.wave_split != 2;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
@@ -268,7 +387,7 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     BwdLauncher launch = bwd_launcher(dtype);
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
-        p.flags = reinterpret_cast<int *>(wsb + 1024 + (size_t)c * flags_bytes);
+        p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
         p.n_bt = pl.n_btiles;
         p.b_base = bt0 * pl.bt;

@@ -120,6 +120,11 @@ struct WsHeader {
 };
 static_assert(sizeof(WsHeader) == 256, "workspace header is 256 bytes");
 
+// Recurrence workspace: header block (1 KiB, WsHeader in front) | 64 KiB of L2 barrier counters of
+// the XCD-local kernels (plans with a cross-CU barrier only) | flags | exchange slots.
+constexpr size_t kWsHeaderBytes = 1024;
+constexpr size_t kWsCounterBytes = 65536;
+
 long long spin_limit_ticks();
 
 }  // namespace fastlstm

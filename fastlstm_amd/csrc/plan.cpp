@@ -61,7 +61,8 @@ int bwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync) {
     return lds;
 }
 
-// Workspace layout: header (1 KiB) | flags of every batch chunk | exchange ring of every chunk.
+// Workspace layout: header (1 KiB) | L2 barrier counters (64 KiB) | flags of every batch chunk |
+// exchange ring of every chunk.  Without a cross-CU barrier: the header only.
 size_t recurrent_flags_bytes(int n_bt, int n_ht) {
     return align_up((size_t)n_bt * align_up((size_t)n_ht, 64) * sizeof(int), 1024);
 }
@@ -72,9 +73,8 @@ size_t recurrent_slot_bytes(int H, int dtype, int bt, int n_bt, bool backward) {
 }
 size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync,
                           int slots) {
-    size_t ws = 1024;  // header (256 B used)
-    if (!sync) return ws;
-    return ws + (size_t)chunks * (recurrent_flags_bytes(n_bt, n_ht) +
+    if (!sync) return kWsHeaderBytes;
+    return kWsHeaderBytes + kWsCounterBytes + (size_t)chunks * (recurrent_flags_bytes(n_bt, n_ht) +
                                   (size_t)slots * recurrent_slot_bytes(H, dtype, bt, n_bt, backward));
 }
 // Slots of a full history ring (one per exchanged version), capped so that one launch's ring
@@ -180,7 +180,7 @@ extern "C" int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int d
     plan->wave_split = best.split;
     plan->lds_bytes = best.lds;
     plan->ws_bytes = recurrent_ws_bytes(H, dtype, best.bt, best.n_bt, best.n_ht, best.chunks, backward != 0, true, 2);
-    plan->ws_zero_bytes = 1024 + (size_t)best.chunks * recurrent_flags_bytes(best.n_bt, best.n_ht);
+    plan->ws_zero_bytes = kWsHeaderBytes + kWsCounterBytes + (size_t)best.chunks * recurrent_flags_bytes(best.n_bt, best.n_ht);
     plan->ring_needs_zero = (B % 16 != 0 || K % KSTEP != 0) ? 1 : 0;
     return FASTLSTM_OK;
 }
@@ -189,6 +189,12 @@ extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, 
     if (!plan || T <= 0 || H <= 0 || !dtype_ok(dtype)) return 0;
     if (plan->wave_split == 2) return plan->ws_bytes;
     const size_t slot = recurrent_slot_bytes(H, dtype, plan->bt, plan->n_btiles, backward != 0);
-    return recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks, backward != 0,
-                              true, recurrent_full_slots(T, slot, backward != 0));
+    const int slots = recurrent_full_slots(T, slot, backward != 0);
+    size_t ws = recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks,
+                                   backward != 0, true, slots);
+    // the XCD-local kernels lay their ring out for batch tiles of 16 or 32 rows: one tile more at most
+    const int KS = cdiv(backward ? 4 * H : H, kstep_of(dtype));
+    ws = std::max(ws, kWsHeaderBytes + kWsCounterBytes +
+                          (size_t)slots * (plan->batch_chunks * slot + 2 * (size_t)KS * kFragBytes));
+    return ws;
 }

@@ -1,0 +1,368 @@
+// Persistent forward kernel, XCD-local form: the hidden tiles of one batch tile all run on ONE
+// of the 8 XCDs of an MI355X and exchange h_t through that XCD's L2 instead of through memory.
+//
+// Same mathematics and the same results as lstm_fwd_persistent_kernel (which replaces
+// fastlstm/kernels.py:414-663); what differs is where the data travels:
+//  * placement: the hardware deals workgroup i to XCD i % 8.  A barrier group takes its members
+//    from the workgroups of one XCD (i % 8 == group % 8); workgroups that are not needed return
+//    at once.  One workgroup fills the register file of a CU, so the up to 32 members of a group
+//    sit on the 32 CUs of their XCD.  The host verifies i % 8 == XCC_ID once per device before
+//    it selects this kernel;
+//  * exchange data: ordinary stores (the vector L1 writes through to L2) and ordinary loads.  A
+//    load may hit in the CU's L1, which nobody keeps coherent, so every timestep writes a slot
+//    of its own (ring of T + 1 slots): an address is only read after its single write;
+//  * barrier: counters in L2.  Atomics execute in the L2, never in an L1: a member adds 1 to
+//    each of kXcdReplicas counters of its group after its stores were acknowledged, and polls
+//    one of them (its index % replicas) with an atomic add of 0;
+//  * W_h: a slice of 4*MT units x 4 gates x H no longer has to fit in LDS next to the peers'
+//    (32 CUs x 160 KiB < 8 MiB for H = 1024): every wave keeps its K-share of the slice, MT x NKW
+//    operand fragments, in registers (up to 256 of the 512 per lane).
+// Requirements (host): H a multiple of the tile width and of 16 bytes' worth of elements,
+// H / (4*MT) <= 32 members, ceil(H / KSTEP) <= 4*NKW k-steps, all batch tiles in one launch.
+#pragma once
+#include <type_traits>
+
+#include "recurrent_common.hpp"
+
+namespace fastlstm {
+
+constexpr int kXcdReplicas = 8;          // counters per barrier group, 128 bytes apart
+constexpr int kXcdCounterStride = 32;    // ints between replicas
+constexpr int kXcdGroupStride = kXcdReplicas * kXcdCounterStride;   // ints between groups (1 KiB)
+constexpr int kXcdMaxGroups = 64;
+static_assert((size_t)kXcdMaxGroups * kXcdGroupStride * sizeof(int) == kWsCounterBytes, "counter region of the workspace");
+
+struct FwdXcdParams {
+    void *ifgo;        // [T,B,4H] in: x.Wx^T+b, out: full pre-activations
+    void *out, *cell;  // [T+1,B,H]
+    const void *Wh;    // [4H,H]
+    WsHeader *hdr;
+    int *counters;        // [groups][kXcdReplicas][kXcdCounterStride], zero at launch
+    unsigned char *xbuf;  // ring: [T+1 slots][groups][NT][KS] operand blocks
+    int T, B, H;
+    int n_ht;          // members of a barrier group (<= 32)
+    int gpx;           // groups per XCD (32 / n_ht)
+    int n_groups;      // batch tiles of this launch (<= 8 * gpx)
+    int KS;            // k-steps covering H
+    long long spin_limit;
+    long long *trace;  // diagnostic build only
+};
+
+// Exchange ring accessed with ordinary (cached) 16-byte loads and ordinary stores.
+struct XchgL2 {
+    __amdgpu_buffer_rsrc_t rsrc;
+    __device__ __forceinline__ XchgL2(unsigned char *b, unsigned bytes)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(b, 0, bytes, 0x00020000)) {}
+    __device__ __forceinline__ u32x4 load16(unsigned off) const {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+    }
+    template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
+        if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rsrc, off, 0, 0);
+        else __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc, off, 0, 0);
+    }
+};
+
+// Lane 0 of the calling wave polls `counter` in L2 until it reaches `target`.  Bounded like
+// wait_versions.
+__device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader *hdr, long long spin_limit,
+                                             int group, int step) {
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        long long t0 = 0;
+        int polls = 0;
+        for (;;) {
+            int v;
+            const int zero = 0;
+            // an atomic with return value: executed by the L2, whatever the L1 holds
+            asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)"
+                         : "=v"(v)
+                         : "v"(counter), "v"(zero)
+                         : "memory");
+            if (v >= target) break;
+            __builtin_amdgcn_s_sleep(1);
+            if (++polls >= 64 || spin_limit <= 1) {
+                polls = 0;
+                if (__hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+                const long long now = (long long)wall_clock64();
+                if (t0 == 0 && spin_limit > 1) {
+                    t0 = now;
+                } else if (now - t0 > spin_limit) {
+                    hdr->timeout_group = group;
+                    hdr->timeout_step = step;
+                    __hip_atomic_store(&hdr->abort_flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // compiler ordering only
+}
+
+// NWV waves per workgroup split K: wave w owns k-steps w, w + NWV, ... (NKW of them).  8 waves (two
+// per SIMD, 256 registers each) halve the fragments a wave has to hold, which leaves registers
+// to keep all operand loads of a step in flight.
+template <typename T, int MT, int NKW, int NTW, int NWV>
+__global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdParams p) {
+    constexpr int NTHR = kWave * NWV;
+    using E = Elem<T>;
+    constexpr bool ACC = (E::DT == FASTLSTM_FP32);
+    constexpr int NT = NTW, TILES = MT * NT;
+    constexpr int IPT = (TILES + NWV - 1) / NWV;     // (tile, lane) items per thread
+    constexpr int HT = 4 * MT, BT = 16 * NT;
+    constexpr int GSEG = HT * E::BYTES;              // bytes of one gate segment of a row (>= 16)
+    static_assert(GSEG >= 16 && GSEG % 16 == 0, "tile I/O needs 16-byte gate segments");
+    constexpr int GROW = 4 * GSEG + 16, SROW = GSEG + 16;
+    constexpr int PPSEG = GSEG / 16;
+    constexpr int GPIECES = BT * 4 * PPSEG, SPIECES = BT * PPSEG;
+    constexpr int IOT = NTHR - kWave;                // waves 1.. move the tiles, wave 0 polls
+    constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, n = lane & 15;
+    const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+
+    // ---- placement: group g lives on XCD g % 8 ------------------------------------------
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int gl = slot / p.n_ht, j = slot % p.n_ht;
+    const int g = gl * kNumXcd + xcd;
+    if (gl >= p.gpx || g >= p.n_groups) return;
+    const int u0 = j * HT, b0 = g * BT;
+
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                  // [NWV][TILES][64]
+    unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * TILES * kWave);   // gates, h, c tiles
+    const int io_tid = tid - kWave;
+
+    T *ifgo = static_cast<T *>(p.ifgo);
+    T *out = static_cast<T *>(p.out);
+    T *cell = static_cast<T *>(p.cell);
+    const T *Wh = static_cast<const T *>(p.Wh);
+
+#ifdef FASTLSTM_TIMELINE
+    long long *tl = reinterpret_cast<long long *>(tiles + BT * GROW + 2 * BT * SROW + 64);
+    for (int idx = tid; idx < 256; idx += NTHR) tl[idx] = 0;
+    __syncthreads();
+    if (tid == 0) {
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        tl[15] = (long long)(xcc & 15u);
+    }
+#define FASTLSTM_TP(ev)                                                                              \
+    do {                                                                                             \
+        if (lane == 0 && wave < 4 && t >= 200 && t < 204) tl[((t - 200) * 4 + wave) * 16 + (ev)] = (long long)wall_clock64(); \
+    } while (0)
+#else
+#define FASTLSTM_TP(ev) do {} while (0)
+#endif
+
+    // ---- prologue 1: this wave's fragments of the W_h slice, global -> registers ---------
+    // fragment (m-tile a, k-step ks): lane (q, r) holds row r = (unit a*4 + r/4, gate r%4),
+    // k = ks*KSTEP + q*EPL .. + EPL-1, i.e. 16 contiguous bytes of W_h
+    u32x4 wreg[MT][NKW];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki) {
+            const int ks = wave + NWV * ki;
+            const int unit = u0 + a * 4 + (n >> 2), gate = n & 3;
+            const int k0 = ks * E::KSTEP + q * E::EPL;
+            const bool ok = ks < KS && k0 < H;   // H % EPL == 0: a piece is inside or outside as a whole
+            const size_t off = ok ? ((size_t)gate * H + unit) * H + k0 : 0;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(Wh + off);
+            wreg[a][ki] = ok ? v : u32x4{0u, 0u, 0u, 0u};
+        }
+
+    // ---- per-thread items: (tile = wave + 4m, lane) -> (unit, batch row) -------------
+    float c_state[IPT];
+    size_t off_h[IPT];
+    int xoff[IPT], goff[IPT], soff[IPT];
+    bool valid[IPT];
+#pragma unroll
+    for (int m = 0; m < IPT; ++m) {
+        const int tile = wave + NWV * m;
+        const int mt = tile / NT, nt = tile % NT;
+        const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
+        valid[m] = (tile < TILES) && b < B;
+        off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
+        xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
+        goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
+        soff[m] = (nt * 16 + n) * SROW + (mt * 4 + q) * E::BYTES;
+        c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
+    }
+
+    // exchange ring: slot v holds h_{v-1}... slot s = version index: h_s for s = 0..T
+    const unsigned xgrp = (unsigned)g * NT * KS * kFragBytes;
+    const size_t xslot = (size_t)p.n_groups * NT * KS * kFragBytes;
+    int *grp_counters = p.counters + (size_t)g * kXcdGroupStride;
+    int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
+
+    auto publish = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's exchange stores have reached the L2
+        __syncthreads();
+        if (tid < kXcdReplicas)
+            __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+
+    // ---- prologue 2: publish h_0 (slot 0) -------------------------------------------------
+    {
+        const XchgL2 x0(p.xbuf, (unsigned)xslot);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m)
+            if (valid[m]) x0.store_elem(xgrp + xoff[m], out[off_h[m]]);
+        publish();
+    }
+
+    const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
+
+    // ---- coalesced tile I/O (see lstm_fwd_persistent_kernel) --------------------------------
+    constexpr int PD = 2;
+    u32x4 gpre[PD][GPT];
+    const size_t tile_org = (size_t)b0 * 4 * H + u0;
+    auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
+        if (io_tid < 0) return;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            const bool ok = pc < GPIECES && b0 + row < B;
+            const size_t off = ok ? (size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES) : 0;
+            dst[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + tile_org + off);
+        }
+    };
+    auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            if (io_tid >= 0 && pc < GPIECES)
+                *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
+        }
+    };
+    auto tiles_to_global = [&](int t, const unsigned char *gt) {
+        const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+                *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
+                                           k * (16 / E::BYTES)) =
+                    *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / PPSEG, k = pc % PPSEG;
+            if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
+                const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
+                *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+            }
+        }
+    };
+    auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (t < T_) fetch_tile(t, gpre[u]);
+    };
+    prefetch(0, std::integral_constant<int, 0>{});
+    prefetch(1, std::integral_constant<int, 1>{});
+
+    auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        unsigned char *gt = tiles;
+        FASTLSTM_TP(0);
+        if (wave == 0) wait_counter(my_counter, p.n_ht * (t + 1), p.hdr, p.spin_limit, g, t);
+        FASTLSTM_TP(1);
+        __syncthreads();
+        FASTLSTM_TP(2);
+
+        // ---- acc[a][i] += Wslice(a) . h_{t-1}(i)^T over this wave's k-steps: all operand blocks
+        // of the wave are requested at once, the weights come from registers
+        const XchgL2 xr(p.xbuf + (size_t)t * xslot, (unsigned)xslot);
+        f32x4 acc[MT][NTW];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        u32x4 bq[NKW][NTW];
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki) {
+            const int ks = min(wave + NWV * ki, KS - 1);   // past the end: any valid block (its weights are zero)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) bq[ki][i] = xr.load16(xgrp + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
+        }
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki)
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
+#ifdef FASTLSTM_TIMELINE
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#endif
+        FASTLSTM_TP(3);
+
+        // ---- partial sums -> LDS, then every (tile, lane) item sums the NWV partials ---------
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) red[(wave * TILES + a * NT + i) * kWave + lane] = acc[a][i];
+        tile_to_lds(gpre[u], gt);
+        FASTLSTM_TP(4);
+        __syncthreads();
+        FASTLSTM_TP(5);
+
+        const XchgL2 xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            const int tile = wave + NWV * m;
+            if (tile < TILES) {
+                f32x4 s = red[tile * kWave + lane];
+#pragma unroll
+                for (int pp = 1; pp < NWV; ++pp) s += red[(pp * TILES + tile) * kWave + lane];
+                if (valid[m]) {
+                    T *gl_ = reinterpret_cast<T *>(gt + goff[m]);   // the item's 4 gates in the LDS tile
+                    const float pi = E::to_f32(gl_[0]) + s[0];
+                    const float pf = E::to_f32(gl_[HT]) + s[1];
+                    const float pg = E::to_f32(gl_[2 * HT]) + s[2];
+                    const float po = E::to_f32(gl_[3 * HT]) + s[3];
+                    const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
+                    const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
+                    c_state[m] = c1;
+                    const T hv = E::from_f32(h1);
+                    xw.store_elem(xgrp + xoff[m], hv);
+                    gl_[0] = E::from_f32(pi);
+                    gl_[HT] = E::from_f32(pf);
+                    gl_[2 * HT] = E::from_f32(pg);
+                    gl_[3 * HT] = E::from_f32(po);
+                    *reinterpret_cast<T *>(gt + BT * GROW + soff[m]) = hv;
+                    *reinterpret_cast<T *>(gt + BT * GROW + BT * SROW + soff[m]) = E::from_f32(c1);
+                }
+            }
+        }
+        FASTLSTM_TP(6);
+#ifdef FASTLSTM_TIMELINE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        FASTLSTM_TP(7);
+#endif
+        if (t + 1 < T_) publish();
+        else __syncthreads();   // last step: the tiles still have to be complete
+        FASTLSTM_TP(8);
+        tiles_to_global(t, gt);
+        prefetch(t + PD, uc);
+        FASTLSTM_TP(9);
+    };
+    for (int t0 = 0; t0 < T_; t0 += PD) {
+        step(t0, std::integral_constant<int, 0>{});
+        if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
+    }
+#ifdef FASTLSTM_TIMELINE
+    __syncthreads();
+    if (p.trace)
+        for (int idx = tid; idx < 256; idx += NTHR) p.trace[(size_t)blockIdx.x * 256 + idx] = tl[idx];
+#endif
+#undef FASTLSTM_TP
+}
+
+}  // namespace fastlstm

@@ -15,7 +15,8 @@ struct OccKey {
 };
 
 template <typename K, typename P>
-hipError_t launch_one(K kern, const P &p, int grid, int lds, hipStream_t s, int *max_blocks_per_cu) {
+hipError_t launch_one(K kern, const P &p, int grid, int lds, hipStream_t s, int *max_blocks_per_cu,
+                      int threads = kThreads) {
     // the LDS attribute and the occupancy of (kernel, LDS size) are looked up once
     static std::map<OccKey, int> cache;
     static std::mutex mu;
@@ -28,7 +29,7 @@ hipError_t launch_one(K kern, const P &p, int grid, int lds, hipStream_t s, int 
             hipError_t e = hipFuncSetAttribute(key.fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
             if (e != hipSuccess) return e;
             int nb = 0;
-            e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, kThreads, (size_t)lds);
+            e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, threads, (size_t)lds);
             if (e != hipSuccess) return e;
             it = cache.emplace(key, nb).first;
         }
@@ -36,7 +37,7 @@ hipError_t launch_one(K kern, const P &p, int grid, int lds, hipStream_t s, int 
     }
     if (max_blocks_per_cu) *max_blocks_per_cu = occ;
     if (grid <= 0) return hipSuccess;  // query only
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), (size_t)lds, s, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), (size_t)lds, s, p);
     return hipGetLastError();
 }
 

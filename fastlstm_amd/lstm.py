@@ -60,20 +60,21 @@ def _plan(device, B, H, code, backward):
     return plan
 
 
-# Largest history ring (one exchange slot per timestep) the backward pass may allocate.
+# Largest exchange ring (one slot per timestep) a recurrent call may allocate.
 RING_MAX_BYTES = 1 << 30
 
 
 def _workspace(plan, T, H, code, backward, device):
-    """Recurrence workspace, flag part zero-filled.
+    """Recurrence workspace, with the part the kernels need zeroed (header, counters, flags).
 
-    Forward: flags + a two-slot exchange buffer (a few hundred KiB).  Backward, when the
-    workgroups synchronise across CUs: a ring with one slot per timestep, sized by
-    fastlstm_recurrent_workspace_bytes(), which lets the kernel read d_ifgo[t] through the caches
-    (one fetch per XCD instead of one per workgroup; ~8 % faster at B=64, H=1024 on MI355X).  The
-    forward kernel exchanges a quarter of the data and measured no faster with a ring."""
-    if backward and plan.wave_split != 2:
-        ring = _lib.load().fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1)
+    Plans whose workgroups synchronise across CUs get a ring with one exchange slot per timestep,
+    sized by fastlstm_recurrent_workspace_bytes(): no address of it is read before its only
+    write, so the kernels can read the exchange data through the caches.  The forward pass then
+    uses the XCD-local kernel where the shape allows (the barrier group on one XCD, exchange
+    through its L2); the backward pass reads d_ifgo[t] once per XCD instead of once per CU.
+    Without room for the ring (RING_MAX_BYTES) the two-slot workspace of the plan is used."""
+    if plan.wave_split != 2:
+        ring = _lib.load().fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1 if backward else 0)
         if plan.ws_bytes < ring <= RING_MAX_BYTES:
             ws = torch.empty(ring, dtype=torch.uint8, device=device)
             zero = ring if plan.ring_needs_zero else plan.ws_zero_bytes

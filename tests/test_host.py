@@ -94,7 +94,7 @@ def test_tiling_rule_invariants(dtype, backward):
             if p.n_htiles > 1:
                 flags = -(-(p.n_btiles * (-(-p.n_htiles // 64) * 64) * 4) // 1024) * 1024
                 xbuf = 2 * p.n_btiles * (p.bt // 16) * ks * 1024
-                assert p.ws_bytes == 1024 + p.batch_chunks * (flags + xbuf)
+                assert p.ws_bytes == 1024 + 65536 + p.batch_chunks * (flags + xbuf)
 
 
 def test_tiling_rule_headline_configs():
