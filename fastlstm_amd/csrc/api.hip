@@ -123,7 +123,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     if (H % kstep) return 1;
     const int KS = H / kstep;
-    int nkw = cdiv(KS, 4) <= 4 ? 4 : (cdiv(KS, 4) <= 8 ? 8 : 0);   // k-steps per wave with 4 waves
+    const int nkw = cdiv(KS, 4) <= 4 ? 4 : (cdiv(KS, 4) <= 8 ? 8 : 0);   // k-steps per K-share (4 shares)
     if (!nkw) return 1;
     int ht = 0, ntw = 0;
     const int hts[3] = {8, 16, 32};
@@ -137,12 +137,11 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     if (!ht) return 1;
     const int mt = ht / 4, n_ht = H / ht, bt = 16 * ntw, n_groups = cdiv(B, bt);
     // more than 32 fragments per wave: 8 waves share the slice, so that registers remain for the operand loads
-    int nwv = 4;
-    if (mt * nkw > 32) { nwv = 8; nkw /= 2; }
+    const int nwv = mt * nkw > 32 ? 8 : 4;
     const size_t xslot = (size_t)n_groups * ntw * KS * kFragBytes;
     if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)(T + 1) * xslot) return 1;
     const int gseg = ht * s;
-    int lds = nwv * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
+    int lds = 4 * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
 #ifdef FASTLSTM_TIMELINE
     lds += 4096;
 #endif

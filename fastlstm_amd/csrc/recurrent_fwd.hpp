@@ -379,6 +379,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
                 for (int i = 0; i < NTW; ++i)
                     bq[ki][i] = xch.template load16<COH>(xb + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
             }
+            __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first MFMA: one round trip, not NKW
 #pragma unroll
             for (int ki = 0; ki < (WREG ? NKW : 0); ++ki)
 #pragma unroll

@@ -97,12 +97,16 @@ __device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader 
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // compiler ordering only
 }
 
-// NWV waves per workgroup split K: wave w owns k-steps w, w + NWV, ... (NKW of them).  8 waves (two
-// per SIMD, 256 registers each) halve the fragments a wave has to hold, which leaves registers
-// to keep all operand loads of a step in flight.
+// The waves split K four ways: wave w owns k-steps w % 4, w % 4 + 4, ... (NKW of them).  With
+// NWV = 8 waves (two per SIMD, 256 registers each) the two waves of a K-share split the MT unit
+// tiles between them, which halves the fragments a wave holds and leaves registers to keep all
+// operand loads of a step in flight.
 template <typename T, int MT, int NKW, int NTW, int NWV>
 __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdParams p) {
     constexpr int NTHR = kWave * NWV;
+    constexpr int MW = NWV / 4, MTW = MT / MW;       // M-split ways, unit tiles per wave
+    static_assert(NWV == 4 || NWV == 8, "4 or 8 waves");
+    static_assert(MT % MW == 0, "unit tiles divide among the waves of a K-share");
     using E = Elem<T>;
     constexpr bool ACC = (E::DT == FASTLSTM_FP32);
     constexpr int NT = NTW, TILES = MT * NT;
@@ -128,8 +132,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     if (gl >= p.gpx || g >= p.n_groups) return;
     const int u0 = j * HT, b0 = g * BT;
 
-    f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                  // [NWV][TILES][64]
-    unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * TILES * kWave);   // gates, h, c tiles
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                  // [4][TILES][64]
+    unsigned char *tiles = reinterpret_cast<unsigned char *>(red + 4 * TILES * kWave);   // gates, h, c tiles
     const int io_tid = tid - kWave;
 
     T *ifgo = static_cast<T *>(p.ifgo);
@@ -157,13 +161,14 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     // ---- prologue 1: this wave's fragments of the W_h slice, global -> registers ---------
     // fragment (m-tile a, k-step ks): lane (q, r) holds row r = (unit a*4 + r/4, gate r%4),
     // k = ks*KSTEP + q*EPL .. + EPL-1, i.e. 16 contiguous bytes of W_h
-    u32x4 wreg[MT][NKW];
+    const int kq = wave & 3, mh = wave >> 2;         // K-share and M-half of this wave
+    u32x4 wreg[MTW][NKW];
 #pragma unroll
-    for (int a = 0; a < MT; ++a)
+    for (int a = 0; a < MTW; ++a)
 #pragma unroll
         for (int ki = 0; ki < NKW; ++ki) {
-            const int ks = wave + NWV * ki;
-            const int unit = u0 + a * 4 + (n >> 2), gate = n & 3;
+            const int ks = kq + 4 * ki;
+            const int unit = u0 + (mh * MTW + a) * 4 + (n >> 2), gate = n & 3;
             const int k0 = ks * E::KSTEP + q * E::EPL;
             const bool ok = ks < KS && k0 < H;   // H % EPL == 0: a piece is inside or outside as a whole
             const size_t off = ok ? ((size_t)gate * H + unit) * H + k0 : 0;
@@ -280,22 +285,23 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         // ---- acc[a][i] += Wslice(a) . h_{t-1}(i)^T over this wave's k-steps: all operand blocks
         // of the wave are requested at once, the weights come from registers
         const XchgL2 xr(p.xbuf + (size_t)t * xslot, (unsigned)xslot);
-        f32x4 acc[MT][NTW];
+        f32x4 acc[MTW][NTW];
 #pragma unroll
-        for (int a = 0; a < MT; ++a)
+        for (int a = 0; a < MTW; ++a)
 #pragma unroll
             for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
         u32x4 bq[NKW][NTW];
 #pragma unroll
         for (int ki = 0; ki < NKW; ++ki) {
-            const int ks = min(wave + NWV * ki, KS - 1);   // past the end: any valid block (its weights are zero)
+            const int ks = min(kq + 4 * ki, KS - 1);   // past the end: any valid block (its weights are zero)
 #pragma unroll
             for (int i = 0; i < NTW; ++i) bq[ki][i] = xr.load16(xgrp + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
         }
+        __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first MFMA: one round trip, not NKW
 #pragma unroll
         for (int ki = 0; ki < NKW; ++ki)
 #pragma unroll
-            for (int a = 0; a < MT; ++a)
+            for (int a = 0; a < MTW; ++a)
 #pragma unroll
                 for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
 #ifdef FASTLSTM_TIMELINE
@@ -303,11 +309,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
 #endif
         FASTLSTM_TP(3);
 
-        // ---- partial sums -> LDS, then every (tile, lane) item sums the NWV partials ---------
+        // ---- partial sums -> LDS, then every (tile, lane) item sums the 4 partials ---------
 #pragma unroll
-        for (int a = 0; a < MT; ++a)
+        for (int a = 0; a < MTW; ++a)
 #pragma unroll
-            for (int i = 0; i < NTW; ++i) red[(wave * TILES + a * NT + i) * kWave + lane] = acc[a][i];
+            for (int i = 0; i < NTW; ++i) red[(kq * TILES + (mh * MTW + a) * NT + i) * kWave + lane] = acc[a][i];
         tile_to_lds(gpre[u], gt);
         FASTLSTM_TP(4);
         __syncthreads();
@@ -320,7 +326,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
             if (tile < TILES) {
                 f32x4 s = red[tile * kWave + lane];
 #pragma unroll
-                for (int pp = 1; pp < NWV; ++pp) s += red[(pp * TILES + tile) * kWave + lane];
+                for (int pp = 1; pp < 4; ++pp) s += red[(pp * TILES + tile) * kWave + lane];
                 if (valid[m]) {
                     T *gl_ = reinterpret_cast<T *>(gt + goff[m]);   // the item's 4 gates in the LDS tile
                     const float pi = E::to_f32(gl_[0]) + s[0];
