@@ -140,8 +140,14 @@ def main():
     plan_f, plan_b = _lib.Plan(), _lib.Plan()
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
-    ws_f = torch.zeros(plan_f.ws_bytes, dtype=torch.uint8, device=dev)   # what lstm.py allocates per call
-    ws_b = torch.zeros(plan_b.ws_bytes, dtype=torch.uint8, device=dev)
+    # the workspaces lstm.py allocates per call (a one-slot-per-timestep exchange ring when it fits)
+    from fastlstm_amd import lstm as _host
+    ws_f = _host._workspace(plan_f, T, H, code, False, dev)
+    ws_b = _host._workspace(plan_b, T, H, code, True, dev)
+
+    def zero_ws(ws, plan):  # the part a call needs zeroed: header, counters, flags
+        n = ws.numel() if (plan.ring_needs_zero or ws.numel() == plan.ws_bytes) else plan.ws_zero_bytes
+        ws[:n].zero_()
 
     def k1():
         _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
@@ -153,7 +159,7 @@ def main():
 
     def rec_fwd_pre():  # the kernel overwrites ifgo in place and needs zeroed flags
         ifgo.copy_(ifgo0)
-        ws_f.zero_()
+        zero_ws(ws_f, plan_f)
 
     if args.stage == "fwd_recurrence":
         # counter runs (rocprofv3 --pmc): the dominant kernel plus a plain copy of known size
@@ -193,7 +199,7 @@ def main():
                                                ws_b.numel(), T, B, H, code, stream), "bwd")
 
     def rec_bwd_pre():
-        ws_b.zero_(); dh_n.zero_(); dc_n.zero_()
+        zero_ws(ws_b, plan_b); dh_n.zero_(); dc_n.zero_()
 
     def k5():
         _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, stream), "k5")

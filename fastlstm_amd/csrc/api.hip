@@ -7,6 +7,7 @@
 #include "internal.hpp"
 #include "recurrent_bwd.hpp"
 #include "recurrent_fwd.hpp"
+#include "recurrent_bwd_xcd.hpp"
 #include "recurrent_fwd_xcd.hpp"
 
 using namespace fastlstm;
@@ -161,6 +162,50 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     if (occ < 1) return 1;
     // every CU gets one workgroup (a workgroup takes the whole register file); those without a role return at once
     if (launch(p, mt, nkw, ntw, nwv, di.num_cus, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    return FASTLSTM_OK;
+}
+
+typedef hipError_t (*BwdXcdLauncher)(const BwdXcdParams &, int, int, int, int, int, hipStream_t, int *);
+
+// The XCD-local reverse kernel under the same conditions as try_fwd_xcd (ring of T slots).
+int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
+                unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream) {
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return 1;
+    const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    if ((4 * H) % kstep || H % 16) return 1;
+    const int KSB = 4 * H / kstep;
+    const int nkw = cdiv(KSB, 8) <= 4 ? 4 : (cdiv(KSB, 8) <= 8 ? 8 : (cdiv(KSB, 8) <= 16 ? 16 : 0));   // per wave, 8 waves
+    if (!nkw) return 1;
+    int ht = 0, ntw = 0;
+    const int hts[2] = {16, 32};
+    for (int hi = 0; hi < 2 && !ht; ++hi) {
+        const int c = hts[hi];
+        if (H % c || H / c > 32 || (c / 16) * nkw > 32) continue;
+        const int groups_max = kNumXcd * (32 / (H / c));
+        if (cdiv(B, 16) <= groups_max) { ht = c; ntw = 1; }
+        else if (cdiv(B, 32) <= groups_max) { ht = c; ntw = 2; }
+    }
+    if (!ht) return 1;
+    const int mt = ht / 16, n_ht = H / ht, bt = 16 * ntw, n_groups = cdiv(B, bt);
+    const size_t xslot = (size_t)n_groups * ntw * KSB * kFragBytes;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * xslot) return 1;
+    const int gseg = ht * s;
+    const int lds = 8 * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
+    BwdXcdParams p{};
+    p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);
+    p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = n_ht; p.gpx = 32 / n_ht; p.n_groups = n_groups; p.KSB = KSB;
+    p.spin_limit = spin_limit_ticks();
+    BwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_bwd_xcd_f32
+                                                   : (dtype == FASTLSTM_FP16 ? launch_bwd_xcd_f16 : launch_bwd_xcd_bf16);
+    int occ = 0;
+    if (launch(p, mt, nkw, ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (occ < 1) return 1;
+    if (launch(p, mt, nkw, ntw, di.num_cus, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
@@ -356,6 +401,11 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     const bool sync = pl.wave_split != 2;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
+    if (sync) {
+        const int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
+                                   static_cast<hipStream_t>(stream));
+        if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
+    }
     BwdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);

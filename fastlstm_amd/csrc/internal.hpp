@@ -10,6 +10,7 @@ struct GemmParams;
 struct FwdParams;
 struct BwdParams;
 struct FwdXcdParams;
+struct BwdXcdParams;
 
 hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hipStream_t s);
 hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
@@ -29,6 +30,8 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_k
     hipError_t launch_fwd_wreg_##SUF(const FwdParams &p, int mt, int ntw, int grid, int lds,        \
                                      hipStream_t s, int *max_blocks_per_cu);                         \
     hipError_t launch_fwd_xcd_##SUF(const FwdXcdParams &p, int mt, int nkw, int ntw, int nwv, int grid, int lds, \
+                                    hipStream_t s, int *max_blocks_per_cu);                          \
+    hipError_t launch_bwd_xcd_##SUF(const BwdXcdParams &p, int mt, int nkw, int ntw, int grid, int lds, \
                                     hipStream_t s, int *max_blocks_per_cu);
 FASTLSTM_DECL_REC(f32)
 FASTLSTM_DECL_REC(f16)

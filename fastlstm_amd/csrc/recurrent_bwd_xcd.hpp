@@ -1,0 +1,302 @@
+// Persistent reverse-time kernel, XCD-local form: the hidden tiles of one batch tile run on one XCD
+// and exchange d_ifgo[t] through that XCD's L2.  Same mathematics and results as
+// lstm_bwd_persistent_kernel (which replaces fastlstm/kernels.py:1201-1409); placement, exchange
+// ring, L2 counter barrier and the register-resident weight slice follow lstm_fwd_xcd_kernel.
+//
+// Per reverse step s (timestep t = T-1-s) a workgroup of NWV waves, owning 16*MT hidden units and
+// 16*NTW batch rows:
+//   gate backward for its (unit, row) items -> d_ifgo[t] tile (LDS) and exchange slot s (L2)
+//   counter barrier over the group
+//   dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over K = 4H:
+//       the waves split K NWV ways; wave w holds A fragments (MT unit tiles x NKW k-steps
+//       w, w + NWV, ...) of Wh^T in registers and requests its NKW*NTW operand blocks at once
+//   cross-wave sum of the NWV partials through LDS
+// K index = 4 * source unit + gate, as in the general kernel.
+#pragma once
+#include <type_traits>
+
+#include "recurrent_fwd_xcd.hpp"
+
+namespace fastlstm {
+
+struct BwdXcdParams {
+    const void *dout;   // [T,B,H]
+    void *dh, *dc;      // [B,H] in: grads of h_T, c_T; out: grads of h_0, c_0
+    const void *ifgo;   // [T,B,4H]
+    const void *cell;   // [T+1,B,H]
+    void *d_ifgo;       // [T,B,4H]
+    const void *Wh;     // [4H,H]
+    WsHeader *hdr;
+    int *counters;         // [groups][kXcdReplicas][kXcdCounterStride], zero at launch
+    unsigned char *xbuf;   // ring: [T slots][groups][NT][KSB] operand blocks
+    int T, B, H;
+    int n_ht, gpx, n_groups;
+    int KSB;            // k-steps covering 4H
+    long long spin_limit;
+};
+
+template <typename T, int MT, int NKW, int NTW, int NWV>
+__global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdParams p) {
+    using E = Elem<T>;
+    constexpr bool ACC = (E::DT == FASTLSTM_FP32);
+    constexpr int NTHR = kWave * NWV;
+    constexpr int NT = NTW, HT = 16 * MT, BT = 16 * NT;
+    constexpr int IPT = (HT * BT + NTHR - 1) / NTHR;   // (unit, batch row) items per thread
+    constexpr int GSEG = HT * E::BYTES;
+    constexpr int GROW = 4 * GSEG + 16, SROW = GSEG + 16;
+    constexpr int PPSEG = GSEG / 16;
+    constexpr int GPIECES = BT * 4 * PPSEG, SPIECES = BT * PPSEG;
+    constexpr int IOT = NTHR - kWave;                  // wave 0 polls, the others move the tiles
+    constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, r = lane & 15;
+    const int KSB = p.KSB, H = p.H, B = p.B, T_ = p.T;
+
+    // ---- placement: group g lives on XCD g % 8 ------------------------------------------
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int gl = slot / p.n_ht, j = slot % p.n_ht;
+    const int g = gl * kNumXcd + xcd;
+    if (gl >= p.gpx || g >= p.n_groups) return;
+    const int u0 = j * HT, b0 = g * BT;
+
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                    // [NWV][MT][NT][64]
+    unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
+    const int io_tid = tid - kWave;
+
+    const T *dout = static_cast<const T *>(p.dout);
+    const T *ifgo = static_cast<const T *>(p.ifgo);
+    const T *cell = static_cast<const T *>(p.cell);
+    T *d_ifgo = static_cast<T *>(p.d_ifgo);
+    const T *Wh = static_cast<const T *>(p.Wh);
+
+    // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
+    // fragment (unit tile a, k-step ks): lane (q, r) holds row r = unit u0 + 16a + r and
+    // k = ks*KSTEP + q*EPL + e, e < EPL, with k = 4 * source unit + gate
+    u32x4 wreg[MT][NKW];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki) {
+            const int ks = wave + NWV * ki;
+            T tmp[E::EPL];
+#pragma unroll
+            for (int e = 0; e < E::EPL; ++e) {
+                const int k = ks * E::KSTEP + q * E::EPL + e;
+                const int uk = k >> 2, gate = k & 3;
+                const bool ok = ks < KSB && uk < H;
+                const T v = Wh[ok ? ((size_t)gate * H + uk) * H + u0 + a * 16 + r : 0];
+                tmp[e] = ok ? v : E::from_f32(0.f);
+            }
+            wreg[a][ki] = *reinterpret_cast<u32x4 *>(tmp);
+        }
+
+    // ---- per-thread items: it = tid + NTHR*m -> (row n, unit ul, n-tile nt) ----------------
+    float dc_state[IPT], dh_rec[IPT], c1v[IPT];
+    size_t off_h[IPT];
+    int xoff[IPT], roff[IPT], goff[IPT], soff[IPT];
+    bool valid[IPT], pair_lead[IPT];
+    const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
+#pragma unroll
+    for (int m = 0; m < IPT; ++m) {
+        const int it = tid + NTHR * m;
+        const int n = it & 15, rest = it >> 4;
+        const int ul = rest % HT, nt = rest / HT;
+        const int unit = u0 + ul, b = b0 + nt * 16 + n;
+        valid[m] = nt < NT && b < B;
+        off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
+        xoff[m] = (nt < NT ? nt : 0) * KSB * kFragBytes + frag_offset<T>(n, unit * 4);
+        pair_lead[m] = valid[m] && ((ul & 1) == 0);
+        const int a = ul >> 4, ur = ul & 15;
+        roff[m] = ((a * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
+        goff[m] = ((nt < NT ? nt : 0) * 16 + n) * GROW + ul * E::BYTES;
+        soff[m] = ((nt < NT ? nt : 0) * 16 + n) * SROW + ul * E::BYTES;
+        dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
+        dc_state[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dc)[off_h[m]]) : 0.f;
+        c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
+    }
+
+    const unsigned xgrp = (unsigned)g * NT * KSB * kFragBytes;
+    const size_t xslot = (size_t)p.n_groups * NT * KSB * kFragBytes;
+    int *grp_counters = p.counters + (size_t)g * kXcdGroupStride;
+    int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
+
+    // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out --------------------
+    constexpr int PD = 2;
+    u32x4 gpre[PD][GPT], cpre[PD][SPT], dpre[PD][SPT];
+    unsigned g_glb[GPT], s_glb[SPT];
+    int g_lds[GPT], s_lds[SPT];
+    bool g_ok[GPT], s_ok[SPT];
+#pragma unroll
+    for (int i = 0; i < GPT; ++i) {
+        const int pc = io_tid + IOT * i;
+        const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+        const int seg = rem / PPSEG, k = rem % PPSEG;
+        g_ok[i] = io_tid >= 0 && pc < GPIECES && b0 + row < B;
+        g_lds[i] = g_ok[i] ? row * GROW + seg * GSEG + k * 16 : 0;
+        g_glb[i] = (unsigned)((size_t)b0 * 4 * H + u0) +
+                   (g_ok[i] ? (unsigned)(row * 4 * H + seg * H + k * (16 / E::BYTES)) : 0u);
+    }
+#pragma unroll
+    for (int i = 0; i < SPT; ++i) {
+        const int pc = io_tid + IOT * i;
+        const int row = pc / PPSEG, k = pc % PPSEG;
+        s_ok[i] = io_tid >= 0 && pc < SPIECES && b0 + row < B;
+        s_lds[i] = s_ok[i] ? row * SROW + k * 16 : 0;
+        s_glb[i] = (unsigned)((size_t)b0 * H + u0) + (s_ok[i] ? (unsigned)(row * H + k * (16 / E::BYTES)) : 0u);
+    }
+    auto fetch_tiles = [&](int t, u32x4(&gp)[GPT], u32x4(&cp)[SPT], u32x4(&dp)[SPT]) {
+        if (io_tid < 0) return;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) gp[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + g_glb[i]);
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            cp[i] = *reinterpret_cast<const u32x4 *>(cell + (size_t)t * BH + s_glb[i]);
+            dp[i] = *reinterpret_cast<const u32x4 *>(dout + (size_t)t * BH + s_glb[i]);
+        }
+    };
+    auto tiles_to_lds = [&](const u32x4(&gp)[GPT], const u32x4(&cp)[SPT], const u32x4(&dp)[SPT]) {
+        unsigned char *stc = tiles + BT * GROW, *std_ = stc + BT * SROW;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i)
+            if (g_ok[i]) *reinterpret_cast<u32x4 *>(tiles + g_lds[i]) = gp[i];
+#pragma unroll
+        for (int i = 0; i < SPT; ++i)
+            if (s_ok[i]) {
+                *reinterpret_cast<u32x4 *>(stc + s_lds[i]) = cp[i];
+                *reinterpret_cast<u32x4 *>(std_ + s_lds[i]) = dp[i];
+            }
+    };
+    auto tile_to_global = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < GPT; ++i)
+            if (g_ok[i])
+                *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
+                    *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
+    };
+    auto prefetch = [&](int s, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (s < T_) fetch_tiles(T_ - 1 - s, gpre[u], cpre[u], dpre[u]);
+    };
+    prefetch(0, std::integral_constant<int, 0>{});
+    tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
+    __syncthreads();
+    prefetch(1, std::integral_constant<int, 1>{});
+
+    auto step = [&](const int s, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        constexpr int un = (u + 1) % PD;
+        const int t = T_ - 1 - s;
+        const XchgL2 xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
+
+        // ---- point-wise gate backward for this thread's items --------------------------
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            T st_d[4];
+            if (valid[m]) {
+                T *gl_ = reinterpret_cast<T *>(tiles + goff[m]);   // the item's 4 gates in the LDS tile
+                const float si = sigmoidf_<ACC>(E::to_f32(gl_[0]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(gl_[HT]));
+                const float tg = tanhf_<ACC>(E::to_f32(gl_[2 * HT]));
+                const float so = sigmoidf_<ACC>(E::to_f32(gl_[3 * HT]));
+                const float tc = tanhf_<ACC>(c1v[m]);
+                const float c0 = E::to_f32(*reinterpret_cast<const T *>(tiles + BT * GROW + soff[m]));
+                const float dh = dh_rec[m] + E::to_f32(*reinterpret_cast<const T *>(tiles + BT * GROW + BT * SROW + soff[m]));
+                const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
+                const float d_o = dh * tc * so * (1.f - so);
+                const float d_f = dc1 * c0 * sf * (1.f - sf);
+                const float d_i = dc1 * tg * si * (1.f - si);
+                const float d_g = dc1 * si * (1.f - tg * tg);
+                dc_state[m] = dc1 * sf;
+                c1v[m] = c0;   // c_{t-1} is the next step's c_t
+                st_d[0] = E::from_f32(d_i);
+                st_d[1] = E::from_f32(d_f);
+                st_d[2] = E::from_f32(d_g);
+                st_d[3] = E::from_f32(d_o);
+                gl_[0] = st_d[0];
+                gl_[HT] = st_d[1];
+                gl_[2 * HT] = st_d[2];
+                gl_[3 * HT] = st_d[3];
+            } else {
+#pragma unroll
+                for (int gt = 0; gt < 4; ++gt) st_d[gt] = E::from_f32(0.f);
+            }
+            // exchange copy: 4 consecutive k = (unit, gate 0..3).  16-bit types: lanes l and l+16
+            // own units u and u+1 of the same batch row; the even-unit lane writes both (16 bytes)
+            if constexpr (E::BYTES == 2) {
+                const u32x2 mine = *reinterpret_cast<u32x2 *>(st_d);
+                u32x2 other;
+                other[0] = (unsigned)__shfl_down((int)mine[0], 16);
+                other[1] = (unsigned)__shfl_down((int)mine[1], 16);
+                if (pair_lead[m])
+                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{mine[0], mine[1], other[0], other[1]}, xch.rsrc,
+                                                           xgrp + xoff[m], 0, 0);
+            } else {
+                if (valid[m])
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<u32x4 *>(st_d), xch.rsrc, xgrp + xoff[m], 0, 0);
+            }
+        }
+        // ---- publish: stores acknowledged by the L2, then the group's counters ----------------
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid < kXcdReplicas)
+            __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        tile_to_global(t);
+        prefetch(s + PD, uc);
+
+        if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, g, s);
+        __syncthreads();
+        // the tile has been drained: the next step's inputs take its place
+        if (s + 1 < T_) tiles_to_lds(gpre[un], cpre[un], dpre[un]);
+
+        // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps
+        f32x4 acc[MT][NTW];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        u32x4 bq[NKW][NTW];
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki) {
+            const int ks = min(wave + NWV * ki, KSB - 1);   // past the end: any valid block (its weights are zero)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) bq[ki][i] = xch.load16(xgrp + (unsigned)((i * KSB + ks) * kWave + lane) * 16u);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first MFMA: one round trip, not NKW
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki)
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int i = 0; i < NTW; ++i) red[((wave * MT + a) * NT + i) * kWave + lane] = acc[a][i];
+        __syncthreads();
+        const float *redf = reinterpret_cast<const float *>(red);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            float v = redf[roff[m]];
+#pragma unroll
+            for (int pp = 1; pp < NWV; ++pp) v += redf[roff[m] + pp * MT * NT * kWave * 4];
+            dh_rec[m] = v;
+        }
+        // the next step's publish barrier orders these reads before the next writes to `red`
+    };
+    for (int s0 = 0; s0 < T_; s0 += PD) {
+        step(s0, std::integral_constant<int, 0>{});
+        if (s0 + 1 < T_) step(s0 + 1, std::integral_constant<int, 1>{});
+    }
+
+    T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
+#pragma unroll
+    for (int m = 0; m < IPT; ++m)
+        if (valid[m]) {
+            dh_out[off_h[m]] = E::from_f32(dh_rec[m]);
+            dc_out[off_h[m]] = E::from_f32(dc_state[m]);
+        }
+}
+
+}  // namespace fastlstm
