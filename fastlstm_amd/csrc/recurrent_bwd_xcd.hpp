@@ -123,8 +123,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
 
     // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out --------------------
-    constexpr int PD = 2;
-    u32x4 gpre[PD][GPT], cpre[PD][SPT], dpre[PD][SPT];
+    // one set of tile pieces in flight: requested right after a step's tile went out, consumed after
+    // the step's K loop (more than an HBM round trip later); registers are scarce next to the weights
+    u32x4 gpre[GPT], cpre[SPT], dpre[SPT];
     unsigned g_glb[GPT], s_glb[SPT];
     int g_lds[GPT], s_lds[SPT];
     bool g_ok[GPT], s_ok[SPT];
@@ -175,18 +176,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
                     *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
     };
-    auto prefetch = [&](int s, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
-        if (s < T_) fetch_tiles(T_ - 1 - s, gpre[u], cpre[u], dpre[u]);
-    };
-    prefetch(0, std::integral_constant<int, 0>{});
-    tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
+    fetch_tiles(T_ - 1, gpre, cpre, dpre);
+    tiles_to_lds(gpre, cpre, dpre);   // step 0 works on the LDS tiles right away
     __syncthreads();
-    prefetch(1, std::integral_constant<int, 1>{});
 
-    auto step = [&](const int s, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
-        constexpr int un = (u + 1) % PD;
+    for (int s = 0; s < T_; ++s) {
         const int t = T_ - 1 - s;
         const XchgL2 xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
 
@@ -243,12 +237,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         if (tid < kXcdReplicas)
             __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         tile_to_global(t);
-        prefetch(s + PD, uc);
+        if (s + 1 < T_) fetch_tiles(t - 1, gpre, cpre, dpre);
 
         if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, g, s);
         __syncthreads();
-        // the tile has been drained: the next step's inputs take its place
-        if (s + 1 < T_) tiles_to_lds(gpre[un], cpre[un], dpre[un]);
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps
         f32x4 acc[MT][NTW];
@@ -256,24 +248,34 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         for (int a = 0; a < MT; ++a)
 #pragma unroll
             for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-        u32x4 bq[NKW][NTW];
+        // the operand blocks of the wave are requested in batches of at most 8 k-steps (registers):
+        // all loads of a batch are issued before its first MFMA -- one round trip per batch
+        constexpr int KB = NKW > 8 ? 8 : NKW;
 #pragma unroll
-        for (int ki = 0; ki < NKW; ++ki) {
-            const int ks = min(wave + NWV * ki, KSB - 1);   // past the end: any valid block (its weights are zero)
+        for (int k0 = 0; k0 < NKW; k0 += KB) {
+            u32x4 bq[KB][NTW];
 #pragma unroll
-            for (int i = 0; i < NTW; ++i) bq[ki][i] = xch.load16(xgrp + (unsigned)((i * KSB + ks) * kWave + lane) * 16u);
+            for (int kk = 0; kk < KB; ++kk) {
+                const int ks = min(wave + NWV * (k0 + kk), KSB - 1);   // past the end: any valid block (its weights are zero)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i)
+                    bq[kk][i] = xch.load16(xgrp + (unsigned)((i * KSB + ks) * kWave + lane) * 16u);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < KB; ++kk)
+#pragma unroll
+                for (int a = 0; a < MT; ++a)
+#pragma unroll
+                    for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][k0 + kk], bq[kk][i], acc[a][i]);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first MFMA: one round trip, not NKW
-#pragma unroll
-        for (int ki = 0; ki < NKW; ++ki)
-#pragma unroll
-            for (int a = 0; a < MT; ++a)
-#pragma unroll
-                for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
 #pragma unroll
         for (int a = 0; a < MT; ++a)
 #pragma unroll
             for (int i = 0; i < NTW; ++i) red[((wave * MT + a) * NT + i) * kWave + lane] = acc[a][i];
+        // the tile was drained before the barrier above: the next step's inputs take its place
+        if (s + 1 < T_) tiles_to_lds(gpre, cpre, dpre);
         __syncthreads();
         const float *redf = reinterpret_cast<const float *>(red);
 #pragma unroll
@@ -284,10 +286,6 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             dh_rec[m] = v;
         }
         // the next step's publish barrier orders these reads before the next writes to `red`
-    };
-    for (int s0 = 0; s0 < T_; s0 += PD) {
-        step(s0, std::integral_constant<int, 0>{});
-        if (s0 + 1 < T_) step(s0 + 1, std::integral_constant<int, 1>{});
     }
 
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
