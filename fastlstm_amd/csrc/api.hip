@@ -113,99 +113,105 @@ BwdLauncher bwd_launcher(int dtype) {
 }
 
 typedef hipError_t (*FwdXcdLauncher)(const FwdXcdParams &, int, int, int, int, int, int, hipStream_t, int *);
+typedef hipError_t (*BwdXcdLauncher)(const BwdXcdParams &, int, int, int, int, int, hipStream_t, int *);
 
-// The XCD-local forward kernel, when the device deals workgroups to XCDs in turn, the shape fits
-// (see recurrent_fwd_xcd.hpp) and the workspace holds a ring of T+1 slots.  Returns 1 when it
-// does not apply, else a fastlstm_status.
+// Shape of an XCD-local launch (see recurrent_fwd_xcd.hpp / recurrent_bwd_xcd.hpp).
+struct XcdCfg {
+    int mt, nkw, ntw, nwv;     // unit tiles per workgroup, k-steps per wave (share), batch tiles, waves
+    int n_ht, gpx, n_groups;   // members of a group, groups per XCD, groups of the launch
+    int ks;                    // k-steps of the contraction
+    int lds;
+    size_t xslot;              // bytes of one ring slot
+};
+
+// The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
+// and the workspace holds a ring with one slot per exchanged version.
+bool select_xcd(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c) {
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
+    const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    const int K = backward ? 4 * H : H;
+    if (K % kstep || (H * s) % 16) return false;
+    c->ks = K / kstep;
+    const int ways = backward ? 8 : 4;   // K-shares
+    const int per = cdiv(c->ks, ways);
+    c->nkw = per <= 4 ? 4 : (per <= 8 ? 8 : ((backward && per <= 16) ? 16 : 0));
+    if (!c->nkw) return false;
+    // hidden units per workgroup: the smallest tile that puts a group on one XCD and all batch tiles in one launch
+    const int hts_f[3] = {8, 16, 32}, hts_b[2] = {16, 32};
+    const int *hts = backward ? hts_b : hts_f;
+    const int n_hts = backward ? 2 : 3, rows = backward ? 16 : 4;   // weight rows per unit tile count as rows/4 fragments
+    int ht = 0;
+    c->ntw = 0;
+    for (int hi = 0; hi < n_hts && !ht; ++hi) {
+        const int cand = hts[hi];
+        const int frags = (cand / rows) * c->nkw;   // per wave (forward: halved again by the unit split of 8 waves)
+        if (H % cand || H / cand > 32 || cand * s < 16 || frags > (backward ? 32 : 64)) continue;
+        const int groups_max = kNumXcd * (32 / (H / cand));
+        if (cdiv(B, 16) <= groups_max) { ht = cand; c->ntw = 1; }
+        else if (cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
+    }
+    if (!ht) return false;
+    c->mt = ht / rows;
+    c->nwv = backward ? 8 : (c->mt * c->nkw > 32 ? 8 : 4);
+    c->n_ht = H / ht;
+    c->gpx = 32 / c->n_ht;
+    const int bt = 16 * c->ntw;
+    c->n_groups = cdiv(B, bt);
+    c->xslot = (size_t)c->n_groups * c->ntw * c->ks * kFragBytes;
+    const size_t slots = backward ? (size_t)T : (size_t)T + 1;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + slots * c->xslot) return false;
+    const int gseg = ht * s;
+    const int red_blocks = backward ? 8 * c->mt * c->ntw : 4 * c->mt * c->ntw;
+    c->lds = red_blocks * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
+#ifdef FASTLSTM_TIMELINE
+    c->lds += 4096;
+#endif
+    return true;
+}
+
+// Returns 1 when the XCD-local kernel does not apply, else a fastlstm_status.
 int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
                 int H, int dtype, hipStream_t stream) {
-    DeviceInfo di;
-    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return 1;
-    const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
-    if (H % kstep) return 1;
-    const int KS = H / kstep;
-    const int nkw = cdiv(KS, 4) <= 4 ? 4 : (cdiv(KS, 4) <= 8 ? 8 : 0);   // k-steps per K-share (4 shares)
-    if (!nkw) return 1;
-    int ht = 0, ntw = 0;
-    const int hts[3] = {8, 16, 32};
-    for (int hi = 0; hi < 3 && !ht; ++hi) {
-        const int c = hts[hi];
-        if (H % c || H / c > 32 || (c / 4) * nkw > 64 || c * s < 16) continue;
-        const int groups_max = kNumXcd * (32 / (H / c));
-        if (cdiv(B, 16) <= groups_max) { ht = c; ntw = 1; }
-        else if (cdiv(B, 32) <= groups_max) { ht = c; ntw = 2; }
-    }
-    if (!ht) return 1;
-    const int mt = ht / 4, n_ht = H / ht, bt = 16 * ntw, n_groups = cdiv(B, bt);
-    // more than 32 fragments per wave: 8 waves share the slice, so that registers remain for the operand loads
-    const int nwv = mt * nkw > 32 ? 8 : 4;
-    const size_t xslot = (size_t)n_groups * ntw * KS * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)(T + 1) * xslot) return 1;
-    const int gseg = ht * s;
-    int lds = 4 * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
-#ifdef FASTLSTM_TIMELINE
-    lds += 4096;
-#endif
+    XcdCfg c;
+    if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c)) return 1;
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
     p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
-    p.n_ht = n_ht; p.gpx = 32 / n_ht; p.n_groups = n_groups; p.KS = KS;
+    p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
     p.trace = g_rec_trace;
     FwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_fwd_xcd_f32
                                                    : (dtype == FASTLSTM_FP16 ? launch_fwd_xcd_f16 : launch_fwd_xcd_bf16);
     int occ = 0;
-    if (launch(p, mt, nkw, ntw, nwv, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.mt, c.nkw, c.ntw, c.nwv, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
-    // every CU gets one workgroup (a workgroup takes the whole register file); those without a role return at once
-    if (launch(p, mt, nkw, ntw, nwv, di.num_cus, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    // one workgroup per CU of the device; those without a role return at once
+    if (launch(p, c.mt, c.nkw, c.ntw, c.nwv, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
-typedef hipError_t (*BwdXcdLauncher)(const BwdXcdParams &, int, int, int, int, int, hipStream_t, int *);
-
-// The XCD-local reverse kernel under the same conditions as try_fwd_xcd (ring of T slots).
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream) {
-    DeviceInfo di;
-    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return 1;
-    const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
-    if ((4 * H) % kstep || H % 16) return 1;
-    const int KSB = 4 * H / kstep;
-    const int nkw = cdiv(KSB, 8) <= 4 ? 4 : (cdiv(KSB, 8) <= 8 ? 8 : (cdiv(KSB, 8) <= 16 ? 16 : 0));   // per wave, 8 waves
-    if (!nkw) return 1;
-    int ht = 0, ntw = 0;
-    const int hts[2] = {16, 32};
-    for (int hi = 0; hi < 2 && !ht; ++hi) {
-        const int c = hts[hi];
-        if (H % c || H / c > 32 || (c / 16) * nkw > 32) continue;
-        const int groups_max = kNumXcd * (32 / (H / c));
-        if (cdiv(B, 16) <= groups_max) { ht = c; ntw = 1; }
-        else if (cdiv(B, 32) <= groups_max) { ht = c; ntw = 2; }
-    }
-    if (!ht) return 1;
-    const int mt = ht / 16, n_ht = H / ht, bt = 16 * ntw, n_groups = cdiv(B, bt);
-    const size_t xslot = (size_t)n_groups * ntw * KSB * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * xslot) return 1;
-    const int gseg = ht * s;
-    const int lds = 8 * mt * ntw * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
+    XcdCfg c;
+    if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
     p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
-    p.n_ht = n_ht; p.gpx = 32 / n_ht; p.n_groups = n_groups; p.KSB = KSB;
+    p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
     p.spin_limit = spin_limit_ticks();
     BwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_bwd_xcd_f32
                                                    : (dtype == FASTLSTM_FP16 ? launch_bwd_xcd_f16 : launch_bwd_xcd_bf16);
     int occ = 0;
-    if (launch(p, mt, nkw, ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.mt, c.nkw, c.ntw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
-    if (launch(p, mt, nkw, ntw, di.num_cus, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
@@ -449,6 +455,13 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
             return FASTLSTM_ERR_HIP;
     }
     return FASTLSTM_OK;
+}
+
+int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (T <= 0 || B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    XcdCfg c;
+    return select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c) ? 1 : 0;
 }
 
 int fastlstm_ws_status(const void *ws_head) {

@@ -122,6 +122,14 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
                         int dtype, void *stream);
 size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
 
+/* Which kernel fastlstm_fwd_persistent (backward = 0) / fastlstm_bwd_persistent (1) will launch on
+ * the current device for this shape and a workspace of ws_bytes: 0 = the general kernel
+ * (exchange through device memory), 1 = the XCD-local kernel (barrier group on one XCD,
+ * exchange through its L2; needs the ring workspace of fastlstm_recurrent_workspace_bytes and a
+ * device that fastlstm_plan_device has probed).  Negative: fastlstm_status.  Diagnostics; no
+ * counterpart in the reference. */
+int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
+
 /* Reads the status word the recurrent kernels leave at the start of their
  * workspace; `ws_head` points to a HOST copy of the first 64 bytes.
  * 0 = ok, FASTLSTM_ERR_TIMEOUT = a barrier wait gave up (the kernel still ran

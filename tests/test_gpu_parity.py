@@ -307,6 +307,99 @@ def test_barrier_timeout_is_reported_not_hung():
     assert torch.isfinite(out.float()).all()
 
 
+XCD_CASES = [
+    # T, B, H, dtype          (hidden tile, members, batch tiles) of the XCD-local launch
+    (20, 64, 1024, torch.float16),    # config B: 32 units x 32 members, 8 waves
+    (9, 40, 512, torch.bfloat16),     # 16 units x 32 members, ragged batch
+    (7, 100, 256, torch.float32),     # fp32, 7 batch tiles on 7 XCDs
+    (5, 300, 256, torch.float16),     # 32-row batch tiles, two groups per XCD
+    (6, 16, 128, torch.float16),      # small H: 8 units (forward) / 16 units (backward) per workgroup
+]
+
+
+@pytest.mark.parametrize("T,B,H,dt", XCD_CASES)
+def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
+    """The C ABI picks the XCD-local kernels when the workspace holds the exchange ring and the
+    general kernels when it does not; both must meet the oracle, on the same inputs."""
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    rm = RM[dt]
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    p = make_problem(T, B, H, H, seed=77 + H)
+    pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}
+    g = {k: dev(v, dt) for k, v in p.items()}
+    o_out, o_cell, o_ifgo = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=rm)
+    st = torch.cuda.current_stream().cuda_stream
+    plans = [_lib.Plan(), _lib.Plan()]
+    for bw in (0, 1):
+        _lib.check(lib.fastlstm_plan_device(0, B, H, code, bw, plans[bw]), "plan")
+    ifgo0 = torch.empty(T, B, 4 * H, device="cuda", dtype=dt)
+    _lib.check(lib.fastlstm_gemm_ifgo(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(), g["bh"].data_ptr(),
+                                      ifgo0.data_ptr(), T, B, H, H, code, st), "k1")
+    results = {}
+    for kind in ("general", "xcd"):
+        sizes = [plans[bw].ws_bytes if kind == "general" else
+                 lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
+        for bw in (0, 1):
+            assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, bw, sizes[bw]) == (1 if kind == "xcd" else 0)
+        ifgo = ifgo0.clone()
+        out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
+        cell = torch.empty_like(out)
+        out[0], cell[0] = g["h0"], g["c0"]
+        ws = torch.zeros(sizes[0], dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), g["Wh"].data_ptr(),
+                                               ws.data_ptr(), ws.numel(), T, B, H, code, st), "fwd")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
+        for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
+            assert rel_err(got, want) < tol, (kind, name)
+        d_ifgo = torch.empty_like(ifgo)
+        dh, dc = g["dh_n"].clone(), g["dc_n"].clone()
+        wsb = torch.zeros(sizes[1], dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_bwd_persistent(g["dout"].data_ptr(), dh.data_ptr(), dc.data_ptr(), ifgo.data_ptr(),
+                                               cell.data_ptr(), d_ifgo.data_ptr(), g["Wh"].data_ptr(), wsb.data_ptr(),
+                                               wsb.numel(), T, B, H, code, st), "bwd")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(wsb[:64].cpu().numpy().tobytes()) == _lib.OK
+        dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
+        r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
+        for name, got, want in (("d_ifgo", d_ifgo, r["d_ifgo"]), ("dh0", dh, r["dh0"]), ("dc0", dc, r["dc0"])):
+            assert rel_err(got, want) < tol, (kind, name)
+        results[kind] = (out, cell, ifgo, d_ifgo, dh, dc)
+    for a, b in zip(results["general"], results["xcd"]):   # two summation orders of the same sums
+        assert rel_err(a, b) < tol
+
+
+def test_xcd_local_barrier_timeout_is_reported_not_hung():
+    """The host-forced failure path of the L2 counter barrier: same contract as the flag barrier."""
+    lib = _lib.load()
+    T, B, H, code = 64, 16, 512, 1
+    plan = _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan), "plan")
+    nbytes = lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0)
+    assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, nbytes) == 1
+    ifgo = torch.randn(T, B, 4 * H, device="cuda").half()
+    out = torch.zeros(T + 1, B, H, device="cuda").half()
+    cell = torch.zeros(T + 1, B, H, device="cuda").half()
+    Wh = (torch.randn(4 * H, H, device="cuda") * 0.03).half()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.clone().data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
+                                               ws.data_ptr(), ws.numel(), T, B, H, code, st), "fwd")
+        torch.cuda.synchronize()  # returns: the grid drained
+        return lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes())
+
+    try:
+        lib.fastlstm_set_spin_limit(1)
+        assert launch() == _lib.ERR_TIMEOUT
+    finally:
+        lib.fastlstm_set_spin_limit(400000000)
+    assert launch() == _lib.OK
+    assert torch.isfinite(out.float()).all()
+
+
 # --------------------------------------------------------------------------------------
 # 4. BASELINE.json configurations at their real shapes
 # --------------------------------------------------------------------------------------
