@@ -38,7 +38,7 @@ PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MF
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the forward recurrence from rocprofv3 FETCH_SIZE + WRITE_SIZE,
 # scaled by a plain copy of known size (profiles/fwd_recurrence_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 982.0e6}
+TRAFFIC_BYTES = {"B": 858.5e6}
 
 
 def main():
@@ -225,13 +225,16 @@ def main():
     # ---- roofline of the dominant kernel: the persistent forward recurrence -------------
     rec_flops = 2.0 * B * H * 4 * H * T          # algorithmic flops of one launch
     ach = rec_flops / (t_rec * 1e-3) / 1e12
-    roofline = {"kernel": "lstm_fwd_persistent_kernel", "bound": "mfma", "achieved": round(ach, 2),
+    xcd_local = lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, ws_f.numel()) == 1
+    roofline = {"kernel": "lstm_fwd_xcd_kernel" if xcd_local else "lstm_fwd_persistent_kernel",
+                "bound": "mfma", "achieved": round(ach, 2),
                 "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dname], 4),
                 "traffic": TRAFFIC_BYTES.get(args.workload),
                 "algorithmic": "2*B*H*4H*T flop per launch = %.1f GFLOP" % (rec_flops / 1e9),
                 "launch_ms": round(t_rec, 4),
-                "note": "latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange; "
-                        "us/step is in kernels.recurrent_fwd_us_per_step"}
+                "note": "latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange "
+                        + ("through the L2 of one XCD" if xcd_local else "through device memory")
+                        + "; us/step is in kernels.recurrent_fwd_us_per_step"}
 
     res = {
         "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
