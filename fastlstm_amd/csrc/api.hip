@@ -278,7 +278,7 @@ static void wgrad_plan(int M, int N, int K, int dtype, int *tile, int *splits, i
     *k_per_split = cdiv(cdiv(K, *splits), bk) * bk;
     *splits = cdiv(K, *k_per_split);
 }
-static int colsum_chunks(int R) { return std::max(1, std::min(64, R / 64)); }
+static int colsum_chunks(int R) { return std::max(1, std::min(256, R / 64)); }
 
 size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
     if (!dtype_ok(dtype) || check_dims(T, B, I, H)) return 0;

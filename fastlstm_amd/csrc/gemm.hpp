@@ -237,7 +237,22 @@ __global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, in
     float s[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) s[e] = 0.f;
-    for (int rr = r0; rr < r1; ++rr) {
+    constexpr int U = 8;   // rows in flight per thread: the kernel is a pure HBM stream
+    int rr = r0;
+    if constexpr (VEC > 1) {
+        for (; rr + U <= r1; rr += U) {
+            u32x4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const u32x4 *>(in + (size_t)(rr + u) * C + c0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const T *tv = reinterpret_cast<const T *>(&v[u]);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s[e] += Elem<T>::to_f32(tv[e]);
+            }
+        }
+    }
+    for (; rr < r1; ++rr) {
         const T *src = in + (size_t)rr * C + c0;
         if constexpr (VEC == 1) {
             s[0] += Elem<T>::to_f32(src[0]);
@@ -252,12 +267,18 @@ __global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, in
     for (int e = 0; e < VEC; ++e) part[(size_t)blockIdx.y * C + c0 + e] = s[e];
 }
 
+// out[c] = sum over chunks of part[chunk][c].  A block of 256 threads covers 64 columns with 4
+// threads each (chunks k = slice, slice + 4, ...), summed through LDS in a fixed order.
 template <typename T> __global__ void colsum_final_kernel(const float *part, T *out, int C, int chunks) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
+    __shared__ float red[4][64];
+    const int cl = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cl;
     float s = 0.f;
-    for (int k = 0; k < chunks; ++k) s += part[(size_t)k * C + c];
-    out[c] = Elem<T>::from_f32(s);
+    if (c < C)
+        for (int k = slice; k < chunks; k += 4) s += part[(size_t)k * C + c];
+    red[slice][cl] = s;
+    __syncthreads();
+    if (slice == 0 && c < C) out[c] = Elem<T>::from_f32((red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]));
 }
 
 }  // namespace fastlstm
