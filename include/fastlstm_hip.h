@@ -13,10 +13,11 @@
  *  - `stream` is a hipStream_t passed as void*; every launch is asynchronous
  *    on it and nothing here synchronises the host;
  *  - the library never allocates device memory: scratch comes in through the
- *    `ws` arguments, sized by the *_workspace_bytes / plan calls; the flag part of a
- *    recurrence workspace must be ZERO-FILLED by the caller before each call (the same
- *    contract as the reference's zero-initialised sync buffer, fastlstm/lstm.py:96-100,
- *    249) -- see fastlstm_recurrent_workspace_bytes;
+ *    `ws` arguments, sized by the *_workspace_bytes / plan calls; the leading part of a
+ *    recurrence workspace (header, barrier counters, flags: plan->ws_zero_bytes) must be
+ *    ZERO-FILLED by the caller before each call (the same contract as the reference's
+ *    zero-initialised sync buffer, fastlstm/lstm.py:96-100, 249) -- see
+ *    fastlstm_recurrent_workspace_bytes;
  *  - return value: 0 on success, a negative fastlstm_status otherwise; argument
  *    validation happens before the first HIP call, so the error paths can be
  *    exercised on a machine without a GPU;
@@ -64,7 +65,7 @@ typedef struct {
     int wave_split;   /* 0: waves split K, 1: waves split batch tiles, 2: waves split W rows */
     int lds_bytes;    /* LDS the kernel will request */
     size_t ws_bytes;  /* smallest workspace the recurrent call accepts (2 exchange slots) */
-    size_t ws_zero_bytes; /* leading bytes of the workspace that must be zero (header + flags) */
+    size_t ws_zero_bytes; /* leading bytes of the workspace that must be zero (header + counters + flags) */
     int ring_needs_zero;  /* 1: B or H leave padding in the exchange blocks -> zero the whole workspace */
 } fastlstm_plan;
 
@@ -75,14 +76,19 @@ typedef struct {
 int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int dtype, int backward,
                       fastlstm_plan *plan);
 
-/* Same, for the current HIP device `device` (queries CU count and LDS size). */
+/* Same, for HIP device `device` (-1: the current one; queries CU count and LDS size).  The first
+ * call for a device also probes, with one tiny kernel and a device synchronisation, whether the
+ * workgroups of a launch are dealt to the 8 XCDs in turn; the XCD-local recurrent kernels are only
+ * used on a device where that was seen.  The launch calls below never synchronise. */
 int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan);
 
-/* Workspace that gives every timestep its own exchange slot (a "history ring" of T+1 forward /
- * T backward slots, capped at 1 GiB per launch).  With it the exchange data is read through
- * the caches (one fetch per XCD); with less, down to plan->ws_bytes, the kernels fall back to
- * cache-bypassing loads.  The first plan->ws_zero_bytes bytes must be zero; the rest only if
- * plan->ring_needs_zero. */
+/* Workspace that gives every timestep its own exchange slot (a ring of T+1 forward / T backward
+ * slots, capped at 1 GiB per launch).  With it no exchange address is read before its only
+ * write, so the kernels read the exchange data through the caches, and where the shape allows
+ * (fastlstm_recurrent_kernel_kind) the XCD-local kernels run: the workgroups that exchange data
+ * sit on one XCD and exchange through its L2.  With less, down to plan->ws_bytes, the general
+ * kernels exchange through device memory with cache-bypassing loads.  The first
+ * plan->ws_zero_bytes bytes must be zero; the rest only if plan->ring_needs_zero. */
 size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype, int backward);
 
 /* K1 -- ifgo[T*B,4H] = x[T*B,I] . Wx[4H,I]^T + (bx + bh).
