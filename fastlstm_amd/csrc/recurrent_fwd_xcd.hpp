@@ -13,7 +13,7 @@
 //    of its own (ring of T + 1 slots): an address is only read after its single write;
 //  * barrier: counters in L2.  Atomics execute in the L2, never in an L1: a member adds 1 to
 //    each of kXcdReplicas counters of its group after its stores were acknowledged, and polls
-//    one of them (its index % replicas) with an atomic add of 0;
+//    one of them (its index % replicas) with scalar loads that bypass the scalar cache;
 //  * W_h: a slice of 4*MT units x 4 gates x H no longer has to fit in LDS next to the peers'
 //    (32 CUs x 160 KiB < 8 MiB for H = 1024): every wave keeps its K-share of the slice, MT x NKW
 //    operand fragments, in registers (up to 256 of the 512 per lane).
@@ -62,35 +62,33 @@ struct XchgL2 {
     }
 };
 
-// Lane 0 of the calling wave polls `counter` in L2 until it reaches `target`.  Bounded like
+// The calling wave polls `counter` in L2 until it reaches `target`.  The poll is a scalar load
+// with the glc bit (it misses the scalar cache and is served by the L2; the vector L1, which
+// could hold a stale line, is not on its path) -- half the round trip of a returning L2 atomic.
+// A stale value can only be too small, i.e. delay the wait, never release it early.  Bounded like
 // wait_versions.
 __device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader *hdr, long long spin_limit,
                                              int group, int step) {
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-        long long t0 = 0;
-        int polls = 0;
-        for (;;) {
-            int v;
-            const int zero = 0;
-            // an atomic with return value: executed by the L2, whatever the L1 holds
-            asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)"
-                         : "=v"(v)
-                         : "v"(counter), "v"(zero)
-                         : "memory");
-            if (v >= target) break;
-            __builtin_amdgcn_s_sleep(1);
-            if (++polls >= 64 || spin_limit <= 1) {
-                polls = 0;
-                if (__hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
-                const long long now = (long long)wall_clock64();
-                if (t0 == 0 && spin_limit > 1) {
-                    t0 = now;
-                } else if (now - t0 > spin_limit) {
+    long long t0 = 0;
+    int polls = 0;
+    for (;;) {
+        int v;
+        asm volatile("s_load_dword %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(counter) : "memory");
+        if (v >= target) break;
+        __builtin_amdgcn_s_sleep(1);
+        if (++polls >= 64 || spin_limit <= 1) {
+            polls = 0;
+            if (__hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+            const long long now = (long long)wall_clock64();
+            if (t0 == 0 && spin_limit > 1) {
+                t0 = now;
+            } else if (now - t0 > spin_limit) {
+                if ((threadIdx.x & (kWave - 1)) == 0) {
                     hdr->timeout_group = group;
                     hdr->timeout_step = step;
                     __hip_atomic_store(&hdr->abort_flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-                    break;
                 }
+                break;
             }
         }
     }
