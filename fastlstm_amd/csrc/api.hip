@@ -114,6 +114,7 @@ BwdLauncher bwd_launcher(int dtype) {
 
 typedef hipError_t (*FwdXcdLauncher)(const FwdXcdParams &, int, int, int, int, int, int, hipStream_t, int *);
 typedef hipError_t (*BwdXcdLauncher)(const BwdXcdParams &, int, int, int, int, int, hipStream_t, int *);
+typedef hipError_t (*FwdXcdHelpLauncher)(const FwdXcdParams &, int, int, int, hipStream_t, int *);
 
 // Shape of an XCD-local launch (see recurrent_fwd_xcd.hpp / recurrent_bwd_xcd.hpp).
 struct XcdCfg {
@@ -170,9 +171,41 @@ bool select_xcd(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, 
     return true;
 }
 
-// Returns 1 when the XCD-local kernel does not apply, else a fastlstm_status.
+// In-kernel input projection: possible when the XCD-local forward kernel is the 8-wave one, at
+// least a quarter of the CUs have no role in the recurrence, and K1 suits the 256 x 256 16-bit
+// tile kernel.  Fills the k1 fields of *p (chunking by time) and returns true.
+bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int T,
+                     int B, int I, int H, int dtype, FwdXcdParams *p) {
+    if (dtype == FASTLSTM_FP32 || c.nwv != 8 || c.mt != 8 || c.nkw != 8) return false;
+    const int n_helpers = kNumXcd * 32 - c.n_groups * c.n_ht;
+    if (n_helpers < kNumXcd * 8) return false;
+    const int M = T * B, N = 4 * H;
+    if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;
+    const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
+    // a chunk: whole timesteps, about one round of the helpers, at most 32 chunks
+    int base = 1;
+    while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
+    int ct = std::max(1, n_helpers / tiles_n / base) * base;
+    while (cdiv(tiles_m, ct) > 32) ct += base;
+    const int steps = ct * 256 / B;
+    if (steps < 2) return false;
+    p->k1 = GemmParams{};
+    p->k1.A = x; p->k1.B = Wx; p->k1.C = ifgo; p->k1.bias0 = bx; p->k1.bias1 = bh;
+    p->k1.M = M; p->k1.N = N; p->k1.K = I;
+    p->k1.lda = I; p->k1.ldb = I; p->k1.ldc = N;
+    p->k1.splits = 1; p->k1.k_per_split = I;
+    p->k1_tiles_m = tiles_m; p->k1_tiles_n = tiles_n;
+    p->k1_chunk_tiles = ct; p->k1_chunk_steps = steps;
+    p->k1_done = p->hdr->reserved;
+    p->k1_ticket = p->hdr->reserved + 32;
+    return true;
+}
+
+// Returns 1 when the XCD-local kernel does not apply, else a fastlstm_status.  With x != nullptr
+// the kernel also has to compute ifgo = x.Wx^T + b (returns 2 when that is not possible in-kernel).
 int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
-                int H, int dtype, hipStream_t stream) {
+                int H, int dtype, hipStream_t stream, const void *x = nullptr, const void *Wx = nullptr,
+                const void *bx = nullptr, const void *bh = nullptr, int I = 0) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c)) return 1;
     FwdXcdParams p{};
@@ -184,6 +217,16 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
     p.trace = g_rec_trace;
+    if (x) {
+        if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p)) return 2;
+        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 4, 2, 2>::LDS_BYTES);
+        FwdXcdHelpLauncher hl = dtype == FASTLSTM_FP16 ? launch_fwd_xcd_help_f16 : launch_fwd_xcd_help_bf16;
+        int occ = 0;
+        if (hl(p, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (occ < 1) return 2;
+        if (hl(p, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+        return FASTLSTM_OK;
+    }
     FwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_fwd_xcd_f32
                                                    : (dtype == FASTLSTM_FP16 ? launch_fwd_xcd_f16 : launch_fwd_xcd_bf16);
     int occ = 0;
@@ -233,6 +276,23 @@ static int plan_device(int device, int B, int H, int dtype, int backward, fastls
 
 int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan) {
     return plan_device(device, B, H, dtype, backward, plan, true);
+}
+
+// K1 on rows [row0, row0 + rows) of x[T*B, I] / ifgo[T*B, 4H]
+static int gemm_ifgo_rows(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, size_t row0,
+                          int rows, int I, int H, int dtype, hipStream_t stream) {
+    const size_t s = elem_bytes(dtype);
+    GemmParams p{};
+    p.A = static_cast<const unsigned char *>(x) + row0 * I * s;
+    p.B = Wx;
+    p.C = static_cast<unsigned char *>(ifgo) + row0 * 4 * H * s;
+    p.bias0 = bx; p.bias1 = bh;
+    p.M = rows; p.N = 4 * H; p.K = I;
+    p.lda = I; p.ldb = I; p.ldc = 4 * H;
+    p.splits = 1; p.k_per_split = I;
+    int tile, splits;
+    gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, false, false, &tile, &splits);
+    return launch_gemm_tiled(dtype, p, false, false, tile, stream) == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
 }
 
 int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int T,
@@ -455,6 +515,34 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
             return FASTLSTM_ERR_HIP;
     }
     return FASTLSTM_OK;
+}
+
+int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
+                       void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                       void *stream) {
+    if (!x || !Wx || !bx || !bh || !Wh || !ifgo || !out || !cell || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(x) || !aligned16(Wx) || !aligned16(ifgo) || !aligned16(out) || !aligned16(cell) || !aligned16(Wh) ||
+        !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    // Where the XCD-local recurrence leaves CUs without a role, those workgroups compute the input
+    // projection inside the same launch, earliest timesteps first, and the recurrence follows them
+    // chunk by chunk; otherwise K1 and the recurrence are two launches back to back.
+#ifndef FASTLSTM_TIMELINE
+    {
+        fastlstm_plan pl;
+        if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
+        if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+        if (pl.wave_split != 2) {
+            const int rc = try_fwd_xcd(ifgo, out, cell, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
+                                       static_cast<hipStream_t>(stream), x, Wx, bx, bh, I);
+            if (rc <= 0) return rc;   // launched, or failed
+        }
+    }
+#endif
+    if (int rc = fastlstm_gemm_ifgo(x, Wx, bx, bh, ifgo, T, B, I, H, dtype, stream)) return rc;
+    return fastlstm_fwd_persistent(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {

@@ -75,30 +75,21 @@ template <int N> __device__ __forceinline__ void wait_vm_at_most() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));
 }
 
+// One BM x BN tile of C (rows m0.., columns n0.., K range of `split`) by a workgroup of
+// 64*WVM*WVN threads with Gemm16Cfg::LDS_BYTES of LDS at `smem`.  All threads of the workgroup
+// call it together; it ends with the tile stored (the caller orders later use of `smem`).
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
-__global__ __launch_bounds__(64 * WVM * WVN) void gemm16_kernel(const GemmParams p) {
+__device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
+                                            unsigned char *smem, const int trace_slot) {
     using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
     constexpr int NWAVES = C::NWAVES, THREADS = C::THREADS;
     constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave / WVN, wn = wave % WVN;
 
     long long t_start = 0, t_loop = 0, t_epi = 0;
     if (p.trace) t_start = (long long)wall_clock64();
-    const int tiles_n = cdiv(p.N, BN), tiles_m = cdiv(p.M, BM);
-    int bid = blockIdx.x;
-    const int split = bid / (tiles_m * tiles_n);
-    bid -= split * tiles_m * tiles_n;
-    // Tile order: every XCD gets a contiguous range of a grouped order in which 8 x 8 blocks
-    // of C tiles are consecutive, so the ~64 workgroups an XCD runs at a time re-use each
-    // other's A and B tiles out of that XCD's L2.
-    constexpr int GM = 8;
-    const int lin = xcd_major_id(bid, tiles_m * tiles_n);
-    const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
-    const int gsz = min(tiles_m - first_m, GM);
-    const int m0 = (first_m + (lin % per_group) % gsz) * BM, n0 = ((lin % per_group) / gsz) * BN;
     const int kb = split * p.k_per_split;
     const int ke = min(p.K, kb + p.k_per_split);
     const int nkt = (ke - kb) / BK;
@@ -272,9 +263,27 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm16_kernel(const GemmParams
         }
     }
     if (p.trace && tid == 0) {
-        long long *t = p.trace + (size_t)blockIdx.x * 4;
+        long long *t = p.trace + (size_t)trace_slot * 4;
         t[0] = t_start; t[1] = t_loop; t[2] = t_epi; t[3] = (long long)wall_clock64();
     }
+}
+
+template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+__global__ __launch_bounds__(64 * WVM * WVN) void gemm16_kernel(const GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tiles_n = cdiv(p.N, BN), tiles_m = cdiv(p.M, BM);
+    int bid = blockIdx.x;
+    const int split = bid / (tiles_m * tiles_n);
+    bid -= split * tiles_m * tiles_n;
+    // Tile order: every XCD gets a contiguous range of a grouped order in which 8 x 8 blocks
+    // of C tiles are consecutive, so the ~64 workgroups an XCD runs at a time re-use each
+    // other's A and B tiles out of that XCD's L2.
+    constexpr int GM = 8;
+    const int lin = xcd_major_id(bid, tiles_m * tiles_n);
+    const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int m0 = (first_m + (lin % per_group) % gsz) * BM, n0 = ((lin % per_group) / gsz) * BN;
+    gemm16_tile<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, split, smem, (int)blockIdx.x);
 }
 
 }  // namespace fastlstm

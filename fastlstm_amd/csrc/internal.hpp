@@ -16,6 +16,7 @@ hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hip
 hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
                          hipStream_t s);
 int gemm_bk(int dtype);
+bool gemm16_eligible(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km);
 void set_gemm_trace(long long *buf);
 void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km, bool allow_split,
                int *tile, int *splits);
@@ -32,7 +33,9 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_k
     hipError_t launch_fwd_xcd_##SUF(const FwdXcdParams &p, int mt, int nkw, int ntw, int nwv, int grid, int lds, \
                                     hipStream_t s, int *max_blocks_per_cu);                          \
     hipError_t launch_bwd_xcd_##SUF(const BwdXcdParams &p, int mt, int nkw, int ntw, int grid, int lds, \
-                                    hipStream_t s, int *max_blocks_per_cu);
+                                    hipStream_t s, int *max_blocks_per_cu);                          \
+    hipError_t launch_fwd_xcd_help_##SUF(const FwdXcdParams &p, int ntw, int grid, int lds, hipStream_t s, \
+                                         int *max_blocks_per_cu);
 FASTLSTM_DECL_REC(f32)
 FASTLSTM_DECL_REC(f16)
 FASTLSTM_DECL_REC(bf16)

@@ -22,6 +22,8 @@
 #pragma once
 #include <type_traits>
 
+#include "gemm.hpp"
+#include "gemm16.hpp"
 #include "recurrent_common.hpp"
 
 namespace fastlstm {
@@ -44,6 +46,15 @@ struct FwdXcdParams {
     int gpx;           // groups per XCD (32 / n_ht)
     int n_groups;      // batch tiles of this launch (<= 8 * gpx)
     int KS;            // k-steps covering H
+    // In-kernel input projection (HELP instantiations, k1_tiles_n > 0): the workgroups without a
+    // role in the recurrence compute ifgo = x.Wx^T + b in 256 x 256 tiles, earliest timesteps first;
+    // k1_done[c] counts the finished tiles of chunk c (k1_chunk_tiles row tiles = k1_chunk_steps
+    // timesteps), and the recurrence requests the gates of a timestep only when its chunk is done.
+    GemmParams k1;        // M = T*B, N = 4H, K = I, A = x, B = Wx, C = ifgo, biases
+    int k1_tiles_m, k1_tiles_n;
+    int k1_chunk_tiles, k1_chunk_steps;
+    int *k1_done;         // [<= 32] device-scope counters, zero at launch
+    int *k1_ticket;       // numbers the helper workgroups, zero at launch
     long long spin_limit;
     long long *trace;  // diagnostic build only
 };
@@ -95,12 +106,36 @@ __device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader 
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // compiler ordering only
 }
 
+// Input projection by a workgroup (8 waves) that has no role in the recurrence.  Helper h of n
+// takes tiles h, h + n, ... of the time-ordered tile list.  A finished tile is made visible to the
+// other XCDs (its stores acknowledged, this XCD's L2 written back: the release of the atomic) before
+// it is counted.
+template <typename T>
+__device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *smem) {
+    int *ticket = reinterpret_cast<int *>(smem);
+    if (threadIdx.x == 0) *ticket = __hip_atomic_fetch_add(p.k1_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int h = *ticket;
+    __syncthreads();
+    const int n_helpers = (int)gridDim.x - p.n_groups * p.n_ht;
+    const int total = p.k1_tiles_m * p.k1_tiles_n;
+    for (int tile = h; tile < total; tile += n_helpers) {
+        const int rt = tile / p.k1_tiles_n, ct = tile % p.k1_tiles_n;
+        gemm16_tile<T, false, false, 256, 256, 2, 4, 2, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // every wave's part of the tile is in the L2 (and the LDS may be reused)
+        if (threadIdx.x == 0)
+            __hip_atomic_fetch_add(p.k1_done + rt / p.k1_chunk_tiles, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // The waves split K four ways: wave w owns k-steps w % 4, w % 4 + 4, ... (NKW of them).  With
 // NWV = 8 waves (two per SIMD, 256 registers each) the two waves of a K-share split the MT unit
 // tiles between them, which halves the fragments a wave holds and leaves registers to keep all
 // operand loads of a step in flight.
-template <typename T, int MT, int NKW, int NTW, int NWV>
+template <typename T, int MT, int NKW, int NTW, int NWV, bool HELP = false>
 __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdParams p) {
+    static_assert(!HELP || (NWV == 8 && sizeof(T) == 2), "the in-kernel GEMM tile is the 8-wave 16-bit one");
     constexpr int NTHR = kWave * NWV;
     constexpr int MW = NWV / 4, MTW = MT / MW;       // M-split ways, unit tiles per wave
     static_assert(NWV == 4 || NWV == 8, "4 or 8 waves");
@@ -127,8 +162,19 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
     const int g = gl * kNumXcd + xcd;
-    if (gl >= p.gpx || g >= p.n_groups) return;
+    if (gl >= p.gpx || g >= p.n_groups) {
+        if constexpr (HELP) {
+            if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);
+        }
+        return;
+    }
     const int u0 = j * HT, b0 = g * BT;
+    const bool k1_live = HELP && p.k1_tiles_n > 0;
+    // chunk c of ifgo is complete when all its tiles were counted
+    auto wait_chunk = [&](int c, int t) {
+        const int rows = min(p.k1_chunk_tiles, p.k1_tiles_m - c * p.k1_chunk_tiles);
+        wait_versions(p.k1_done + c, 1, rows * p.k1_tiles_n, p.hdr, p.spin_limit, g, t);
+    };
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                  // [4][TILES][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + 4 * TILES * kWave);   // gates, h, c tiles
@@ -268,6 +314,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         constexpr int u = decltype(uc)::value;
         if (t < T_) fetch_tile(t, gpre[u]);
     };
+    if (k1_live) {   // the first chunk of the input projection has to be there
+        if (wave == 0) wait_chunk(0, 0);
+        __syncthreads();
+    }
     prefetch(0, std::integral_constant<int, 0>{});
     prefetch(1, std::integral_constant<int, 1>{});
 
@@ -275,6 +325,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         constexpr int u = decltype(uc)::value;
         unsigned char *gt = tiles;
         FASTLSTM_TP(0);
+        // the gates of step t + PD are requested at the end of this step: their chunk must have landed
+        // (the barrier below orders the poll before the request)
+        if (k1_live && t + PD < T_ && (t + PD) % p.k1_chunk_steps == 0 && wave == 0)
+            wait_chunk((t + PD) / p.k1_chunk_steps, t);
         if (wave == 0) wait_counter(my_counter, p.n_ht * (t + 1), p.hdr, p.spin_limit, g, t);
         FASTLSTM_TP(1);
         __syncthreads();

@@ -125,14 +125,12 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
         plan = _plan(x.device, batch_size, hidden_size, code, False)
         ws = _workspace(plan, seq_len, hidden_size, code, False, x.device)
         stream = _stream()
-        _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(),
-                                          ifgo.data_ptr(), seq_len, batch_size, input_size, hidden_size,
-                                          code, stream), "fastlstm_gemm_ifgo")
-        _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(),
-                                               Wh.data_ptr(), ws.data_ptr(), ws.numel(), seq_len,
-                                               batch_size, hidden_size, code, stream),
-                   "fastlstm_fwd_persistent")
-        _check_ws(ws, "fastlstm_fwd_persistent")
+        # input projection + time loop in one call (the library fuses the two where CUs would idle)
+        _lib.check(lib.fastlstm_fwd_layer(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
+                                          ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws.data_ptr(),
+                                          ws.numel(), seq_len, batch_size, input_size, hidden_size, code, stream),
+                   "fastlstm_fwd_layer")
+        _check_ws(ws, "fastlstm_fwd_layer")
     return out, cell, ifgo
 
 

@@ -105,6 +105,16 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
 int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws,
                             size_t ws_bytes, int T, int B, int H, int dtype, void *stream);
 
+/* K1 + K2/K3 for one layer in one call: the same results as fastlstm_gemm_ifgo followed by
+ * fastlstm_fwd_persistent (same arguments, same workspace contract).  Where the XCD-local
+ * recurrence leaves CUs without a role (few batch tiles), the workgroups on those CUs compute the
+ * input projection inside the same launch, earliest timesteps first, and the recurrence follows
+ * them chunk by chunk; otherwise the two stages are launched back to back.  Replaces
+ * fastlstm/lstm.py:66-68 together with 131-142. */
+int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh,
+                       void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I,
+                       int H, int dtype, void *stream);
+
 /* K4 -- the reverse time loop.  In: dout[T,B,H]; dh,dc [B,H] hold the gradients
  * flowing into h_T, c_T; ifgo, cell as written by the forward.  Out: d_ifgo[T,B,4H];
  * dh, dc overwritten with the gradients of h_0, c_0.  ws: see
