@@ -370,6 +370,44 @@ def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H
         assert rel_err(a, b) < tol
 
 
+@pytest.mark.parametrize("T,B,I,H,dt", [(96, 64, 1024, 1024, torch.float16),    # helpers compute K1 inside the launch
+                                        (40, 32, 512, 1024, torch.bfloat16),   # same, 8 timesteps per row tile
+                                        (12, 40, 96, 512, torch.float16),      # 4-wave kernel: two launches
+                                        (9, 20, 50, 72, torch.float32)])       # general kernels
+def test_fwd_layer_equals_projection_then_recurrence(T, B, I, H, dt):
+    """fastlstm_fwd_layer must give bit-identical results to fastlstm_gemm_ifgo followed by
+    fastlstm_fwd_persistent, whichever way it schedules the two stages."""
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    p = make_problem(T, B, I, H, seed=5 + T)
+    g = {k: dev(v, dt) for k, v in p.items()}
+    st = torch.cuda.current_stream().cuda_stream
+    plan = _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan), "plan")
+    nbytes = lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0)
+    res = []
+    for fused in (False, True):
+        ifgo = torch.empty(T, B, 4 * H, device="cuda", dtype=dt)
+        out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
+        cell = torch.empty_like(out)
+        out[0], cell[0] = g["h0"], g["c0"]
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        if fused:
+            _lib.check(lib.fastlstm_fwd_layer(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(),
+                                              g["bh"].data_ptr(), g["Wh"].data_ptr(), ifgo.data_ptr(), out.data_ptr(),
+                                              cell.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H, code, st), "layer")
+        else:
+            _lib.check(lib.fastlstm_gemm_ifgo(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(),
+                                              g["bh"].data_ptr(), ifgo.data_ptr(), T, B, I, H, code, st), "k1")
+            _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(),
+                                                   g["Wh"].data_ptr(), ws.data_ptr(), ws.numel(), T, B, H, code, st), "fwd")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
+        res.append((out, cell, ifgo))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+
+
 def test_xcd_local_barrier_timeout_is_reported_not_hung():
     """The host-forced failure path of the L2 counter barrier: same contract as the flag barrier."""
     lib = _lib.load()
