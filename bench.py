@@ -36,9 +36,9 @@ WORKLOADS = {
 }
 PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the forward recurrence from rocprofv3 FETCH_SIZE + WRITE_SIZE,
-# scaled by a plain copy of known size (profiles/fwd_recurrence_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 858.5e6}
+# HBM bytes per launch of the fused forward layer kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE,
+# scaled by a plain copy of known size (profiles/fwd_layer_B_pmc.md); None = not measured
+TRAFFIC_BYTES = {"B": 1768.6e6}
 
 
 def main():
@@ -161,6 +161,11 @@ def main():
         ifgo.copy_(ifgo0)
         zero_ws(ws_f, plan_f)
 
+    def layer_fwd():   # what lstm_persistent_fwd calls: projection + recurrence, fused where CUs would idle
+        _lib.check(lib.fastlstm_fwd_layer(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
+                                          ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws_f.data_ptr(),
+                                          ws_f.numel(), T, B, I, H, code, stream), "fwd_layer")
+
     if args.stage == "fwd_recurrence":
         # counter runs (rocprofv3 --pmc): the dominant kernel plus a plain copy of known size
         # (2 x 256 MiB of traffic) that calibrates FETCH_SIZE / WRITE_SIZE
@@ -169,15 +174,19 @@ def main():
         cal_dst = torch.empty_like(cal_src)
         for _ in range(3):
             rec_fwd_pre()
-            rec_fwd()
+            rec_fwd()            # the recurrence alone (ifgo complete at launch)
+            zero_ws(ws_f, plan_f)
+            layer_fwd()          # projection + recurrence in one launch where the library fuses them
             cal_dst.copy_(cal_src)
         torch.cuda.synchronize()
         return
 
     t_k1 = ev_time(k1)
     t_rec = ev_time(rec_fwd, pre=rec_fwd_pre)
+    t_layer = ev_time(layer_fwd, pre=lambda: zero_ws(ws_f, plan_f))
     kernels = {"gemm_ifgo_ms": round(t_k1, 4), "recurrent_fwd_ms": round(t_rec, 4),
                "recurrent_fwd_us_per_step": round(t_rec * 1e3 / T, 3),
+               "fwd_layer_ms": round(t_layer, 4),
                "gemm_ifgo_tflops": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12, 2),
                "gemm_ifgo_frac_of_mfma_peak": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
                "plan_fwd": plan_f.as_dict(), "plan_bwd": plan_b.as_dict()}
@@ -222,19 +231,29 @@ def main():
         "gemm_wgrad_tflops": round(2.0 * T * B * 4 * H * (I + H) / (t_k89 * 1e-3) / 1e12, 2),
     })
 
-    # ---- roofline of the dominant kernel: the persistent forward recurrence -------------
-    rec_flops = 2.0 * B * H * 4 * H * T          # algorithmic flops of one launch
-    ach = rec_flops / (t_rec * 1e-3) / 1e12
+    # ---- roofline of the dominant kernel of the headline (forward) path ------------------
+    # XCD-local path with idle CUs: ONE launch does projection + recurrence (fastlstm_fwd_layer);
+    # otherwise the recurrence launch dominates.  Either way the bound is latency (T sequential
+    # steps), which the low MFMA fraction shows.
+    rec_flops = 2.0 * B * H * 4 * H * T          # algorithmic flops of the recurrence
+    k1_flops = 2.0 * T * B * I * 4 * H           # ... of the input projection
     xcd_local = lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, ws_f.numel()) == 1
-    roofline = {"kernel": "lstm_fwd_xcd_kernel" if xcd_local else "lstm_fwd_persistent_kernel",
-                "bound": "mfma", "achieved": round(ach, 2),
+    fused = xcd_local and t_layer < 0.9 * (t_k1 + t_rec)
+    if fused:
+        flops, t_dom, kname = rec_flops + k1_flops, t_layer, "lstm_fwd_xcd_kernel<..., HELP=true> (projection + recurrence)"
+        alg = "2*B*H*4H*T + 2*T*B*I*4H flop per launch = %.1f GFLOP" % (flops / 1e9)
+    else:
+        flops, t_dom = rec_flops, t_rec
+        kname = "lstm_fwd_xcd_kernel" if xcd_local else "lstm_fwd_persistent_kernel"
+        alg = "2*B*H*4H*T flop per launch = %.1f GFLOP" % (flops / 1e9)
+    ach = flops / (t_dom * 1e-3) / 1e12
+    roofline = {"kernel": kname, "bound": "mfma", "achieved": round(ach, 2),
                 "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dname], 4),
-                "traffic": TRAFFIC_BYTES.get(args.workload),
-                "algorithmic": "2*B*H*4H*T flop per launch = %.1f GFLOP" % (rec_flops / 1e9),
-                "launch_ms": round(t_rec, 4),
+                "traffic": TRAFFIC_BYTES.get(args.workload) if fused else None,
+                "algorithmic": alg, "launch_ms": round(t_dom, 4),
                 "note": "latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange "
                         + ("through the L2 of one XCD" if xcd_local else "through device memory")
-                        + "; us/step is in kernels.recurrent_fwd_us_per_step"}
+                        + "; us/step of the recurrence alone is in kernels.recurrent_fwd_us_per_step"}
 
     res = {
         "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
