@@ -237,8 +237,37 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     return FASTLSTM_OK;
 }
 
+// In-kernel dx = d_ifgo . Wx by the workgroups without a role (see BwdXcdParams).
+bool plan_k5_helpers(const XcdCfg &c, const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
+                     BwdXcdParams *p) {
+    if (dtype == FASTLSTM_FP32 || !((c.mt == 2 && c.nkw == 16) || (c.mt == 1 && c.nkw == 8))) return false;
+    const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - n_active;
+    if (n_helpers < kNumXcd * 8) return false;
+    const int M = T * B, N = I, K = 4 * H;
+    if (!gemm16_eligible(dtype, M, N, K, K, N, false, true) || N % 8) return false;
+    const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
+    int base = 1;
+    while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
+    int ct = std::max(1, n_helpers / tiles_n / base) * base;
+    while (cdiv(tiles_m, ct) > 32) ct += base;
+    p->k5 = GemmParams{};
+    p->k5.A = d_ifgo; p->k5.B = Wx; p->k5.C = dx;
+    p->k5.M = M; p->k5.N = N; p->k5.K = K;
+    p->k5.lda = K; p->k5.ldb = N; p->k5.ldc = N;
+    p->k5.splits = 1; p->k5.k_per_split = K;
+    p->k5_tiles_m = tiles_m; p->k5_tiles_n = tiles_n;
+    p->k5_chunk_tiles = ct; p->k5_chunk_steps = ct * 256 / B; p->k5_chunks = cdiv(tiles_m, ct);
+    p->n_active = n_active;
+    p->chunk_done = p->hdr->reserved;
+    p->ticket = p->hdr->reserved + 32;
+    return true;
+}
+
+// With dx != nullptr the kernel also has to compute dx = d_ifgo . Wx (returns 2 when that is not
+// possible in-kernel).
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
-                unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream) {
+                unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
+                const void *Wx = nullptr, void *dx = nullptr, int I = 0) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
     BwdXcdParams p{};
@@ -249,6 +278,16 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
     p.spin_limit = spin_limit_ticks();
+    if (dx) {
+        if (!plan_k5_helpers(c, d_ifgo, Wx, dx, T, B, I, H, dtype, &p)) return 2;
+        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 4, 2, 2>::LDS_BYTES);
+        BwdXcdLauncher hl = dtype == FASTLSTM_FP16 ? launch_bwd_xcd_help_f16 : launch_bwd_xcd_help_bf16;
+        int occ = 0;
+        if (hl(p, c.mt, c.nkw, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (occ < 1) return 2;
+        if (hl(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+        return FASTLSTM_OK;
+    }
     BwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_bwd_xcd_f32
                                                    : (dtype == FASTLSTM_FP16 ? launch_bwd_xcd_f16 : launch_bwd_xcd_bf16);
     int occ = 0;
@@ -543,6 +582,32 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
 #endif
     if (int rc = fastlstm_gemm_ifgo(x, Wx, bx, bh, ifgo, T, B, I, H, dtype, stream)) return rc;
     return fastlstm_fwd_persistent(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream);
+}
+
+int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
+                       const void *Wh, const void *Wx, void *dx, void *ws, size_t ws_bytes, int T, int B, int I, int H,
+                       int dtype, void *stream) {
+    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !dx || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(dout) || !aligned16(dh) || !aligned16(dc) || !aligned16(ifgo) || !aligned16(cell) ||
+        !aligned16(d_ifgo) || !aligned16(Wh) || !aligned16(Wx) || !aligned16(dx) || !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    // Where the XCD-local reverse recurrence leaves CUs without a role, those workgroups compute dx
+    // inside the same launch, chunk by chunk behind the recurrence; otherwise two launches.
+    {
+        fastlstm_plan pl;
+        if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
+        if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+        if (pl.wave_split != 2) {
+            const int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes,
+                                       T, B, H, dtype, static_cast<hipStream_t>(stream), Wx, dx, I);
+            if (rc <= 0) return rc;   // launched, or failed
+        }
+    }
+    if (int rc = fastlstm_bwd_persistent(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
+        return rc;
+    return fastlstm_gemm_dx(d_ifgo, Wx, dx, T, B, I, H, dtype, stream);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {

@@ -32,11 +32,50 @@ struct BwdXcdParams {
     int T, B, H;
     int n_ht, gpx, n_groups;
     int KSB;            // k-steps covering 4H
+    // In-kernel dx = d_ifgo . Wx (HELP instantiations, k5_tiles_n > 0): the workgroups without a role
+    // in the recurrence compute it in 256 x 256 tiles, latest timesteps first, as soon as the
+    // recurrence has finished a chunk of k5_chunk_steps timesteps (k5_chunk_tiles row tiles);
+    // chunk_done[c] counts the recurrence workgroups (n_active) whose part of chunk c is in memory.
+    GemmParams k5;      // M = T*B, N = I, K = 4H, A = d_ifgo, B = Wx (K-major), C = dx
+    int k5_tiles_m, k5_tiles_n;
+    int k5_chunk_tiles, k5_chunk_steps, k5_chunks;
+    int n_active;
+    int *chunk_done;    // [<= 32] device-scope counters, zero at launch
+    int *ticket;        // numbers the helper workgroups, zero at launch
     long long spin_limit;
 };
 
-template <typename T, int MT, int NKW, int NTW, int NWV>
+// dx tiles by a workgroup (8 waves) that has no role in the recurrence.  Chunks become available
+// in reverse time order; helper h of n takes tiles h, h + n, ... of the list ordered that way.
+template <typename T>
+__device__ __forceinline__ void k5_helper(const BwdXcdParams &p, unsigned char *smem) {
+    int *ticket = reinterpret_cast<int *>(smem);
+    if (threadIdx.x == 0) *ticket = __hip_atomic_fetch_add(p.ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int h = *ticket;
+    __syncthreads();
+    const int n_helpers = (int)gridDim.x - p.n_active;
+    const int per_chunk = p.k5_chunk_tiles * p.k5_tiles_n;
+    const int total = p.k5_chunks * per_chunk;
+    int seen = -1;   // last chunk this workgroup has waited for
+    for (int i = h; i < total; i += n_helpers) {
+        const int k = i / per_chunk, r = i % per_chunk;
+        const int c = p.k5_chunks - 1 - k;                       // chunk in forward time
+        const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
+        if (rt >= p.k5_tiles_m) continue;
+        if (c != seen) {   // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
+            if ((threadIdx.x >> 6) == 0) wait_versions(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
+            __syncthreads();
+            seen = c;
+        }
+        gemm16_tile<T, false, true, 256, 256, 2, 4, 2, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
+        __syncthreads();   // the LDS is reused by the next tile
+    }
+}
+
+template <typename T, int MT, int NKW, int NTW, int NWV, bool HELP = false>
 __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdParams p) {
+    static_assert(!HELP || (NWV == 8 && sizeof(T) == 2), "the in-kernel GEMM tile is the 8-wave 16-bit one");
     using E = Elem<T>;
     constexpr bool ACC = (E::DT == FASTLSTM_FP32);
     constexpr int NTHR = kWave * NWV;
@@ -58,8 +97,14 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
     const int g = gl * kNumXcd + xcd;
-    if (gl >= p.gpx || g >= p.n_groups) return;
+    if (gl >= p.gpx || g >= p.n_groups) {
+        if constexpr (HELP) {
+            if (p.k5_tiles_n > 0) k5_helper<T>(p, smem);
+        }
+        return;
+    }
     const int u0 = j * HT, b0 = g * BT;
+    const bool k5_live = HELP && p.k5_tiles_n > 0;
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                    // [NWV][MT][NT][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
@@ -236,6 +281,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         __syncthreads();
         if (tid < kXcdReplicas)
             __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        // every store of the previous steps (d_ifgo tiles included) has been acknowledged: when the
+        // previous step closed a chunk, hand the chunk to the dx helpers (release: this XCD's L2 is
+        // written back so that the other XCDs can read it)
+        if (k5_live && tid == kWave && s > 0 && (t + 1) % p.k5_chunk_steps == 0)
+            __hip_atomic_fetch_add(p.chunk_done + (t + 1) / p.k5_chunk_steps, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         tile_to_global(t);
         if (s + 1 < T_) fetch_tiles(t - 1, gpre, cpre, dpre);
 
@@ -288,6 +338,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         // the next step's publish barrier orders these reads before the next writes to `red`
     }
 
+    if (k5_live) {   // the last chunk (timesteps 0 ..)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == kWave) __hip_atomic_fetch_add(p.chunk_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
 #pragma unroll
     for (int m = 0; m < IPT; ++m)

@@ -174,16 +174,14 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
         plan = _plan(x.device, batch_size, hidden_size, code, True)
         ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
-        _lib.check(lib.fastlstm_bwd_persistent(dh.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(),
-                                               ifgo.data_ptr(), cell.data_ptr(), d_ifgo.data_ptr(),
-                                               Wh.data_ptr(), ws.data_ptr(), ws.numel(), seq_len,
-                                               batch_size, hidden_size, code, stream),
-                   "fastlstm_bwd_persistent")
-        _check_ws(ws, "fastlstm_bwd_persistent")
         d_x = torch.empty_like(x)
-        _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), d_x.data_ptr(), seq_len,
-                                        batch_size, input_size, hidden_size, code, stream),
-                   "fastlstm_gemm_dx")
+        # reverse time loop + dx in one call (the library fuses the two where CUs would idle)
+        _lib.check(lib.fastlstm_bwd_layer(dh.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
+                                          cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), Wx.data_ptr(),
+                                          d_x.data_ptr(), ws.data_ptr(), ws.numel(), seq_len, batch_size,
+                                          input_size, hidden_size, code, stream),
+                   "fastlstm_bwd_layer")
+        _check_ws(ws, "fastlstm_bwd_layer")
         dbx, dbh, dWx, dWh = Wgrad(d_ifgo, x, h)
     return d_x, dh_n, dc_n, dWx, dbx, dWh, dbh
 
