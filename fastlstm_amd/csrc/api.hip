@@ -197,7 +197,6 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     p->k1_tiles_m = tiles_m; p->k1_tiles_n = tiles_n;
     p->k1_chunk_tiles = ct; p->k1_chunk_steps = steps;
     p->k1_done = p->hdr->reserved;
-    p->k1_ticket = p->hdr->reserved + 32;
     return true;
 }
 
@@ -237,37 +236,60 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     return FASTLSTM_OK;
 }
 
-// In-kernel dx = d_ifgo . Wx by the workgroups without a role (see BwdXcdParams).
-bool plan_k5_helpers(const XcdCfg &c, const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
-                     BwdXcdParams *p) {
+// What the reverse launch may compute besides the recurrence (fastlstm_bwd_layer).
+struct BwdExtras {
+    const void *Wx, *x, *h;
+    void *dx, *dWx, *dWh;
+    int I;
+};
+
+// In-kernel dx (and, where the shapes suit the 16-bit tile kernel, dWx and dWh) by the workgroups
+// without a role in the recurrence (see BwdXcdParams).  *wgrad_fused tells whether the weight
+// gradients are part of the launch.
+bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, int T, int B, int H, int dtype,
+                      BwdXcdParams *p, bool *wgrad_fused) {
+    *wgrad_fused = false;
     if (dtype == FASTLSTM_FP32 || !((c.mt == 2 && c.nkw == 16) || (c.mt == 1 && c.nkw == 8))) return false;
     const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - n_active;
     if (n_helpers < kNumXcd * 8) return false;
-    const int M = T * B, N = I, K = 4 * H;
-    if (!gemm16_eligible(dtype, M, N, K, K, N, false, true) || N % 8) return false;
-    const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
+    const int I = e.I, M = T * B, K = 4 * H;
+    if (!gemm16_eligible(dtype, M, I, K, K, I, false, true) || I % 8) return false;
+    const int tiles_m = cdiv(M, 256), tiles_n = cdiv(I, 256);
+    // a chunk: whole timesteps, about 8 row tiles (a short tail behind the recurrence), at most 32 chunks
     int base = 1;
-    while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
-    int ct = std::max(1, n_helpers / tiles_n / base) * base;
+    while ((base * 256) % B) ++base;
+    int ct = base >= 8 ? base : (8 / base) * base;
     while (cdiv(tiles_m, ct) > 32) ct += base;
     p->k5 = GemmParams{};
-    p->k5.A = d_ifgo; p->k5.B = Wx; p->k5.C = dx;
-    p->k5.M = M; p->k5.N = N; p->k5.K = K;
-    p->k5.lda = K; p->k5.ldb = N; p->k5.ldc = N;
+    p->k5.A = d_ifgo; p->k5.B = e.Wx; p->k5.C = e.dx;
+    p->k5.M = M; p->k5.N = I; p->k5.K = K;
+    p->k5.lda = K; p->k5.ldb = I; p->k5.ldc = I;
     p->k5.splits = 1; p->k5.k_per_split = K;
     p->k5_tiles_m = tiles_m; p->k5_tiles_n = tiles_n;
     p->k5_chunk_tiles = ct; p->k5_chunk_steps = ct * 256 / B; p->k5_chunks = cdiv(tiles_m, ct);
     p->n_active = n_active;
     p->chunk_done = p->hdr->reserved;
-    p->ticket = p->hdr->reserved + 32;
+    p->wg_tiles = 0;
+    if (e.dWx && gemm16_eligible(dtype, K, I, M, K, I, true, true) && gemm16_eligible(dtype, K, H, M, K, H, true, true) &&
+        H % 8 == 0) {
+        GemmParams g{};
+        g.A = d_ifgo; g.M = K; g.K = M; g.lda = K; g.splits = 1; g.k_per_split = M;
+        p->k8 = g; p->k8.B = e.x; p->k8.C = e.dWx; p->k8.N = I; p->k8.ldb = I; p->k8.ldc = I;
+        p->k9 = g; p->k9.B = e.h; p->k9.C = e.dWh; p->k9.N = H; p->k9.ldb = H; p->k9.ldc = H;
+        p->wg_tiles_m = cdiv(K, 256);
+        p->k8_tiles_n = cdiv(I, 256); p->k9_tiles_n = cdiv(H, 256);
+        p->wg_tiles = p->wg_tiles_m * (p->k8_tiles_n + p->k9_tiles_n);
+        *wgrad_fused = true;
+    }
     return true;
 }
 
-// With dx != nullptr the kernel also has to compute dx = d_ifgo . Wx (returns 2 when that is not
-// possible in-kernel).
+// With `extras` the launch also computes dx (returns 2 when that is not possible in-kernel) and, if
+// it can, the weight gradients: returns 0 when they were part of the launch, 3 when they are still
+// to be computed.
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
-                const void *Wx = nullptr, void *dx = nullptr, int I = 0) {
+                const BwdExtras *extras = nullptr) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
     BwdXcdParams p{};
@@ -278,15 +300,16 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
     p.spin_limit = spin_limit_ticks();
-    if (dx) {
-        if (!plan_k5_helpers(c, d_ifgo, Wx, dx, T, B, I, H, dtype, &p)) return 2;
+    if (extras) {
+        bool wgrad_fused = false;
+        if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused)) return 2;
         const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 4, 2, 2>::LDS_BYTES);
         BwdXcdLauncher hl = dtype == FASTLSTM_FP16 ? launch_bwd_xcd_help_f16 : launch_bwd_xcd_help_bf16;
         int occ = 0;
         if (hl(p, c.mt, c.nkw, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (occ < 1) return 2;
         if (hl(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
-        return FASTLSTM_OK;
+        return wgrad_fused ? FASTLSTM_OK : 3;
     }
     BwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_bwd_xcd_f32
                                                    : (dtype == FASTLSTM_FP16 ? launch_bwd_xcd_f16 : launch_bwd_xcd_bf16);
@@ -585,29 +608,45 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
 }
 
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
-                       const void *Wh, const void *Wx, void *dx, void *ws, size_t ws_bytes, int T, int B, int I, int H,
-                       int dtype, void *stream) {
-    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !dx || !ws) return FASTLSTM_ERR_NULL;
+                       const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
+                       void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
+                       int H, int dtype, void *stream) {
+    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !x || !h || !dx || !dWx || !dWh || !db ||
+        !ws || !wgrad_ws)
+        return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
     if (!aligned16(dout) || !aligned16(dh) || !aligned16(dc) || !aligned16(ifgo) || !aligned16(cell) ||
-        !aligned16(d_ifgo) || !aligned16(Wh) || !aligned16(Wx) || !aligned16(dx) || !aligned16(ws))
+        !aligned16(d_ifgo) || !aligned16(Wh) || !aligned16(Wx) || !aligned16(x) || !aligned16(h) || !aligned16(dx) ||
+        !aligned16(dWx) || !aligned16(dWh) || !aligned16(ws) || !aligned16(wgrad_ws))
         return FASTLSTM_ERR_ALIGN;
+    if (wgrad_ws_bytes < fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype)) return FASTLSTM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
     // Where the XCD-local reverse recurrence leaves CUs without a role, those workgroups compute dx
-    // inside the same launch, chunk by chunk behind the recurrence; otherwise two launches.
-    {
-        fastlstm_plan pl;
-        if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
-        if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
-        if (pl.wave_split != 2) {
-            const int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes,
-                                       T, B, H, dtype, static_cast<hipStream_t>(stream), Wx, dx, I);
-            if (rc <= 0) return rc;   // launched, or failed
-        }
+    // and the weight gradients inside the same launch, chunk of timesteps by chunk behind the
+    // recurrence; otherwise the stages are launched back to back.
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
+    if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+    int rc = 1;
+    if (pl.wave_split != 2) {
+        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I};
+        rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
+                         s, &e);
+        if (rc < 0) return rc;
     }
-    if (int rc = fastlstm_bwd_persistent(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
-        return rc;
-    return fastlstm_gemm_dx(d_ifgo, Wx, dx, T, B, I, H, dtype, stream);
+    if (rc == 0) {   // everything but the bias gradient was part of the launch
+        const int chunks = colsum_chunks(T * B);
+        return launch_colsum(dtype, d_ifgo, db, static_cast<float *>(wgrad_ws), T * B, 4 * H, chunks, s) == hipSuccess
+                   ? FASTLSTM_OK
+                   : FASTLSTM_ERR_HIP;
+    }
+    if (rc != 3) {   // nothing was launched: recurrence, then dx
+        if (int r2 = fastlstm_bwd_persistent(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
+            return r2;
+        if (int r2 = fastlstm_gemm_dx(d_ifgo, Wx, dx, T, B, I, H, dtype, stream)) return r2;
+    }
+    return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {

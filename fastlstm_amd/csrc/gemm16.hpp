@@ -75,23 +75,19 @@ template <int N> __device__ __forceinline__ void wait_vm_at_most() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));
 }
 
-// One BM x BN tile of C (rows m0.., columns n0.., K range of `split`) by a workgroup of
-// 64*WVM*WVN threads with Gemm16Cfg::LDS_BYTES of LDS at `smem`.  All threads of the workgroup
-// call it together; it ends with the tile stored (the caller orders later use of `smem`).
+// acc += A(rows m0.., k in [kb, ke)) . B(columns n0.., same k) for one BM x BN tile, by a workgroup
+// of 64*WVM*WVN threads with Gemm16Cfg::LDS_BYTES of LDS at `smem`; ke - kb a multiple of BK.  All
+// threads of the workgroup call it together; it ends behind a workgroup barrier (the LDS is free).
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
-__device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
-                                            unsigned char *smem, const int trace_slot) {
+__device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m0, const int n0, const int kb,
+                                                const int ke, unsigned char *smem,
+                                                f32x4 (&acc)[BM / WVM / 16][BN / WVN / 16]) {
     using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
-    constexpr int NWAVES = C::NWAVES, THREADS = C::THREADS;
+    constexpr int NWAVES = C::NWAVES;
     constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave / WVN, wn = wave % WVN;
-
-    long long t_start = 0, t_loop = 0, t_epi = 0;
-    if (p.trace) t_start = (long long)wall_clock64();
-    const int kb = split * p.k_per_split;
-    const int ke = min(p.K, kb + p.k_per_split);
     const int nkt = (ke - kb) / BK;
 
     const unsigned a_bytes = (unsigned)((A_KM ? (size_t)p.K : (size_t)p.M) * p.lda * 2);
@@ -161,12 +157,6 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
         }
     };
 
-    f32x4 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
     // NS-stage pipeline: the loads of k-tiles kt+1 .. kt+NS-1 are in flight while k-tile kt is
     // multiplied (memory latency, not bandwidth, bounds a short loop: ~2 us per round trip).
     // Per iteration: wait for this wave's own loads of tile kt (everything issued later may
@@ -177,7 +167,6 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
 #pragma unroll
     for (int d = 0; d < D; ++d)
         if (d < nkt) gload(d, d);
-    if (p.trace) t_loop = (long long)wall_clock64();
     for (int kt = 0; kt < nkt; ++kt) {
         if (kt + D <= nkt) wait_vm_at_most<(D - 1) * LPT>();   // D-1 younger tiles may stay in flight
         else wait_vm_at_most<0>();                             // tail: fewer tiles behind this one
@@ -198,9 +187,20 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
             }
         }
     }
-    __syncthreads();  // all waves are done reading the stages before the C tile reuses them
+    __syncthreads();  // all waves are done reading the stages before the LDS is reused
+}
 
-    if (p.trace) t_epi = (long long)wall_clock64();
+// Stores the accumulated tile: fp32 partials of `split` when p.splits > 1, else bias + rounding,
+// staged through LDS and written with 16-byte row-contiguous stores.
+template <typename T, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+__device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m0, const int n0, const int split,
+                                                unsigned char *smem,
+                                                const f32x4 (&acc)[BM / WVM / 16][BN / WVN / 16]) {
+    using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
+    constexpr int THREADS = C::THREADS, TM = C::TM, TN = C::TN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, r = lane & 15;
+    const int wm = wave / WVN, wn = wave % WVN;
     // ---- epilogue -----------------------------------------------------------------------
     // lane holds C[m = tile row r][n = 4q .. 4q+3] of each 16x16 tile
     if (p.splits > 1) {
@@ -262,9 +262,27 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
                 if (n + e < p.N) dst[e] = tv[e];
         }
     }
-    if (p.trace && tid == 0) {
+}
+
+// One BM x BN tile of C (rows m0.., columns n0.., K range of `split`): main loop + epilogue.
+template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+__device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
+                                            unsigned char *smem, const int trace_slot) {
+    constexpr int TM = BM / WVM / 16, TN = BN / WVN / 16;
+    long long t_start = 0, t_epi = 0;
+    if (p.trace) t_start = (long long)wall_clock64();
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int kb = split * p.k_per_split;
+    gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(p.K, kb + p.k_per_split), smem, acc);
+    if (p.trace) t_epi = (long long)wall_clock64();
+    gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, split, smem, acc);
+    if (p.trace && threadIdx.x == 0) {   // stamps: start, main loop entered (= start), main loop left, done
         long long *t = p.trace + (size_t)trace_slot * 4;
-        t[0] = t_start; t[1] = t_loop; t[2] = t_epi; t[3] = (long long)wall_clock64();
+        t[0] = t_start; t[1] = t_start; t[2] = t_epi; t[3] = (long long)wall_clock64();
     }
 }
 

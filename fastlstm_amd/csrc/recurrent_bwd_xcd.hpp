@@ -39,37 +39,67 @@ struct BwdXcdParams {
     GemmParams k5;      // M = T*B, N = I, K = 4H, A = d_ifgo, B = Wx (K-major), C = dx
     int k5_tiles_m, k5_tiles_n;
     int k5_chunk_tiles, k5_chunk_steps, k5_chunks;
+    // In-kernel weight gradients (wg_tiles > 0): dWx = d_ifgo^T . x and dWh = d_ifgo^T . h, 256 x 256
+    // output tiles, the first n_helpers of them one per helper: a helper adds the K range (rows of
+    // T*B) of every finished chunk to its accumulators and stores the tile after the last chunk.
+    GemmParams k8, k9;  // M = 4H, N = I | H, K = T*B, A = d_ifgo (K-major), B = x | h (K-major), C = dWx | dWh
+    int k8_tiles_n, k9_tiles_n, wg_tiles_m, wg_tiles;
     int n_active;
     int *chunk_done;    // [<= 32] device-scope counters, zero at launch
-    int *ticket;        // numbers the helper workgroups, zero at launch
     long long spin_limit;
 };
 
-// dx tiles by a workgroup (8 waves) that has no role in the recurrence.  Chunks become available
-// in reverse time order; helper h of n takes tiles h, h + n, ... of the list ordered that way.
+// The workgroups (8 waves) without a role in the recurrence.  Chunks of timesteps become available
+// in reverse time order.  Helper h of n owns weight-gradient tile h (if there is one), which it
+// accumulates chunk by chunk, and takes the dx tiles h, h + n, ... of the list ordered by chunk.
 template <typename T>
-__device__ __forceinline__ void k5_helper(const BwdXcdParams &p, unsigned char *smem) {
-    int *ticket = reinterpret_cast<int *>(smem);
-    if (threadIdx.x == 0) *ticket = __hip_atomic_fetch_add(p.ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const int h = *ticket;
-    __syncthreads();
-    const int n_helpers = (int)gridDim.x - p.n_active;
+__device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char *smem) {
+    constexpr int TM = 4, TN = 8;   // 16 x 16 tiles per wave of the 256 x 256 tile, 8 waves as 4 x 2
+    int n_helpers;
+    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups, &n_helpers);
     const int per_chunk = p.k5_chunk_tiles * p.k5_tiles_n;
-    const int total = p.k5_chunks * per_chunk;
-    int seen = -1;   // last chunk this workgroup has waited for
-    for (int i = h; i < total; i += n_helpers) {
-        const int k = i / per_chunk, r = i % per_chunk;
-        const int c = p.k5_chunks - 1 - k;                       // chunk in forward time
-        const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
-        if (rt >= p.k5_tiles_m) continue;
-        if (c != seen) {   // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
-            if ((threadIdx.x >> 6) == 0) wait_versions(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
-            __syncthreads();
-            seen = c;
+    // the weight-gradient tile of this helper: tiles of dWx first, then those of dWh
+    const int n8 = p.wg_tiles_m * p.k8_tiles_n;
+    const bool own = h < p.wg_tiles;
+    const bool is8 = h < n8;
+    const GemmParams &wp = is8 ? p.k8 : p.k9;
+    const int wi = is8 ? h : h - n8, wtn = is8 ? p.k8_tiles_n : p.k9_tiles_n;
+    const int wm0 = (wi / wtn) * 256, wn0 = (wi % wtn) * 256;
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int k = 0; k < p.k5_chunks; ++k) {
+        const int c = p.k5_chunks - 1 - k;   // chunk in forward time
+        // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
+        if ((threadIdx.x >> 6) == 0) wait_versions(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
+        __syncthreads();
+        if (own) {
+            const int kb = c * p.k5_chunk_tiles * 256, ke = min(wp.K, kb + p.k5_chunk_tiles * 256);
+            gemm16_mainloop<T, true, true, 256, 256, 2, 4, 2, 2>(wp, wm0, wn0, kb, ke, smem, acc);
         }
-        gemm16_tile<T, false, true, 256, 256, 2, 4, 2, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
-        __syncthreads();   // the LDS is reused by the next tile
+        for (int i = k * per_chunk + ((h - k * per_chunk) % n_helpers + n_helpers) % n_helpers; i < (k + 1) * per_chunk;
+             i += n_helpers) {
+            const int r = i - k * per_chunk;
+            const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
+            if (rt >= p.k5_tiles_m) continue;
+            gemm16_tile<T, false, true, 256, 256, 2, 4, 2, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
+            __syncthreads();   // the LDS is reused by the next tile
+        }
+    }
+    if (own) {
+        gemm16_epilogue<T, 256, 256, 2, 4, 2, 2>(wp, wm0, wn0, 0, smem, acc);
+        __syncthreads();
+    }
+    // weight-gradient tiles beyond one per helper: everything they need is in memory now
+    for (int w = h + n_helpers; w < p.wg_tiles; w += n_helpers) {
+        const bool w8 = w < n8;
+        const GemmParams &q = w8 ? p.k8 : p.k9;
+        const int qi = w8 ? w : w - n8, qtn = w8 ? p.k8_tiles_n : p.k9_tiles_n;
+        gemm16_tile<T, true, true, 256, 256, 2, 4, 2, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
+        __syncthreads();
     }
 }
 
@@ -99,7 +129,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int g = gl * kNumXcd + xcd;
     if (gl >= p.gpx || g >= p.n_groups) {
         if constexpr (HELP) {
-            if (p.k5_tiles_n > 0) k5_helper<T>(p, smem);
+            if (p.k5_tiles_n > 0) bwd_helper<T>(p, smem);
         }
         return;
     }

@@ -54,7 +54,6 @@ struct FwdXcdParams {
     int k1_tiles_m, k1_tiles_n;
     int k1_chunk_tiles, k1_chunk_steps;
     int *k1_done;         // [<= 32] device-scope counters, zero at launch
-    int *k1_ticket;       // numbers the helper workgroups, zero at launch
     long long spin_limit;
     long long *trace;  // diagnostic build only
 };
@@ -106,18 +105,32 @@ __device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader 
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");   // compiler ordering only
 }
 
+// Rank of the calling workgroup among the workgroups of the launch that have no role in the
+// recurrence, counted XCD by XCD, and their number: helpers with consecutive ranks share an L2.
+// (Roles: see the placement rule at the top of the kernels.)
+__device__ __forceinline__ int helper_rank(int n_ht, int gpx, int n_groups, int *n_helpers) {
+    const int my_xcd = blockIdx.x % kNumXcd, my_slot = blockIdx.x / kNumXcd;
+    const int slots = gridDim.x / kNumXcd;
+    int rank = 0, total = 0;
+    for (int x = 0; x < kNumXcd; ++x)
+        for (int sl = 0; sl < slots; ++sl) {
+            const int gl = sl / n_ht;
+            const bool idle = gl >= gpx || gl * kNumXcd + x >= n_groups;
+            total += idle;
+            rank += idle && (x < my_xcd || (x == my_xcd && sl < my_slot));
+        }
+    *n_helpers = total;
+    return rank;
+}
+
 // Input projection by a workgroup (8 waves) that has no role in the recurrence.  Helper h of n
 // takes tiles h, h + n, ... of the time-ordered tile list.  A finished tile is made visible to the
 // other XCDs (its stores acknowledged, this XCD's L2 written back: the release of the atomic) before
 // it is counted.
 template <typename T>
 __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *smem) {
-    int *ticket = reinterpret_cast<int *>(smem);
-    if (threadIdx.x == 0) *ticket = __hip_atomic_fetch_add(p.k1_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const int h = *ticket;
-    __syncthreads();
-    const int n_helpers = (int)gridDim.x - p.n_groups * p.n_ht;
+    int n_helpers;
+    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups, &n_helpers);
     const int total = p.k1_tiles_m * p.k1_tiles_n;
     for (int tile = h; tile < total; tile += n_helpers) {
         const int rt = tile / p.k1_tiles_n, ct = tile % p.k1_tiles_n;

@@ -174,15 +174,24 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
         plan = _plan(x.device, batch_size, hidden_size, code, True)
         ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
+        x, h = x.contiguous(), h.contiguous()
         d_x = torch.empty_like(x)
-        # reverse time loop + dx in one call (the library fuses the two where CUs would idle)
+        G = 4 * hidden_size
+        dWx = torch.empty((G, input_size), device=x.device, dtype=x.dtype)
+        dWh = torch.empty((G, hidden_size), device=x.device, dtype=x.dtype)
+        db = torch.empty((G,), device=x.device, dtype=x.dtype)
+        wws = torch.empty(lib.fastlstm_wgrad_workspace_bytes(seq_len, batch_size, input_size, hidden_size, code),
+                          dtype=torch.uint8, device=x.device)
+        # reverse time loop + dx + weight gradients in one call (the library fuses them where CUs would idle)
         _lib.check(lib.fastlstm_bwd_layer(dh.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
                                           cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), Wx.data_ptr(),
-                                          d_x.data_ptr(), ws.data_ptr(), ws.numel(), seq_len, batch_size,
-                                          input_size, hidden_size, code, stream),
+                                          x.data_ptr(), h.data_ptr(), d_x.data_ptr(), dWx.data_ptr(),
+                                          dWh.data_ptr(), db.data_ptr(), ws.data_ptr(), ws.numel(),
+                                          wws.data_ptr(), wws.numel(), seq_len, batch_size, input_size,
+                                          hidden_size, code, stream),
                    "fastlstm_bwd_layer")
         _check_ws(ws, "fastlstm_bwd_layer")
-        dbx, dbh, dWx, dWh = Wgrad(d_ifgo, x, h)
+        dbx = dbh = db   # the same tensor twice, as Wgrad returns it (fastlstm/lstm.py:501)
     return d_x, dh_n, dc_n, dWx, dbx, dWh, dbh
 
 

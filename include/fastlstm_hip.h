@@ -125,14 +125,18 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
                             const void *cell, void *d_ifgo, const void *Wh, void *ws,
                             size_t ws_bytes, int T, int B, int H, int dtype, void *stream);
 
-/* K4 + K5 for one layer in one call: the same results as fastlstm_bwd_persistent followed by
- * fastlstm_gemm_dx (same arguments, same workspace contract).  Where the XCD-local reverse
- * recurrence leaves CUs without a role, the workgroups on those CUs compute dx inside the same
- * launch, chunk of timesteps by chunk behind the recurrence; otherwise the two stages are launched
- * back to back.  Replaces fastlstm/lstm.py:277-290 together with 294. */
+/* K4 + K5 + K6..K9 for one layer in one call: the same results as fastlstm_bwd_persistent,
+ * fastlstm_gemm_dx and fastlstm_gemm_wgrad one after the other (same arguments and workspace
+ * contracts; dWx and dWh to the rounding of a different summation order).  Where the XCD-local
+ * reverse recurrence leaves CUs without a role, the workgroups on those CUs compute dx and the
+ * weight gradients inside the same launch, chunk of timesteps by chunk behind the recurrence;
+ * otherwise the stages are launched back to back.  Replaces fastlstm/lstm.py:277-290, 294 and
+ * 494-501 together. */
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
-                       void *d_ifgo, const void *Wh, const void *Wx, void *dx, void *ws, size_t ws_bytes,
-                       int T, int B, int I, int H, int dtype, void *stream);
+                       void *d_ifgo, const void *Wh, const void *Wx, const void *x, const void *h,
+                       void *dx, void *dWx, void *dWh, void *db, void *ws, size_t ws_bytes,
+                       void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H, int dtype,
+                       void *stream);
 
 /* K5 -- dx[T*B,I] = d_ifgo[T*B,4H] . Wx[4H,I].   Replaces fastlstm/lstm.py:294. */
 int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H,

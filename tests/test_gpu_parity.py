@@ -412,11 +412,13 @@ def test_fwd_layer_equals_projection_then_recurrence(T, B, I, H, dt):
                                         (40, 32, 512, 1024, torch.bfloat16),
                                         (24, 48, 256, 512, torch.float16),     # 16 units per workgroup
                                         (9, 20, 50, 72, torch.float32)])       # general kernels, two launches
-def test_bwd_layer_equals_recurrence_then_dx(T, B, I, H, dt):
-    """fastlstm_bwd_layer must give bit-identical results to fastlstm_bwd_persistent followed by
-    fastlstm_gemm_dx, whichever way it schedules the two stages."""
+def test_bwd_layer_equals_separate_stages(T, B, I, H, dt):
+    """fastlstm_bwd_layer must give the results of fastlstm_bwd_persistent, fastlstm_gemm_dx and
+    fastlstm_gemm_wgrad run one after the other, whichever way it schedules the stages: bit-identical
+    d_ifgo, dx, dh_0, dc_0, db; dWx and dWh to the rounding of a different summation order."""
     lib = _lib.load()
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
     p = make_problem(T, B, I, H, seed=11 + T)
     g = {k: dev(v, dt) for k, v in p.items()}
     out, cell, ifgo = L.lstm_persistent_fwd(g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"])
@@ -424,26 +426,37 @@ def test_bwd_layer_equals_recurrence_then_dx(T, B, I, H, dt):
     plan = _lib.Plan()
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan), "plan")
     nbytes = lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1)
+    wbytes = lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code)
     res = []
     for fused in (False, True):
         d_ifgo = torch.empty_like(ifgo)
         dx = torch.empty(T, B, I, device="cuda", dtype=dt)
+        dWx, dWh, db = torch.empty_like(g["Wx"]), torch.empty_like(g["Wh"]), torch.empty_like(g["bx"])
         dh, dc = g["dh_n"].clone(), g["dc_n"].clone()
         ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        wws = torch.empty(wbytes, dtype=torch.uint8, device="cuda")
         if fused:
             _lib.check(lib.fastlstm_bwd_layer(g["dout"].data_ptr(), dh.data_ptr(), dc.data_ptr(), ifgo.data_ptr(),
                                               cell.data_ptr(), d_ifgo.data_ptr(), g["Wh"].data_ptr(), g["Wx"].data_ptr(),
-                                              dx.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H, code, st), "layer")
+                                              g["x"].data_ptr(), out.data_ptr(), dx.data_ptr(), dWx.data_ptr(),
+                                              dWh.data_ptr(), db.data_ptr(), ws.data_ptr(), ws.numel(), wws.data_ptr(),
+                                              wws.numel(), T, B, I, H, code, st), "layer")
         else:
             _lib.check(lib.fastlstm_bwd_persistent(g["dout"].data_ptr(), dh.data_ptr(), dc.data_ptr(), ifgo.data_ptr(),
                                                    cell.data_ptr(), d_ifgo.data_ptr(), g["Wh"].data_ptr(), ws.data_ptr(),
                                                    ws.numel(), T, B, H, code, st), "bwd")
             _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), g["Wx"].data_ptr(), dx.data_ptr(), T, B, I, H, code, st), "dx")
+            _lib.check(lib.fastlstm_gemm_wgrad(d_ifgo.data_ptr(), g["x"].data_ptr(), out.data_ptr(), dWx.data_ptr(),
+                                               dWh.data_ptr(), db.data_ptr(), wws.data_ptr(), wws.numel(), T, B, I, H,
+                                               code, st), "wgrad")
         torch.cuda.synchronize()
         assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
-        res.append((d_ifgo, dx, dh, dc))
-    for a, b in zip(*res):
-        assert torch.equal(a, b)
+        res.append((d_ifgo, dx, dh, dc, db, dWx, dWh))
+    for i, (a, b) in enumerate(zip(*res)):
+        if i < 5:
+            assert torch.equal(a, b), i
+        else:
+            assert rel_err(a, b) < tol, i
 
 
 def test_xcd_local_barrier_timeout_is_reported_not_hung():
