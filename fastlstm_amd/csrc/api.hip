@@ -218,7 +218,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.trace = g_rec_trace;
     if (x) {
         if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p)) return 2;
-        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 4, 2, 2>::LDS_BYTES);
+        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
         FwdXcdHelpLauncher hl = dtype == FASTLSTM_FP16 ? launch_fwd_xcd_help_f16 : launch_fwd_xcd_help_bf16;
         int occ = 0;
         if (hl(p, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
@@ -241,6 +241,8 @@ struct BwdExtras {
     const void *Wx, *x, *h;
     void *dx, *dWx, *dWh;
     int I;
+    void *scratch;          // device memory for parked fp32 accumulator tiles (the wgrad workspace)
+    size_t scratch_bytes;
 };
 
 // In-kernel dx (and, where the shapes suit the 16-bit tile kernel, dWx and dWh) by the workgroups
@@ -279,7 +281,10 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
         p->wg_tiles_m = cdiv(K, 256);
         p->k8_tiles_n = cdiv(I, 256); p->k9_tiles_n = cdiv(H, 256);
         p->wg_tiles = p->wg_tiles_m * (p->k8_tiles_n + p->k9_tiles_n);
-        *wgrad_fused = true;
+        p->wg_scratch = static_cast<float *>(e.scratch);
+        const size_t need = (size_t)std::min(p->wg_tiles, n_helpers) * 256 * 256 * sizeof(float);
+        if (e.scratch && need <= e.scratch_bytes) *wgrad_fused = true;
+        else p->wg_tiles = 0;
     }
     return true;
 }
@@ -303,7 +308,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     if (extras) {
         bool wgrad_fused = false;
         if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused)) return 2;
-        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 4, 2, 2>::LDS_BYTES);
+        const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
         BwdXcdLauncher hl = dtype == FASTLSTM_FP16 ? launch_bwd_xcd_help_f16 : launch_bwd_xcd_help_bf16;
         int occ = 0;
         if (hl(p, c.mt, c.nkw, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
@@ -630,7 +635,7 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     int rc = 1;
     if (pl.wave_split != 2) {
-        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I};
+        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I, wgrad_ws, wgrad_ws_bytes};
         rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
                          s, &e);
         if (rc < 0) return rc;

@@ -23,6 +23,7 @@
 //  * Epilogue: the C tile is staged through LDS (padded rows, conflict-free) and written
 //    with 16-byte row-contiguous stores; bias is added in fp32 before rounding.
 #pragma once
+#include <type_traits>
 #include "common.hpp"
 #include "gemm.hpp"
 
@@ -30,16 +31,56 @@ namespace fastlstm {
 
 #define FASTLSTM_LDS_PTR __attribute__((address_space(3)))
 
-template <typename T> __device__ __forceinline__ u32x2 lds_read_tr16(const unsigned char *p);
-template <> __device__ __forceinline__ u32x2 lds_read_tr16<_Float16>(const unsigned char *p) {
-    typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 v4;
-    auto lp = (FASTLSTM_LDS_PTR v4 *)(p);
-    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16(lp));
+// Transposing LDS read (ds_read_b64_tr_b16, the same instruction for both 16-bit types) of the
+// 8 bytes at `p + OFF`.  Written as inline assembly on purpose: the compiler orders every LDS
+// read it knows of behind ALL LDS-direct global loads in flight (s_waitcnt vmcnt(0)), which
+// would serialise the prefetch of the next k-tile with the multiplication of this one.  The
+// result is valid only behind lds_reads_landed_but() (below), which counts the reads issued since.
+template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16(const unsigned char *p) {
+    u32x2 v = {0u, 0u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned addr = (unsigned)(size_t)((FASTLSTM_LDS_PTR const unsigned char *)p);
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+#else
+    (void)p;
+#endif
+    return v;
 }
-template <> __device__ __forceinline__ u32x2 lds_read_tr16<__bf16>(const unsigned char *p) {
-    typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 v4;
-    auto lp = (FASTLSTM_LDS_PTR v4 *)(p);
-    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4bf16(lp));
+// Plain 16-byte LDS read, as inline assembly for the same reason.
+template <int OFF> __device__ __forceinline__ u32x4 lds_read_b128_asm(const unsigned char *p) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned addr = (unsigned)(size_t)((FASTLSTM_LDS_PTR const unsigned char *)p);
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+#else
+    (void)p;
+#endif
+    return v;
+}
+// Waits until at most N LDS operations of this wave are in flight (they complete in order, so
+// everything but the N youngest has landed); `f` passes through it so that no use of the fragment
+// can be scheduled ahead of the wait.  Operations the compiler issued on its own (LDS or scalar
+// memory) only make the wait stricter.
+template <int N> __device__ __forceinline__ void lds_reads_landed_but(u32x4 &f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(f) : "n"(N));
+#else
+    (void)f;
+#endif
+}
+// Waits for every LDS operation of this wave; the fragments pass through it so that no use of
+// them can be scheduled ahead of the wait.
+template <int N> __device__ __forceinline__ void lds_reads_landed(u32x4 (&f)[N]) {
+    static_assert(N == 4 || N == 8, "fragments per wave tile edge");
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (N == 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
+#else
+    (void)f;
+#endif
 }
 
 // 16 bytes per lane, global -> LDS, destination = lds_block + 16 * lane.  (The 16-byte form
@@ -50,6 +91,20 @@ __device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t rsrc, u
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (FASTLSTM_LDS_PTR void *)lds_block, 16, voffset, soffset, 0, 0);
 #else
     (void)rsrc; (void)lds_block; (void)voffset; (void)soffset;
+#endif
+}
+
+// acc += a . b with the accumulator pinned to the accumulation registers (AGPRs).  With more
+// than 128 accumulators per lane the register allocator otherwise shuttles them between the two
+// halves of the register file around every MFMA.
+template <typename T> __device__ __forceinline__ void mfma_kstep_agpr(const u32x4 a, const u32x4 b, f32x4 &c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (Elem<T>::DT == FASTLSTM_BF16)
+        asm("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else
+        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#else
+    (void)a; (void)b; (void)c;
 #endif
 }
 
@@ -100,16 +155,24 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     // and the rows of neighbouring lane groups (k & 8), land in different banks.
     auto swz = [](int k) { return ((k & 3) << 1) ^ (((k >> 3) & 1) << 3); };
 
+    // K-contiguous operand tile in LDS: rows of BK elements (LPR 16-byte chunks), chunk c of row r
+    // at position c ^ kswz(r % 16): the 16 lanes of a fragment read (16 rows, one chunk index) hit
+    // 16 different 16-byte bank groups.
+    constexpr int LPR = 4 * KSPT, RPB = 64 / LPR;   // chunks per row; rows per 1 KiB block
+    static_assert(KSPT == 1 || KSPT == 2 || KSPT == 4, "row of a k-tile: 64, 128 or 256 bytes");
+    auto kswz = [](int r16) { return (r16 >> (KSPT == 1 ? 2 : KSPT == 2 ? 1 : 0)) & (LPR - 1); };
+
     // 1 KiB LDS block `blk` of a k-tile is filled by one wave instruction; wave w fills
     // blocks w, w + NWAVES, ...  Lane l of block blk fetches:
-    //   K-contiguous operand (operand order): row = 16 (blk / KSPT) + l % 16, k = 32 (blk % KSPT) + 8 (l / 16)
+    //   K-contiguous operand: row = RPB blk + l / LPR, whole rows of the k-tile (full cache lines),
+    //                         chunk (l % LPR) ^ kswz(row)
     //   K-major operand: chunk position P = 64 blk + l -> k-row P / CPR, column chunk (P % CPR) ^ swz(k)
     unsigned goff_a[C::A_LOADS], goff_b[C::B_LOADS];
 #pragma unroll
     for (int i = 0; i < C::A_LOADS; ++i) {
         const int blk = wave + NWAVES * i;
         if constexpr (!A_KM) {
-            const int row = (blk / KSPT) * 16 + r, k = (blk % KSPT) * 32 + q * 8;
+            const int row = blk * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
             goff_a[i] = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * 2);
         } else {
             constexpr int CPR = BM / 8;
@@ -121,7 +184,7 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     for (int i = 0; i < C::B_LOADS; ++i) {
         const int blk = wave + NWAVES * i;
         if constexpr (!B_KM) {
-            const int row = (blk / KSPT) * 16 + r, k = (blk % KSPT) * 32 + q * 8;
+            const int row = blk * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
             goff_b[i] = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * 2);
         } else {
             constexpr int CPR = BN / 8;
@@ -143,47 +206,153 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
             load_block_to_lds(rb_rsrc, sb + (wave + NWAVES * i) * kFragBytes, goff_b[i], kt * b_kstep);
     };
     // fragment of rows [tile16*16, +16) of the operand tile, k-step ks
-    auto frag = [&](const unsigned char *tile, bool km, int ld, int tile16, int ks) -> u32x4 {
-        if (!km) {
-            return *reinterpret_cast<const u32x4 *>(tile + ((tile16 * KSPT + ks) * 64 + lane) * 16);
+    auto frag = [&](const unsigned char *tile, auto km_, auto ld_, int tile16, int ks) -> u32x4 {
+        constexpr bool km = decltype(km_)::value;
+        constexpr int LD = decltype(ld_)::value, ld = LD;
+        if constexpr (!km) {
+            const unsigned char *src = tile + ((tile16 * 16 + r) * LPR + ((ks * 4 + q) ^ kswz(r))) * 16;
+            if constexpr (A_KM || B_KM) return lds_read_b128_asm<0>(src);   // see the streamed loop below
+            else return *reinterpret_cast<const u32x4 *>(src);
         } else {
             // lane (a, b) of a 16-lane group addresses 4 consecutive m of k-row a; rows k and
             // k + 4 (second read) share k & 3 and k & 8, hence the swizzle
             const int a = r >> 2, b = r & 3;
             const int k = ks * 32 + q * 8 + a;
             const unsigned char *base = tile + k * ld + (((tile16 * 2 + (b >> 1)) ^ swz(k)) * 16) + (b & 1) * 8;
-            const u32x2 lo = lds_read_tr16<T>(base), hi = lds_read_tr16<T>(base + 4 * ld);
+            const u32x2 lo = lds_read_tr16<0>(base), hi = lds_read_tr16<4 * LD>(base);
             return u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
     };
 
     // NS-stage pipeline: the loads of k-tiles kt+1 .. kt+NS-1 are in flight while k-tile kt is
     // multiplied (memory latency, not bandwidth, bounds a short loop: ~2 us per round trip).
-    // Per iteration: wait for this wave's own loads of tile kt (everything issued later may
-    // stay in flight), barrier (every wave's part of tile kt has landed, and every wave is
-    // done reading the stage that tile kt+NS-1 is about to overwrite), issue, multiply.
+    // The fragments of k-step s+1 are read from LDS while k-step s is multiplied (two register
+    // sets).  Where s+1 is the first k-step of the next k-tile, the wave first waits for its own
+    // loads of that tile (everything issued later may stay in flight) and meets the others at a
+    // barrier (every wave's part of the tile has landed, and every wave has READ the last
+    // fragments of the stage that the next global loads overwrite); the multiplications of the
+    // k-tile's last k-step then cover the barrier skew and the LDS latency.
     constexpr int D = NS - 1;                         // prefetch distance in k-tiles
     constexpr int LPT = C::A_LOADS + C::B_LOADS;      // loads per k-tile per wave
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-        if (d < nkt) gload(d, d);
-    for (int kt = 0; kt < nkt; ++kt) {
+    static_assert(KSPT % 2 == 0, "fragment register sets alternate by k-step parity");
+    auto tile_ready = [&](int kt) {   // k-tile kt has landed in LDS; the stage of k-tile kt-1 is free
         if (kt + D <= nkt) wait_vm_at_most<(D - 1) * LPT>();   // D-1 younger tiles may stay in flight
         else wait_vm_at_most<0>();                             // tail: fewer tiles behind this one
         __builtin_amdgcn_s_barrier();
         if (kt + D < nkt) gload(kt + D, (kt + D) % NS);
-        const int st = kt % NS;
-        const unsigned char *sa = smem + st * C::STAGE, *sb = sa + C::A_BYTES;
+    };
+    if constexpr (A_KM || B_KM) {
+        // Products with a K-major operand: all fragment reads are inline assembly (see
+        // lds_read_tr16) and this loop counts them itself.  Registers: the B fragments of both
+        // k-steps of a k-tile (TN each), the A fragments of its second k-step (TM), and two
+        // registers through which the A fragments of its first k-step stream, one ahead of the
+        // multiplications.
+        //   first k-step, iteration i:  read A fragment i + 1 of this k-step, B fragment i / (TM / TN)
+        //       (every TM / TN-th i) and A fragment i of the second k-step; wait for A fragment i
+        //       (everything issued behind it may stay in flight); multiply.
+        //   second k-step: its fragments are all in registers before the barrier that hands the
+        //       stage of this k-tile to the global loads; the iterations read the next k-tile's
+        //       first-k-step B fragments and, at the end, its A fragment 0.
+        // Behind the last k-tile those reads still happen (fixed counts), from a stage that exists.
+        static_assert(KSPT == 2, "one streamed and one register-resident k-step per k-tile");
+        static_assert(TM % TN == 0, "B fragments are read every TM / TN-th iteration");
+        constexpr int NA = A_KM ? 2 : 1, NB = B_KM ? 2 : 1, EVERY = TM / TN;   // LDS instructions per fragment
+        u32x4 fs[2], fa1[TM], fb[2][TN];
+        auto rd_a = [&](int kt, int ks, int i) {
+            return frag(smem + (kt % NS) * C::STAGE, std::bool_constant<A_KM>{}, std::integral_constant<int, C::A_LD>{},
+                        wm * TM + i, ks);
+        };
+        auto rd_b = [&](int kt, int ks, int j) {
+            return frag(smem + (kt % NS) * C::STAGE + C::A_BYTES, std::bool_constant<B_KM>{},
+                        std::integral_constant<int, C::B_LD>{}, wn * TN + j, ks);
+        };
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (d < nkt) gload(d, d);
+        tile_ready(0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = rd_b(0, 0, j);
+        fs[0] = rd_a(0, 0, 0);
+        for (int kt = 0; kt < nkt; ++kt) {
+            auto step0 = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                constexpr bool rdb = i % EVERY == 0, rdb_prev = i > 0 && (i - 1) % EVERY == 0;
+                if constexpr (i + 1 < TM) fs[(i + 1) & 1] = rd_a(kt, 0, i + 1);
+                if constexpr (rdb) fb[1][i / EVERY] = rd_b(kt, 1, i / EVERY);
+                fa1[i] = rd_a(kt, 1, i);
+                // issued behind the read of A fragment i: the rest of iteration i - 1, and this iteration
+                constexpr int behind = (i > 0 ? (rdb_prev ? NB : 0) + NA : 0) + (i + 1 < TM ? NA : 0) + (rdb ? NB : 0) + NA;
+                lds_reads_landed_but<behind>(fs[i & 1]);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma_kstep<T>(fb[0][j], fs[i & 1], acc[i][j]);
+            };
+            auto step1 = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i % EVERY == 0) fb[0][i / EVERY] = rd_b(kt + 1, 0, i / EVERY);
+                if constexpr (i == TM - 1) fs[0] = rd_a(kt + 1, 0, 0);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma_kstep<T>(fb[1][j], fa1[i], acc[i][j]);
+            };
+            static_assert(TM == 4 || TM == 8, "wave tile rows");
+            step0(std::integral_constant<int, 0>{}); step0(std::integral_constant<int, 1>{});
+            step0(std::integral_constant<int, 2>{}); step0(std::integral_constant<int, 3>{});
+            if constexpr (TM == 8) {
+                step0(std::integral_constant<int, 4>{}); step0(std::integral_constant<int, 5>{});
+                step0(std::integral_constant<int, 6>{}); step0(std::integral_constant<int, 7>{});
+            }
+            // every fragment of the second k-step is in registers: the stage can be handed over
+            lds_reads_landed(fa1);
+            lds_reads_landed(fb[1]);
+            if (kt + 1 < nkt) tile_ready(kt + 1);
+            step1(std::integral_constant<int, 0>{}); step1(std::integral_constant<int, 1>{});
+            step1(std::integral_constant<int, 2>{}); step1(std::integral_constant<int, 3>{});
+            if constexpr (TM == 8) {
+                step1(std::integral_constant<int, 4>{}); step1(std::integral_constant<int, 5>{});
+                step1(std::integral_constant<int, 6>{}); step1(std::integral_constant<int, 7>{});
+            }
+        }
+        // the reads behind the last k-tile are still in flight: nothing may reuse the LDS before them
+        lds_reads_landed_but<0>(fs[0]);
+        __syncthreads();
+        return;
+    }
+    u32x4 fa[2][TM], fb[2][TN];
+    auto read_a = [&](int kt, int ks, int i) {
+        fa[ks & 1][i] = frag(smem + (kt % NS) * C::STAGE, std::bool_constant<A_KM>{},
+                             std::integral_constant<int, C::A_LD>{}, wm * TM + i, ks);
+    };
+    auto read_b = [&](int kt, int ks, int j) {
+        fb[ks & 1][j] = frag(smem + (kt % NS) * C::STAGE + C::A_BYTES, std::bool_constant<B_KM>{},
+                             std::integral_constant<int, C::B_LD>{}, wn * TN + j, ks);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (d < nkt) gload(d, d);
+    tile_ready(0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) read_a(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) read_b(0, 0, j);
+    for (int kt = 0; kt < nkt; ++kt) {
 #pragma unroll
         for (int ks = 0; ks < KSPT; ++ks) {
-            u32x4 fa[TM];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = frag(sa, A_KM, C::A_LD, wm * TM + i, ks);
+            const bool last = ks + 1 == KSPT;
+            const bool more = !last || kt + 1 < nkt;
+            const int nkt_ = last ? kt + 1 : kt, nks = last ? 0 : ks + 1;   // the k-step after this one
+            if (last && more) tile_ready(kt + 1);
+            // column j of the wave tile is multiplied while the next k-step's fragments stream in
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const u32x4 fb = frag(sb, B_KM, C::B_LD, wn * TN + j, ks);
+                if (more) {
+                    read_b(nkt_, nks, j);
 #pragma unroll
-                for (int i = 0; i < TM; ++i) acc[i][j] = mfma_kstep<T>(fb, fa[i], acc[i][j]);
+                    for (int i = j; i < TM; i += TN) read_a(nkt_, nks, i);
+                }
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    if constexpr (TM * TN > 32) mfma_kstep_agpr<T>(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+                    else acc[i][j] = mfma_kstep<T>(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+                }
             }
         }
     }
@@ -225,22 +394,46 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
         return;
     }
     const T *bias0 = static_cast<const T *>(p.bias0), *bias1 = static_cast<const T *>(p.bias1);
+    // the 4 bias elements of every tile column group: one 8-byte load each where the row of
+    // biases allows it (all loads in flight together), element loads at a ragged edge
+    float bv[TN][4];
+    {
+        u32x2 raw0[TN], raw1[TN];
+        const bool vec = (p.N & 3) == 0 && ((reinterpret_cast<size_t>(bias0) | reinterpret_cast<size_t>(bias1)) & 7) == 0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + (wn * TN + j) * 16 + q * 4;
+            raw0[j] = raw1[j] = u32x2{0u, 0u};
+            if (bias0 && vec && n < p.N) {
+                raw0[j] = *reinterpret_cast<const u32x2 *>(bias0 + n);
+                if (bias1) raw1[j] = *reinterpret_cast<const u32x2 *>(bias1 + n);
+            } else if (bias0) {
+                T t0[4], t1[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    t0[e] = n + e < p.N ? bias0[n + e] : Elem<T>::from_f32(0.f);
+                    t1[e] = bias1 && n + e < p.N ? bias1[n + e] : Elem<T>::from_f32(0.f);
+                }
+                raw0[j] = *reinterpret_cast<u32x2 *>(t0);
+                raw1[j] = *reinterpret_cast<u32x2 *>(t1);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const T *t0 = reinterpret_cast<const T *>(&raw0[j]), *t1 = reinterpret_cast<const T *>(&raw1[j]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[j][e] = Elem<T>::to_f32(t0[e]) + Elem<T>::to_f32(t1[e]);
+        }
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int nl = (wn * TN + j) * 16 + q * 4;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias0) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (n0 + nl + e < p.N)
-                    bv[e] = Elem<T>::to_f32(bias0[n0 + nl + e]) + (bias1 ? Elem<T>::to_f32(bias1[n0 + nl + e]) : 0.f);
-        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int ml = (wm * TM + i) * 16 + r;
             const f32x4 v = acc[i][j];
-            T pk[4] = {Elem<T>::from_f32(v[0] + bv[0]), Elem<T>::from_f32(v[1] + bv[1]),
-                       Elem<T>::from_f32(v[2] + bv[2]), Elem<T>::from_f32(v[3] + bv[3])};
+            T pk[4] = {Elem<T>::from_f32(v[0] + bv[j][0]), Elem<T>::from_f32(v[1] + bv[j][1]),
+                       Elem<T>::from_f32(v[2] + bv[j][2]), Elem<T>::from_f32(v[3] + bv[j][3])};
             *reinterpret_cast<u32x2 *>(smem + (size_t)ml * C::C_LD + nl * 2) = *reinterpret_cast<u32x2 *>(pk);
         }
     }

@@ -45,6 +45,7 @@ struct BwdXcdParams {
     GemmParams k8, k9;  // M = 4H, N = I | H, K = T*B, A = d_ifgo (K-major), B = x | h (K-major), C = dWx | dWh
     int k8_tiles_n, k9_tiles_n, wg_tiles_m, wg_tiles;
     int n_active;
+    float *wg_scratch;  // 256 KiB per helper that owns a weight-gradient tile
     int *chunk_done;    // [<= 32] device-scope counters, zero at launch
     long long spin_limit;
 };
@@ -52,9 +53,13 @@ struct BwdXcdParams {
 // The workgroups (8 waves) without a role in the recurrence.  Chunks of timesteps become available
 // in reverse time order.  Helper h of n owns weight-gradient tile h (if there is one), which it
 // accumulates chunk by chunk, and takes the dx tiles h, h + n, ... of the list ordered by chunk.
+// The 128 accumulator registers of the weight-gradient tile and those of a dx tile do not fit
+// side by side: between chunks the helper parks the weight-gradient accumulators in its 256 KiB of
+// wg_scratch (lane-major, 16-byte accesses; ~0.5 MiB of traffic per 80 us chunk) instead of
+// leaving that to register spills inside the GEMM loops.
 template <typename T>
 __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char *smem) {
-    constexpr int TM = 4, TN = 8;   // 16 x 16 tiles per wave of the 256 x 256 tile, 8 waves as 4 x 2
+    constexpr int WVM = 2, WVN = 4, TM = 256 / WVM / 16, TN = 256 / WVN / 16;   // 8 waves, 128 x 64 each
     int n_helpers;
     const int h = helper_rank(p.n_ht, p.gpx, p.n_groups, &n_helpers);
     const int per_chunk = p.k5_chunk_tiles * p.k5_tiles_n;
@@ -65,11 +70,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
     const GemmParams &wp = is8 ? p.k8 : p.k9;
     const int wi = is8 ? h : h - n8, wtn = is8 ? p.k8_tiles_n : p.k9_tiles_n;
     const int wm0 = (wi / wtn) * 256, wn0 = (wi % wtn) * 256;
-    f32x4 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 *park = reinterpret_cast<f32x4 *>(p.wg_scratch) + (size_t)h * (256 * 256 / 4) + threadIdx.x;
 
     for (int k = 0; k < p.k5_chunks; ++k) {
         const int c = p.k5_chunks - 1 - k;   // chunk in forward time
@@ -77,28 +78,39 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
         if ((threadIdx.x >> 6) == 0) wait_versions(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
         __syncthreads();
         if (own) {
+            f32x4 acc[TM][TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = k == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : park[(i * TN + j) * (kWave * 8)];
             const int kb = c * p.k5_chunk_tiles * 256, ke = min(wp.K, kb + p.k5_chunk_tiles * 256);
-            gemm16_mainloop<T, true, true, 256, 256, 2, 4, 2, 2>(wp, wm0, wn0, kb, ke, smem, acc);
+            gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc);
+            if (k + 1 < p.k5_chunks) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) park[(i * TN + j) * (kWave * 8)] = acc[i][j];
+            } else {
+                gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, 0, smem, acc);
+                __syncthreads();
+            }
         }
         for (int i = k * per_chunk + ((h - k * per_chunk) % n_helpers + n_helpers) % n_helpers; i < (k + 1) * per_chunk;
              i += n_helpers) {
             const int r = i - k * per_chunk;
             const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
             if (rt >= p.k5_tiles_m) continue;
-            gemm16_tile<T, false, true, 256, 256, 2, 4, 2, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
+            gemm16_tile<T, false, true, 256, 256, 2, WVM, WVN, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
             __syncthreads();   // the LDS is reused by the next tile
         }
-    }
-    if (own) {
-        gemm16_epilogue<T, 256, 256, 2, 4, 2, 2>(wp, wm0, wn0, 0, smem, acc);
-        __syncthreads();
     }
     // weight-gradient tiles beyond one per helper: everything they need is in memory now
     for (int w = h + n_helpers; w < p.wg_tiles; w += n_helpers) {
         const bool w8 = w < n8;
         const GemmParams &q = w8 ? p.k8 : p.k9;
         const int qi = w8 ? w : w - n8, qtn = w8 ? p.k8_tiles_n : p.k9_tiles_n;
-        gemm16_tile<T, true, true, 256, 256, 2, 4, 2, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
+        gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
         __syncthreads();
     }
 }

@@ -134,7 +134,7 @@ __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *
     const int total = p.k1_tiles_m * p.k1_tiles_n;
     for (int tile = h; tile < total; tile += n_helpers) {
         const int rt = tile / p.k1_tiles_n, ct = tile % p.k1_tiles_n;
-        gemm16_tile<T, false, false, 256, 256, 2, 4, 2, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
+        gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // every wave's part of the tile is in the L2 (and the LDS may be reused)
         if (threadIdx.x == 0)
