@@ -241,8 +241,6 @@ struct BwdExtras {
     const void *Wx, *x, *h;
     void *dx, *dWx, *dWh;
     int I;
-    void *scratch;          // device memory for parked fp32 accumulator tiles (the wgrad workspace)
-    size_t scratch_bytes;
 };
 
 // In-kernel dx (and, where the shapes suit the 16-bit tile kernel, dWx and dWh) by the workgroups
@@ -281,10 +279,7 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
         p->wg_tiles_m = cdiv(K, 256);
         p->k8_tiles_n = cdiv(I, 256); p->k9_tiles_n = cdiv(H, 256);
         p->wg_tiles = p->wg_tiles_m * (p->k8_tiles_n + p->k9_tiles_n);
-        p->wg_scratch = static_cast<float *>(e.scratch);
-        const size_t need = (size_t)std::min(p->wg_tiles, n_helpers) * 256 * 256 * sizeof(float);
-        if (e.scratch && need <= e.scratch_bytes) *wgrad_fused = true;
-        else p->wg_tiles = 0;
+        *wgrad_fused = true;
     }
     return true;
 }
@@ -635,7 +630,7 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     int rc = 1;
     if (pl.wave_split != 2) {
-        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I, wgrad_ws, wgrad_ws_bytes};
+        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I};
         rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
                          s, &e);
         if (rc < 0) return rc;

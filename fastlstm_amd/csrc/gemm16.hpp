@@ -136,11 +136,14 @@ template <int N> __device__ __forceinline__ void wait_vm_at_most() {
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
 __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m0, const int n0, const int kb,
                                                 const int ke, unsigned char *smem,
-                                                f32x4 (&acc)[BM / WVM / 16][BN / WVN / 16]) {
+                                                f32x4 (&acc)[BM / WVM / 16][BN / WVN / 16], const int tid_salt = 0) {
     using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
     constexpr int NWAVES = C::NWAVES;
     constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // tid_salt is zero.  A caller inside a loop passes one the compiler cannot see through, so that the
+    // per-lane address arithmetic below is redone per call instead of being kept in registers (or
+    // spilled and reloaded inside the k loop) across the caller's loop.
+    const int tid = threadIdx.x + tid_salt, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave / WVN, wn = wave % WVN;
     const int nkt = (ke - kb) / BK;
@@ -167,31 +170,29 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     //   K-contiguous operand: row = RPB blk + l / LPR, whole rows of the k-tile (full cache lines),
     //                         chunk (l % LPR) ^ kswz(row)
     //   K-major operand: chunk position P = 64 blk + l -> k-row P / CPR, column chunk (P % CPR) ^ swz(k)
-    unsigned goff_a[C::A_LOADS], goff_b[C::B_LOADS];
-#pragma unroll
-    for (int i = 0; i < C::A_LOADS; ++i) {
-        const int blk = wave + NWAVES * i;
-        if constexpr (!A_KM) {
-            const int row = blk * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
-            goff_a[i] = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * 2);
-        } else {
-            constexpr int CPR = BM / 8;
-            const int P = blk * 64 + lane, k = P / CPR, mc = (P % CPR) ^ swz(k);
-            goff_a[i] = (unsigned)(((size_t)(kb + k) * p.lda + m0 + mc * 8) * 2);
-        }
+    // Blocks w + NWAVES i, i = 0, 1, ..., of a wave differ by whole groups of rows that leave both
+    // swizzles unchanged: one per-lane offset per operand, the rest is a scalar offset.
+    static_assert((NWAVES * RPB) % 16 == 0 && (NWAVES * 64) % (BM / 8) == 0 && (NWAVES * 64) % (BN / 8) == 0 &&
+                  (NWAVES * 64 / (BM / 8)) % 16 == 0 && (NWAVES * 64 / (BN / 8)) % 16 == 0, "row groups per block");
+    unsigned goff_a, goff_b;
+    if constexpr (!A_KM) {
+        const int row = wave * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
+        goff_a = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * 2);
+    } else {
+        constexpr int CPR = BM / 8;
+        const int P = wave * 64 + lane, k = P / CPR, mc = (P % CPR) ^ swz(k);
+        goff_a = (unsigned)(((size_t)(kb + k) * p.lda + m0 + mc * 8) * 2);
     }
-#pragma unroll
-    for (int i = 0; i < C::B_LOADS; ++i) {
-        const int blk = wave + NWAVES * i;
-        if constexpr (!B_KM) {
-            const int row = blk * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
-            goff_b[i] = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * 2);
-        } else {
-            constexpr int CPR = BN / 8;
-            const int P = blk * 64 + lane, k = P / CPR, nc = (P % CPR) ^ swz(k);
-            goff_b[i] = (unsigned)(((size_t)(kb + k) * p.ldb + n0 + nc * 8) * 2);
-        }
+    if constexpr (!B_KM) {
+        const int row = wave * RPB + lane / LPR, k = ((lane % LPR) ^ kswz(row & 15)) * 8;
+        goff_b = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * 2);
+    } else {
+        constexpr int CPR = BN / 8;
+        const int P = wave * 64 + lane, k = P / CPR, nc = (P % CPR) ^ swz(k);
+        goff_b = (unsigned)(((size_t)(kb + k) * p.ldb + n0 + nc * 8) * 2);
     }
+    const unsigned a_istep = (unsigned)(A_KM ? NWAVES * 64 / (BM / 8) : NWAVES * RPB) * p.lda * 2;  // bytes per block index
+    const unsigned b_istep = (unsigned)(B_KM ? NWAVES * 64 / (BN / 8) : NWAVES * RPB) * p.ldb * 2;
     const unsigned a_kstep = A_KM ? (unsigned)BK * p.lda * 2 : BK * 2;  // byte advance per k-tile
     const unsigned b_kstep = B_KM ? (unsigned)BK * p.ldb * 2 : BK * 2;
 
@@ -200,10 +201,10 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
         unsigned char *sa = smem + stage * C::STAGE, *sb = sa + C::A_BYTES;
 #pragma unroll
         for (int i = 0; i < C::A_LOADS; ++i)
-            load_block_to_lds(ra_rsrc, sa + (wave + NWAVES * i) * kFragBytes, goff_a[i], kt * a_kstep);
+            load_block_to_lds(ra_rsrc, sa + (wave + NWAVES * i) * kFragBytes, goff_a, kt * a_kstep + i * a_istep);
 #pragma unroll
         for (int i = 0; i < C::B_LOADS; ++i)
-            load_block_to_lds(rb_rsrc, sb + (wave + NWAVES * i) * kFragBytes, goff_b[i], kt * b_kstep);
+            load_block_to_lds(rb_rsrc, sb + (wave + NWAVES * i) * kFragBytes, goff_b, kt * b_kstep + i * b_istep);
     };
     // fragment of rows [tile16*16, +16) of the operand tile, k-step ks
     auto frag = [&](const unsigned char *tile, auto km_, auto ld_, int tile16, int ks) -> u32x4 {

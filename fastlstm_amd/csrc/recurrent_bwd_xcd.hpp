@@ -45,18 +45,38 @@ struct BwdXcdParams {
     GemmParams k8, k9;  // M = 4H, N = I | H, K = T*B, A = d_ifgo (K-major), B = x | h (K-major), C = dWx | dWh
     int k8_tiles_n, k9_tiles_n, wg_tiles_m, wg_tiles;
     int n_active;
-    float *wg_scratch;  // 256 KiB per helper that owns a weight-gradient tile
     int *chunk_done;    // [<= 32] device-scope counters, zero at launch
     long long spin_limit;
 };
 
+// One 256 x 256 tile of dx = d_ifgo . Wx as a real function call.  The caller keeps the 128
+// accumulator registers of its weight-gradient tile across the call: the calling convention saves
+// and restores them around it (once per dx tile), where inlining would spill inside the GEMM
+// loops of both products.  Arguments of a function arrive in vector registers; every one of them
+// is the same in all lanes and goes back to scalar registers first.
+__device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename P> __device__ __forceinline__ P *uniform_ptr(P *ptr) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return reinterpret_cast<P *>(((unsigned long long)hi << 32) | lo);
+}
+template <typename T>
+__device__ __attribute__((noinline)) void helper_dx_tile(const void *A, const void *B, void *C, int M, int N, int K,
+                                                         int m0, int n0, FASTLSTM_LDS_PTR unsigned char *lds) {
+    GemmParams g{};
+    g.A = uniform_ptr(A); g.B = uniform_ptr(B); g.C = uniform_ptr(C);
+    g.M = uniform_int(M); g.N = uniform_int(N); g.K = uniform_int(K);
+    g.lda = g.K; g.ldb = g.N; g.ldc = g.N;
+    g.splits = 1; g.k_per_split = g.K;
+    unsigned char *smem = (unsigned char *)(FASTLSTM_LDS_PTR unsigned char *)uniform_int((int)(size_t)lds);
+    gemm16_tile<T, false, true, 256, 256, 2, 2, 4, 2>(g, uniform_int(m0), uniform_int(n0), 0, smem, 0);
+    __syncthreads();   // the LDS is reused by the caller
+}
+
 // The workgroups (8 waves) without a role in the recurrence.  Chunks of timesteps become available
 // in reverse time order.  Helper h of n owns weight-gradient tile h (if there is one), which it
-// accumulates chunk by chunk, and takes the dx tiles h, h + n, ... of the list ordered by chunk.
-// The 128 accumulator registers of the weight-gradient tile and those of a dx tile do not fit
-// side by side: between chunks the helper parks the weight-gradient accumulators in its 256 KiB of
-// wg_scratch (lane-major, 16-byte accesses; ~0.5 MiB of traffic per 80 us chunk) instead of
-// leaving that to register spills inside the GEMM loops.
+// accumulates chunk by chunk in registers, and takes the dx tiles h, h + n, ... of the list ordered
+// by chunk.
 template <typename T>
 __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char *smem) {
     constexpr int WVM = 2, WVN = 4, TM = 256 / WVM / 16, TN = 256 / WVN / 16;   // 8 waves, 128 x 64 each
@@ -70,41 +90,51 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
     const GemmParams &wp = is8 ? p.k8 : p.k9;
     const int wi = is8 ? h : h - n8, wtn = is8 ? p.k8_tiles_n : p.k9_tiles_n;
     const int wm0 = (wi / wtn) * 256, wn0 = (wi % wtn) * 256;
-    f32x4 *park = reinterpret_cast<f32x4 *>(p.wg_scratch) + (size_t)h * (256 * 256 / 4) + threadIdx.x;
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+#ifdef FASTLSTM_BWD_STAMPS
+    long long *stamps = reinterpret_cast<long long *>(p.counters + 8192) + blockIdx.x * 4;
+    long long waited = 0;
+    if (threadIdx.x == 0) stamps[0] = (long long)wall_clock64();
+#endif
     for (int k = 0; k < p.k5_chunks; ++k) {
         const int c = p.k5_chunks - 1 - k;   // chunk in forward time
         // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
-        if ((threadIdx.x >> 6) == 0) wait_versions(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
+#ifdef FASTLSTM_BWD_STAMPS
+        const long long w0 = (long long)wall_clock64();
+#endif
+        if ((threadIdx.x >> 6) == 0) wait_versions<100>(p.chunk_done + c, 1, p.n_active, p.hdr, p.spin_limit, -1, c);
         __syncthreads();
+#ifdef FASTLSTM_BWD_STAMPS
+        waited += (long long)wall_clock64() - w0;
+        if (threadIdx.x == 0 && k == p.k5_chunks - 1) stamps[3] = (long long)wall_clock64();
+#endif
         if (own) {
-            f32x4 acc[TM][TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = k == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : park[(i * TN + j) * (kWave * 8)];
             const int kb = c * p.k5_chunk_tiles * 256, ke = min(wp.K, kb + p.k5_chunk_tiles * 256);
-            gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc);
-            if (k + 1 < p.k5_chunks) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) park[(i * TN + j) * (kWave * 8)] = acc[i][j];
-            } else {
-                gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, 0, smem, acc);
-                __syncthreads();
-            }
+            int salt = 0;
+            asm volatile("" : "+v"(salt));   // opaque zero: see gemm16_mainloop
+            gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc, salt);
         }
         for (int i = k * per_chunk + ((h - k * per_chunk) % n_helpers + n_helpers) % n_helpers; i < (k + 1) * per_chunk;
              i += n_helpers) {
             const int r = i - k * per_chunk;
             const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
             if (rt >= p.k5_tiles_m) continue;
-            gemm16_tile<T, false, true, 256, 256, 2, WVM, WVN, 2>(p.k5, rt * 256, ct * 256, 0, smem, 0);
-            __syncthreads();   // the LDS is reused by the next tile
+            helper_dx_tile<T>(p.k5.A, p.k5.B, p.k5.C, p.k5.M, p.k5.N, p.k5.K, rt * 256, ct * 256,
+                              (FASTLSTM_LDS_PTR unsigned char *)smem);
         }
     }
+    if (own) {
+        gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, 0, smem, acc);
+        __syncthreads();
+    }
+#ifdef FASTLSTM_BWD_STAMPS
+    if (threadIdx.x == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = waited; }
+#endif
     // weight-gradient tiles beyond one per helper: everything they need is in memory now
     for (int w = h + n_helpers; w < p.wg_tiles; w += n_helpers) {
         const bool w8 = w < n8;
@@ -141,12 +171,18 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int g = gl * kNumXcd + xcd;
     if (gl >= p.gpx || g >= p.n_groups) {
         if constexpr (HELP) {
+#ifndef FASTLSTM_DBG_NOHELPWORK
             if (p.k5_tiles_n > 0) bwd_helper<T>(p, smem);
+#endif
         }
         return;
     }
     const int u0 = j * HT, b0 = g * BT;
     const bool k5_live = HELP && p.k5_tiles_n > 0;
+#ifdef FASTLSTM_BWD_STAMPS
+    long long *stamps = reinterpret_cast<long long *>(p.counters + 8192) + blockIdx.x * 4;
+    if (tid == 0) stamps[0] = (long long)wall_clock64();
+#endif
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                    // [NWV][MT][NT][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
@@ -210,9 +246,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
 
     // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out --------------------
-    // one set of tile pieces in flight: requested right after a step's tile went out, consumed after
-    // the step's K loop (more than an HBM round trip later); registers are scarce next to the weights
-    u32x4 gpre[GPT], cpre[SPT], dpre[SPT];
+    // two sets of tile pieces in flight: the tiles of step s + 2 are requested right after step s's
+    // tile went out (into the set that held step s's own tiles) and go to the LDS behind step s + 1's
+    // K loop -- almost two steps later, which also covers the memory latency while the workgroups
+    // without a role in the recurrence stream their GEMM operands
+    u32x4 gpre[2][GPT], cpre[2][SPT], dpre[2][SPT];
     unsigned g_glb[GPT], s_glb[SPT];
     int g_lds[GPT], s_lds[SPT];
     bool g_ok[GPT], s_ok[SPT];
@@ -263,11 +301,14 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
                     *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
     };
-    fetch_tiles(T_ - 1, gpre, cpre, dpre);
-    tiles_to_lds(gpre, cpre, dpre);   // step 0 works on the LDS tiles right away
+    fetch_tiles(T_ - 1, gpre[0], cpre[0], dpre[0]);
+    if (T_ > 1) fetch_tiles(T_ - 2, gpre[1], cpre[1], dpre[1]);
+    tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
     __syncthreads();
 
-    for (int s = 0; s < T_; ++s) {
+    // one reverse step; PAR = s % 2 picks the register sets at compile time
+    auto step = [&](const int s, auto par) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par)::value;
         const int t = T_ - 1 - s;
         const XchgL2 xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
 
@@ -323,16 +364,19 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         __syncthreads();
         if (tid < kXcdReplicas)
             __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        // every store of the previous steps (d_ifgo tiles included) has been acknowledged: when the
-        // previous step closed a chunk, hand the chunk to the dx helpers (release: this XCD's L2 is
-        // written back so that the other XCDs can read it)
-        if (k5_live && tid == kWave && s > 0 && (t + 1) % p.k5_chunk_steps == 0)
-            __hip_atomic_fetch_add(p.chunk_done + (t + 1) / p.k5_chunk_steps, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         tile_to_global(t);
-        if (s + 1 < T_) fetch_tiles(t - 1, gpre, cpre, dpre);
+        if (s + 2 < T_) fetch_tiles(t - 2, gpre[PAR], cpre[PAR], dpre[PAR]);
 
         if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, g, s);
         __syncthreads();
+        // Every workgroup of the group has passed this step's publish point, where its stores of the
+        // previous steps (d_ifgo tiles included) were acknowledged by the L2.  When the previous step
+        // closed a chunk, ONE workgroup hands the group's share of it to the helpers: the release
+        // writes this XCD's L2 back (all of it, whichever CU wrote the lines), so that the other
+        // XCDs can read the chunk, and counts for all n_ht workgroups.
+        if (k5_live && j == 0 && tid == kWave && s > 0 && (t + 1) % p.k5_chunk_steps == 0)
+            __hip_atomic_fetch_add(p.chunk_done + (t + 1) / p.k5_chunk_steps, p.n_ht, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps
         f32x4 acc[MT][NTW];
@@ -367,7 +411,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
 #pragma unroll
             for (int i = 0; i < NTW; ++i) red[((wave * MT + a) * NT + i) * kWave + lane] = acc[a][i];
         // the tile was drained before the barrier above: the next step's inputs take its place
-        if (s + 1 < T_) tiles_to_lds(gpre, cpre, dpre);
+        if (s + 1 < T_) tiles_to_lds(gpre[PAR ^ 1], cpre[PAR ^ 1], dpre[PAR ^ 1]);
         __syncthreads();
         const float *redf = reinterpret_cast<const float *>(red);
 #pragma unroll
@@ -378,6 +422,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             dh_rec[m] = v;
         }
         // the next step's publish barrier orders these reads before the next writes to `red`
+    };
+    for (int s = 0; s < T_; s += 2) {
+        step(s, std::integral_constant<int, 0>{});
+        if (s + 1 < T_) step(s + 1, std::integral_constant<int, 1>{});
     }
 
     if (k5_live) {   // the last chunk (timesteps 0 ..)
@@ -385,6 +433,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         __syncthreads();
         if (tid == kWave) __hip_atomic_fetch_add(p.chunk_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
+#ifdef FASTLSTM_BWD_STAMPS
+    if (tid == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = -1; }
+#endif
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
 #pragma unroll
     for (int m = 0; m < IPT; ++m)

@@ -79,7 +79,10 @@ struct XchgLds {
 };
 
 
-// Called by wave 0 of a workgroup.  flags: the n flags of this barrier group.
+// Called by wave 0 of a workgroup.  flags: the n flags of this barrier group.  NAP: s_sleep units
+// (64 clocks each) between polls; waits that are expected to last many microseconds nap longer so
+// that their polling stays out of the way of the traffic they wait for.
+template <int NAP = 1>
 __device__ __forceinline__ void wait_versions(const int *flags, int n, int target, WsHeader *hdr,
                                               long long spin_limit, int group, int step) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -90,7 +93,7 @@ __device__ __forceinline__ void wait_versions(const int *flags, int n, int targe
         for (int j = lane; j < n; j += kWave)
             ok &= (__hip_atomic_load(flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target);
         if (__all(ok)) break;
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(NAP);
         // a spin limit <= 1 means "give up at the first failed poll" (host-forced failure path)
         if (++polls >= 32 || spin_limit <= 1) {
             polls = 0;
