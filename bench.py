@@ -38,7 +38,7 @@ PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MF
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the fused forward layer kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE,
 # scaled by a plain copy of known size (profiles/fwd_layer_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 1768.6e6}
+TRAFFIC_BYTES = {"B": 1761.3e6}
 
 
 def main():
@@ -218,9 +218,17 @@ def main():
                                            dWh_.data_ptr(), db.data_ptr(), ws_w.data_ptr(), ws_w.numel(), T, B, I, H,
                                            code, stream), "wgrad")
 
+    def layer_bwd():   # what lstm_persistent_bwd calls: recurrence + dx + dWx + dWh + db, fused where CUs would idle
+        _lib.check(lib.fastlstm_bwd_layer(dout.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
+                                          cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), Wx.data_ptr(),
+                                          x.data_ptr(), out.data_ptr(), dx.data_ptr(), dWx.data_ptr(), dWh_.data_ptr(),
+                                          db.data_ptr(), ws_b.data_ptr(), ws_b.numel(), ws_w.data_ptr(), ws_w.numel(),
+                                          T, B, I, H, code, stream), "bwd_layer")
+
     t_rb = ev_time(rec_bwd, reps=5, pre=rec_bwd_pre)
     t_k5 = ev_time(k5, reps=5)
     t_k89 = ev_time(k89, reps=5)
+    t_lb = ev_time(layer_bwd, reps=5, pre=rec_bwd_pre)
     torch.cuda.synchronize()
     _lib.check(lib.fastlstm_ws_status(ws_b[:64].cpu().numpy().tobytes()), "backward barrier status")
     kernels.update({
@@ -229,6 +237,7 @@ def main():
         "gemm_dx_tflops": round(2.0 * T * B * I * 4 * H / (t_k5 * 1e-3) / 1e12, 2),
         "gemm_wgrad_ms": round(t_k89, 4),
         "gemm_wgrad_tflops": round(2.0 * T * B * 4 * H * (I + H) / (t_k89 * 1e-3) / 1e12, 2),
+        "bwd_layer_ms": round(t_lb, 4),
     })
 
     # ---- roofline of the dominant kernel of the headline (forward) path ------------------
