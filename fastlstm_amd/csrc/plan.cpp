@@ -192,9 +192,10 @@ extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, 
     const int slots = recurrent_full_slots(T, slot, backward != 0);
     size_t ws = recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks,
                                    backward != 0, true, slots);
-    // the XCD-local kernels lay their ring out for batch tiles of 16 or 32 rows: one tile more at most
+    // the XCD-local kernels lay their ring out for batch tiles of 16 or 32 rows, which covers at most
+    // 16 rows (one operand block per k-step) more than the tiles of the plan
     const int KS = cdiv(backward ? 4 * H : H, kstep_of(dtype));
     ws = std::max(ws, kWsHeaderBytes + kWsCounterBytes +
-                          (size_t)slots * (plan->batch_chunks * slot + 2 * (size_t)KS * kFragBytes));
+                          (size_t)slots * (plan->batch_chunks * slot + (size_t)KS * kFragBytes));
     return ws;
 }

@@ -61,7 +61,7 @@ def _plan(device, B, H, code, backward):
 
 
 # Largest exchange ring (one slot per timestep) a recurrent call may allocate.
-RING_MAX_BYTES = 1 << 30
+RING_MAX_BYTES = 2 << 30
 
 
 def _workspace(plan, T, H, code, backward, device):
