@@ -236,6 +236,51 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     return FASTLSTM_OK;
 }
 
+// Shape of a launch of the register-resident kernels whose barrier groups span several XCDs
+// (recurrent_fwd_wide.hpp): 16 units x 64 batch rows per workgroup, H / 16 workgroups per group.
+struct WideCfg {
+    int nkw, n_ht, xpg, n_groups, ks, lds;
+    size_t xslot;
+};
+bool select_wide(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c) {
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
+    if (dtype == FASTLSTM_FP32 || backward) return false;
+    if (H % 256 || (H != 1536 && H != 2048)) return false;
+    c->nkw = H / 256;
+    c->n_ht = H / 16;
+    if (c->n_ht % 32 || c->n_ht > kXcdGroupStride) return false;
+    c->xpg = c->n_ht / 32;
+    c->n_groups = cdiv(B, 64);
+    if (c->n_groups * c->xpg > kNumXcd) return false;
+    c->ks = H / 32;
+    c->xslot = (size_t)c->n_groups * 4 * c->ks * kFragBytes;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + 1) * c->xslot) return false;
+    c->lds = 8 * 16 * kFragBytes + 64 * (4 * 32 + 16) + 2 * 64 * (32 + 16);
+    return true;
+}
+
+// Returns 1 when the kernel does not apply, else a fastlstm_status.
+int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
+                 int H, int dtype, hipStream_t stream) {
+    WideCfg c;
+    if (!select_wide(T, B, H, dtype, false, ws_bytes, &c)) return 1;
+    FwdXcdParams p{};
+    p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);   // here: one flag per workgroup
+    p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KS = c.ks;
+    p.spin_limit = spin_limit_ticks();
+    auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
+    int occ = 0;
+    if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (occ < 1) return 1;
+    if (launch(p, c.nkw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    return FASTLSTM_OK;
+}
+
 // What the reverse launch may compute besides the recurrence (fastlstm_bwd_layer).
 struct BwdExtras {
     const void *Wx, *x, *h;
@@ -457,7 +502,8 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (sync) {
-        const int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+        int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+        if (rc == 1) rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     FwdParams p{};
@@ -653,7 +699,9 @@ int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward,
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (T <= 0 || B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
     XcdCfg c;
-    return select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c) ? 1 : 0;
+    if (select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c)) return 1;
+    WideCfg w;
+    return select_wide(T, B, H, dtype, backward != 0, ws_bytes, &w) ? 2 : 0;
 }
 
 int fastlstm_ws_status(const void *ws_head) {

@@ -68,7 +68,7 @@ __device__ __attribute__((noinline)) void helper_dx_tile(const void *A, const vo
     g.M = uniform_int(M); g.N = uniform_int(N); g.K = uniform_int(K);
     g.lda = g.K; g.ldb = g.N; g.ldc = g.N;
     g.splits = 1; g.k_per_split = g.K;
-    unsigned char *smem = (unsigned char *)(FASTLSTM_LDS_PTR unsigned char *)uniform_int((int)(size_t)lds);
+    unsigned char *smem = (unsigned char *)(FASTLSTM_LDS_PTR unsigned char *)(size_t)(unsigned)uniform_int((int)(size_t)lds);
     gemm16_tile<T, false, true, 256, 256, 2, 2, 4, 2>(g, uniform_int(m0), uniform_int(n0), 0, smem, 0);
     __syncthreads();   // the LDS is reused by the caller
 }

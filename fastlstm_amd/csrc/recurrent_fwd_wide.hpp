@@ -1,0 +1,263 @@
+// Persistent forward kernel for hidden sizes whose W_h does not fit the CUs of one XCD
+// (H = 1536, 2048 with 16-bit elements): weight slice in registers, barrier groups of H / 16
+// workgroups that span several whole XCDs.
+//
+// Same mathematics and the same results as lstm_fwd_persistent_kernel (which replaces
+// fastlstm/kernels.py:414-663).  The general kernel keeps a workgroup's slice of W_h in LDS, which
+// for H = 2048 leaves room for 8 hidden units per CU only: one barrier group of 256 workgroups, each
+// of which has to read the h_t of ALL batch rows every step (512 KiB per CU and step for B = 128).
+// Here a workgroup of 8 waves holds 16 units x 4 gates x H (256 KiB for H = 2048) in registers, as
+// the XCD-local kernel does, so a group needs H / 16 workgroups (128) and the launch has room for two
+// groups of 64 batch rows: half the operand volume per CU.
+//  * placement: group g takes the workgroups of XCDs [g * xpg, (g + 1) * xpg), xpg = H / 16 / 32, so
+//    an XCD's L2 only ever holds the exchange data of one group;
+//  * exchange: device-scope (write-through) stores into a ring with one slot per timestep, ordinary
+//    cached loads (no address is read before its only write; the 32 CUs of an XCD share one fetch);
+//  * barrier: one flag per workgroup, raised with a device-scope store, polled by wave 0 of every
+//    member (wait_versions); h_t goes from the LDS tile to the exchange slot in whole 16-byte pieces;
+//  * the 8 waves split K eight ways (no wave loads an operand block that another wave of the
+//    workgroup loads too); the 4 batch tiles of 16 rows are multiplied one after the other, the operand
+//    blocks of the next one in flight meanwhile: weights (128 registers), two sets of operand blocks
+//    (64) and accumulators (16) stay within 256 registers.
+// Requirements (host): 16-bit elements, H = 256 * NKW, H / 16 a multiple of 32, groups * xpg <= 8.
+#pragma once
+#include <type_traits>
+
+#include "recurrent_fwd_xcd.hpp"
+#ifndef FASTLSTM_WIDE_ABL
+#define FASTLSTM_WIDE_ABL 0
+#endif
+
+namespace fastlstm {
+
+template <typename T, int NKW>
+__global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdParams p) {
+    static_assert(sizeof(T) == 2, "16-bit element types");
+    using E = Elem<T>;
+    constexpr int NWV = 8, NTHR = kWave * NWV;
+    constexpr int MT = 4, NT = 4, TILES = MT * NT;           // unit tiles, batch tiles of 16 rows
+    constexpr int IPT = TILES / NWV;                         // (tile, lane) items per thread
+    constexpr int HT = 4 * MT, BT = 16 * NT;
+    constexpr int GSEG = HT * E::BYTES;                      // bytes of one gate segment of a row
+    constexpr int GROW = 4 * GSEG + 16, SROW = GSEG + 16;
+    constexpr int PPSEG = GSEG / 16;
+    constexpr int GPIECES = BT * 4 * PPSEG, SPIECES = BT * PPSEG;
+    constexpr int IOT = NTHR - kWave;                        // waves 1.. move the tiles, wave 0 polls
+    constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, n = lane & 15;
+    const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+
+    // ---- placement: group g on XCDs g*xpg .. (hardware deals workgroup i to XCD i % 8) --------
+    const int xpg = p.gpx;   // XCDs per group
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int g = xcd / xpg, j = (xcd % xpg) * 32 + slot;
+    if (g >= p.n_groups || j >= p.n_ht) return;
+    const int u0 = j * HT, b0 = g * BT;
+
+    f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                       // [8][TILES][64]
+    unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * TILES * kWave);   // gates, h, c tiles
+    const int io_tid = tid - kWave;
+
+    T *ifgo = static_cast<T *>(p.ifgo);
+    T *out = static_cast<T *>(p.out);
+    T *cell = static_cast<T *>(p.cell);
+    const T *Wh = static_cast<const T *>(p.Wh);
+
+    // ---- prologue 1: this wave's fragments of the W_h slice, global -> registers ---------
+    // fragment (m-tile a, k-step ks = wave + 8 ki): lane (q, r) holds row r = (unit a*4 + r/4, gate r%4),
+    // k = ks*KSTEP + q*EPL .. + EPL-1, i.e. 16 contiguous bytes of W_h
+    u32x4 wreg[MT][NKW];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int ki = 0; ki < NKW; ++ki) {
+            const int ks = wave + NWV * ki;
+            const int unit = u0 + a * 4 + (n >> 2), gate = n & 3;
+            const int k0 = ks * E::KSTEP + q * E::EPL;
+            wreg[a][ki] = *reinterpret_cast<const u32x4 *>(Wh + ((size_t)gate * H + unit) * H + k0);
+        }
+
+    // ---- per-thread items: (tile = wave + 8m, lane) -> (unit, batch row) -------------
+    float c_state[IPT];
+    size_t off_h[IPT];
+    int xoff[IPT], goff[IPT], soff[IPT];   // xoff: prologue only
+    bool valid[IPT];
+#pragma unroll
+    for (int m = 0; m < IPT; ++m) {
+        const int tile = wave + NWV * m;
+        const int mt = tile / NT, nt = tile % NT;
+        const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
+        valid[m] = b < B;
+        off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
+        xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
+        goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
+        soff[m] = (nt * 16 + n) * SROW + (mt * 4 + q) * E::BYTES;
+        c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
+    }
+
+    // exchange ring: slot s holds h_s, s = 0..T
+    const unsigned xgrp = (unsigned)g * NT * KS * kFragBytes;
+    const size_t xslot = (size_t)p.n_groups * NT * KS * kFragBytes;
+    int *grp_flags = p.counters + (size_t)g * kXcdGroupStride;   // n_ht <= kXcdGroupStride flags per group
+    auto publish = [&](int version) { publish_version(grp_flags + j, version); };
+
+    // ---- prologue 2: publish h_0 (slot 0) as version 1 -------------------------------------
+    {
+        const XchgGlobal x0(p.xbuf, (unsigned)xslot);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m)
+            if (valid[m]) x0.store_elem(xgrp + xoff[m], out[off_h[m]]);
+        publish(1);
+    }
+
+    const size_t B4H = (size_t)B * 4 * H;
+
+    // ---- coalesced tile I/O (see lstm_fwd_persistent_kernel) --------------------------------
+    constexpr int PD = 2;
+    u32x4 gpre[PD][GPT];
+    const size_t tile_org = (size_t)b0 * 4 * H + u0;
+    auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
+        if (io_tid < 0) return;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            const bool ok = pc < GPIECES && b0 + row < B;
+            const size_t off = ok ? (size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES) : 0;
+            dst[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + tile_org + off);
+        }
+    };
+    auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            if (io_tid >= 0 && pc < GPIECES)
+                *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
+        }
+    };
+    auto tiles_to_global = [&](int t, const unsigned char *gt) {
+        const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+#pragma unroll
+        for (int i = 0; i < GPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+                *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
+                                           k * (16 / E::BYTES)) =
+                    *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / PPSEG, k = pc % PPSEG;
+            if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
+                const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
+                *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+            }
+        }
+    };
+    auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (t < T_) fetch_tile(t, gpre[u]);
+    };
+    prefetch(0, std::integral_constant<int, 0>{});
+    prefetch(1, std::integral_constant<int, 1>{});
+
+    auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        unsigned char *gt = tiles;
+#if FASTLSTM_WIDE_ABL != 2
+        if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
+#endif
+        __syncthreads();
+
+        // ---- partial(a, i) = Wslice(a, this wave's k-steps) . h_{t-1}(i)^T, one batch tile i per pass.
+        // The operand blocks of pass i + 1 are requested before pass i is multiplied (two register
+        // sets): one exposed round trip per step, the others hide behind the MFMAs.
+        const XchgGlobal xr(p.xbuf + (size_t)t * xslot, (unsigned)xslot);
+        u32x4 bq[2][NKW];
+        auto request = [&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+#pragma unroll
+            for (int ki = 0; ki < NKW; ++ki)
+                bq[i & 1][ki] = xr.template load16<false>(xgrp + (unsigned)((i * KS + wave + NWV * ki) * kWave + lane) * 16u);
+        };
+        auto pass = [&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value;
+            if constexpr (i + 1 < NT) request(std::integral_constant<int, i + 1>{});
+            __builtin_amdgcn_sched_barrier(0);   // the next pass's loads are issued before this pass's first MFMA
+            f32x4 acc[MT];
+#pragma unroll
+            for (int a = 0; a < MT; ++a) acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ki = 0; ki < NKW; ++ki)
+#pragma unroll
+                for (int a = 0; a < MT; ++a) acc[a] = mfma_kstep<T>(wreg[a][ki], bq[i & 1][ki], acc[a]);
+#pragma unroll
+            for (int a = 0; a < MT; ++a) red[(wave * TILES + a * NT + i) * kWave + lane] = acc[a];
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#if FASTLSTM_WIDE_ABL != 1
+        request(std::integral_constant<int, 0>{});
+        pass(std::integral_constant<int, 0>{}); pass(std::integral_constant<int, 1>{});
+        pass(std::integral_constant<int, 2>{}); pass(std::integral_constant<int, 3>{});
+#endif
+        tile_to_lds(gpre[u], gt);
+        __syncthreads();
+
+        // ---- every (tile, lane) item sums the 8 partials and applies the gates -------------------
+        const XchgGlobal xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) {
+            const int tile = wave + NWV * m;
+            f32x4 s = red[tile * kWave + lane];
+#pragma unroll
+            for (int pp = 1; pp < NWV; ++pp) s += red[(pp * TILES + tile) * kWave + lane];
+            if (valid[m]) {
+                T *gl_ = reinterpret_cast<T *>(gt + goff[m]);   // the item's 4 gates in the LDS tile
+                const float pi = E::to_f32(gl_[0]) + s[0];
+                const float pf = E::to_f32(gl_[HT]) + s[1];
+                const float pg = E::to_f32(gl_[2 * HT]) + s[2];
+                const float po = E::to_f32(gl_[3 * HT]) + s[3];
+                const float c1 = sigmoidf_<false>(pf) * c_state[m] + sigmoidf_<false>(pi) * tanhf_<false>(pg);
+                const float h1 = sigmoidf_<false>(po) * tanhf_<false>(c1);
+                c_state[m] = c1;
+                const T hv = E::from_f32(h1);
+                gl_[0] = E::from_f32(pi);
+                gl_[HT] = E::from_f32(pf);
+                gl_[2 * HT] = E::from_f32(pg);
+                gl_[3 * HT] = E::from_f32(po);
+                *reinterpret_cast<T *>(gt + BT * GROW + soff[m]) = hv;
+                *reinterpret_cast<T *>(gt + BT * GROW + BT * SROW + soff[m]) = E::from_f32(c1);
+            }
+        }
+        __syncthreads();   // the h tile is complete in LDS
+        if (t + 1 < T_) {
+            // h_t to the exchange slot in 16-byte pieces (8 consecutive units of one batch row are 16
+            // contiguous bytes of an operand block): write-through stores of whole pieces, not of elements
+            const unsigned char *sth = gt + BT * GROW;
+            for (int pc = io_tid; io_tid >= 0 && pc < BT * PPSEG; pc += IOT) {
+                const int row = pc / PPSEG, c = pc % PPSEG;
+                if (b0 + row < B)
+                    xw.store16(xgrp + (unsigned)((row >> 4) * KS * kFragBytes + frag_offset<T>(row & 15, u0 + c * E::EPL)),
+                               *reinterpret_cast<const u32x4 *>(sth + row * SROW + c * 16));
+            }
+            publish(t + 2);
+        }
+        tiles_to_global(t, gt);
+        prefetch(t + PD, uc);
+    };
+    for (int t0 = 0; t0 < T_; t0 += PD) {
+        step(t0, std::integral_constant<int, 0>{});
+        if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
+    }
+}
+
+}  // namespace fastlstm

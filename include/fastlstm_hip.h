@@ -155,8 +155,9 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
  * the current device for this shape and a workspace of ws_bytes: 0 = the general kernel
  * (exchange through device memory), 1 = the XCD-local kernel (barrier group on one XCD,
  * exchange through its L2; needs the ring workspace of fastlstm_recurrent_workspace_bytes and a
- * device that fastlstm_plan_device has probed).  Negative: fastlstm_status.  Diagnostics; no
- * counterpart in the reference. */
+ * device that fastlstm_plan_device has probed), 2 = the register-resident kernel for H = 1536 and
+ * 2048 with 16-bit elements (barrier groups of H / 16 workgroups over several XCDs, 64 batch rows
+ * each; same needs as 1).  Negative: fastlstm_status.  Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
 /* Reads the status word the recurrent kernels leave at the start of their

@@ -307,6 +307,67 @@ def test_barrier_timeout_is_reported_not_hung():
     assert torch.isfinite(out.float()).all()
 
 
+WIDE_CASES = [
+    # T, B, H, dtype: hidden sizes whose barrier groups span several XCDs (weights in registers, 64-row groups)
+    (5, 128, 2048, torch.bfloat16),   # config C's B and H: two groups of 128 workgroups
+    (4, 100, 1536, torch.float16),    # 96 workgroups per group, ragged second group
+    (3, 40, 2048, torch.float16),     # one partly filled group
+]
+
+
+@pytest.mark.parametrize("T,B,H,dt", WIDE_CASES)
+def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
+    """H = 1536 / 2048: with the ring workspace the C ABI runs the register-resident kernels whose
+    groups span several XCDs (kernel kind 2), without it the general kernels; both must meet the
+    oracle on the same inputs."""
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    rm = RM[dt]
+    p = make_problem(T, B, 64, H, seed=5 + H + B)
+    pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}
+    g = {k: dev(v, dt) for k, v in p.items()}
+    o_out, o_cell, o_ifgo = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=rm)
+    st = torch.cuda.current_stream().cuda_stream
+    plans = [_lib.Plan(), _lib.Plan()]
+    for bw in (0, 1):
+        _lib.check(lib.fastlstm_plan_device(0, B, H, code, bw, plans[bw]), "plan")
+    ifgo0 = torch.empty(T, B, 4 * H, device="cuda", dtype=dt)
+    _lib.check(lib.fastlstm_gemm_ifgo(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(), g["bh"].data_ptr(),
+                                      ifgo0.data_ptr(), T, B, 64, H, code, st), "k1")
+    results = {}
+    for kind in ("general", "wide"):
+        sizes = [plans[bw].ws_bytes if kind == "general" else
+                 lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
+        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (2 if kind == "wide" else 0)
+        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 1, sizes[1]) in ((0, 2) if kind == "wide" else (0,))
+        ifgo = ifgo0.clone()
+        out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
+        cell = torch.empty_like(out)
+        out[0], cell[0] = g["h0"], g["c0"]
+        ws = torch.zeros(sizes[0], dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), g["Wh"].data_ptr(),
+                                               ws.data_ptr(), ws.numel(), T, B, H, code, st), "fwd")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
+        for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
+            assert rel_err(got, want) < HALF_TOL, (kind, name)
+        d_ifgo = torch.empty_like(ifgo)
+        dh, dc = g["dh_n"].clone(), g["dc_n"].clone()
+        wsb = torch.zeros(sizes[1], dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_bwd_persistent(g["dout"].data_ptr(), dh.data_ptr(), dc.data_ptr(), ifgo.data_ptr(),
+                                               cell.data_ptr(), d_ifgo.data_ptr(), g["Wh"].data_ptr(), wsb.data_ptr(),
+                                               wsb.numel(), T, B, H, code, st), "bwd")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(wsb[:64].cpu().numpy().tobytes()) == _lib.OK
+        dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
+        r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
+        for name, got, want in (("d_ifgo", d_ifgo, r["d_ifgo"]), ("dh0", dh, r["dh0"]), ("dc0", dc, r["dc0"])):
+            assert rel_err(got, want) < HALF_TOL, (kind, name)
+        results[kind] = (out, cell, ifgo, d_ifgo, dh, dc)
+    for a, b in zip(results["general"], results["wide"]):   # two summation orders of the same sums
+        assert rel_err(a, b) < HALF_TOL
+
+
 XCD_CASES = [
     # T, B, H, dtype          (hidden tile, members, batch tiles) of the XCD-local launch
     (20, 64, 1024, torch.float16),    # config B: 32 units x 32 members, 8 waves
