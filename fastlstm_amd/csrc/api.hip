@@ -8,6 +8,7 @@
 #include "recurrent_bwd.hpp"
 #include "recurrent_fwd.hpp"
 #include "recurrent_bwd_xcd.hpp"
+#include "recurrent_bwd_wide.hpp"
 #include "recurrent_fwd_xcd.hpp"
 
 using namespace fastlstm;
@@ -245,18 +246,19 @@ struct WideCfg {
 bool select_wide(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c) {
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
-    if (dtype == FASTLSTM_FP32 || backward) return false;
+    if (dtype == FASTLSTM_FP32) return false;
     if (H % 256 || (H != 1536 && H != 2048)) return false;
-    c->nkw = H / 256;
+    c->nkw = backward ? H / 64 : H / 256;
     c->n_ht = H / 16;
     if (c->n_ht % 32 || c->n_ht > kXcdGroupStride) return false;
     c->xpg = c->n_ht / 32;
     c->n_groups = cdiv(B, 64);
     if (c->n_groups * c->xpg > kNumXcd) return false;
-    c->ks = H / 32;
+    c->ks = (backward ? 4 * H : H) / 32;
     c->xslot = (size_t)c->n_groups * 4 * c->ks * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + 1) * c->xslot) return false;
-    c->lds = 8 * 16 * kFragBytes + 64 * (4 * 32 + 16) + 2 * 64 * (32 + 16);
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + (backward ? 0 : 1)) * c->xslot) return false;
+    const int tiles = 64 * (4 * 32 + 16) + 2 * 64 * (32 + 16);   // gates + two state tiles of 64 rows x 16 units
+    c->lds = backward ? 8 * 4 * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 16 * kFragBytes + tiles;
     return true;
 }
 
@@ -274,6 +276,26 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
     auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
+    int occ = 0;
+    if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (occ < 1) return 1;
+    if (launch(p, c.nkw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    return FASTLSTM_OK;
+}
+
+int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
+                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream) {
+    WideCfg c;
+    if (!select_wide(T, B, H, dtype, true, ws_bytes, &c)) return 1;
+    BwdXcdParams p{};
+    p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
+    p.hdr = reinterpret_cast<WsHeader *>(wsb);
+    p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);   // here: one flag per workgroup
+    p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
+    p.T = T; p.B = B; p.H = H;
+    p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KSB = c.ks;
+    p.spin_limit = spin_limit_ticks();
+    auto launch = dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16;
     int occ = 0;
     if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
@@ -576,8 +598,11 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (sync) {
-        const int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
-                                   static_cast<hipStream_t>(stream));
+        int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
+                             static_cast<hipStream_t>(stream));
+        if (rc == 1)
+            rc = try_bwd_wide(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
+                              static_cast<hipStream_t>(stream));
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     BwdParams p{};
