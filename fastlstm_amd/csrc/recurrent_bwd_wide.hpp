@@ -19,7 +19,7 @@
 
 namespace fastlstm {
 
-constexpr int kWideRing = 12;   // LDS blocks (1 KiB) per wave for operand blocks in flight
+constexpr int kWideRing = 12;   // LDS blocks (1 KiB) per wave for operand blocks in flight (8 and 14: same step time)
 
 // number of k-steps per wave NKW = 4H / KSTEP / 8 (24 for H = 1536, 32 for H = 2048)
 template <typename T, int NKW>

@@ -96,6 +96,9 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // FASTLSTM_BWD_STAMPS (diagnostic builds only): per workgroup {start, end, clocks spent waiting for
+    // chunks | -1 for a recurrence workgroup, time the last chunk arrived} of the 100 MHz clock, in the
+    // second half of the counter region of the workspace
 #ifdef FASTLSTM_BWD_STAMPS
     long long *stamps = reinterpret_cast<long long *>(p.counters + 8192) + blockIdx.x * 4;
     long long waited = 0;
@@ -171,9 +174,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int g = gl * kNumXcd + xcd;
     if (gl >= p.gpx || g >= p.n_groups) {
         if constexpr (HELP) {
-#ifndef FASTLSTM_DBG_NOHELPWORK
             if (p.k5_tiles_n > 0) bwd_helper<T>(p, smem);
-#endif
         }
         return;
     }

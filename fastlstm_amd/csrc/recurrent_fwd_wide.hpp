@@ -24,9 +24,6 @@
 #include <type_traits>
 
 #include "recurrent_fwd_xcd.hpp"
-#ifndef FASTLSTM_WIDE_ABL
-#define FASTLSTM_WIDE_ABL 0
-#endif
 
 namespace fastlstm {
 
@@ -173,9 +170,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
         unsigned char *gt = tiles;
-#if FASTLSTM_WIDE_ABL != 2
         if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
-#endif
         __syncthreads();
 
         // ---- partial(a, i) = Wslice(a, this wave's k-steps) . h_{t-1}(i)^T, one batch tile i per pass.
@@ -204,11 +199,9 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
             for (int a = 0; a < MT; ++a) red[(wave * TILES + a * NT + i) * kWave + lane] = acc[a];
             __builtin_amdgcn_sched_barrier(0);
         };
-#if FASTLSTM_WIDE_ABL != 1
         request(std::integral_constant<int, 0>{});
         pass(std::integral_constant<int, 0>{}); pass(std::integral_constant<int, 1>{});
         pass(std::integral_constant<int, 2>{}); pass(std::integral_constant<int, 3>{});
-#endif
         tile_to_lds(gpre[u], gt);
         __syncthreads();
 
