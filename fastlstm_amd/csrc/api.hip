@@ -175,11 +175,20 @@ bool select_xcd(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, 
 // In-kernel input projection: possible when the XCD-local forward kernel is the 8-wave one, at
 // least a quarter of the CUs have no role in the recurrence, and K1 suits the 256 x 256 16-bit
 // tile kernel.  Fills the k1 fields of *p (chunking by time) and returns true.
+// The second layer of a stack that shares the launch (see FwdXcdParams::n_layers).
+struct SecondLayer {
+    const void *Wx, *bx, *bh, *Wh;
+    void *ifgo, *out, *cell;
+};
+
 bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int T,
-                     int B, int I, int H, int dtype, FwdXcdParams *p) {
+                     int B, int I, int H, int dtype, FwdXcdParams *p, const SecondLayer *second = nullptr) {
     if (dtype == FASTLSTM_FP32 || c.nwv != 8 || c.mt != 8 || c.nkw != 8) return false;
-    const int n_helpers = kNumXcd * 32 - c.n_groups * c.n_ht;
+    const int layers = second ? 2 : 1;
+    if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
+    const int n_helpers = kNumXcd * 32 - layers * c.n_groups * c.n_ht;
     if (n_helpers < kNumXcd * 8) return false;
+    const int max_chunks = second ? 20 : 32;   // counters in the workspace header: 60 ints
     const int M = T * B, N = 4 * H;
     if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
@@ -187,9 +196,23 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     int base = 1;
     while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
     int ct = std::max(1, n_helpers / tiles_n / base) * base;
-    while (cdiv(tiles_m, ct) > 32) ct += base;
+    while (cdiv(tiles_m, ct) > max_chunks) ct += base;
     const int steps = ct * 256 / B;
     if (steps < 2) return false;
+    p->n_layers = layers;
+    p->n_active = c.n_groups * c.n_ht;
+    if (second) {
+        if (!gemm16_eligible(dtype, M, N, H, H, H, false, false)) return false;
+        p->ifgo2 = second->ifgo; p->out2 = second->out; p->cell2 = second->cell; p->Wh2 = second->Wh;
+        p->k1b = GemmParams{};
+        p->k1b.A = static_cast<const unsigned char *>(p->out) + (size_t)B * H * elem_bytes(dtype);   // out[1:] of the first layer
+        p->k1b.B = second->Wx; p->k1b.C = second->ifgo; p->k1b.bias0 = second->bx; p->k1b.bias1 = second->bh;
+        p->k1b.M = M; p->k1b.N = N; p->k1b.K = H;
+        p->k1b.lda = H; p->k1b.ldb = H; p->k1b.ldc = N;
+        p->k1b.splits = 1; p->k1b.k_per_split = H;
+        p->k1_done2 = p->hdr->reserved + 20;
+        p->out_ready = p->hdr->reserved + 40;
+    }
     p->k1 = GemmParams{};
     p->k1.A = x; p->k1.B = Wx; p->k1.C = ifgo; p->k1.bias0 = bx; p->k1.bias1 = bh;
     p->k1.M = M; p->k1.N = N; p->k1.K = I;
@@ -205,9 +228,11 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
 // the kernel also has to compute ifgo = x.Wx^T + b (returns 2 when that is not possible in-kernel).
 int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
                 int H, int dtype, hipStream_t stream, const void *x = nullptr, const void *Wx = nullptr,
-                const void *bx = nullptr, const void *bh = nullptr, int I = 0) {
+                const void *bx = nullptr, const void *bh = nullptr, int I = 0, const SecondLayer *second = nullptr,
+                bool dry_run = false) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c)) return 1;
+    if (second && ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + 1) * 2 * c.xslot) return 2;
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -217,13 +242,15 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
     p.trace = g_rec_trace;
+    p.n_layers = 1;
     if (x) {
-        if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p)) return 2;
+        if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p, second)) return 2;
         const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
         FwdXcdHelpLauncher hl = dtype == FASTLSTM_FP16 ? launch_fwd_xcd_help_f16 : launch_fwd_xcd_help_bf16;
         int occ = 0;
         if (hl(p, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (occ < 1) return 2;
+        if (dry_run) return FASTLSTM_OK;
         if (hl(p, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
         return FASTLSTM_OK;
     }
@@ -235,6 +262,12 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     // one workgroup per CU of the device; those without a role return at once
     if (launch(p, c.mt, c.nkw, c.ntw, c.nwv, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
+}
+
+// Clears the part of a workspace that a recurrent call needs zeroed (a kernel, not hipMemsetAsync:
+// callers may capture the stream into a graph).
+__global__ void zero_words_kernel(unsigned *p, size_t n) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
 // Shape of a launch of the register-resident kernels whose barrier groups span several XCDs
@@ -676,6 +709,58 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
 #endif
     if (int rc = fastlstm_gemm_ifgo(x, Wx, bx, bh, ifgo, T, B, I, H, dtype, stream)) return rc;
     return fastlstm_fwd_persistent(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream);
+}
+
+size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
+    const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 0);
+    if (!plan || one == 0 || plan->wave_split == 2) return one;
+    const size_t head = kWsHeaderBytes + kWsCounterBytes;
+    return one > head ? head + 2 * (one - head) : one;
+}
+
+int fastlstm_fwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    unsigned char *fake = reinterpret_cast<unsigned char *>(static_cast<size_t>(4096));   // never dereferenced
+    const SecondLayer second{fake, fake, fake, fake, fake, fake, fake};
+    const int rc = try_fwd_xcd(fake, fake, fake, fake, fake, ws_bytes, T, B, H, dtype, nullptr, fake, fake, fake, fake, I,
+                               &second, true);
+    return rc == FASTLSTM_OK ? 1 : (rc < 0 ? rc : 0);
+}
+
+int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0, void *ifgo0,
+                        void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1, const void *Wh1,
+                        void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream) {
+    if (!x || !Wx0 || !bx0 || !bh0 || !Wh0 || !ifgo0 || !out0 || !cell0 || !Wx1 || !bx1 || !bh1 || !Wh1 || !ifgo1 ||
+        !out1 || !cell1 || !ws)
+        return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(x) || !aligned16(Wx0) || !aligned16(ifgo0) || !aligned16(out0) || !aligned16(cell0) ||
+        !aligned16(Wh0) || !aligned16(Wx1) || !aligned16(ifgo1) || !aligned16(out1) || !aligned16(cell1) ||
+        !aligned16(Wh1) || !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
+    if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#ifndef FASTLSTM_TIMELINE
+    if (pl.wave_split != 2) {
+        const SecondLayer second{Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1};
+        const int rc = try_fwd_xcd(ifgo0, out0, cell0, Wh0, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype, s, x,
+                                   Wx0, bx0, bh0, I, &second);
+        if (rc <= 0) return rc;   // both layers in one launch, or failed
+    }
+#endif
+    // one layer after the other, the second on the first one's out[1:]; the workspace is cleared in between
+    if (int rc = fastlstm_fwd_layer(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, ws, ws_bytes, T, B, I, H, dtype, stream))
+        return rc;
+    const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
+    zero_words_kernel<<<256, 256, 0, s>>>(static_cast<unsigned *>(ws), zero / 4);
+    if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+    const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
+    return fastlstm_fwd_layer(x1, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws, ws_bytes, T, B, H, H, dtype, stream);
 }
 
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,

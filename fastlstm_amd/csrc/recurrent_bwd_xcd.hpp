@@ -54,12 +54,6 @@ struct BwdXcdParams {
 // and restores them around it (once per dx tile), where inlining would spill inside the GEMM
 // loops of both products.  Arguments of a function arrive in vector registers; every one of them
 // is the same in all lanes and goes back to scalar registers first.
-__device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }
-template <typename P> __device__ __forceinline__ P *uniform_ptr(P *ptr) {
-    const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
-    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
-    return reinterpret_cast<P *>(((unsigned long long)hi << 32) | lo);
-}
 template <typename T>
 __device__ __attribute__((noinline)) void helper_dx_tile(const void *A, const void *B, void *C, int M, int N, int K,
                                                          int m0, int n0, FASTLSTM_LDS_PTR unsigned char *lds) {

@@ -79,6 +79,14 @@ struct XchgLds {
 };
 
 
+// A value that is the same in all lanes, moved to scalar registers (the compiler cannot always tell).
+__device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename P> __device__ __forceinline__ P *uniform_ptr(P *ptr) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return reinterpret_cast<P *>(((unsigned long long)hi << 32) | lo);
+}
+
 // Called by wave 0 of a workgroup.  flags: the n flags of this barrier group.  NAP: s_sleep units
 // (64 clocks each) between polls; waits that are expected to last many microseconds nap longer so
 // that their polling stays out of the way of the traffic they wait for.

@@ -54,6 +54,18 @@ struct FwdXcdParams {
     int k1_tiles_m, k1_tiles_n;
     int k1_chunk_tiles, k1_chunk_steps;
     int *k1_done;         // [<= 32] device-scope counters, zero at launch
+    // Two stacked layers in one launch (n_layers == 2, HELP instantiations): the second layer's barrier
+    // groups follow the first layer's in the group numbering (so they sit on other XCDs or CUs), its
+    // input projection reads the first layer's out[1:] chunk by chunk as that layer produces it
+    // (out_ready[c] counts the first layer's workgroups whose h of chunk c are in memory), and its
+    // recurrence follows its own projection like the first layer's does.
+    int n_layers;
+    void *ifgo2, *out2, *cell2;
+    const void *Wh2;
+    GemmParams k1b;       // M = T*B, N = 4H, K = H, A = out[1:] of the first layer, B = Wx2, C = ifgo2, biases
+    int *k1_done2;        // chunk counters of the second projection
+    int *out_ready;       // [<= 20] device-scope counters, zero at launch
+    int n_active;         // workgroups of one layer's recurrence (groups * members)
     long long spin_limit;
     long long *trace;  // diagnostic build only
 };
@@ -81,6 +93,7 @@ __device__ __forceinline__ void wait_counter(int *counter, int target, WsHeader 
                                              int group, int step) {
     long long t0 = 0;
     int polls = 0;
+    counter = uniform_ptr(counter);   // the scalar load needs its address in scalar registers
     for (;;) {
         int v;
         asm volatile("s_load_dword %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(counter) : "memory");
@@ -124,21 +137,47 @@ __device__ __forceinline__ int helper_rank(int n_ht, int gpx, int n_groups, int 
 }
 
 // Input projection by a workgroup (8 waves) that has no role in the recurrence.  Helper h of n
-// takes tiles h, h + n, ... of the time-ordered tile list.  A finished tile is made visible to the
-// other XCDs (its stores acknowledged, this XCD's L2 written back: the release of the atomic) before
-// it is counted.
+// takes tiles h, h + n, ... of the time-ordered tile list of each layer.  A finished tile is made
+// visible to the other XCDs (its stores acknowledged, this XCD's L2 written back: the release of the
+// atomic) before it is counted.  With two layers a helper prefers the second layer's next tile
+// whenever the first layer has delivered the timesteps that tile reads (one poll), and otherwise
+// goes on with the first layer's list, which never has to wait for anything.
 template <typename T>
 __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *smem) {
     int n_helpers;
-    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups, &n_helpers);
+    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups * p.n_layers, &n_helpers);
     const int total = p.k1_tiles_m * p.k1_tiles_n;
-    for (int tile = h; tile < total; tile += n_helpers) {
+    int i0 = h, i1 = p.n_layers > 1 ? h : total;
+    int *ready_flag = reinterpret_cast<int *>(smem);
+    while (i0 < total || i1 < total) {
+        bool second = false;
+        if (i1 < total) {
+            const int c1 = (i1 / p.k1_tiles_n) / p.k1_chunk_tiles;
+            if (i0 < total) {   // one poll: is the chunk there?
+                if (threadIdx.x == 0)
+                    *ready_flag = __hip_atomic_load(p.out_ready + c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= p.n_active;
+                __syncthreads();
+                second = *ready_flag != 0;
+                __syncthreads();   // the flag's LDS word is part of the GEMM stages
+            } else {            // nothing else to do: wait for it
+                if ((threadIdx.x >> 6) == 0)
+                    wait_versions<100>(p.out_ready + c1, 1, p.n_active, p.hdr, p.spin_limit, -2, c1);
+                __syncthreads();
+                second = true;
+            }
+            if (second) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the first layer's h, written on other XCDs
+        }
+        const int tile = second ? i1 : i0;
         const int rt = tile / p.k1_tiles_n, ct = tile % p.k1_tiles_n;
-        gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
+        if (second) gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1b, rt * 256, ct * 256, 0, smem, 0);
+        else gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // every wave's part of the tile is in the L2 (and the LDS may be reused)
         if (threadIdx.x == 0)
-            __hip_atomic_fetch_add(p.k1_done + rt / p.k1_chunk_tiles, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add((second ? p.k1_done2 : p.k1_done) + rt / p.k1_chunk_tiles, 1, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        if (second) i1 += n_helpers;
+        else i0 += n_helpers;
     }
 }
 
@@ -174,29 +213,33 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     // ---- placement: group g lives on XCD g % 8 ------------------------------------------
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
-    const int g = gl * kNumXcd + xcd;
-    if (gl >= p.gpx || g >= p.n_groups) {
+    const int vg = gl * kNumXcd + xcd;          // group index over all layers of the launch
+    const int n_layers = HELP ? p.n_layers : 1;
+    if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
             if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);
         }
         return;
     }
+    const int layer = vg / p.n_groups, g = vg % p.n_groups;   // layer 1: the second of a stack
     const int u0 = j * HT, b0 = g * BT;
     const bool k1_live = HELP && p.k1_tiles_n > 0;
     // chunk c of ifgo is complete when all its tiles were counted
     auto wait_chunk = [&](int c, int t) {
         const int rows = min(p.k1_chunk_tiles, p.k1_tiles_m - c * p.k1_chunk_tiles);
-        wait_versions(p.k1_done + c, 1, rows * p.k1_tiles_n, p.hdr, p.spin_limit, g, t);
+        wait_versions((layer ? p.k1_done2 : p.k1_done) + c, 1, rows * p.k1_tiles_n, p.hdr, p.spin_limit, vg, t);
     };
+    // a first layer tells the helpers which chunks of its h are in memory (see the step loop)
+    const bool feeds = HELP && n_layers > 1 && layer == 0;
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                  // [4][TILES][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + 4 * TILES * kWave);   // gates, h, c tiles
     const int io_tid = tid - kWave;
 
-    T *ifgo = static_cast<T *>(p.ifgo);
-    T *out = static_cast<T *>(p.out);
-    T *cell = static_cast<T *>(p.cell);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    T *ifgo = static_cast<T *>(layer ? p.ifgo2 : p.ifgo);
+    T *out = static_cast<T *>(layer ? p.out2 : p.out);
+    T *cell = static_cast<T *>(layer ? p.cell2 : p.cell);
+    const T *Wh = static_cast<const T *>(layer ? p.Wh2 : p.Wh);
 
 #ifdef FASTLSTM_TIMELINE
     long long *tl = reinterpret_cast<long long *>(tiles + BT * GROW + 2 * BT * SROW + 64);
@@ -252,9 +295,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     }
 
     // exchange ring: slot v holds h_{v-1}... slot s = version index: h_s for s = 0..T
-    const unsigned xgrp = (unsigned)g * NT * KS * kFragBytes;
-    const size_t xslot = (size_t)p.n_groups * NT * KS * kFragBytes;
-    int *grp_counters = p.counters + (size_t)g * kXcdGroupStride;
+    const unsigned xgrp = (unsigned)vg * NT * KS * kFragBytes;
+    const size_t xslot = (size_t)p.n_groups * n_layers * NT * KS * kFragBytes;
+    int *grp_counters = p.counters + (size_t)vg * kXcdGroupStride;
     int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
 
     auto publish = [&]() {
@@ -342,10 +385,16 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         // (the barrier below orders the poll before the request)
         if (k1_live && t + PD < T_ && (t + PD) % p.k1_chunk_steps == 0 && wave == 0)
             wait_chunk((t + PD) / p.k1_chunk_steps, t);
-        if (wave == 0) wait_counter(my_counter, p.n_ht * (t + 1), p.hdr, p.spin_limit, g, t);
+        if (wave == 0) wait_counter(my_counter, p.n_ht * (t + 1), p.hdr, p.spin_limit, vg, t);
         FASTLSTM_TP(1);
         __syncthreads();
         FASTLSTM_TP(2);
+        // Every workgroup of the group has published h_t, behind the acknowledgement of everything it
+        // stored before: out[t-1] (stored in step t-2) is in this XCD's L2.  When step t-2 closed a chunk,
+        // ONE workgroup writes the L2 back (release) and counts the chunk for the whole group.
+        if (feeds && j == 0 && tid == kWave && t >= 2 && (t - 1) % p.k1_chunk_steps == 0)
+            __hip_atomic_fetch_add(p.out_ready + (t - 1) / p.k1_chunk_steps - 1, p.n_ht, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- acc[a][i] += Wslice(a) . h_{t-1}(i)^T over this wave's k-steps: all operand blocks
         // of the wave are requested at once, the weights come from registers
@@ -427,6 +476,16 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     for (int t0 = 0; t0 < T_; t0 += PD) {
         step(t0, std::integral_constant<int, 0>{});
         if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
+    }
+    if (feeds) {   // the chunks that no step has counted: every workgroup counts its own part
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        // in-loop: chunk c was counted at step (c + 1) * chunk_steps + 1 if that step exists
+        const int chunks = (T_ + p.k1_chunk_steps - 1) / p.k1_chunk_steps;
+        const int counted = T_ >= 2 ? (T_ - 2) / p.k1_chunk_steps : 0;   // chunks 0 .. counted-1 are done
+        if (tid == kWave)
+            for (int c = counted; c < chunks; ++c)
+                __hip_atomic_fetch_add(p.out_ready + c, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
 #ifdef FASTLSTM_TIMELINE
     __syncthreads();

@@ -134,6 +134,76 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
     return out, cell, ifgo
 
 
+def _stack2_workspace(plan, T, H, code, device):
+    """Workspace for fastlstm_fwd_stack2 (ring slots for both layers), or None if it would exceed
+    RING_MAX_BYTES; the part the kernels need zeroed is zeroed."""
+    n = _lib.load().fastlstm_stack2_workspace_bytes(plan, T, H, code)
+    if plan.wave_split == 2 or not plan.ws_bytes < n <= RING_MAX_BYTES:
+        return None
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    ws[:(n if plan.ring_needs_zero else plan.ws_zero_bytes)].zero_()
+    return ws
+
+
+def stack2_runs_in_one_launch(T, B, I, H, dtype, device):
+    """True if two stacked layers of this shape run as one launch (fastlstm_fwd_stack2_fused)."""
+    if dtype not in _DTYPE_CODE or torch.device(device).type != "cuda":
+        return False
+    lib = _lib.load()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(device):
+        plan = _plan(torch.device(device), B, H, code, False)
+        n = lib.fastlstm_stack2_workspace_bytes(plan, T, H, code)
+        if plan.wave_split == 2 or not plan.ws_bytes < n <= RING_MAX_BYTES:
+            return False
+        return lib.fastlstm_fwd_stack2_fused(T, B, I, H, code, n) == 1
+
+
+def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1):
+    """Two stacked layers (the second reads the first one's h): returns
+    (out0, cell0, ifgo0, out1, cell1, ifgo1) with the layouts of lstm_persistent_fwd.  The same
+    results as two calls of lstm_persistent_fwd (two iterations of the layer loop at
+    fastlstm/lstm.py:685-696); one launch where the library can run both recurrences side by side."""
+    if x.dim() == 2:
+        x = x[None]
+    _require_gpu(x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1, h0a, c0a, h0b, c0b)
+    code = _code(x)
+    T, B, I = x.shape
+    H = Wh0.shape[1]
+    assert x.is_contiguous() and Wh0.is_contiguous() and Wh1.is_contiguous()
+    assert Wx0.shape == (4 * H, I) and Wh0.shape == (4 * H, H) and Wx1.shape == (4 * H, H) and Wh1.shape == (4 * H, H)
+    for w in (Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1):
+        if w.dtype != x.dtype:
+            raise TypeError("weights must have the dtype of x (%s), got %s" % (x.dtype, w.dtype))
+    Wx0, bx0, bh0, Wx1, bx1, bh1 = (t.contiguous() for t in (Wx0, bx0, bh0, Wx1, bx1, bh1))
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        bufs = []
+        for h0, c0 in ((h0a, c0a), (h0b, c0b)):
+            ifgo = torch.empty((T, B, 4 * H), device=x.device, dtype=x.dtype)
+            out = torch.empty((T + 1, B, H), device=x.device, dtype=x.dtype)
+            cell = torch.empty_like(out)
+            if h0 is not None:
+                out[0] = h0
+                cell[0] = c0
+            else:
+                out[0].zero_()
+                cell[0].zero_()
+            bufs.append((out, cell, ifgo))
+        (out0, cell0, ifgo0), (out1, cell1, ifgo1) = bufs
+        plan = _plan(x.device, B, H, code, False)
+        ws = _stack2_workspace(plan, T, H, code, x.device)
+        if ws is None:
+            ws = _workspace(plan, T, H, code, False, x.device)
+        _lib.check(lib.fastlstm_fwd_stack2(x.data_ptr(), Wx0.data_ptr(), bx0.data_ptr(), bh0.data_ptr(), Wh0.data_ptr(),
+                                           ifgo0.data_ptr(), out0.data_ptr(), cell0.data_ptr(), Wx1.data_ptr(),
+                                           bx1.data_ptr(), bh1.data_ptr(), Wh1.data_ptr(), ifgo1.data_ptr(),
+                                           out1.data_ptr(), cell1.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H,
+                                           code, _stream()), "fastlstm_fwd_stack2")
+        _check_ws(ws, "fastlstm_fwd_stack2")
+    return out0, cell0, ifgo0, out1, cell1, ifgo1
+
+
 def Wgrad(d_ifgo, x, h):
     """(dbx, dbh, dWx, dWh) from d_ifgo[T,B,4H], x[T,B,I], h[T+1,B,H]
     (fastlstm/lstm.py:494-501; the same db tensor is returned twice)."""
@@ -235,6 +305,43 @@ class PersistentLSTMfn(torch.autograd.Function):
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
 
 
+class PersistentLSTMStack2fn(torch.autograd.Function):
+    """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2 (one
+    launch where the shapes allow), backward layer by layer through lstm_persistent_bwd.  Same
+    results and the same contract as two PersistentLSTMfn nodes in a row (fastlstm/lstm.py:685-696):
+    returns out[T,B,H] of the second layer and the (h_T, c_T) pairs of both layers, which carry no
+    gradient."""
+
+    @staticmethod
+    @custom_fwd(device_type="cuda")
+    def forward(ctx, x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1):
+        if torch.is_autocast_enabled():
+            target = torch.get_autocast_dtype("cuda")
+            x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1 = (t.to(target) for t in (x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1))
+        out0, cell0, ifgo0, out1, cell1, ifgo1 = lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b,
+                                                                            Wx1, bx1, Wh1, bh1)
+        ctx.no_state = (h0a is None, h0b is None)
+        if x.dim() == 2:
+            x = x[None]
+        ctx.save_for_backward(x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
+        return out1[1:], (out0[-1], cell0[-1]), (out1[-1], cell1[-1])
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, dh, d_state0, d_state1):
+        x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1 = ctx.saved_tensors
+        if d_state0 is not None or d_state1 is not None:
+            raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
+        z = lambda: torch.zeros_like(cell0[0])
+        d_x1, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1 = lstm_persistent_bwd(dh, z(), z(), out0[1:], out1, cell1, ifgo1, Wx1, Wh1)
+        d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0 = lstm_persistent_bwd(d_x1, z(), z(), x, out0, cell0, ifgo0, Wx0, Wh0)
+        if ctx.no_state[0]:
+            dh0a = dc0a = None
+        if ctx.no_state[1]:
+            dh0b = dc0b = None
+        return d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1
+
+
 class FastLSTM(nn.Module):
     """nn.LSTM-compatible parameters (names, shapes, order, seeded values) and the
     reference's forward contract (fastlstm/lstm.py:586-698): sequence-first input
@@ -272,7 +379,21 @@ class FastLSTM(nn.Module):
             raise ValueError(f"Not Implemnted: {self.version}")
         fn = PersistentLSTMfn.apply
         h_n, c_n = [], []
-        for layer in range(self.num_layers):
+        layer = 0
+        while layer < self.num_layers:
+            # two layers at a time where the library runs them as one launch (the second layer's
+            # recurrence a chunk of timesteps behind the first); the results do not depend on it
+            if layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda and stack2_runs_in_one_launch(
+                    x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
+                    torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device):
+                w = [getattr(self, f"{n}_l{k}") for k in (layer, layer + 1)
+                     for n in ("weight_ih", "bias_ih", "weight_hh", "bias_hh")]
+                x, (h_a, c_a), (h_b, c_b) = PersistentLSTMStack2fn.apply(
+                    x, h_0[layer], c_0[layer], *w[:4], h_0[layer + 1], c_0[layer + 1], *w[4:])
+                h_n += [h_a, h_b]
+                c_n += [c_a, c_b]
+                layer += 2
+                continue
             x, (h_i, c_i) = fn(
                 x,
                 h_0[layer],
@@ -284,6 +405,7 @@ class FastLSTM(nn.Module):
             )
             h_n += [h_i]
             c_n += [c_i]
+            layer += 1
         return x, (torch.stack(h_n), torch.stack(c_n))
 
     def extra_repr(self):

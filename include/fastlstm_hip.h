@@ -115,6 +115,25 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
                        void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I,
                        int H, int dtype, void *stream);
 
+/* Two stacked layers in one call: the second layer's input is out0[1:] (its input size is H).  The
+ * same results as fastlstm_fwd_layer for the first layer followed by fastlstm_fwd_layer for the
+ * second.  Where the XCD-local recurrences of BOTH layers fit the device next to each other and
+ * leave CUs without a role (fastlstm_fwd_stack2_fused returns 1: e.g. H = 1024, B <= 32), the two
+ * layers run in ONE launch: the idle workgroups compute both input projections, the second one
+ * chunk by chunk behind the first layer's recurrence, and the second layer's recurrence follows a
+ * chunk of timesteps behind the first -- the wall time of one layer instead of two.  Otherwise the
+ * layers run one after the other.  ws: fastlstm_stack2_workspace_bytes (ring slots for both layers),
+ * zeroed like any recurrent workspace.  Replaces two iterations of the layer loop at
+ * fastlstm/lstm.py:685-696 (which the reference runs strictly one after the other, README.md:94). */
+int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0,
+                        void *ifgo0, void *out0, void *cell0, const void *Wx1, const void *bx1,
+                        const void *bh1, const void *Wh1, void *ifgo1, void *out1, void *cell1, void *ws,
+                        size_t ws_bytes, int T, int B, int I, int H, int dtype, void *stream);
+size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype);
+/* 1 if fastlstm_fwd_stack2 runs both layers in one launch for this shape and workspace size on the
+ * current device, 0 if it runs them one after the other; negative: fastlstm_status. */
+int fastlstm_fwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes);
+
 /* K4 -- the reverse time loop.  In: dout[T,B,H]; dh,dc [B,H] hold the gradients
  * flowing into h_T, c_T; ifgo, cell as written by the forward.  Out: d_ifgo[T,B,4H];
  * dh, dc overwritten with the gradients of h_0, c_0.  ws: see

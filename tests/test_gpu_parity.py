@@ -469,6 +469,89 @@ def test_fwd_layer_equals_projection_then_recurrence(T, B, I, H, dt):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("T,B,I,H,dt,one_launch", [
+    (200, 32, 1024, 1024, torch.float16, True),    # config E's layer shape: 4 chunks of 64 timesteps
+    (131, 16, 512, 1024, torch.bfloat16, True),    # one group per layer, I != H, ragged last chunk
+    (3, 24, 256, 1024, torch.float16, True),       # shorter than a chunk
+    (30, 64, 256, 1024, torch.float16, False),     # 2 x 4 groups leave no idle CUs: one layer after the other
+    (9, 20, 50, 72, torch.float32, False),         # general kernels
+])
+def test_fwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
+    """fastlstm_fwd_stack2 must give bit-identical results to fastlstm_fwd_layer for the first layer
+    followed by fastlstm_fwd_layer for the second on out0[1:], whether it runs the two layers in one
+    launch (the second a chunk of timesteps behind the first) or one after the other."""
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    p0 = make_problem(T, B, I, H, seed=21 + T)
+    p1 = make_problem(T, B, H, H, seed=22 + T)
+    g0 = {k: dev(v, dt) for k, v in p0.items()}
+    g1 = {k: dev(v, dt) for k, v in p1.items()}
+    st = torch.cuda.current_stream().cuda_stream
+    plan = _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan), "plan")
+    n1 = lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0)
+    n2 = lib.fastlstm_stack2_workspace_bytes(plan, T, H, code)
+    assert lib.fastlstm_fwd_stack2_fused(T, B, I, H, code, n2) == (1 if one_launch else 0)
+
+    def buffers(g):
+        ifgo = torch.empty(T, B, 4 * H, device="cuda", dtype=dt)
+        out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
+        cell = torch.empty_like(out)
+        out[0], cell[0] = g["h0"], g["c0"]
+        return ifgo, out, cell
+
+    def layer(x, g, bufs, in_size):
+        ifgo, out, cell = bufs
+        ws = torch.zeros(n1, dtype=torch.uint8, device="cuda")
+        _lib.check(lib.fastlstm_fwd_layer(x.data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(), g["bh"].data_ptr(),
+                                          g["Wh"].data_ptr(), ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(),
+                                          ws.data_ptr(), ws.numel(), T, B, in_size, H, code, st), "layer")
+        torch.cuda.synchronize()
+        assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
+
+    ref0, ref1 = buffers(g0), buffers(g1)
+    layer(g0["x"], g0, ref0, I)
+    layer(ref0[1][1:], g1, ref1, H)
+    got0, got1 = buffers(g0), buffers(g1)
+    ws = torch.zeros(n2, dtype=torch.uint8, device="cuda")
+    _lib.check(lib.fastlstm_fwd_stack2(
+        g0["x"].data_ptr(), g0["Wx"].data_ptr(), g0["bx"].data_ptr(), g0["bh"].data_ptr(), g0["Wh"].data_ptr(),
+        got0[0].data_ptr(), got0[1].data_ptr(), got0[2].data_ptr(),
+        g1["Wx"].data_ptr(), g1["bx"].data_ptr(), g1["bh"].data_ptr(), g1["Wh"].data_ptr(),
+        got1[0].data_ptr(), got1[1].data_ptr(), got1[2].data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H, code, st), "stack2")
+    torch.cuda.synchronize()
+    assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
+    for a, b in zip(ref0 + ref1, got0 + got1):
+        assert torch.equal(a, b)
+
+
+def test_two_layer_module_one_launch_matches_layer_by_layer():
+    """FastLSTM with two layers of a shape that runs as one launch: outputs, final states and all
+    gradients equal those of the layer-by-layer path (two PersistentLSTMfn nodes), bit for bit."""
+    T, B, I, H = 130, 32, 1024, 1024
+    assert L.stack2_runs_in_one_launch(T, B, I, H, torch.float16, torch.device("cuda", 0))
+    torch.manual_seed(3)
+    m = L.FastLSTM(I, H, num_layers=2, device="cuda", dtype=torch.float16)
+    x = (torch.randn(T, B, I, device="cuda") * 0.5).half().requires_grad_(True)
+    w = torch.randn(T, B, H, device="cuda").half()
+    out, (h_n, c_n) = m(x)
+    (out * w).sum().backward()
+    got = [out.detach(), h_n.detach(), c_n.detach(), x.grad.clone()] + [q.grad.clone() for q in m.parameters()]
+    x.grad = None
+    m.zero_grad(set_to_none=True)
+    y = x
+    hs, cs = [], []
+    for k in range(2):
+        y, (h_i, c_i) = L.PersistentLSTMfn.apply(y, None, None, getattr(m, f"weight_ih_l{k}"), getattr(m, f"bias_ih_l{k}"),
+                                                 getattr(m, f"weight_hh_l{k}"), getattr(m, f"bias_hh_l{k}"))
+        hs.append(h_i)
+        cs.append(c_i)
+    (y * w).sum().backward()
+    want = [y.detach(), torch.stack(hs).detach(), torch.stack(cs).detach(), x.grad.clone()] + [q.grad.clone() for q in m.parameters()]
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("T,B,I,H,dt", [(96, 64, 1024, 1024, torch.float16),    # helpers compute dx inside the launch
                                         (40, 32, 512, 1024, torch.bfloat16),
                                         (24, 48, 256, 512, torch.float16),     # 16 units per workgroup
