@@ -346,12 +346,28 @@ struct BwdExtras {
 // In-kernel dx (and, where the shapes suit the 16-bit tile kernel, dWx and dWh) by the workgroups
 // without a role in the recurrence (see BwdXcdParams).  *wgrad_fused tells whether the weight
 // gradients are part of the launch.
+// The lower layer of a stack that shares the reverse launch (see BwdXcdParams::n_layers): its state
+// gradients, saved activations, d_ifgo, weights; dx may be null (not wanted); I = its input size.
+struct LowerLayer {
+    void *dh, *dc;
+    const void *ifgo, *cell;
+    void *d_ifgo;
+    const void *Wh, *Wx;
+    void *dx;
+    int I;
+    void *scratch;          // device memory for the parked fp32 weight-gradient tiles (the wgrad workspace)
+    size_t scratch_bytes;
+};
+
 bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, int T, int B, int H, int dtype,
-                      BwdXcdParams *p, bool *wgrad_fused) {
+                      BwdXcdParams *p, bool *wgrad_fused, const LowerLayer *lower = nullptr) {
     *wgrad_fused = false;
     if (dtype == FASTLSTM_FP32 || !((c.mt == 2 && c.nkw == 16) || (c.mt == 1 && c.nkw == 8))) return false;
-    const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - n_active;
+    const int layers = lower ? 2 : 1;
+    if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
+    const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - layers * n_active;
     if (n_helpers < kNumXcd * 8) return false;
+    const int max_chunks = lower ? 20 : 32;   // counters in the workspace header: 60 ints
     const int I = e.I, M = T * B, K = 4 * H;
     if (!gemm16_eligible(dtype, M, I, K, K, I, false, true) || I % 8) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(I, 256);
@@ -359,7 +375,24 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     int base = 1;
     while ((base * 256) % B) ++base;
     int ct = base >= 8 ? base : (8 / base) * base;
-    while (cdiv(tiles_m, ct) > 32) ct += base;
+    while (cdiv(tiles_m, ct) > max_chunks) ct += base;
+    p->n_layers = layers;
+    if (lower) {
+        if (e.I != H) return false;   // the upper layer's dx is the lower layer's dout
+        p->dh_lo = lower->dh; p->dc_lo = lower->dc; p->ifgo_lo = lower->ifgo; p->cell_lo = lower->cell;
+        p->d_ifgo_lo = lower->d_ifgo; p->Wh_lo = lower->Wh;
+        p->k5_lo = GemmParams{};
+        if (lower->dx) {
+            if (!gemm16_eligible(dtype, M, lower->I, K, K, lower->I, false, true) || lower->I % 8) return false;
+            p->k5_lo.A = lower->d_ifgo; p->k5_lo.B = lower->Wx; p->k5_lo.C = lower->dx;
+            p->k5_lo.M = M; p->k5_lo.N = lower->I; p->k5_lo.K = K;
+            p->k5_lo.lda = K; p->k5_lo.ldb = lower->I; p->k5_lo.ldc = lower->I;
+            p->k5_lo.splits = 1; p->k5_lo.k_per_split = K;
+        }
+        p->k5_lo_tiles_n = cdiv(lower->I, 256);
+        p->chunk_done_lo = p->hdr->reserved + 20;
+        p->dx_done = p->hdr->reserved + 40;
+    }
     p->k5 = GemmParams{};
     p->k5.A = d_ifgo; p->k5.B = e.Wx; p->k5.C = e.dx;
     p->k5.M = M; p->k5.N = I; p->k5.K = K;
@@ -380,6 +413,13 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
         p->k8_tiles_n = cdiv(I, 256); p->k9_tiles_n = cdiv(H, 256);
         p->wg_tiles = p->wg_tiles_m * (p->k8_tiles_n + p->k9_tiles_n);
         *wgrad_fused = true;
+        if (lower) {   // the stacked helpers park their accumulators between chunks
+            p->wg_scratch = static_cast<float *>(lower->scratch);
+            if ((size_t)std::min(p->wg_tiles, n_helpers) * 256 * 256 * sizeof(float) > lower->scratch_bytes) {
+                p->wg_tiles = 0;
+                *wgrad_fused = false;
+            }
+        }
     }
     return true;
 }
@@ -389,9 +429,10 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
 // to be computed.
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
-                const BwdExtras *extras = nullptr) {
+                const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
+    if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * 2 * c.xslot) return 2;
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -400,14 +441,16 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
     p.spin_limit = spin_limit_ticks();
+    p.n_layers = 1;
     if (extras) {
         bool wgrad_fused = false;
-        if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused)) return 2;
+        if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused, lower)) return 2;
         const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
         BwdXcdLauncher hl = dtype == FASTLSTM_FP16 ? launch_bwd_xcd_help_f16 : launch_bwd_xcd_help_bf16;
         int occ = 0;
         if (hl(p, c.mt, c.nkw, c.ntw, 0, lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (occ < 1) return 2;
+        if (dry_run) return wgrad_fused ? FASTLSTM_OK : 3;
         if (hl(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
         return wgrad_fused ? FASTLSTM_OK : 3;
     }
@@ -803,6 +846,77 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
         if (int r2 = fastlstm_gemm_dx(d_ifgo, Wx, dx, T, B, I, H, dtype, stream)) return r2;
     }
     return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
+}
+
+size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
+    const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 1);
+    if (!plan || one == 0 || plan->wave_split == 2) return one;
+    const size_t head = kWsHeaderBytes + kWsCounterBytes;
+    return one > head ? head + 2 * (one - head) : one;
+}
+
+int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    unsigned char *fake = reinterpret_cast<unsigned char *>(static_cast<size_t>(4096));   // never dereferenced
+    const BwdExtras e{fake, fake, fake, fake, fake, fake, H};
+    const LowerLayer lower{fake, fake, fake, fake, fake, fake, fake, fake, I, fake, (size_t)1 << 40};
+    const int rc = try_bwd_xcd(fake, fake, fake, fake, fake, fake, fake, fake, ws_bytes, T, B, H, dtype, nullptr, &e, &lower,
+                               true);
+    return (rc == FASTLSTM_OK || rc == 3) ? 1 : (rc < 0 ? rc : 0);
+}
+
+int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1, void *d_ifgo1,
+                        const void *Wh1, const void *Wx1, const void *out1, void *dWx1, void *dWh1, void *db1, void *dx1,
+                        void *dh0, void *dc0, const void *ifgo0, const void *cell0, void *d_ifgo0, const void *Wh0,
+                        const void *Wx0, const void *x, const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0,
+                        void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream) {
+    if (!dout || !dh1 || !dc1 || !ifgo1 || !cell1 || !d_ifgo1 || !Wh1 || !Wx1 || !out1 || !dWx1 || !dWh1 || !db1 || !dx1 ||
+        !dh0 || !dc0 || !ifgo0 || !cell0 || !d_ifgo0 || !Wh0 || !Wx0 || !x || !out0 || !dx0 || !dWx0 || !dWh0 || !db0 ||
+        !ws || !wgrad_ws)
+        return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    const void *ptrs[] = {dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, out1, dWx1, dWh1, dx1, dh0, dc0, ifgo0, cell0,
+                          d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, ws, wgrad_ws};
+    for (const void *q : ptrs)
+        if (!aligned16(q)) return FASTLSTM_ERR_ALIGN;
+    const size_t need = std::max(fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype), fastlstm_wgrad_workspace_bytes(T, B, H, H, dtype));
+    if (wgrad_ws_bytes < need) return FASTLSTM_ERR_WORKSPACE;
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
+    if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // the upper layer's input is the lower layer's h: x1 = out0[1:]
+    const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
+    if (pl.wave_split != 2) {
+        const BwdExtras e{Wx1, x1, out1, dx1, dWx1, dWh1, H};
+        const LowerLayer lower{dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, dx0, I, wgrad_ws, wgrad_ws_bytes};
+        const int rc = try_bwd_xcd(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, static_cast<unsigned char *>(ws), ws_bytes, T, B,
+                                   H, dtype, s, &e, &lower);
+        if (rc < 0) return rc;
+        if (rc == 0) {   // both recurrences, both dx and the upper weight gradients were one launch
+            const int chunks = colsum_chunks(T * B);
+            if (launch_colsum(dtype, d_ifgo1, db1, static_cast<float *>(wgrad_ws), T * B, 4 * H, chunks, s) != hipSuccess)
+                return FASTLSTM_ERR_HIP;
+        } else if (rc == 3) {   // ... but for the upper weight gradients (T*B not a multiple of the GEMM k-tile)
+            if (int r2 = fastlstm_gemm_wgrad(d_ifgo1, x1, out1, dWx1, dWh1, db1, wgrad_ws, wgrad_ws_bytes, T, B, H, H, dtype,
+                                             stream))
+                return r2;
+        }
+        if (rc == 0 || rc == 3)
+            return fastlstm_gemm_wgrad(d_ifgo0, x, out0, dWx0, dWh0, db0, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
+    }
+    // one layer after the other; the workspace is cleared in between
+    if (int rc = fastlstm_bwd_layer(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, x1, out1, dx1, dWx1, dWh1, db1, ws,
+                                    ws_bytes, wgrad_ws, wgrad_ws_bytes, T, B, H, H, dtype, stream))
+        return rc;
+    const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
+    zero_words_kernel<<<256, 256, 0, s>>>(static_cast<unsigned *>(ws), zero / 4);
+    if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+    return fastlstm_bwd_layer(dx1, dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, db0, ws, ws_bytes,
+                              wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {

@@ -245,20 +245,19 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     if constexpr (A_KM || B_KM) {
         // Products with a K-major operand: all fragment reads are inline assembly (see
         // lds_read_tr16) and this loop counts them itself.  Registers: the B fragments of both
-        // k-steps of a k-tile (TN each), the A fragments of its second k-step (TM), and two
-        // registers through which the A fragments of its first k-step stream, one ahead of the
-        // multiplications.
-        //   first k-step, iteration i:  read A fragment i + 1 of this k-step, B fragment i / (TM / TN)
-        //       (every TM / TN-th i) and A fragment i of the second k-step; wait for A fragment i
-        //       (everything issued behind it may stay in flight); multiply.
-        //   second k-step: its fragments are all in registers before the barrier that hands the
-        //       stage of this k-tile to the global loads; the iterations read the next k-tile's
-        //       first-k-step B fragments and, at the end, its A fragment 0.
-        // Behind the last k-tile those reads still happen (fixed counts), from a stage that exists.
-        static_assert(KSPT == 2, "one streamed and one register-resident k-step per k-tile");
-        static_assert(TM % TN == 0, "B fragments are read every TM / TN-th iteration");
+        // k-steps of a k-tile (TN each) and two registers through which the A fragments stream, one
+        // ahead of the multiplications.
+        //   iteration i of a k-step: read B fragment i / (TM / TN) of the next k-step (first k-step
+        //       only, every TM / TN-th i), read the next A fragment, wait for A fragment i
+        //       (everything issued behind it may stay in flight), multiply.
+        //   The last two A fragments of a k-tile are in registers when iteration TM - 2 of its second
+        //       k-step starts: there the wave waits for all its reads, passes the barrier that hands
+        //       the stage to the global loads, and requests the next k-tile's first fragments, whose
+        //       latency the remaining two iterations' multiplications cover.
+        static_assert(KSPT == 2, "two k-steps per k-tile");
+        static_assert(TM % TN == 0 && TM >= 4, "B fragments are read every TM / TN-th iteration");
         constexpr int NA = A_KM ? 2 : 1, NB = B_KM ? 2 : 1, EVERY = TM / TN;   // LDS instructions per fragment
-        u32x4 fs[2], fa1[TM], fb[2][TN];
+        u32x4 fs[2], fb[2][TN];
         auto rd_a = [&](int kt, int ks, int i) {
             return frag(smem + (kt % NS) * C::STAGE, std::bool_constant<A_KM>{}, std::integral_constant<int, C::A_LD>{},
                         wm * TM + i, ks);
@@ -275,24 +274,37 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
         for (int j = 0; j < TN; ++j) fb[0][j] = rd_b(0, 0, j);
         fs[0] = rd_a(0, 0, 0);
         for (int kt = 0; kt < nkt; ++kt) {
+            const bool more = kt + 1 < nkt;
             auto step0 = [&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                constexpr bool rdb = i % EVERY == 0, rdb_prev = i > 0 && (i - 1) % EVERY == 0;
-                if constexpr (i + 1 < TM) fs[(i + 1) & 1] = rd_a(kt, 0, i + 1);
+                constexpr bool rdb = i % EVERY == 0;
                 if constexpr (rdb) fb[1][i / EVERY] = rd_b(kt, 1, i / EVERY);
-                fa1[i] = rd_a(kt, 1, i);
-                // issued behind the read of A fragment i: the rest of iteration i - 1, and this iteration
-                constexpr int behind = (i > 0 ? (rdb_prev ? NB : 0) + NA : 0) + (i + 1 < TM ? NA : 0) + (rdb ? NB : 0) + NA;
-                lds_reads_landed_but<behind>(fs[i & 1]);
+                if constexpr (i + 1 < TM) fs[(i + 1) & 1] = rd_a(kt, 0, i + 1);
+                else fs[(i + 1) & 1] = rd_a(kt, 1, 0);
+                lds_reads_landed_but<(rdb ? NB : 0) + NA>(fs[i & 1]);   // behind A fragment i: this iteration's reads
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = mfma_kstep<T>(fb[0][j], fs[i & 1], acc[i][j]);
             };
             auto step1 = [&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
-                if constexpr (i % EVERY == 0) fb[0][i / EVERY] = rd_b(kt + 1, 0, i / EVERY);
-                if constexpr (i == TM - 1) fs[0] = rd_a(kt + 1, 0, 0);
+                if constexpr (i < TM - 2) {
+                    fs[(i + 1) & 1] = rd_a(kt, 1, i + 1);
+                    lds_reads_landed_but<NA>(fs[i & 1]);
+                } else if constexpr (i == TM - 2) {
+                    fs[(i + 1) & 1] = rd_a(kt, 1, i + 1);
+                    lds_reads_landed_but<0>(fs[0]);   // every read of this k-tile has landed (fs[1] passes below)
+                    lds_reads_landed_but<0>(fs[1]);
+                    if (more) {
+                        tile_ready(kt + 1);
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma_kstep<T>(fb[1][j], fa1[i], acc[i][j]);
+                        for (int j = 0; j < TN; ++j) fb[0][j] = rd_b(kt + 1, 0, j);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma_kstep<T>(fb[1][j], fs[i & 1], acc[i][j]);
+                // A fragment TM - 2 has been multiplied: its register takes the next k-tile's first A fragment
+                if constexpr (i == TM - 2)
+                    if (more) fs[0] = rd_a(kt + 1, 0, 0);
             };
             static_assert(TM == 4 || TM == 8, "wave tile rows");
             step0(std::integral_constant<int, 0>{}); step0(std::integral_constant<int, 1>{});
@@ -301,10 +313,6 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
                 step0(std::integral_constant<int, 4>{}); step0(std::integral_constant<int, 5>{});
                 step0(std::integral_constant<int, 6>{}); step0(std::integral_constant<int, 7>{});
             }
-            // every fragment of the second k-step is in registers: the stage can be handed over
-            lds_reads_landed(fa1);
-            lds_reads_landed(fb[1]);
-            if (kt + 1 < nkt) tile_ready(kt + 1);
             step1(std::integral_constant<int, 0>{}); step1(std::integral_constant<int, 1>{});
             step1(std::integral_constant<int, 2>{}); step1(std::integral_constant<int, 3>{});
             if constexpr (TM == 8) {
@@ -312,9 +320,7 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
                 step1(std::integral_constant<int, 6>{}); step1(std::integral_constant<int, 7>{});
             }
         }
-        // the reads behind the last k-tile are still in flight: nothing may reuse the LDS before them
-        lds_reads_landed_but<0>(fs[0]);
-        __syncthreads();
+        __syncthreads();   // every wave has read its last fragments (waited for above)
         return;
     }
     u32x4 fa[2][TM], fb[2][TN];

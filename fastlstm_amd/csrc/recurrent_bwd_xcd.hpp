@@ -44,8 +44,25 @@ struct BwdXcdParams {
     // T*B) of every finished chunk to its accumulators and stores the tile after the last chunk.
     GemmParams k8, k9;  // M = 4H, N = I | H, K = T*B, A = d_ifgo (K-major), B = x | h (K-major), C = dWx | dWh
     int k8_tiles_n, k9_tiles_n, wg_tiles_m, wg_tiles;
-    int n_active;
+    int n_active;       // workgroups of one layer's recurrence
     int *chunk_done;    // [<= 32] device-scope counters, zero at launch
+    // Two stacked layers in one launch (n_layers == 2, HELP instantiations).  The fields above describe
+    // the UPPER layer, whose groups come first in the group numbering.  The lower layer's recurrence
+    // reads the upper layer's dx (k5.C) as its dout: the helpers write it chunk by chunk, latest
+    // timesteps first (dx_done[c] counts the finished tiles of chunk c), and the lower recurrence
+    // requests the dout of a timestep only when its chunk is complete.  The helpers also compute the
+    // lower layer's dx (k5_lo, when its C is not null) behind that recurrence; the lower layer's weight
+    // gradients are left to the caller.
+    int n_layers;
+    void *dh_lo, *dc_lo;
+    const void *ifgo_lo, *cell_lo;
+    void *d_ifgo_lo;
+    const void *Wh_lo;
+    GemmParams k5_lo;   // M = T*B, N = I of the lower layer, K = 4H, A = d_ifgo_lo, B = Wx_lo (K-major), C = dx_lo
+    int k5_lo_tiles_n;
+    int *chunk_done_lo; // [<= 20]
+    int *dx_done;       // [<= 20]
+    float *wg_scratch;  // stacked launches: 256 KiB per helper that owns a weight-gradient tile
     long long spin_limit;
 };
 
@@ -67,15 +84,75 @@ __device__ __attribute__((noinline)) void helper_dx_tile(const void *A, const vo
     __syncthreads();   // the LDS is reused by the caller
 }
 
+// Stacked launch: one chunk's K range added to the helper's weight-gradient tile, whose fp32
+// accumulators live in `park` (256 KiB, lane-major, 16-byte accesses) between the chunks; with
+// `last` the tile is stored instead of parked.  A function call for the same reason as
+// helper_dx_tile: inlined next to the stacked helper's other work, the GEMM loop spills.
+template <typename T>
+__device__ __attribute__((noinline)) void helper_wgrad_chunk(const void *A, const void *B, void *C, int M, int N, int K,
+                                                             int ldb, int m0, int n0, int kb, int ke, f32x4 *park, int first,
+                                                             int last, FASTLSTM_LDS_PTR unsigned char *lds) {
+    constexpr int WVM = 2, WVN = 4, TM = 256 / WVM / 16, TN = 256 / WVN / 16;
+    GemmParams g{};
+    g.A = uniform_ptr(A); g.B = uniform_ptr(B); g.C = uniform_ptr(C);
+    g.M = uniform_int(M); g.N = uniform_int(N); g.K = uniform_int(K);
+    g.lda = g.M; g.ldb = uniform_int(ldb); g.ldc = g.N;
+    g.splits = 1; g.k_per_split = g.K;
+    unsigned char *smem = (unsigned char *)(FASTLSTM_LDS_PTR unsigned char *)(size_t)(unsigned)uniform_int((int)(size_t)lds);
+    park = uniform_ptr(park) + threadIdx.x;
+    m0 = uniform_int(m0); n0 = uniform_int(n0);
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            acc[i][j] = uniform_int(first) ? f32x4{0.f, 0.f, 0.f, 0.f} : park[(i * TN + j) * (kWave * 8)];
+    gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(g, m0, n0, uniform_int(kb), uniform_int(ke), smem, acc);
+    if (uniform_int(last)) {
+        gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(g, m0, n0, 0, smem, acc);
+        __syncthreads();
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) park[(i * TN + j) * (kWave * 8)] = acc[i][j];
+    }
+}
+
+// Stacked launch: waits until the lower layer has finished chunk c (the k-th in reverse time) and
+// computes this helper's share of the chunk's dx tiles of the lower layer.  A function call for the
+// same reason as helper_dx_tile.
+template <typename T>
+__device__ __attribute__((noinline)) void helper_lower_dx(int *chunk_done, int n_active, WsHeader *hdr, long long spin_limit,
+                                                          const void *A, const void *B, void *C, int M, int N, int K,
+                                                          int chunk_tiles, int tiles_n, int tiles_m, int c, int k, int h,
+                                                          int n_helpers, FASTLSTM_LDS_PTR unsigned char *lds) {
+    chunk_done = uniform_ptr(chunk_done); hdr = uniform_ptr(hdr);
+    n_active = uniform_int(n_active); chunk_tiles = uniform_int(chunk_tiles); tiles_n = uniform_int(tiles_n);
+    tiles_m = uniform_int(tiles_m); c = uniform_int(c); k = uniform_int(k); h = uniform_int(h); n_helpers = uniform_int(n_helpers);
+    if ((threadIdx.x >> 6) == 0) wait_versions<100>(chunk_done, 1, n_active, hdr, spin_limit, -3, c);
+    __syncthreads();
+    if (!uniform_ptr(C)) return;
+    const int per = chunk_tiles * tiles_n;
+    for (int i = k * per + ((h - k * per) % n_helpers + n_helpers) % n_helpers; i < (k + 1) * per; i += n_helpers) {
+        const int r = i - k * per;
+        const int rt = c * chunk_tiles + r / tiles_n, ct = r % tiles_n;
+        if (rt >= tiles_m) continue;
+        helper_dx_tile<T>(A, B, C, M, N, K, rt * 256, ct * 256, lds);
+    }
+}
+
 // The workgroups (8 waves) without a role in the recurrence.  Chunks of timesteps become available
 // in reverse time order.  Helper h of n owns weight-gradient tile h (if there is one), which it
 // accumulates chunk by chunk in registers, and takes the dx tiles h, h + n, ... of the list ordered
 // by chunk.
-template <typename T>
+// STACKED: two layers share the launch (a separate instantiation: the single-layer code keeps the
+// register allocation of its GEMM loops).
+template <typename T, bool STACKED>
 __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char *smem) {
     constexpr int WVM = 2, WVN = 4, TM = 256 / WVM / 16, TN = 256 / WVN / 16;   // 8 waves, 128 x 64 each
     int n_helpers;
-    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups, &n_helpers);
+    const int h = helper_rank(p.n_ht, p.gpx, p.n_groups * (STACKED ? 2 : 1), &n_helpers);
     const int per_chunk = p.k5_chunk_tiles * p.k5_tiles_n;
     // the weight-gradient tile of this helper: tiles of dWx first, then those of dWh
     const int n8 = p.wg_tiles_m * p.k8_tiles_n;
@@ -84,20 +161,24 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
     const GemmParams &wp = is8 ? p.k8 : p.k9;
     const int wi = is8 ? h : h - n8, wtn = is8 ? p.k8_tiles_n : p.k9_tiles_n;
     const int wm0 = (wi / wtn) * 256, wn0 = (wi % wtn) * 256;
+    constexpr bool stacked = STACKED;
+    const int lag = 2;   // the lower layer's chunks are taken this many chunks behind the upper layer's
     f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // FASTLSTM_BWD_STAMPS (diagnostic builds only): per workgroup {start, end, clocks spent waiting for
-    // chunks | -1 for a recurrence workgroup, time the last chunk arrived} of the 100 MHz clock, in the
-    // second half of the counter region of the workspace
 #ifdef FASTLSTM_BWD_STAMPS
     long long *stamps = reinterpret_cast<long long *>(p.counters + 8192) + blockIdx.x * 4;
     long long waited = 0;
     if (threadIdx.x == 0) stamps[0] = (long long)wall_clock64();
 #endif
+    // the lower layer's dx tiles of the k-th chunk in reverse time, this helper's share
+    auto lower_dx = [&](int k) {
+        helper_lower_dx<T>(p.chunk_done_lo + (p.k5_chunks - 1 - k), p.n_active, p.hdr, p.spin_limit, p.k5_lo.A, p.k5_lo.B,
+                           p.k5_lo.C, p.k5_lo.M, p.k5_lo.N, p.k5_lo.K, p.k5_chunk_tiles, p.k5_lo_tiles_n, p.k5_tiles_m,
+                           p.k5_chunks - 1 - k, k, h, n_helpers, (FASTLSTM_LDS_PTR unsigned char *)smem);
+    };
     for (int k = 0; k < p.k5_chunks; ++k) {
         const int c = p.k5_chunks - 1 - k;   // chunk in forward time
         // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
@@ -112,9 +193,15 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
 #endif
         if (own) {
             const int kb = c * p.k5_chunk_tiles * 256, ke = min(wp.K, kb + p.k5_chunk_tiles * 256);
-            int salt = 0;
-            asm volatile("" : "+v"(salt));   // opaque zero: see gemm16_mainloop
-            gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc, salt);
+            if constexpr (STACKED) {
+                helper_wgrad_chunk<T>(wp.A, wp.B, wp.C, wp.M, wp.N, wp.K, wp.ldb, wm0, wn0, kb, ke,
+                                      reinterpret_cast<f32x4 *>(p.wg_scratch) + (size_t)h * (256 * 256 / 4), k == 0,
+                                      k + 1 == p.k5_chunks, (FASTLSTM_LDS_PTR unsigned char *)smem);
+            } else {
+                int salt = 0;
+                asm volatile("" : "+v"(salt));   // opaque zero: see gemm16_mainloop
+                gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc, salt);
+            }
         }
         for (int i = k * per_chunk + ((h - k * per_chunk) % n_helpers + n_helpers) % n_helpers; i < (k + 1) * per_chunk;
              i += n_helpers) {
@@ -123,12 +210,20 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
             if (rt >= p.k5_tiles_m) continue;
             helper_dx_tile<T>(p.k5.A, p.k5.B, p.k5.C, p.k5.M, p.k5.N, p.k5.K, rt * 256, ct * 256,
                               (FASTLSTM_LDS_PTR unsigned char *)smem);
+            if (stacked) {   // the tile's stores acknowledged, this XCD's L2 written back, then counted
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (threadIdx.x == 0) __hip_atomic_fetch_add(p.dx_done + c, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
+        if (stacked && k >= lag) lower_dx(k - lag);
     }
-    if (own) {
+    if (own && !STACKED) {
         gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, 0, smem, acc);
         __syncthreads();
     }
+    if (stacked)
+        for (int k = max(p.k5_chunks - lag, 0); k < p.k5_chunks; ++k) lower_dx(k);
 #ifdef FASTLSTM_BWD_STAMPS
     if (threadIdx.x == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = waited; }
 #endif
@@ -142,7 +237,9 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
     }
 }
 
-template <typename T, int MT, int NKW, int NTW, int NWV, bool HELP = false>
+// HELP: 0 = recurrence only; 1 = the workgroups without a role compute dx and the weight gradients;
+// 2 = the same for two stacked layers that share the launch.
+template <typename T, int MT, int NKW, int NTW, int NWV, int HELP = 0>
 __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdParams p) {
     static_assert(!HELP || (NWV == 8 && sizeof(T) == 2), "the in-kernel GEMM tile is the 8-wave 16-bit one");
     using E = Elem<T>;
@@ -165,15 +262,25 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     // ---- placement: group g lives on XCD g % 8 ------------------------------------------
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
-    const int g = gl * kNumXcd + xcd;
-    if (gl >= p.gpx || g >= p.n_groups) {
-        if constexpr (HELP) {
-            if (p.k5_tiles_n > 0) bwd_helper<T>(p, smem);
+    const int vg = gl * kNumXcd + xcd;          // group index over the layers of the launch
+    constexpr int n_layers = HELP == 2 ? 2 : 1;
+    if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
+        if constexpr (HELP != 0) {
+            if (p.k5_tiles_n > 0) bwd_helper<T, HELP == 2>(p, smem);
         }
         return;
     }
+    const bool lower = HELP == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
+    const int g = lower ? vg - p.n_groups : vg;
     const int u0 = j * HT, b0 = g * BT;
     const bool k5_live = HELP && p.k5_tiles_n > 0;
+    int *chunk_done = lower ? p.chunk_done_lo : p.chunk_done;
+    // chunk c of the upper layer's dx (this layer's dout) is complete when all its tiles were counted
+    auto wait_dout = [&](int tt) {
+        const int c = tt / p.k5_chunk_steps;
+        const int rows = min(p.k5_chunk_tiles, p.k5_tiles_m - c * p.k5_chunk_tiles);
+        wait_versions(p.dx_done + c, 1, rows * p.k5_tiles_n, p.hdr, p.spin_limit, vg, tt);
+    };
 #ifdef FASTLSTM_BWD_STAMPS
     long long *stamps = reinterpret_cast<long long *>(p.counters + 8192) + blockIdx.x * 4;
     if (tid == 0) stamps[0] = (long long)wall_clock64();
@@ -183,11 +290,12 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
     const int io_tid = tid - kWave;
 
-    const T *dout = static_cast<const T *>(p.dout);
-    const T *ifgo = static_cast<const T *>(p.ifgo);
-    const T *cell = static_cast<const T *>(p.cell);
-    T *d_ifgo = static_cast<T *>(p.d_ifgo);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    const T *dout = static_cast<const T *>(lower ? p.k5.C : p.dout);
+    const T *ifgo = static_cast<const T *>(lower ? p.ifgo_lo : p.ifgo);
+    const T *cell = static_cast<const T *>(lower ? p.cell_lo : p.cell);
+    T *d_ifgo = static_cast<T *>(lower ? p.d_ifgo_lo : p.d_ifgo);
+    const T *Wh = static_cast<const T *>(lower ? p.Wh_lo : p.Wh);
+    T *dh_state = static_cast<T *>(lower ? p.dh_lo : p.dh), *dc_state_buf = static_cast<T *>(lower ? p.dc_lo : p.dc);
 
     // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
     // fragment (unit tile a, k-step ks): lane (q, r) holds row r = unit u0 + 16a + r and
@@ -230,14 +338,14 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         roff[m] = ((a * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
         goff[m] = ((nt < NT ? nt : 0) * 16 + n) * GROW + ul * E::BYTES;
         soff[m] = ((nt < NT ? nt : 0) * 16 + n) * SROW + ul * E::BYTES;
-        dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
-        dc_state[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dc)[off_h[m]]) : 0.f;
+        dh_rec[m] = valid[m] ? E::to_f32(dh_state[off_h[m]]) : 0.f;
+        dc_state[m] = valid[m] ? E::to_f32(dc_state_buf[off_h[m]]) : 0.f;
         c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
     }
 
-    const unsigned xgrp = (unsigned)g * NT * KSB * kFragBytes;
-    const size_t xslot = (size_t)p.n_groups * NT * KSB * kFragBytes;
-    int *grp_counters = p.counters + (size_t)g * kXcdGroupStride;
+    const unsigned xgrp = (unsigned)vg * NT * KSB * kFragBytes;
+    const size_t xslot = (size_t)p.n_groups * n_layers * NT * KSB * kFragBytes;
+    int *grp_counters = p.counters + (size_t)vg * kXcdGroupStride;
     int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
 
     // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out --------------------
@@ -296,6 +404,13 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
                     *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
     };
+    if (lower) {   // the latest chunk(s) of this layer's dout have to be there
+        if (wave == 0) {
+            wait_dout(T_ - 1);
+            if (T_ > 1) wait_dout(T_ - 2);
+        }
+        __syncthreads();
+    }
     fetch_tiles(T_ - 1, gpre[0], cpre[0], dpre[0]);
     if (T_ > 1) fetch_tiles(T_ - 2, gpre[1], cpre[1], dpre[1]);
     tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
@@ -306,6 +421,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         constexpr int PAR = decltype(par)::value;
         const int t = T_ - 1 - s;
         const XchgL2 xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
+        // the dout of timestep t - 2 is requested behind this step's publish barrier: when it is the
+        // latest timestep of a chunk, that chunk of the upper layer's dx must be complete
+        if (lower && wave == 0 && t >= 2 && (t - 2) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - 2);
 
         // ---- point-wise gate backward for this thread's items --------------------------
 #pragma unroll
@@ -362,7 +480,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         tile_to_global(t);
         if (s + 2 < T_) fetch_tiles(t - 2, gpre[PAR], cpre[PAR], dpre[PAR]);
 
-        if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, g, s);
+        if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, vg, s);
         __syncthreads();
         // Every workgroup of the group has passed this step's publish point, where its stores of the
         // previous steps (d_ifgo tiles included) were acknowledged by the L2.  When the previous step
@@ -370,7 +488,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         // writes this XCD's L2 back (all of it, whichever CU wrote the lines), so that the other
         // XCDs can read the chunk, and counts for all n_ht workgroups.
         if (k5_live && j == 0 && tid == kWave && s > 0 && (t + 1) % p.k5_chunk_steps == 0)
-            __hip_atomic_fetch_add(p.chunk_done + (t + 1) / p.k5_chunk_steps, p.n_ht, __ATOMIC_RELEASE,
+            __hip_atomic_fetch_add(chunk_done + (t + 1) / p.k5_chunk_steps, p.n_ht, __ATOMIC_RELEASE,
                                    __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps
@@ -426,17 +544,16 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     if (k5_live) {   // the last chunk (timesteps 0 ..)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == kWave) __hip_atomic_fetch_add(p.chunk_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == kWave) __hip_atomic_fetch_add(chunk_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
 #ifdef FASTLSTM_BWD_STAMPS
     if (tid == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = -1; }
 #endif
-    T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
 #pragma unroll
     for (int m = 0; m < IPT; ++m)
         if (valid[m]) {
-            dh_out[off_h[m]] = E::from_f32(dh_rec[m]);
-            dc_out[off_h[m]] = E::from_f32(dc_state[m]);
+            dh_state[off_h[m]] = E::from_f32(dh_rec[m]);
+            dc_state_buf[off_h[m]] = E::from_f32(dc_state[m]);
         }
 }
 

@@ -265,6 +265,48 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
     return d_x, dh_n, dc_n, dWx, dbx, dWh, dbh
 
 
+def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1):
+    """Reverse pass of two stacked layers (suffix 1: upper, 0: lower); dh[T,B,H] is the gradient of
+    out1[1:], no gradient flows into the final states.  The same results as lstm_persistent_bwd for
+    the upper layer followed by lstm_persistent_bwd for the lower layer on the upper layer's d_x;
+    one launch for both recurrences where the library can run them side by side.
+    Returns ((d_x, dh_0, dc_0, dWx, dbx, dWh, dbh) of the lower layer, the same of the upper layer)."""
+    _require_gpu(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
+    code = _code(ifgo1)
+    T, B, H = dh.shape
+    I = Wx0.shape[1]
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        dh = dh.contiguous()
+        if dh.dtype != ifgo1.dtype:
+            dh = dh.to(ifgo1.dtype)
+        x = x.contiguous()
+        new = lambda *shape: torch.empty(shape, device=x.device, dtype=x.dtype)
+        zeros = lambda: torch.zeros((B, H), device=x.device, dtype=x.dtype)
+        G = 4 * H
+        d_ifgo1, d_ifgo0 = torch.empty_like(ifgo1), torch.empty_like(ifgo0)
+        dh1, dc1, dh0, dc0 = zeros(), zeros(), zeros(), zeros()
+        dx1, dx0 = new(T, B, H), torch.empty_like(x)
+        dWx1, dWh1, db1 = new(G, H), new(G, H), new(G)
+        dWx0, dWh0, db0 = new(G, I), new(G, H), new(G)
+        plan = _plan(x.device, B, H, code, True)
+        n = lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)
+        if plan.wave_split != 2 and plan.ws_bytes < n <= RING_MAX_BYTES:
+            ws = torch.empty(n, dtype=torch.uint8, device=x.device)
+            ws[:(n if plan.ring_needs_zero else plan.ws_zero_bytes)].zero_()
+        else:
+            ws = _workspace(plan, T, H, code, True, x.device)
+        wws = torch.empty(max(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code),
+                              lib.fastlstm_wgrad_workspace_bytes(T, B, H, H, code)), dtype=torch.uint8, device=x.device)
+        p = lambda t: t.data_ptr()
+        _lib.check(lib.fastlstm_bwd_stack2(
+            p(dh), p(dh1), p(dc1), p(ifgo1), p(cell1), p(d_ifgo1), p(Wh1), p(Wx1), p(out1), p(dWx1), p(dWh1), p(db1), p(dx1),
+            p(dh0), p(dc0), p(ifgo0), p(cell0), p(d_ifgo0), p(Wh0), p(Wx0), p(x), p(out0), p(dx0), p(dWx0), p(dWh0), p(db0),
+            p(ws), ws.numel(), p(wws), wws.numel(), T, B, I, H, code, _stream()), "fastlstm_bwd_stack2")
+        _check_ws(ws, "fastlstm_bwd_stack2")
+    return (dx0, dh0, dc0, dWx0, db0, dWh0, db0), (dx1, dh1, dc1, dWx1, db1, dWh1, db1)
+
+
 class PersistentLSTMfn(torch.autograd.Function):
     """apply(x, h_0|None, c_0|None, Wx[4H,I], bx[4H], Wh[4H,H], bh[4H]) ->
     (out[T,B,H], (h_T[B,H], c_T[B,H])).  The nested tuple makes h_T/c_T
@@ -306,8 +348,8 @@ class PersistentLSTMfn(torch.autograd.Function):
 
 
 class PersistentLSTMStack2fn(torch.autograd.Function):
-    """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2 (one
-    launch where the shapes allow), backward layer by layer through lstm_persistent_bwd.  Same
+    """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2, backward
+    through lstm_persistent_bwd_stack2 (one launch each where the shapes allow).  Same
     results and the same contract as two PersistentLSTMfn nodes in a row (fastlstm/lstm.py:685-696):
     returns out[T,B,H] of the second layer and the (h_T, c_T) pairs of both layers, which carry no
     gradient."""
@@ -332,9 +374,8 @@ class PersistentLSTMStack2fn(torch.autograd.Function):
         x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1 = ctx.saved_tensors
         if d_state0 is not None or d_state1 is not None:
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
-        z = lambda: torch.zeros_like(cell0[0])
-        d_x1, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1 = lstm_persistent_bwd(dh, z(), z(), out0[1:], out1, cell1, ifgo1, Wx1, Wh1)
-        d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0 = lstm_persistent_bwd(d_x1, z(), z(), x, out0, cell0, ifgo0, Wx0, Wh0)
+        (d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0), (_, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1) = lstm_persistent_bwd_stack2(
+            dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
         if ctx.no_state[0]:
             dh0a = dc0a = None
         if ctx.no_state[1]:

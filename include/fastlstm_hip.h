@@ -170,6 +170,28 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
                         int dtype, void *stream);
 size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
 
+/* The reverse pass of two stacked layers in one call (suffix 1: upper layer, 0: lower layer; the
+ * upper layer's input is out0[1:]).  The same results as fastlstm_bwd_layer for the upper layer
+ * followed by fastlstm_bwd_layer for the lower layer with dout = dx1 (dW to the rounding of a
+ * different summation order).  dx1 [T,B,H] is the gradient that flows from the upper into the lower
+ * layer (written, then read).  Where both XCD-local reverse recurrences fit the device side by side
+ * and leave CUs without a role (fastlstm_bwd_stack2_fused returns 1), ONE launch runs both: the idle
+ * workgroups compute dx1 chunk by chunk behind the upper recurrence, the lower recurrence follows
+ * dx1 a few chunks behind, and the same workgroups accumulate dWx1, dWh1 and compute dx0; db1 and the
+ * lower layer's weight gradients follow as separate launches.  ws:
+ * fastlstm_stack2_bwd_workspace_bytes, zeroed like any recurrent workspace; wgrad_ws: the larger of
+ * the two layers' fastlstm_wgrad_workspace_bytes.  Replaces two backward nodes of the layer loop at
+ * fastlstm/lstm.py:685-696 (each lstm.py:236-334 + 494-501). */
+int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1,
+                        void *d_ifgo1, const void *Wh1, const void *Wx1, const void *out1, void *dWx1,
+                        void *dWh1, void *db1, void *dx1, void *dh0, void *dc0, const void *ifgo0,
+                        const void *cell0, void *d_ifgo0, const void *Wh0, const void *Wx0, const void *x,
+                        const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0, void *ws,
+                        size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream);
+size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype);
+int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes);
+
 /* Which kernel fastlstm_fwd_persistent (backward = 0) / fastlstm_bwd_persistent (1) will launch on
  * the current device for this shape and a workspace of ws_bytes: 0 = the general kernel
  * (exchange through device memory), 1 = the XCD-local kernel (barrier group on one XCD,
