@@ -132,6 +132,20 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         }
     }
     __syncthreads();
+    // One hidden tile per workgroup: this wave's unit tile of Wh^T, all k-steps, in registers (the LDS
+    // copy was a chain of dependent round trips per step).  Waves without a unit tile hold zeros.
+    constexpr int KSB2 = 256 / E::KSTEP;   // k-steps that cover 4H for H = 64
+    u32x4 wb2[SPLIT == 2 ? KSB2 : 1];
+    if constexpr (SPLIT == 2) {
+        const int q_ = lane >> 4, r_ = lane & 15;
+#pragma unroll
+        for (int ks = 0; ks < KSB2; ++ks) {
+            const bool ok = ks < KSB && wave < n_utiles;
+            const unsigned char *wp = ok ? Wl + ((((size_t)wave * KSB + ks) * 4 + q_) * RPT + (r_ % RPT)) * 16
+                                         : Wl + zero_off + lane * 16;
+            wb2[ks] = *reinterpret_cast<const u32x4 *>(wp);
+        }
+    }
 
     // ---- per-thread items: it = tid + 256 m -> (row n, unit ul, n-tile nt) --------------
     float dc_state[IPT], dh_rec[IPT], c1v[IPT];
@@ -426,7 +440,23 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 }
             }
         };
-        if (coherent) kloop(std::true_type{});
+        // one hidden tile per workgroup (SPLIT == 2, H <= 64): the wave's unit tile x all k-steps comes
+        // from registers and the (at most KSB2) operand blocks are requested at once
+        auto kloop_single = [&]() {
+            u32x4 bq[KSB2][NTW];
+#pragma unroll
+            for (int ks = 0; ks < KSB2; ++ks)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i)   // past the end: any valid block (its weights are zero)
+                    bq[ks][i] = xch.template load16<false>(xb + (unsigned)((i * KSB + min(ks, KSB - 1)) * kWave + lane) * 16u);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KSB2; ++ks)
+#pragma unroll
+                for (int i = 0; i < NTW; ++i) acc[i] = mfma_kstep<T>(wb2[SPLIT == 2 ? ks : 0], bq[ks][i], acc[i]);
+        };
+        if constexpr (SPLIT == 2) kloop_single();
+        else if (coherent) kloop(std::true_type{});
         else kloop(std::false_type{});
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {
