@@ -499,7 +499,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             for (int i = 0; i < NTW; ++i) acc[a][i] = f32x4{0.f, 0.f, 0.f, 0.f};
         // the operand blocks of the wave are requested in batches of at most 8 k-steps (registers):
         // all loads of a batch are issued before its first MFMA -- one round trip per batch
-        constexpr int KB = NKW > 8 ? 8 : NKW;
+        constexpr int KB = NKW > 8 ? 8 : NKW;   // (all 16 at once: slower, the L2 is the bound, not the round trips)
 #pragma unroll
         for (int k0 = 0; k0 < NKW; k0 += KB) {
             u32x4 bq[KB][NTW];
