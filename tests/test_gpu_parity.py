@@ -700,6 +700,42 @@ def test_xcd_local_barrier_timeout_is_reported_not_hung():
     assert torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("T,B,I,H,dt", [(70, 32, 256, 1024, torch.float16),     # two stacked layers per launch
+                                        (6, 128, 128, 2048, torch.bfloat16)])   # register-resident H = 2048 kernels
+def test_stacked_and_wide_launches_drain_on_timeout(T, B, I, H, dt):
+    """Host-forced failure path for the launches with chunk counters and multi-XCD flag barriers:
+    with a spin limit of one poll every wait gives up, the grids drain, the status word reports the
+    time-out (the host mirror raises), and the next call is healthy."""
+    lib = _lib.load()
+    torch.manual_seed(T)
+    x = (torch.randn(T, B, I, device="cuda") * 0.5).to(dt)
+    mk = lambda *shape: ((torch.rand(*shape, device="cuda") * 2 - 1) / H ** 0.5).to(dt)
+    W0, U0, W1, U1, b = mk(4 * H, I), mk(4 * H, H), mk(4 * H, H), mk(4 * H, H), mk(4 * H)
+    dh = torch.randn(T, B, H, device="cuda").to(dt)
+
+    def run():
+        o = L.lstm_persistent_fwd_stack2(x, None, None, W0, b, U0, b, None, None, W1, b, U1, b)
+        torch.cuda.synchronize()
+        r = L.lstm_persistent_bwd_stack2(dh, x, o[0], o[1], o[2], W0, U0, o[3], o[4], o[5], W1, U1)
+        torch.cuda.synchronize()
+        return o, r
+
+    old = L.CHECK_STATUS
+    try:
+        L.CHECK_STATUS = True
+        lib.fastlstm_set_spin_limit(1)
+        with pytest.raises(RuntimeError):
+            run()
+    finally:
+        lib.fastlstm_set_spin_limit(400000000)
+    try:
+        o, r = run()   # healthy again, still with status checks
+    finally:
+        L.CHECK_STATUS = old
+    assert all(torch.isfinite(t.float()).all() for t in o)
+    assert torch.isfinite(r[0][0].float()).all() and torch.isfinite(r[1][3].float()).all()
+
+
 # --------------------------------------------------------------------------------------
 # 4. BASELINE.json configurations at their real shapes
 # --------------------------------------------------------------------------------------
