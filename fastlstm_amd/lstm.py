@@ -109,6 +109,7 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
         if w.dtype != x.dtype:
             raise TypeError("weights must have the dtype of x (%s), got %s" % (x.dtype, w.dtype))
     Wx, bx, bh = Wx.contiguous(), bx.contiguous(), bh.contiguous()
+    x = _aligned(x)
     lib = _lib.load()
     with torch.cuda.device(x.device):
         ifgo = torch.empty((seq_len, batch_size, 4 * hidden_size), device=x.device, dtype=x.dtype)
@@ -159,6 +160,12 @@ def stack2_runs_in_one_launch(T, B, I, H, dtype, device):
         return lib.fastlstm_fwd_stack2_fused(T, B, I, H, code, n) == 1
 
 
+def _aligned(t):
+    """t itself, or a copy when its first byte is not 16-byte aligned (a slice such as out[1:] with
+    an odd B*H): the library takes base pointers on 16-byte boundaries only."""
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1):
     """Two stacked layers (the second reads the first one's h): returns
     (out0, cell0, ifgo0, out1, cell1, ifgo1) with the layouts of lstm_persistent_fwd.  The same
@@ -176,6 +183,7 @@ def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, b
         if w.dtype != x.dtype:
             raise TypeError("weights must have the dtype of x (%s), got %s" % (x.dtype, w.dtype))
     Wx0, bx0, bh0, Wx1, bx1, bh1 = (t.contiguous() for t in (Wx0, bx0, bh0, Wx1, bx1, bh1))
+    x = _aligned(x)
     lib = _lib.load()
     with torch.cuda.device(x.device):
         bufs = []
@@ -213,7 +221,7 @@ def Wgrad(d_ifgo, x, h):
     H, I = G // 4, x.shape[-1]
     lib = _lib.load()
     with torch.cuda.device(x.device):
-        d_ifgo, x, h = d_ifgo.contiguous(), x.contiguous(), h.contiguous()
+        d_ifgo, x, h = _aligned(d_ifgo.contiguous()), _aligned(x.contiguous()), _aligned(h.contiguous())
         dWx = torch.empty((G, I), device=x.device, dtype=x.dtype)
         dWh = torch.empty((G, H), device=x.device, dtype=x.dtype)
         db = torch.empty((G,), device=x.device, dtype=x.dtype)
@@ -239,12 +247,13 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
         dh = dh.contiguous()
         if dh.dtype != ifgo.dtype:
             dh = dh.to(ifgo.dtype)
+        dh = _aligned(dh)
         assert dc_n.is_contiguous() and dh_n.is_contiguous()
         d_ifgo = torch.empty_like(ifgo)
         plan = _plan(x.device, batch_size, hidden_size, code, True)
         ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
-        x, h = x.contiguous(), h.contiguous()
+        x, h = _aligned(x.contiguous()), h.contiguous()
         d_x = torch.empty_like(x)
         G = 4 * hidden_size
         dWx = torch.empty((G, input_size), device=x.device, dtype=x.dtype)
@@ -265,9 +274,11 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
     return d_x, dh_n, dc_n, dWx, dbx, dWh, dbh
 
 
-def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1):
+def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1,
+                               d_state0=None, d_state1=None):
     """Reverse pass of two stacked layers (suffix 1: upper, 0: lower); dh[T,B,H] is the gradient of
-    out1[1:], no gradient flows into the final states.  The same results as lstm_persistent_bwd for
+    out1[1:]; d_state0 / d_state1 are optional (dh_n, dc_n) pairs, the gradients flowing into the
+    final states of the lower / upper layer (zero when None).  The same results as lstm_persistent_bwd for
     the upper layer followed by lstm_persistent_bwd for the lower layer on the upper layer's d_x;
     one launch for both recurrences where the library can run them side by side.
     Returns ((d_x, dh_0, dc_0, dWx, dbx, dWh, dbh) of the lower layer, the same of the upper layer)."""
@@ -280,12 +291,13 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         dh = dh.contiguous()
         if dh.dtype != ifgo1.dtype:
             dh = dh.to(ifgo1.dtype)
-        x = x.contiguous()
+        dh, x = _aligned(dh), _aligned(x.contiguous())
         new = lambda *shape: torch.empty(shape, device=x.device, dtype=x.dtype)
         zeros = lambda: torch.zeros((B, H), device=x.device, dtype=x.dtype)
         G = 4 * H
         d_ifgo1, d_ifgo0 = torch.empty_like(ifgo1), torch.empty_like(ifgo0)
-        dh1, dc1, dh0, dc0 = zeros(), zeros(), zeros(), zeros()
+        state = lambda d, k: zeros() if d is None else d[k].to(x.dtype).reshape(B, H).clone()
+        dh1, dc1, dh0, dc0 = state(d_state1, 0), state(d_state1, 1), state(d_state0, 0), state(d_state0, 1)
         dx1, dx0 = new(T, B, H), torch.empty_like(x)
         dWx1, dWh1, db1 = new(G, H), new(G, H), new(G)
         dWx0, dWh0, db0 = new(G, I), new(G, H), new(G)
@@ -307,6 +319,15 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
     return (dx0, dh0, dc0, dWx0, db0, dWh0, db0), (dx1, dh1, dc1, dWx1, db1, dWh1, db1)
 
 
+def _autocast_operands(*tensors):
+    """x and the parameters in the autocast dtype when autocast is on (fastlstm/lstm.py:509-515;
+    the initial states are not cast)."""
+    if torch.is_autocast_enabled():
+        target = torch.get_autocast_dtype("cuda")
+        return tuple(t.to(target) for t in tensors)
+    return tensors
+
+
 class PersistentLSTMfn(torch.autograd.Function):
     """apply(x, h_0|None, c_0|None, Wx[4H,I], bx[4H], Wh[4H,H], bh[4H]) ->
     (out[T,B,H], (h_T[B,H], c_T[B,H])).  The nested tuple makes h_T/c_T
@@ -315,13 +336,7 @@ class PersistentLSTMfn(torch.autograd.Function):
     @staticmethod
     @custom_fwd(device_type="cuda")
     def forward(ctx, x, h_0, c_0, Wx, bx, Wh, bh):
-        if torch.is_autocast_enabled():  # fastlstm/lstm.py:509-515 (h_0/c_0 are not cast)
-            target = torch.get_autocast_dtype("cuda")
-            x = x.to(target)
-            Wx = Wx.to(target)
-            Wh = Wh.to(target)
-            bx = bx.to(target)
-            bh = bh.to(target)
+        x, Wx, bx, Wh, bh = _autocast_operands(x, Wx, bx, Wh, bh)
         out, cell, ifgo = lstm_persistent_fwd(x, h_0, c_0, Wx, bx, Wh, bh)
         ctx.h0_is_nan = h_0 is None
         if x.dim() == 2:
@@ -347,49 +362,90 @@ class PersistentLSTMfn(torch.autograd.Function):
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
 
 
+class PersistentLSTMStatefn(torch.autograd.Function):
+    """PersistentLSTMfn with differentiable final states: apply(...) -> (out[T,B,H], h_T[B,H], c_T[B,H]),
+    a flat tuple, so gradients with respect to h_T and c_T reach the reverse kernel as its dh_n / dc_n
+    operands (the reference raises ValueError there, fastlstm/lstm.py:528-531, and its nested tuple
+    never delivers them).  This is what carrying a state across segments and training through it needs."""
+
+    @staticmethod
+    @custom_fwd(device_type="cuda")
+    def forward(ctx, x, h_0, c_0, Wx, bx, Wh, bh):
+        x, Wx, bx, Wh, bh = _autocast_operands(x, Wx, bx, Wh, bh)
+        out, cell, ifgo = lstm_persistent_fwd(x, h_0, c_0, Wx, bx, Wh, bh)
+        ctx.no_state = h_0 is None
+        if x.dim() == 2:
+            x = x[None]
+        ctx.save_for_backward(x, out, cell, ifgo, Wx, Wh)
+        return out[1:], out[-1].clone(), cell[-1].clone()
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, dh, dh_n, dc_n):
+        x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
+        # the kernel overwrites its state operands with the gradients of the initial state
+        dh_n = dh_n.to(cell.dtype).contiguous().clone()
+        dc_n = dc_n.to(cell.dtype).contiguous().clone()
+        d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh)
+        if ctx.no_state:
+            dh_0 = dc_0 = None
+        return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
+
+
 class PersistentLSTMStack2fn(torch.autograd.Function):
     """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2, backward
     through lstm_persistent_bwd_stack2 (one launch each where the shapes allow).  Same
     results and the same contract as two PersistentLSTMfn nodes in a row (fastlstm/lstm.py:685-696):
     returns out[T,B,H] of the second layer and the (h_T, c_T) pairs of both layers, which carry no
-    gradient."""
+    gradient; with state_grads=True the result is the flat tuple (out, h_T0, c_T0, h_T1, c_T1) and
+    the final states are differentiable, as with PersistentLSTMStatefn."""
 
     @staticmethod
     @custom_fwd(device_type="cuda")
-    def forward(ctx, x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1):
-        if torch.is_autocast_enabled():
-            target = torch.get_autocast_dtype("cuda")
-            x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1 = (t.to(target) for t in (x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1))
+    def forward(ctx, x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, state_grads):
+        x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1 = _autocast_operands(x, Wx0, bx0, Wh0, bh0, Wx1, bx1, Wh1, bh1)
         out0, cell0, ifgo0, out1, cell1, ifgo1 = lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b,
                                                                             Wx1, bx1, Wh1, bh1)
         ctx.no_state = (h0a is None, h0b is None)
         if x.dim() == 2:
             x = x[None]
         ctx.save_for_backward(x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
+        if state_grads:
+            return out1[1:], out0[-1].clone(), cell0[-1].clone(), out1[-1].clone(), cell1[-1].clone()
         return out1[1:], (out0[-1], cell0[-1]), (out1[-1], cell1[-1])
 
     @staticmethod
     @custom_bwd(device_type="cuda")
-    def backward(ctx, dh, d_state0, d_state1):
+    def backward(ctx, dh, *d_states):
         x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1 = ctx.saved_tensors
-        if d_state0 is not None or d_state1 is not None:
+        d_state0 = d_state1 = None
+        if len(d_states) == 4:
+            d_state0, d_state1 = d_states[:2], d_states[2:]
+        elif any(d is not None for d in d_states):
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
         (d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0), (_, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1) = lstm_persistent_bwd_stack2(
-            dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
+            dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1)
         if ctx.no_state[0]:
             dh0a = dc0a = None
         if ctx.no_state[1]:
             dh0b = dc0b = None
-        return d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1
+        return d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1, None
 
 
 class FastLSTM(nn.Module):
     """nn.LSTM-compatible parameters (names, shapes, order, seeded values) and the
     reference's forward contract (fastlstm/lstm.py:586-698): sequence-first input
-    x[T,B,I], optional (h_0[L,B,H], c_0[L,B,H]); returns out[T,B,H], (h_n, c_n)."""
+    x[T,B,I], optional (h_0[L,B,H], c_0[L,B,H]); returns out[T,B,H], (h_n, c_n).
+
+    Keyword-only additions with nn.LSTM's meaning, all off by default so that the defaults are the
+    reference's module (which lists them as unsupported, README.md:92-93): bias=False (no bias
+    parameters), batch_first=True (x and out are [B,T,*]), bidirectional=True (a second set of
+    `*_reverse` parameters runs the same kernels over the time-reversed sequence; out is [T,B,2H]
+    and the states are [2L,B,H] in nn.LSTM's order).  state_grads=True makes h_n and c_n
+    differentiable (PersistentLSTMStatefn)."""
 
     def __init__(self, input_size, hidden_size, num_layers=1, version="persistent", device=None,
-                 dtype=None):
+                 dtype=None, *, bias=True, batch_first=False, bidirectional=False, state_grads=False):
         super().__init__()
         self.input_size = input_size
         self.hidden_size = hidden_size
@@ -397,57 +453,93 @@ class FastLSTM(nn.Module):
         self.version = version
         self.device = device
         self.dtype = dtype
+        self.bias = bias
+        self.batch_first = batch_first
+        self.bidirectional = bidirectional
+        self.state_grads = state_grads
         sqrt_k_inv = 1 / hidden_size**0.5
-        # same RNG consumption order as nn.LSTM: w_ih, w_hh, b_ih, b_hh per layer
+        directions = 2 if bidirectional else 1
+        # same RNG consumption order as nn.LSTM: w_ih, w_hh, b_ih, b_hh per layer and direction
         for layer in range(num_layers):
-            shapes = [
-                ("weight_ih_l%d" % layer, (4 * hidden_size, input_size if layer == 0 else hidden_size)),
-                ("weight_hh_l%d" % layer, (4 * hidden_size, hidden_size)),
-                ("bias_ih_l%d" % layer, (4 * hidden_size,)),
-                ("bias_hh_l%d" % layer, (4 * hidden_size,)),
-            ]
-            for name, shape in shapes:
-                value = torch.rand(*shape, device=device, dtype=dtype) * 2 * sqrt_k_inv - sqrt_k_inv
-                setattr(self, name, nn.Parameter(value))
+            for suffix in ("", "_reverse")[:directions]:
+                shapes = [
+                    ("weight_ih_l%d%s" % (layer, suffix),
+                     (4 * hidden_size, input_size if layer == 0 else hidden_size * directions)),
+                    ("weight_hh_l%d%s" % (layer, suffix), (4 * hidden_size, hidden_size)),
+                ]
+                if bias:
+                    shapes += [("bias_ih_l%d%s" % (layer, suffix), (4 * hidden_size,)),
+                               ("bias_hh_l%d%s" % (layer, suffix), (4 * hidden_size,))]
+                for name, shape in shapes:
+                    value = torch.rand(*shape, device=device, dtype=dtype) * 2 * sqrt_k_inv - sqrt_k_inv
+                    setattr(self, name, nn.Parameter(value))
+
+    def _layer_operands(self, layer, suffix=""):
+        """(Wx, bx, Wh, bh) of one layer and direction; zero biases when the module has none."""
+        Wx = getattr(self, f"weight_ih_l{layer}{suffix}")
+        Wh = getattr(self, f"weight_hh_l{layer}{suffix}")
+        if self.bias:
+            return Wx, getattr(self, f"bias_ih_l{layer}{suffix}"), Wh, getattr(self, f"bias_hh_l{layer}{suffix}")
+        zero = torch.zeros(4 * self.hidden_size, device=Wx.device, dtype=Wx.dtype)
+        return Wx, zero, Wh, zero
 
     def forward(self, x, h_c_0=None):
+        directions = 2 if self.bidirectional else 1
         if h_c_0 is None:
-            h_0, c_0 = [None] * self.num_layers, [None] * self.num_layers
+            h_0, c_0 = [None] * (self.num_layers * directions), [None] * (self.num_layers * directions)
         else:
             h_0, c_0 = h_c_0
         if self.version != "persistent":
             # the reference also offers "graph", "naive-pt" and "v1"; this build has one path
             raise ValueError(f"Not Implemnted: {self.version}")
-        fn = PersistentLSTMfn.apply
+        if self.batch_first and x.dim() == 3:
+            x = x.transpose(0, 1).contiguous()
+        if self.state_grads:
+            def fn(*operands):
+                out, h_i, c_i = PersistentLSTMStatefn.apply(*operands)
+                return out, (h_i, c_i)
+        else:
+            fn = PersistentLSTMfn.apply
         h_n, c_n = [], []
         layer = 0
         while layer < self.num_layers:
             # two layers at a time where the library runs them as one launch (the second layer's
             # recurrence a chunk of timesteps behind the first); the results do not depend on it
-            if layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda and stack2_runs_in_one_launch(
-                    x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
-                    torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device):
-                w = [getattr(self, f"{n}_l{k}") for k in (layer, layer + 1)
-                     for n in ("weight_ih", "bias_ih", "weight_hh", "bias_hh")]
-                x, (h_a, c_a), (h_b, c_b) = PersistentLSTMStack2fn.apply(
-                    x, h_0[layer], c_0[layer], *w[:4], h_0[layer + 1], c_0[layer + 1], *w[4:])
+            if (directions == 1 and layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda
+                    and stack2_runs_in_one_launch(
+                        x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
+                        torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device)):
+                w = self._layer_operands(layer) + self._layer_operands(layer + 1)
+                res = PersistentLSTMStack2fn.apply(
+                    x, h_0[layer], c_0[layer], *w[:4], h_0[layer + 1], c_0[layer + 1], *w[4:], self.state_grads)
+                if self.state_grads:
+                    x, h_a, c_a, h_b, c_b = res
+                else:
+                    x, (h_a, c_a), (h_b, c_b) = res
                 h_n += [h_a, h_b]
                 c_n += [c_a, c_b]
                 layer += 2
                 continue
-            x, (h_i, c_i) = fn(
-                x,
-                h_0[layer],
-                c_0[layer],
-                getattr(self, f"weight_ih_l{layer}"),
-                getattr(self, f"bias_ih_l{layer}"),
-                getattr(self, f"weight_hh_l{layer}"),
-                getattr(self, f"bias_hh_l{layer}"),
-            )
+            k = layer * directions
+            y, (h_i, c_i) = fn(x, h_0[k], c_0[k], *self._layer_operands(layer))
             h_n += [h_i]
             c_n += [c_i]
+            if directions == 2:
+                # the same kernels over the time-reversed sequence; its final state belongs to t = 0
+                y_r, (h_r, c_r) = fn(x.flip(0) if x.dim() == 3 else x, h_0[k + 1], c_0[k + 1],
+                                     *self._layer_operands(layer, "_reverse"))
+                y = torch.cat((y, y_r.flip(0)), dim=-1)
+                h_n += [h_r]
+                c_n += [c_r]
+            x = y
             layer += 1
+        if self.batch_first:
+            x = x.transpose(0, 1)
         return x, (torch.stack(h_n), torch.stack(c_n))
 
     def extra_repr(self):
-        return "%d, %d, num_layers=%d" % (self.input_size, self.hidden_size, self.num_layers)
+        s = "%d, %d, num_layers=%d" % (self.input_size, self.hidden_size, self.num_layers)
+        for name in ("bias", "batch_first", "bidirectional", "state_grads"):
+            if getattr(self, name) != (name == "bias"):
+                s += ", %s=%s" % (name, getattr(self, name))
+        return s

@@ -737,6 +737,92 @@ def test_stacked_and_wide_launches_drain_on_timeout(T, B, I, H, dt):
 
 
 # --------------------------------------------------------------------------------------
+# 3b. options beyond the reference's module (its README.md:92-93 lists them as unsupported):
+#     nn.LSTM's bias / batch_first / bidirectional and gradients through h_n, c_n
+# --------------------------------------------------------------------------------------
+def _option_pair(I, H, layers, dt, seed, **kw):
+    torch.manual_seed(seed)
+    m = FastLSTM(I, H, num_layers=layers, **kw)
+    kw.pop("state_grads", None)
+    ref = torch.nn.LSTM(I, H, num_layers=layers, **kw)
+    with torch.no_grad():
+        for n, prm in m.named_parameters():
+            prm.copy_(prm.to(dt).float())
+            getattr(ref, n).copy_(prm)
+    return m.to("cuda", dt), ref
+
+
+@pytest.mark.parametrize("kw", [dict(bias=False), dict(batch_first=True), dict(bidirectional=True),
+                                dict(bias=False, batch_first=True, bidirectional=True)])
+def test_option_surface_vs_nn_lstm(kw):
+    T, B, I, H, layers = 12, 5, 9, 20, 2
+    m, ref = _option_pair(I, H, layers, torch.float32, 31, **kw)
+    D = 2 if kw.get("bidirectional") else 1
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn((B, T, I) if kw.get("batch_first") else (T, B, I), generator=g)
+    h0, c0 = torch.randn(layers * D, B, H, generator=g) * 0.3, torch.randn(layers * D, B, H, generator=g) * 0.3
+    w = torch.randn(x.shape[0], x.shape[1], D * H, generator=g)
+    xg, xr = x.cuda().requires_grad_(True), x.clone().requires_grad_(True)
+    y, (hn, cn) = m(xg, (h0.cuda(), c0.cuda()))
+    yr, (hr, cr) = ref(xr, (h0, c0))
+    assert y.shape == yr.shape and hn.shape == hr.shape
+    assert_close32(y, yr); assert_close32(hn, hr); assert_close32(cn, cr)
+    (y * w.cuda()).sum().backward(); (yr * w).sum().backward()
+    assert_close32(xg.grad, xr.grad, scale_atol=max(1.0, float(xr.grad.abs().max())))
+    assert [n for n, _ in m.named_parameters()] == [n for n, _ in ref.named_parameters()]
+    for n, prm in m.named_parameters():
+        rg = getattr(ref, n).grad
+        assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
+
+
+@pytest.mark.parametrize("T,B,I,H,layers,dt", [(9, 7, 11, 33, 1, torch.float32), (14, 5, 6, 65, 3, torch.float32),
+                                               (70, 32, 256, 1024, 2, torch.float16)])   # one launch per pair
+def test_state_gradients_vs_nn_lstm(T, B, I, H, layers, dt):
+    """state_grads=True: a loss on out, h_n and c_n together, with h_0 and c_0 as leaves; every
+    gradient against nn.LSTM in fp32 on the CPU.  (The reference's nested tuple carries no gradient to
+    h_n / c_n and its backward raises for one, fastlstm/lstm.py:522-531.)"""
+    m, ref = _option_pair(I, H, layers, dt, 77, state_grads=True)
+    g = torch.Generator().manual_seed(3)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dt).float()
+    x, h0, c0 = rnd(T, B, I), rnd(layers, B, H) * 0.3, rnd(layers, B, H) * 0.3
+    wy, wh, wc = rnd(T, B, H), rnd(layers, B, H), rnd(layers, B, H)
+    leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
+    leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
+    y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
+    yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
+    assert hn.requires_grad and cn.requires_grad
+    ((y.float() * wy.cuda()).sum() + (hn.float() * wh.cuda()).sum() + (cn.float() * wc.cuda()).sum()).backward()
+    ((yr * wy).sum() + (hr * wh).sum() + (cr * wc).sum()).backward()
+    pairs = [(a.grad, b.grad, n) for a, b, n in zip(leaves, leaves_r, ("x", "h0", "c0"))]
+    pairs += [(prm.grad, getattr(ref, n).grad, n) for n, prm in m.named_parameters()]
+    for got, want, name in [(y, yr, "y"), (hn, hr, "hn"), (cn, cr, "cn")] + pairs:
+        if dt == torch.float32:
+            assert_close32(got, want, scale_atol=max(1.0, float(want.detach().abs().max())))
+        else:
+            assert rel_err(got, want) < HALF_TOL, name
+
+
+def test_state_carried_across_segments_trains_like_the_whole_sequence():
+    """Two segments with the state handed over (not detached) give the gradients of the whole sequence:
+    the reverse kernel's dh_n / dc_n operands carry the second segment's gradient into the first."""
+    T, B, I, H = 24, 6, 10, 48
+    torch.manual_seed(5)
+    m = FastLSTM(I, H, num_layers=2, state_grads=True).cuda()
+    x = torch.randn(T, B, I, device="cuda")
+    w = torch.randn(T, B, H, device="cuda")
+    y, _ = m(x)
+    (y * w).sum().backward()
+    whole = {n: p.grad.clone() for n, p in m.named_parameters()}
+    m.zero_grad()
+    y1, state = m(x[:10])
+    y2, _ = m(x[10:], state)
+    assert torch.equal(torch.cat((y1, y2)), y)
+    (torch.cat((y1, y2)) * w).sum().backward()
+    for n, p in m.named_parameters():
+        assert_close32(p.grad, whole[n].cpu(), scale_atol=max(1.0, float(whole[n].abs().max())))
+
+
+# --------------------------------------------------------------------------------------
 # 4. BASELINE.json configurations at their real shapes
 # --------------------------------------------------------------------------------------
 def _module_pair(I, H, layers, dt, seed):

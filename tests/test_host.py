@@ -176,6 +176,24 @@ def test_init_matches_nn_lstm():  # reference: tests/test_lstm.py:116-129
         torch.testing.assert_close(p, getattr(m2, n))
 
 
+@pytest.mark.parametrize("kw", [dict(bias=False), dict(bidirectional=True), dict(bias=False, bidirectional=True),
+                                dict(batch_first=True)])
+def test_option_surface_parameters_match_nn_lstm(kw):
+    """bias / bidirectional change the parameter set: same names, order, shapes and seeded values as
+    nn.LSTM (the reference lists these options as unsupported, README.md:92-93), and state dicts load
+    in both directions."""
+    torch.manual_seed(7)
+    m1 = FastLSTM(6, 5, num_layers=3, **kw)
+    torch.manual_seed(7)
+    m2 = torch.nn.LSTM(6, 5, num_layers=3, **kw)
+    assert [n for n, _ in m1.named_parameters()] == [n for n, _ in m2.named_parameters()]
+    for n, p in m1.named_parameters():
+        torch.testing.assert_close(p, getattr(m2, n))
+    m2.load_state_dict(m1.state_dict())
+    m1.load_state_dict(m2.state_dict())
+    assert "num_layers=3" in m1.extra_repr() and all(k in m1.extra_repr() for k in kw)
+
+
 def test_state_dict_interop_with_nn_lstm():
     m1 = FastLSTM(5, 7, num_layers=2)
     m2 = torch.nn.LSTM(5, 7, num_layers=2)
