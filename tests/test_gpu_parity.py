@@ -118,6 +118,56 @@ def test_stages_vs_oracle(oracle, T, B, I, H, dt):
         assert rel_err(got, want) < tol, name
 
 
+def _random_shape(rng):
+    """One (T, B, I, H, dtype) from four families: barrier-free sizes, ragged mid sizes, the tile
+    multiples that select the XCD-local / register-resident kernels, and batches of many launches'
+    worth of rows."""
+    import random  # noqa: F401  (rng is a random.Random)
+    kind = rng.choice(["small", "mid", "mid", "tile", "tile", "bigB"])
+    dt = rng.choice([torch.float32, torch.float16, torch.bfloat16])
+    if kind == "small":
+        return rng.randint(1, 40), rng.randint(1, 70), rng.randint(1, 90), rng.randint(1, 64), dt
+    if kind == "mid":
+        return rng.randint(1, 24), rng.randint(1, 130), rng.randint(1, 300), rng.randint(65, 700), dt
+    if kind == "tile":
+        H = rng.choice([128, 256, 384, 512, 768, 1024, 1024, 1536, 2048])
+        if dt == torch.float32:
+            H = min(H, 1024)
+        return (rng.randint(1, 6), rng.choice([1, 8, 16, 31, 32, 33, 64, 65, 96, 128, 160, 256]),
+                rng.choice([64, 100, 256, 1024]), H, dt)
+    return rng.randint(1, 4), rng.randint(200, 700), rng.randint(8, 128), rng.choice([64, 200, 256, 512, 1024]), dt
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_vs_oracle(oracle, seed):
+    """40 seeded random shapes per seed through both layer entry points, each stage against the oracle
+    (the backward fed with the GPU's stored activations), with the status word checked after every launch."""
+    import random
+    rng = random.Random(seed)
+    old, L.CHECK_STATUS = L.CHECK_STATUS, True
+    try:
+        for case in range(40):
+            T, B, I, H, dt = _random_shape(rng)
+            tag = f"seed {seed} case {case}: T={T} B={B} I={I} H={H} {dt}"
+            print(tag, flush=True)
+            p = make_problem(T, B, I, H, seed=seed * 1000 + case)
+            pr = {k: v.to(dt).double() for k, v in p.items()}
+            g = {k: dev(v, dt) for k, v in p.items()}
+            rm, tol = RM[dt], (FP32_TOL if dt == torch.float32 else HALF_TOL)
+            o_out, o_cell, o_ifgo = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=rm)
+            out, cell, ifgo = L.lstm_persistent_fwd(g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"])
+            for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
+                assert rel_err(got, want) < tol, (tag, name)
+            dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
+            r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
+            got = L.lstm_persistent_bwd(g["dout"], g["dc_n"].clone(), g["dh_n"].clone(), g["x"], out, cell, ifgo,
+                                        g["Wx"], g["Wh"])
+            for name, k in (("dx", 0), ("dh0", 1), ("dc0", 2), ("dWx", 3), ("db", 4), ("dWh", 5)):
+                assert rel_err(got[k], r[name]) < tol, (tag, name)
+    finally:
+        L.CHECK_STATUS = old
+
+
 @pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 4, 3), (130, 260, 70), (257, 123, 515), (512, 1024, 256)])
 def test_gemm_stages_vs_matmul(dt, M, N, K):
@@ -820,6 +870,57 @@ def test_state_carried_across_segments_trains_like_the_whole_sequence():
     (torch.cat((y1, y2)) * w).sum().backward()
     for n, p in m.named_parameters():
         assert_close32(p.grad, whole[n].cpu(), scale_atol=max(1.0, float(whole[n].abs().max())))
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_modules_vs_nn_lstm(seed):
+    """30 seeded random modules per seed (1-4 layers, every option, with and without an initial state,
+    ragged shapes and shapes whose layer pairs run as one launch): outputs, states and every gradient
+    against nn.LSTM in fp32 on the CPU."""
+    import random
+    rng = random.Random(seed)
+    old, L.CHECK_STATUS = L.CHECK_STATUS, True
+    try:
+        for case in range(30):
+            dt = rng.choice([torch.float32, torch.float16, torch.bfloat16])
+            layers = rng.randint(1, 4)
+            kw = dict(bias=rng.random() < 0.8, batch_first=rng.random() < 0.3, bidirectional=rng.random() < 0.3,
+                      state_grads=rng.random() < 0.5)
+            if rng.random() < 0.5:
+                T, B, I, H = rng.randint(20, 90), rng.choice([16, 32, 48, 64]), rng.choice([64, 256, 100]), rng.choice([256, 512, 1024])
+            else:
+                T, B, I, H = rng.randint(1, 30), rng.randint(1, 70), rng.randint(1, 100), rng.randint(1, 300)
+            with_state = rng.random() < 0.5
+            tag = f"seed {seed} case {case}: T={T} B={B} I={I} H={H} L={layers} {dt} {kw} state={with_state}"
+            print(tag, flush=True)
+            m, ref = _option_pair(I, H, layers, dt, seed * 1000 + case, **dict(kw))
+            D = 2 if kw["bidirectional"] else 1
+            g = torch.Generator().manual_seed(case)
+            rnd = lambda *shape: torch.randn(*shape, generator=g).to(dt).float()
+            x = rnd(B, T, I) if kw["batch_first"] else rnd(T, B, I)
+            h0, c0 = rnd(layers * D, B, H) * 0.3, rnd(layers * D, B, H) * 0.3
+            wy, wh, wc = rnd(*x.shape[:2], D * H), rnd(layers * D, B, H), rnd(layers * D, B, H)
+            leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
+            leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
+            if with_state:
+                y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
+                yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
+            else:
+                y, (hn, cn) = m(leaves[0])
+                yr, (hr, cr) = ref(leaves_r[0])
+            loss, loss_r = (y.float() * wy.cuda()).sum(), (yr * wy).sum()
+            if kw["state_grads"]:
+                loss = loss + (hn.float() * wh.cuda()).sum() + (cn.float() * wc.cuda()).sum()
+                loss_r = loss_r + (hr * wh).sum() + (cr * wc).sum()
+            loss.backward(); loss_r.backward()
+            pairs = [("y", y, yr), ("hn", hn, hr), ("cn", cn, cr)]
+            pairs += [(n, a.grad, b.grad) for n, a, b in zip(("dx", "dh0", "dc0"), leaves, leaves_r)][:3 if with_state else 1]
+            pairs += [(n, prm.grad, getattr(ref, n).grad) for n, prm in m.named_parameters()]
+            tol = FP32_TOL if dt == torch.float32 else HALF_TOL   # max-norm relative error
+            for name, got, want in pairs:
+                assert rel_err(got, want) < tol, (tag, name)
+    finally:
+        L.CHECK_STATUS = old
 
 
 # --------------------------------------------------------------------------------------
