@@ -35,6 +35,7 @@ SIGNATURES = {
     "fastlstm_recurrent_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i, _i]),
     "fastlstm_recurrent_kernel_kind": (_i, [_i, _i, _i, _i, _i, _sz]),
     "fastlstm_fwd_stack2": (_i, [_vp] * 16 + [_sz, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_fwd_stack2_infer": (_i, [_vp] * 16 + [_sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_stack2_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i]),
     "fastlstm_fwd_stack2_fused": (_i, [_i, _i, _i, _i, _i, _sz]),
     "fastlstm_bwd_stack2": (_i, [_vp] * 27 + [_sz, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
@@ -43,6 +44,7 @@ SIGNATURES = {
     "fastlstm_gemm_ifgo": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_layer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_fwd_layer_infer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_layer": (_i, [_vp] * 15 + [_sz, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_gemm_dx": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -15,6 +15,15 @@ using namespace fastlstm;
 
 namespace fastlstm {
 
+// What the forward launches of the calling thread store besides out: 1 = gate pre-activations and
+// every cell state (the reverse pass reads them), 0 = inference.  Set for the duration of one of
+// the *_infer entry points.
+static thread_local int t_keep_activations = 1;
+struct InferenceScope {
+    InferenceScope() { t_keep_activations = 0; }
+    ~InferenceScope() { t_keep_activations = 1; }
+};
+
 static long long *g_rec_trace = nullptr;
 static std::atomic<long long> g_spin_limit{400000000ll};  // 4 s of the 100 MHz clock
 long long spin_limit_ticks() { return g_spin_limit.load(); }
@@ -241,6 +250,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
+    p.keep = t_keep_activations;
     p.trace = g_rec_trace;
     p.n_layers = 1;
     if (x) {
@@ -308,6 +318,7 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KS = c.ks;
     p.spin_limit = spin_limit_ticks();
+    p.keep = t_keep_activations;
     auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
     int occ = 0;
     if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
@@ -612,6 +623,7 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
     p.KS = cdiv(H, kstep);
     p.spin_limit = spin_limit_ticks();
+    p.keep = t_keep_activations;
     p.trace = g_rec_trace;
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
@@ -754,6 +766,13 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
     return fastlstm_fwd_persistent(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream);
 }
 
+int fastlstm_fwd_layer_infer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
+                             void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                             void *stream) {
+    const InferenceScope scope;
+    return fastlstm_fwd_layer(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream);
+}
+
 size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
     const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 0);
     if (!plan || one == 0 || plan->wave_split == 2) return one;
@@ -804,6 +823,15 @@ int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const v
     if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
     const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
     return fastlstm_fwd_layer(x1, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws, ws_bytes, T, B, H, H, dtype, stream);
+}
+
+int fastlstm_fwd_stack2_infer(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0,
+                              void *ifgo0, void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1,
+                              const void *Wh1, void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T,
+                              int B, int I, int H, int dtype, void *stream) {
+    const InferenceScope scope;
+    return fastlstm_fwd_stack2(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws,
+                               ws_bytes, T, B, I, H, dtype, stream);
 }
 
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,

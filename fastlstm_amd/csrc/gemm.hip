@@ -141,11 +141,7 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p_in, bool a_km, bool 
         return dtype == FASTLSTM_FP16 ? launch_gemm16_dt<_Float16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s) \
                                       : launch_gemm16_dt<__bf16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s);
     FASTLSTM_TILE_CASE(128, 128, 128, 2, 2, 2, 2)   // 2 workgroups per CU
-#ifdef FASTLSTM_G256M
-    FASTLSTM_TILE_CASE(256, 256, 256, 2, FASTLSTM_G256M, FASTLSTM_G256N, 2)
-#else
     FASTLSTM_TILE_CASE(256, 256, 256, 2, 2, 4, 2)   // 8 waves, 128 x 64 per wave, 2 x 64 KiB stages
-#endif
 #undef FASTLSTM_TILE_CASE
     return launch_gemm(dtype, p, a_km, b_km, s);
 }

@@ -68,20 +68,6 @@ template <int N> __device__ __forceinline__ void lds_reads_landed_but(u32x4 &f) 
     (void)f;
 #endif
 }
-// Waits for every LDS operation of this wave; the fragments pass through it so that no use of
-// them can be scheduled ahead of the wait.
-template <int N> __device__ __forceinline__ void lds_reads_landed(u32x4 (&f)[N]) {
-    static_assert(N == 4 || N == 8, "fragments per wave tile edge");
-#if defined(__HIP_DEVICE_COMPILE__)
-    if constexpr (N == 4)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
-    else
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
-#else
-    (void)f;
-#endif
-}
 
 // 16 bytes per lane, global -> LDS, destination = lds_block + 16 * lane.  (The 16-byte form
 // exists on gfx950 only; the host pass of hipcc must not see the builtin.)

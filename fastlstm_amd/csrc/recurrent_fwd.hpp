@@ -43,6 +43,8 @@ struct FwdParams {
     int coherent_loads;  // 1: read the exchange data with device-scope loads
     int vec_io;        // 1: move the ifgo / out / cell tiles through LDS with 16-byte accesses
     int w_regs;        // > 0: k-steps per wave of the W_h slice held in registers (NKW instantiation)
+    int keep;          // 1: store the gate pre-activations and every cell state (what the reverse pass reads);
+                       // 0: inference, ifgo stays the input projection and only cell[T] is written
     long long spin_limit;
     long long *trace;  // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
 };
@@ -72,6 +74,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, n = lane & 15;
     const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+    const bool keep = p.keep != 0;   // training: gate pre-activations and every cell state are stored
 
     int g, j;
     if constexpr (SYNC) {
@@ -279,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             const int pc = io_tid + IOT * i;
             const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
             const int seg = rem / PPSEG, k = rem % PPSEG;
-            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+            if (keep && io_tid >= 0 && pc < GPIECES && b0 + row < B)
                 *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
                                            k * (16 / E::BYTES)) =
                     *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
@@ -291,7 +294,8 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
                 const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
                 *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
-                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+                if (keep || t + 1 == T_)
+                    *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
             }
         }
     };
@@ -498,13 +502,15 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
             for (int m = 0; m < IPT; ++m) {
                 if (valid[m]) {
-                    T *dst = ifgo + (size_t)t * B4H + off_p[m];
-                    dst[0] = st_p[m][0];
-                    dst[(size_t)H] = st_p[m][1];
-                    dst[(size_t)2 * H] = st_p[m][2];
-                    dst[(size_t)3 * H] = st_p[m][3];
+                    if (keep) {
+                        T *dst = ifgo + (size_t)t * B4H + off_p[m];
+                        dst[0] = st_p[m][0];
+                        dst[(size_t)H] = st_p[m][1];
+                        dst[(size_t)2 * H] = st_p[m][2];
+                        dst[(size_t)3 * H] = st_p[m][3];
+                    }
                     out[(size_t)(t + 1) * BH + off_h[m]] = st_h[m];
-                    cell[(size_t)(t + 1) * BH + off_h[m]] = st_c[m];
+                    if (keep || t + 1 == T_) cell[(size_t)(t + 1) * BH + off_h[m]] = st_c[m];
                 }
             }
         };

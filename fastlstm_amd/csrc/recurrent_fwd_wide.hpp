@@ -46,6 +46,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, n = lane & 15;
     const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+    const bool keep = p.keep != 0;   // training: gate pre-activations and every cell state are stored
 
     // ---- placement: group g on XCDs g*xpg .. (hardware deals workgroup i to XCD i % 8) --------
     const int xpg = p.gpx;   // XCDs per group
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
             const int pc = io_tid + IOT * i;
             const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
             const int seg = rem / PPSEG, k = rem % PPSEG;
-            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+            if (keep && io_tid >= 0 && pc < GPIECES && b0 + row < B)
                 *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
                                            k * (16 / E::BYTES)) =
                     *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
@@ -156,7 +157,8 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
             if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
                 const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
                 *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
-                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+                if (keep || t + 1 == T_)
+                    *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
             }
         }
     };

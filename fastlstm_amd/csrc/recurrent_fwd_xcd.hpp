@@ -66,6 +66,7 @@ struct FwdXcdParams {
     int *k1_done2;        // chunk counters of the second projection
     int *out_ready;       // [<= 20] device-scope counters, zero at launch
     int n_active;         // workgroups of one layer's recurrence (groups * members)
+    int keep;             // 1: store pre-activations and every cell state (training); 0: inference, only cell[T]
     long long spin_limit;
     long long *trace;  // diagnostic build only
 };
@@ -209,6 +210,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q = lane >> 4, n = lane & 15;
     const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
+    const bool keep = p.keep != 0;   // training: gate pre-activations and every cell state are stored
 
     // ---- placement: group g lives on XCD g % 8 ------------------------------------------
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
             const int pc = io_tid + IOT * i;
             const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
             const int seg = rem / PPSEG, k = rem % PPSEG;
-            if (io_tid >= 0 && pc < GPIECES && b0 + row < B)
+            if (keep && io_tid >= 0 && pc < GPIECES && b0 + row < B)
                 *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
                                            k * (16 / E::BYTES)) =
                     *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
@@ -362,7 +364,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
             if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
                 const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
                 *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
-                *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+                if (keep || t + 1 == T_)
+                    *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
             }
         }
     };

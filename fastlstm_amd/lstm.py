@@ -89,12 +89,15 @@ def _check_ws(ws, what):
         _lib.check(_lib.load().fastlstm_ws_status(head), what)
 
 
-def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
+def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None, keep_activations=True):
     """x[T,B,I] (or [B,I]) -> (out[T+1,B,H], cell[T+1,B,H], ifgo[T,B,4H]).
 
     out[0]/cell[0] hold the initial state (zeros when h0 is None); ifgo holds
     the full gate pre-activations of every step (kept for the backward pass).
     `version` is accepted for signature compatibility; there is one path.
+    keep_activations=False is the forward pass no backward pass follows: out and
+    cell[-1] are the same bits, cell[1:-1] is uninitialised and ifgo holds the input
+    projection only (the reference stores everything regardless, fastlstm/lstm.py:507-522).
     """
     if x.dim() == 2:  # fastlstm/lstm.py:33-34
         x = x[None]
@@ -127,9 +130,10 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None):
         ws = _workspace(plan, seq_len, hidden_size, code, False, x.device)
         stream = _stream()
         # input projection + time loop in one call (the library fuses the two where CUs would idle)
-        _lib.check(lib.fastlstm_fwd_layer(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
-                                          ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws.data_ptr(),
-                                          ws.numel(), seq_len, batch_size, input_size, hidden_size, code, stream),
+        entry = lib.fastlstm_fwd_layer if keep_activations else lib.fastlstm_fwd_layer_infer
+        _lib.check(entry(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
+                         ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws.data_ptr(),
+                         ws.numel(), seq_len, batch_size, input_size, hidden_size, code, stream),
                    "fastlstm_fwd_layer")
         _check_ws(ws, "fastlstm_fwd_layer")
     return out, cell, ifgo
@@ -166,7 +170,7 @@ def _aligned(t):
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
-def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1):
+def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, keep_activations=True):
     """Two stacked layers (the second reads the first one's h): returns
     (out0, cell0, ifgo0, out1, cell1, ifgo1) with the layouts of lstm_persistent_fwd.  The same
     results as two calls of lstm_persistent_fwd (two iterations of the layer loop at
@@ -203,11 +207,12 @@ def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, b
         ws = _stack2_workspace(plan, T, H, code, x.device)
         if ws is None:
             ws = _workspace(plan, T, H, code, False, x.device)
-        _lib.check(lib.fastlstm_fwd_stack2(x.data_ptr(), Wx0.data_ptr(), bx0.data_ptr(), bh0.data_ptr(), Wh0.data_ptr(),
-                                           ifgo0.data_ptr(), out0.data_ptr(), cell0.data_ptr(), Wx1.data_ptr(),
-                                           bx1.data_ptr(), bh1.data_ptr(), Wh1.data_ptr(), ifgo1.data_ptr(),
-                                           out1.data_ptr(), cell1.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H,
-                                           code, _stream()), "fastlstm_fwd_stack2")
+        entry = lib.fastlstm_fwd_stack2 if keep_activations else lib.fastlstm_fwd_stack2_infer
+        _lib.check(entry(x.data_ptr(), Wx0.data_ptr(), bx0.data_ptr(), bh0.data_ptr(), Wh0.data_ptr(),
+                         ifgo0.data_ptr(), out0.data_ptr(), cell0.data_ptr(), Wx1.data_ptr(),
+                         bx1.data_ptr(), bh1.data_ptr(), Wh1.data_ptr(), ifgo1.data_ptr(),
+                         out1.data_ptr(), cell1.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H,
+                         code, _stream()), "fastlstm_fwd_stack2")
         _check_ws(ws, "fastlstm_fwd_stack2")
     return out0, cell0, ifgo0, out1, cell1, ifgo1
 
@@ -494,7 +499,16 @@ class FastLSTM(nn.Module):
             raise ValueError(f"Not Implemnted: {self.version}")
         if self.batch_first and x.dim() == 3:
             x = x.transpose(0, 1).contiguous()
-        if self.state_grads:
+        # no backward pass can follow (grad mode off, or nothing that enters requires a gradient): the
+        # kernels skip the stores only the reverse pass reads; the outputs are the same bits
+        tensors = [x] + [p for p in self.parameters()] + [t for t in list(h_0) + list(c_0) if t is not None]
+        inference = not (torch.is_grad_enabled() and any(t.requires_grad for t in tensors))
+        if inference:
+            def fn(xi, h_i, c_i, Wx, bx, Wh, bh):
+                xi, Wx, bx, Wh, bh = _autocast_operands(xi, Wx, bx, Wh, bh)
+                out, cell, _ = lstm_persistent_fwd(xi, h_i, c_i, Wx, bx, Wh, bh, keep_activations=False)
+                return out[1:], (out[-1], cell[-1])
+        elif self.state_grads:
             def fn(*operands):
                 out, h_i, c_i = PersistentLSTMStatefn.apply(*operands)
                 return out, (h_i, c_i)
@@ -510,6 +524,16 @@ class FastLSTM(nn.Module):
                         x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
                         torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device)):
                 w = self._layer_operands(layer) + self._layer_operands(layer + 1)
+                if inference:
+                    xi, *wc = _autocast_operands(x, *w)
+                    out0, cell0, _, out1, cell1, _ = lstm_persistent_fwd_stack2(
+                        xi, h_0[layer], c_0[layer], *wc[:4], h_0[layer + 1], c_0[layer + 1], *wc[4:],
+                        keep_activations=False)
+                    x = out1[1:]
+                    h_n += [out0[-1], out1[-1]]
+                    c_n += [cell0[-1], cell1[-1]]
+                    layer += 2
+                    continue
                 res = PersistentLSTMStack2fn.apply(
                     x, h_0[layer], c_0[layer], *w[:4], h_0[layer + 1], c_0[layer + 1], *w[4:], self.state_grads)
                 if self.state_grads:

@@ -115,6 +115,22 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
                        void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I,
                        int H, int dtype, void *stream);
 
+/* fastlstm_fwd_layer for a forward pass that no reverse pass follows (the reference decides this per
+ * call from torch.is_grad_enabled / requires_grad and still stores everything, fastlstm/lstm.py:
+ * 507-522): out[1..T] and cell[T] are the same bits as fastlstm_fwd_layer writes; the recurrence
+ * does NOT write the gate pre-activations back (ifgo keeps the input projection x.Wx^T + bx + bh)
+ * and does not store cell[1..T-1], which stay as the caller left them.  Same arguments, workspace
+ * and launch shape; 5 of the 13 bytes per element and timestep the training pass moves are not
+ * written.  fastlstm_fwd_stack2_infer is the same for fastlstm_fwd_stack2. */
+int fastlstm_fwd_layer_infer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh,
+                             void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B,
+                             int I, int H, int dtype, void *stream);
+int fastlstm_fwd_stack2_infer(const void *x, const void *Wx0, const void *bx0, const void *bh0,
+                              const void *Wh0, void *ifgo0, void *out0, void *cell0, const void *Wx1,
+                              const void *bx1, const void *bh1, const void *Wh1, void *ifgo1, void *out1,
+                              void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                              void *stream);
+
 /* Two stacked layers in one call: the second layer's input is out0[1:] (its input size is H).  The
  * same results as fastlstm_fwd_layer for the first layer followed by fastlstm_fwd_layer for the
  * second.  Where the XCD-local recurrences of BOTH layers fit the device next to each other and

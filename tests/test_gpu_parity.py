@@ -923,6 +923,55 @@ def test_random_modules_vs_nn_lstm(seed):
         L.CHECK_STATUS = old
 
 
+@pytest.mark.parametrize("T,B,I,H,dt", [(6, 20, 64, 64, torch.float16),       # single-tile kernel
+                                        (5, 33, 70, 300, torch.float32),      # general kernel, element-wise stores
+                                        (7, 40, 64, 512, torch.float32),      # general kernel, tile stores
+                                        (40, 64, 256, 1024, torch.float16),   # XCD-local, projection inside the launch
+                                        (3, 128, 128, 2048, torch.bfloat16),  # register-resident H = 2048
+                                        (3, 300, 64, 1024, torch.float16)])   # several launches over the batch
+def test_inference_forward_is_the_training_forward_without_the_stores(T, B, I, H, dt):
+    """keep_activations=False (fastlstm_fwd_layer_infer): out and the final cell state bit for bit, the
+    gate buffer left as the input projection, cell[1:-1] untouched."""
+    p = make_problem(T, B, I, H, seed=T + H)
+    g = {k: dev(v, dt) for k, v in p.items()}
+    args = (g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"])
+    out, cell, ifgo = L.lstm_persistent_fwd(*args)
+    out_i, cell_i, ifgo_i = L.lstm_persistent_fwd(*args, keep_activations=False)
+    assert torch.equal(out_i, out)
+    assert torch.equal(cell_i[-1], cell[-1]) and torch.equal(cell_i[0], cell[0])
+    proj = torch.empty_like(ifgo)
+    lib = _lib.load()
+    _lib.check(lib.fastlstm_gemm_ifgo(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(), g["bh"].data_ptr(),
+                                      proj.data_ptr(), T, B, I, H, L._code(g["x"]), L._stream()), "gemm_ifgo")
+    assert torch.equal(ifgo_i, proj) and not torch.equal(ifgo_i, ifgo)
+
+
+@pytest.mark.parametrize("kw,T,B,I,H", [(dict(num_layers=2), 70, 32, 256, 1024),          # layer pair in one launch
+                                        (dict(num_layers=3, bidirectional=True), 9, 5, 12, 40)])
+def test_module_without_grad_takes_the_inference_path_same_bits(kw, T, B, I, H, monkeypatch):
+    torch.manual_seed(3)
+    m = FastLSTM(I, H, **kw).to("cuda", torch.float16)
+    x = torch.randn(T, B, I, device="cuda").half()
+    calls = []
+    for name in ("lstm_persistent_fwd", "lstm_persistent_fwd_stack2"):
+        orig = getattr(L, name)
+        monkeypatch.setattr(L, name, lambda *a, _o=orig, **k: (calls.append(k.get("keep_activations", True)), _o(*a, **k))[1])
+    y, (hn, cn) = m(x)
+    assert calls and all(calls)
+    calls.clear()
+    with torch.no_grad():
+        y2, (hn2, cn2) = m(x)
+    assert calls and not any(calls)
+    assert torch.equal(y2, y) and torch.equal(hn2, hn) and torch.equal(cn2, cn)
+    calls.clear()
+    m.requires_grad_(False)
+    y3, _ = m(x)                                   # nothing that enters requires a gradient
+    assert calls and not any(calls) and torch.equal(y3, y)
+    calls.clear()
+    y4, _ = m(x.clone().requires_grad_(True))      # ... unless the input does
+    assert calls and all(calls) and y4.requires_grad
+
+
 # --------------------------------------------------------------------------------------
 # 4. BASELINE.json configurations at their real shapes
 # --------------------------------------------------------------------------------------
