@@ -397,6 +397,33 @@ class PersistentLSTMStatefn(torch.autograd.Function):
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
 
 
+class PersistentLSTMHistoryfn(torch.autograd.Function):
+    """apply(...) -> (out[T,B,H], cell[T,B,H]): the layer with its whole cell-state history as a second,
+    non-differentiable result.  Sequences of different lengths padded to one T read their final states
+    out of the two histories (row b at step len_b - 1); a gradient reaches h_n through out."""
+
+    @staticmethod
+    @custom_fwd(device_type="cuda")
+    def forward(ctx, x, h_0, c_0, Wx, bx, Wh, bh):
+        x, Wx, bx, Wh, bh = _autocast_operands(x, Wx, bx, Wh, bh)
+        out, cell, ifgo = lstm_persistent_fwd(x, h_0, c_0, Wx, bx, Wh, bh)
+        ctx.no_state = h_0 is None
+        ctx.save_for_backward(x, out, cell, ifgo, Wx, Wh)
+        history = cell[1:]
+        ctx.mark_non_differentiable(history)
+        return out[1:], history
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, dh, _):
+        x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
+        d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(
+            dh, torch.zeros_like(cell[0]), torch.zeros_like(cell[0]), x, out, cell, ifgo, Wx, Wh)
+        if ctx.no_state:
+            dh_0 = dc_0 = None
+        return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
+
+
 class PersistentLSTMStack2fn(torch.autograd.Function):
     """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2, backward
     through lstm_persistent_bwd_stack2 (one launch each where the shapes allow).  Same
@@ -447,7 +474,8 @@ class FastLSTM(nn.Module):
     parameters), batch_first=True (x and out are [B,T,*]), bidirectional=True (a second set of
     `*_reverse` parameters runs the same kernels over the time-reversed sequence; out is [T,B,2H]
     and the states are [2L,B,H] in nn.LSTM's order).  state_grads=True makes h_n and c_n
-    differentiable (PersistentLSTMStatefn)."""
+    differentiable (PersistentLSTMStatefn).  A PackedSequence input gives a PackedSequence output and the
+    states at each row's own last step, as nn.LSTM does."""
 
     def __init__(self, input_size, hidden_size, num_layers=1, version="persistent", device=None,
                  dtype=None, *, bias=True, batch_first=False, bidirectional=False, state_grads=False):
@@ -488,6 +516,39 @@ class FastLSTM(nn.Module):
         zero = torch.zeros(4 * self.hidden_size, device=Wx.device, dtype=Wx.dtype)
         return Wx, zero, Wh, zero
 
+    def _forward_packed(self, packed, h_0, c_0):
+        """PackedSequence input, nn.LSTM's contract: the sequences are padded to the longest, every layer
+        runs over the padded batch (a row's steps behind its own end change nothing before it), the
+        reverse direction runs over each row reversed within its own length, and the final states are
+        row b's out / cell at step len_b - 1.  The result is packed like the input."""
+        from torch.nn.utils.rnn import PackedSequence, pack_padded_sequence, pad_packed_sequence
+        x, lengths = pad_packed_sequence(packed)                 # [T,B,I], original batch order
+        T, B = x.shape[0], x.shape[1]
+        directions = 2 if self.bidirectional else 1
+        lengths_dev = lengths.to(x.device)
+        steps = torch.arange(T, device=x.device)[:, None]
+        last = (lengths_dev - 1)[None, :, None]                   # [1,B,1] index of a row's last step
+        # time index that reverses row b within its length and leaves its padding in place
+        flip = torch.where(steps < lengths_dev[None, :], lengths_dev[None, :] - 1 - steps, steps)[:, :, None]
+        h_n, c_n = [], []
+        for layer in range(self.num_layers):
+            ys = []
+            for d, suffix in enumerate(("", "_reverse")[:directions]):
+                k = layer * directions + d
+                xi = x if d == 0 else x.gather(0, flip.expand(T, B, x.shape[2]))
+                y, cells = PersistentLSTMHistoryfn.apply(xi.contiguous(), h_0[k], c_0[k],
+                                                         *self._layer_operands(layer, suffix))
+                H = self.hidden_size
+                h_n.append(y.gather(0, last.expand(1, B, H))[0])
+                c_n.append(cells.gather(0, last.expand(1, B, H))[0])
+                ys.append(y if d == 0 else y.gather(0, flip.expand(T, B, H)))
+            x = ys[0] if directions == 1 else torch.cat(ys, dim=-1)
+        if packed.sorted_indices is not None:
+            x, lengths = x.index_select(1, packed.sorted_indices), lengths[packed.sorted_indices.cpu()]
+        data = pack_padded_sequence(x, lengths, enforce_sorted=True).data
+        out = PackedSequence(data, packed.batch_sizes, packed.sorted_indices, packed.unsorted_indices)
+        return out, (torch.stack(h_n), torch.stack(c_n))
+
     def forward(self, x, h_c_0=None):
         directions = 2 if self.bidirectional else 1
         if h_c_0 is None:
@@ -497,6 +558,8 @@ class FastLSTM(nn.Module):
         if self.version != "persistent":
             # the reference also offers "graph", "naive-pt" and "v1"; this build has one path
             raise ValueError(f"Not Implemnted: {self.version}")
+        if isinstance(x, nn.utils.rnn.PackedSequence):
+            return self._forward_packed(x, h_0, c_0)
         if self.batch_first and x.dim() == 3:
             x = x.transpose(0, 1).contiguous()
         # no backward pass can follow (grad mode off, or nothing that enters requires a gradient): the

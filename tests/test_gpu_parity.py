@@ -825,6 +825,35 @@ def test_option_surface_vs_nn_lstm(kw):
         assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
 
 
+@pytest.mark.parametrize("kw,lengths", [(dict(), [5, 9, 1, 9, 3, 7]),
+                                        (dict(bidirectional=True), [4, 4, 12, 1, 7]),
+                                        (dict(bidirectional=True, bias=False), [6])])
+def test_packed_sequence_vs_nn_lstm(kw, lengths):
+    """PackedSequence in, PackedSequence out (unsorted lengths with ties): packed data, the states at each
+    row's own last step and every gradient against nn.LSTM; the loss also reads h_n."""
+    from torch.nn.utils.rnn import pack_sequence
+    I, H, layers = 7, 24, 2
+    m, ref = _option_pair(I, H, layers, torch.float32, 41, **kw)
+    D = 2 if kw.get("bidirectional") else 1
+    g = torch.Generator().manual_seed(9)
+    seqs = [torch.randn(n, I, generator=g) for n in lengths]
+    B = len(lengths)
+    h0, c0 = torch.randn(layers * D, B, H, generator=g) * 0.3, torch.randn(layers * D, B, H, generator=g) * 0.3
+    w, wh = torch.randn(sum(lengths), D * H, generator=g), torch.randn(layers * D, B, H, generator=g)
+    xr = pack_sequence(seqs, enforce_sorted=False)
+    xg = pack_sequence([t.cuda() for t in seqs], enforce_sorted=False)
+    y, (hn, cn) = m(xg, (h0.cuda(), c0.cuda()))
+    yr, (hr, cr) = ref(xr, (h0, c0))
+    assert torch.equal(y.batch_sizes, yr.batch_sizes) and torch.equal(y.sorted_indices.cpu(), yr.sorted_indices)
+    assert torch.equal(y.unsorted_indices.cpu(), yr.unsorted_indices)
+    assert_close32(y.data, yr.data); assert_close32(hn, hr); assert_close32(cn, cr)
+    ((y.data * w.cuda()).sum() + (hn * wh.cuda()).sum()).backward()
+    ((yr.data * w).sum() + (hr * wh).sum()).backward()
+    for n, prm in m.named_parameters():
+        rg = getattr(ref, n).grad
+        assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
+
+
 @pytest.mark.parametrize("T,B,I,H,layers,dt", [(9, 7, 11, 33, 1, torch.float32), (14, 5, 6, 65, 3, torch.float32),
                                                (70, 32, 256, 1024, 2, torch.float16)])   # one launch per pair
 def test_state_gradients_vs_nn_lstm(T, B, I, H, layers, dt):
