@@ -135,6 +135,13 @@ __device__ __forceinline__ void publish_version(int *flag, int version) {
     }
 }
 
+// Unsigned vector type of N bytes, for moving N / sizeof(T) neighbouring elements with one access.
+template <int N> struct VecBytes;
+template <> struct VecBytes<2> { using type = unsigned short; };
+template <> struct VecBytes<4> { using type = unsigned; };
+template <> struct VecBytes<8> { using type = u32x2; };
+template <> struct VecBytes<16> { using type = u32x4; };
+
 // Byte offset of element k of matrix row r inside a run of fragment blocks
 // (block = 64 lanes x 16 B; lane = 16*(lane group) + row).
 template <typename T> __device__ __forceinline__ int frag_offset(int r, int k) {

@@ -144,7 +144,10 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
         for (int idx = tid; idx < total; idx += kThreads) {
             const int row = idx / chunks_per_row, kc = idx % chunks_per_row;
             const int mt = row >> 4, r = row & 15;
-            const int unit = u0 + mt * 4 + (r >> 2), gate = r & 3;
+            // row r of an m-tile is gate r % 4 of the tile's unit r / 4.  One hidden tile per workgroup:
+            // the MT tiles of a wave interleave, so that a lane's MT results are MT consecutive units
+            const int unit = u0 + (SPLIT == 2 ? (mt / MT) * 4 * MT + (r >> 2) * MT + mt % MT : mt * 4 + (r >> 2));
+            const int gate = r & 3;
             const int k0 = kc * E::EPL;
             u32x4 v = {0u, 0u, 0u, 0u};
             if (unit < H && k0 < H) {
@@ -204,16 +207,18 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     bool valid[IPT];
 #pragma unroll
     for (int m = 0; m < IPT; ++m) {
-        const int tl = wave + 4 * m;
+        // SPLIT 2: the item is the lane's own accumulator of the wave's m-tile m (see the weight rows above)
+        const int tl = SPLIT == 2 ? wave * MT + m : wave + 4 * m;
         const int mt = tl / NT, nt = tl % NT;
-        const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
+        const int ul = SPLIT == 2 ? wave * 4 * MT + q * MT + m : mt * 4 + q;   // unit inside the hidden tile
+        const int unit = u0 + ul, b = b0 + nt * 16 + n;
         valid[m] = (tl < TILES) && unit < H && b < B;
         // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
         off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
         off_p[m] = valid[m] ? (size_t)b * 4 * H + unit : (size_t)b0 * 4 * H + u0;
         xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
-        goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
-        soff[m] = (nt * 16 + n) * SROW + (mt * 4 + q) * E::BYTES;
+        goff[m] = (nt * 16 + n) * GROW + ul * E::BYTES;
+        soff[m] = (nt * 16 + n) * SROW + ul * E::BYTES;
         c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
     }
 
@@ -314,11 +319,106 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     }
 
     int slot_r = 0;  // ring slot that holds h_{t-1}
+    if constexpr (SPLIT == 2 && VIO) {   // the gates tile of step 0 (every later one is moved a step ahead)
+        tile_to_lds(gpre[0], tiles);
+        __syncthreads();
+    }
     // One timestep; u = t % PD selects the prefetch ring entry at compile time.
     auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
         const int slot_w = (slot_r + 1 == n_slots) ? 0 : slot_r + 1;
         unsigned char *gt = tiles + (SYNC ? 0 : (t & 1) * TILE_BYTES);
+        if constexpr (SPLIT == 2) {
+            // One hidden tile per workgroup.  A lane's accumulators ARE its items: accumulator m holds the
+            // four gates of unit (first unit of the lane) + m for batch row n, so nothing is reduced and
+            // nothing but h_t crosses waves; the lane moves its MT consecutive units of every tile row
+            // with one LDS access.  One workgroup barrier per step: behind it h_t (operand blocks), this
+            // step's result tiles and the next step's gates tile are all in LDS.
+            using V = typename VecBytes<MT * E::BYTES>::type;
+            const unsigned xb = (unsigned)slot_r * xslot, xn = (unsigned)slot_w * xslot;
+            f32x4 acc[MT];
+            {
+                u32x4 bq[KS2];
+#pragma unroll
+                for (int ks = 0; ks < KS2; ++ks)   // past the end: any valid block (its weights are zero)
+                    bq[ks] = xch.template load16<false>(xb + (unsigned)(min(ks, KS - 1) * kWave + lane) * 16u);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int a = 0; a < MT; ++a) acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                    for (int a = 0; a < MT; ++a) acc[a] = mfma_kstep<T>(w2[a][ks], bq[ks], acc[a]);
+            }
+            T x4[4][MT], st_p[IPT][4], st_h[IPT], st_c[IPT];
+#pragma unroll
+            for (int gg = 0; gg < 4; ++gg) {
+                if constexpr (VIO) {
+                    const V v = *reinterpret_cast<const V *>(gt + goff[0] + gg * GSEG);
+                    __builtin_memcpy(x4[gg], &v, sizeof(V));
+                } else {
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) x4[gg][m] = pre[u][m][gg];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const float pi = E::to_f32(x4[0][m]) + acc[m][0];
+                const float pf = E::to_f32(x4[1][m]) + acc[m][1];
+                const float pg = E::to_f32(x4[2][m]) + acc[m][2];
+                const float po = E::to_f32(x4[3][m]) + acc[m][3];
+                const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
+                const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
+                c_state[m] = c1;
+                // units past H and rows past B stay zero in the operand blocks (their weights are zero,
+                // but 0 x NaN is not)
+                st_h[m] = E::from_f32(valid[m] ? h1 : 0.f);
+                st_p[m][0] = E::from_f32(pi);
+                st_p[m][1] = E::from_f32(pf);
+                st_p[m][2] = E::from_f32(pg);
+                st_p[m][3] = E::from_f32(po);
+                st_c[m] = E::from_f32(c1);
+            }
+            V vh, vc;
+            __builtin_memcpy(&vh, st_h, sizeof(V));
+            __builtin_memcpy(&vc, st_c, sizeof(V));
+            *reinterpret_cast<V *>(xl + xn + xoff[0]) = vh;
+            if constexpr (VIO) {
+#pragma unroll
+                for (int gg = 0; gg < 4; ++gg) {
+                    T pk[MT];
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) pk[m] = st_p[m][gg];
+                    V vp;
+                    __builtin_memcpy(&vp, pk, sizeof(V));
+                    *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = vp;
+                }
+                *reinterpret_cast<V *>(gt + BT * GROW + soff[0]) = vh;
+                *reinterpret_cast<V *>(gt + BT * GROW + BT * SROW + soff[0]) = vc;
+                if (t + 1 < T_) tile_to_lds(gpre[(u + 1) % PD], tiles + ((t + 1) & 1) * TILE_BYTES);
+                __syncthreads();
+                tiles_to_global(t, gt);
+            } else {
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    if (valid[m]) {
+                        if (keep) {
+                            T *dst = ifgo + (size_t)t * B4H + off_p[m];
+                            dst[0] = st_p[m][0];
+                            dst[(size_t)H] = st_p[m][1];
+                            dst[(size_t)2 * H] = st_p[m][2];
+                            dst[(size_t)3 * H] = st_p[m][3];
+                        }
+                        out[(size_t)(t + 1) * BH + off_h[m]] = st_h[m];
+                        if (keep || t + 1 == T_) cell[(size_t)(t + 1) * BH + off_h[m]] = st_c[m];
+                    }
+                }
+                __syncthreads();
+            }
+            prefetch(t + PD, uc);
+            slot_r = slot_w;
+            return;
+        }
         long long tr0 = 0, tr1 = 0, tr2 = 0, tr3 = 0;
         if (p.trace) tr0 = (long long)wall_clock64();
         FASTLSTM_TP(0);
