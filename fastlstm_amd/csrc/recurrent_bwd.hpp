@@ -156,9 +156,11 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 #pragma unroll
     for (int m = 0; m < IPT; ++m) {
+        // SPLIT 2: the item is element m of the lane's own accumulator -- unit 4 * (lane / 16) + m of the
+        // wave's unit tile, batch row lane % 16 -- so the product of a step lands where it is used
         const int it = tid + kThreads * m;
-        const int n = it & 15, rest = it >> 4;
-        const int ul = rest % HT, nt = rest / HT;
+        const int n = SPLIT == 2 ? (lane & 15) : (it & 15), rest = it >> 4;
+        const int ul = SPLIT == 2 ? wave * 16 + (lane >> 4) * 4 + m : rest % HT, nt = SPLIT == 2 ? 0 : rest / HT;
         const int unit = u0 + ul, b = b0 + nt * 16 + n;
         valid[m] = nt < NT && unit < H && b < B;
         // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
@@ -289,6 +291,114 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         if (p.trace) tr0 = (long long)wall_clock64();
         unsigned char *gt = tiles + (SYNC ? 0 : (s & 1) * TILE_BYTES);         // VIO: this step's tiles
         unsigned char *gt_next = tiles + (SYNC ? 0 : ((s + 1) & 1) * TILE_BYTES);
+        if constexpr (SPLIT == 2) {
+            // One hidden tile per workgroup.  The lane's four items are four consecutive units of one batch
+            // row: every tile row is touched with one LDS access per gate, the lane writes whole operand
+            // slots of the exchange copy, and the product comes back in the lane's own accumulator (nothing
+            // is reduced).  One workgroup barrier per step: behind it the exchange copy, the d_ifgo tile
+            // and the next step's input tiles are all in LDS.
+            using V = typename VecBytes<4 * E::BYTES>::type;
+            constexpr int un_ = (u + 1) % PD;
+            T xg[4][4], xc[4], xd[4], st_d[4][4];
+            if constexpr (VIO) {
+#pragma unroll
+                for (int gg = 0; gg < 4; ++gg) {
+                    const V v = *reinterpret_cast<const V *>(gt + goff[0] + gg * GSEG);
+                    __builtin_memcpy(xg[gg], &v, sizeof(V));
+                }
+                const V vc = *reinterpret_cast<const V *>(gt + BT * GROW + soff[0]);
+                const V vd = *reinterpret_cast<const V *>(gt + BT * GROW + BT * SROW + soff[0]);
+                __builtin_memcpy(xc, &vc, sizeof(V));
+                __builtin_memcpy(xd, &vd, sizeof(V));
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) xg[gg][m] = pre[u][m][gg];
+                    xc[m] = c0r[u][m];
+                    xd[m] = dor[u][m];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float si = sigmoidf_<ACC>(E::to_f32(xg[0][m]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(xg[1][m]));
+                const float tg = tanhf_<ACC>(E::to_f32(xg[2][m]));
+                const float so = sigmoidf_<ACC>(E::to_f32(xg[3][m]));
+                const float tc = tanhf_<ACC>(c1v[m]);
+                const float c0 = E::to_f32(xc[m]);
+                const float dh = dh_rec[m] + E::to_f32(xd[m]);
+                const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
+                const float d_o = dh * tc * so * (1.f - so);
+                const float d_f = dc1 * c0 * sf * (1.f - sf);
+                const float d_i = dc1 * tg * si * (1.f - si);
+                const float d_g = dc1 * si * (1.f - tg * tg);
+                dc_state[m] = dc1 * sf;
+                c1v[m] = c0;  // c_{t-1} is the next step's c_t
+                // items past H or B: zeros (they are operands of the product below)
+                st_d[m][0] = E::from_f32(valid[m] ? d_i : 0.f);
+                st_d[m][1] = E::from_f32(valid[m] ? d_f : 0.f);
+                st_d[m][2] = E::from_f32(valid[m] ? d_g : 0.f);
+                st_d[m][3] = E::from_f32(valid[m] ? d_o : 0.f);
+            }
+            // exchange copy: k = 4 * unit + gate, whole 16-byte operand slots (two units of a 16-bit
+            // type, one of fp32); slots past 4H do not exist in the blocks and are left alone
+            if constexpr (E::BYTES == 2) {
+#pragma unroll
+                for (int m = 0; m < 4; m += 2)
+                    if (valid[m]) {
+                        u32x4 v;
+                        __builtin_memcpy(&v, st_d[m], 16);
+                        xch.store16(xw + xoff[m], v);
+                    }
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    if (valid[m]) {
+                        u32x4 v;
+                        __builtin_memcpy(&v, st_d[m], 16);
+                        xch.store16(xw + xoff[m], v);
+                    }
+            }
+            if constexpr (VIO) {
+#pragma unroll
+                for (int gg = 0; gg < 4; ++gg) {
+                    T pk[4];
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) pk[m] = st_d[m][gg];
+                    V v;
+                    __builtin_memcpy(&v, pk, sizeof(V));
+                    *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = v;
+                }
+                if (s + 1 < T_) tiles_to_lds(gpre[un_], cpre[un_], dpre[un_], gt_next);
+                __syncthreads();
+                tile_to_global(t, gt);
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    if (valid[m]) {
+                        T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
+                        dst[0] = st_d[m][0];
+                        dst[(size_t)H] = st_d[m][1];
+                        dst[(size_t)2 * H] = st_d[m][2];
+                        dst[(size_t)3 * H] = st_d[m][3];
+                    }
+                __syncthreads();
+            }
+            prefetch(s + PD, uc);
+            // dh_rec(units of this wave, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over K = 4H
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+            u32x4 bq[KSB2];
+#pragma unroll
+            for (int ks = 0; ks < KSB2; ++ks)   // past the end: any valid block (its weights are zero)
+                bq[ks] = xch.template load16<false>(xw + (unsigned)(min(ks, KSB - 1) * kWave + lane) * 16u);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KSB2; ++ks) acc = mfma_kstep<T>(wb2[ks], bq[ks], acc);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) dh_rec[m] = acc[m];
+            return;
+        }
         // ---- point-wise gate backward for this thread's items --------------------------
         T st_d[IPT][4];
 #pragma unroll
