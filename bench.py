@@ -272,6 +272,20 @@ def main():
                         + ("through the L2 of one XCD" if xcd_local else "through device memory")
                         + "; us/step of the recurrence alone is in kernels.recurrent_fwd_us_per_step"}
 
+    if plan_f.wave_split == 2:
+        # one hidden tile per workgroup (H <= 64): no exchange between CUs at all; the kernel streams the
+        # gate tiles through (read + write-back) and writes out / cell -- priced against HBM
+        sz = 2 if dname != "fp32" else 4
+        nbytes = sz * (2.0 * T * B * 4 * H + 2.0 * T * B * H + 4.0 * H * H)
+        ach = nbytes / (t_rec * 1e-3) / 1e9
+        roofline = {"kernel": "lstm_fwd_persistent_kernel<SPLIT=2> (one hidden tile per workgroup)", "bound": "hbm",
+                    "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                    "traffic": None,
+                    "algorithmic": "s*(2*T*B*4H + 2*T*B*H + 4H*H) bytes per launch = %.1f MB" % (nbytes / 1e6),
+                    "launch_ms": round(t_rec, 4),
+                    "note": "latency-bound, not HBM-bound: %d independent workgroups (16 batch rows each) walk through "
+                            "T sequential steps; us/step is in kernels.recurrent_fwd_us_per_step" % plan_f.n_btiles}
+
     res = {
         "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),

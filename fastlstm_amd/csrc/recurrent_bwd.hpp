@@ -550,23 +550,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 }
             }
         };
-        // one hidden tile per workgroup (SPLIT == 2, H <= 64): the wave's unit tile x all k-steps comes
-        // from registers and the (at most KSB2) operand blocks are requested at once
-        auto kloop_single = [&]() {
-            u32x4 bq[KSB2][NTW];
-#pragma unroll
-            for (int ks = 0; ks < KSB2; ++ks)
-#pragma unroll
-                for (int i = 0; i < NTW; ++i)   // past the end: any valid block (its weights are zero)
-                    bq[ks][i] = xch.template load16<false>(xb + (unsigned)((i * KSB + min(ks, KSB - 1)) * kWave + lane) * 16u);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int ks = 0; ks < KSB2; ++ks)
-#pragma unroll
-                for (int i = 0; i < NTW; ++i) acc[i] = mfma_kstep<T>(wb2[SPLIT == 2 ? ks : 0], bq[ks][i], acc[i]);
-        };
-        if constexpr (SPLIT == 2) kloop_single();
-        else if (coherent) kloop(std::true_type{});
+        if (coherent) kloop(std::true_type{});
         else kloop(std::false_type{});
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {

@@ -506,25 +506,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
                     for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
         };
-        // one hidden tile per workgroup: weights in registers, the (at most KS2) operand blocks at once
-        auto kloop_single = [&]() {
-            u32x4 bq[KS2][NTW];
-#pragma unroll
-            for (int ks = 0; ks < KS2; ++ks)
-#pragma unroll
-                for (int i = 0; i < NTW; ++i)   // past the end: any valid block (its weights are zero)
-                    bq[ks][i] = xch.template load16<false>(xb + (unsigned)((i * KS + min(ks, KS - 1)) * kWave + lane) * 16u);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int ks = 0; ks < KS2; ++ks)
-#pragma unroll
-                for (int a = 0; a < (SPLIT == 2 ? MT : 0); ++a)
-#pragma unroll
-                    for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(w2[a][ks], bq[ks][i], acc[a][i]);
-        };
-        if constexpr (SPLIT == 2) {
-            kloop_single();
-        } else if constexpr (WREG) {
+        if constexpr (WREG) {
             if (coherent) kloop_wreg(std::true_type{});
             else kloop_wreg(std::false_type{});
         } else {
