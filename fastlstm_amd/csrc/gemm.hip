@@ -24,7 +24,7 @@ hipError_t launch_gemm_t(const GemmParams &p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (p.splits > 1) {
         const size_t total = (size_t)p.M * p.N;
-        const int blocks = (int)std::min<size_t>((total + 255) / 256, 4096);
+        const int blocks = (int)((total + 63) / 64);   // 64 outputs per block
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, p.Cpart,
                            static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits);
         e = hipGetLastError();
@@ -49,7 +49,7 @@ hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (p.splits > 1) {
         const size_t total = (size_t)p.M * p.N;
-        const int blocks = (int)std::min<size_t>((total + 255) / 256, 4096);
+        const int blocks = (int)((total + 63) / 64);   // 64 outputs per block
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, p.Cpart,
                            static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits);
         e = hipGetLastError();
@@ -76,14 +76,22 @@ template <typename T>
 hipError_t launch_colsum_t(const void *in, void *out, float *part, int R, int C, int chunks, hipStream_t s) {
     using E = Elem<T>;
     const int rpc = cdiv(R, chunks);
+    // column groups per block: the power of two that covers the columns, at most the whole block
+    auto col_threads = [](int groups) {
+        int ct = 1;
+        while (ct < 128 && ct < groups) ct *= 2;
+        return ct;
+    };
     if (C % E::EPL == 0) {
-        dim3 grid(cdiv(C, 128 * E::EPL), chunks);
+        const int ct = col_threads(C / E::EPL);
+        dim3 grid(cdiv(C, ct * E::EPL), chunks);
         hipLaunchKernelGGL((colsum_partial_kernel<T, E::EPL>), grid, dim3(128), 0, s,
-                           static_cast<const T *>(in), part, R, C, rpc);
+                           static_cast<const T *>(in), part, R, C, rpc, ct);
     } else {
-        dim3 grid(cdiv(C, 128), chunks);
+        const int ct = col_threads(C);
+        dim3 grid(cdiv(C, ct), chunks);
         hipLaunchKernelGGL((colsum_partial_kernel<T, 1>), grid, dim3(128), 0, s, static_cast<const T *>(in),
-                           part, R, C, rpc);
+                           part, R, C, rpc, ct);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

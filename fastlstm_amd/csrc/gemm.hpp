@@ -219,31 +219,52 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 // C[m][n] = sum_s part[s][m][n]  (deterministic split-K finish), cast to T.
 template <typename T>
 __global__ void splitk_reduce_kernel(const float *part, T *C, int M, int N, int ldc, int splits) {
+    // 256 threads = 64 outputs x 4 slices of the splits (k = slice, slice + 4, ...), eight loads in
+    // flight per thread, combined through LDS in a fixed order
+    __shared__ float red[4][64];
     const size_t total = (size_t)M * N;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        float s = 0.f;
-        for (int k = 0; k < splits; ++k) s += part[(size_t)k * total + i];
-        C[(i / N) * ldc + (i % N)] = Elem<T>::from_f32(s);
+    const int ol = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const size_t i = (size_t)blockIdx.x * 64 + ol;
+    float s = 0.f;
+    if (i < total) {
+        int k = slice;
+        for (; k + 28 < splits; k += 32) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(k + 4 * u) * total + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; k < splits; k += 4) s += part[(size_t)k * total + i];
     }
+    red[slice][ol] = s;
+    __syncthreads();
+    if (slice == 0 && i < total)
+        C[(i / N) * ldc + (i % N)] = Elem<T>::from_f32((red[0][ol] + red[1][ol]) + (red[2][ol] + red[3][ol]));
 }
 
 // Column sums of in[R][C] (db = sum over time and batch of d_ifgo, lstm.py:497), two
 // deterministic stages: part[chunk][C] in fp32, then the sum over chunks.
 template <typename T, int VEC>
-__global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, int rows_per_chunk) {
-    const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-    if (c0 >= C) return;
+__global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, int rows_per_chunk, int col_threads) {
+    // 128 threads = col_threads column groups (VEC columns each) x 128 / col_threads row lanes: a narrow
+    // matrix still fills the block; row lane y takes rows r0 + y, r0 + y + lanes, ... of the chunk and the
+    // lanes are summed through LDS in a fixed order
+    __shared__ float red[128][VEC];
+    const int tx = threadIdx.x % col_threads, ty = threadIdx.x / col_threads, lanes = 128 / col_threads;
+    const int c0 = (blockIdx.x * col_threads + tx) * VEC;
+    const bool live = c0 < C;
     const int r0 = blockIdx.y * rows_per_chunk, r1 = min(R, r0 + rows_per_chunk);
     float s[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) s[e] = 0.f;
     constexpr int U = 8;   // rows in flight per thread: the kernel is a pure HBM stream
-    int rr = r0;
+    int rr = r0 + ty;
     if constexpr (VEC > 1) {
-        for (; rr + U <= r1; rr += U) {
+        for (; live && rr + (U - 1) * lanes < r1; rr += U * lanes) {
             u32x4 v[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const u32x4 *>(in + (size_t)(rr + u) * C + c0);
+            for (int u = 0; u < U; ++u) v[u] = *reinterpret_cast<const u32x4 *>(in + (size_t)(rr + u * lanes) * C + c0);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const T *tv = reinterpret_cast<const T *>(&v[u]);
@@ -252,7 +273,7 @@ __global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, in
             }
         }
     }
-    for (; rr < r1; ++rr) {
+    for (; live && rr < r1; rr += lanes) {
         const T *src = in + (size_t)rr * C + c0;
         if constexpr (VEC == 1) {
             s[0] += Elem<T>::to_f32(src[0]);
@@ -263,8 +284,18 @@ __global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, in
             for (int e = 0; e < VEC; ++e) s[e] += Elem<T>::to_f32(tv[e]);
         }
     }
+    if (lanes > 1) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) part[(size_t)blockIdx.y * C + c0 + e] = s[e];
+        for (int e = 0; e < VEC; ++e) red[threadIdx.x][e] = s[e];
+        __syncthreads();
+        if (ty == 0)
+            for (int y = 1; y < lanes; ++y)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s[e] += red[y * col_threads + tx][e];
+    }
+    if (live && ty == 0)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) part[(size_t)blockIdx.y * C + c0 + e] = s[e];
 }
 
 // out[c] = sum over chunks of part[chunk][c].  A block of 256 threads covers 64 columns with 4
