@@ -197,11 +197,11 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
     const int n_helpers = kNumXcd * 32 - layers * c.n_groups * c.n_ht;
     if (n_helpers < kNumXcd * 8) return false;
-    const int max_chunks = second ? 20 : 32;   // counters in the workspace header: 60 ints
+    const int max_chunks = kMaxChunks;
     const int M = T * B, N = 4 * H;
     if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
-    // a chunk: whole timesteps, about one round of the helpers, at most 32 chunks
+    // a chunk: whole timesteps, about one round of the helpers, at most kMaxChunks chunks
     int base = 1;
     while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
     int ct = std::max(1, n_helpers / tiles_n / base) * base;
@@ -219,8 +219,8 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
         p->k1b.M = M; p->k1b.N = N; p->k1b.K = H;
         p->k1b.lda = H; p->k1b.ldb = H; p->k1b.ldc = N;
         p->k1b.splits = 1; p->k1b.k_per_split = H;
-        p->k1_done2 = p->hdr->reserved + 20;
-        p->out_ready = p->hdr->reserved + 40;
+        p->k1_done2 = ws_chunk_counters(p->hdr, 1);
+        p->out_ready = ws_chunk_counters(p->hdr, 2);
     }
     p->k1 = GemmParams{};
     p->k1.A = x; p->k1.B = Wx; p->k1.C = ifgo; p->k1.bias0 = bx; p->k1.bias1 = bh;
@@ -229,7 +229,7 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     p->k1.splits = 1; p->k1.k_per_split = I;
     p->k1_tiles_m = tiles_m; p->k1_tiles_n = tiles_n;
     p->k1_chunk_tiles = ct; p->k1_chunk_steps = steps;
-    p->k1_done = p->hdr->reserved;
+    p->k1_done = ws_chunk_counters(p->hdr, 0);
     return true;
 }
 
@@ -378,11 +378,11 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
     const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - layers * n_active;
     if (n_helpers < kNumXcd * 8) return false;
-    const int max_chunks = lower ? 20 : 32;   // counters in the workspace header: 60 ints
+    const int max_chunks = kMaxChunks;
     const int I = e.I, M = T * B, K = 4 * H;
     if (!gemm16_eligible(dtype, M, I, K, K, I, false, true) || I % 8) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(I, 256);
-    // a chunk: whole timesteps, about 8 row tiles (a short tail behind the recurrence), at most 32 chunks
+    // a chunk: whole timesteps, about 8 row tiles (a short tail behind the recurrence), at most kMaxChunks chunks
     int base = 1;
     while ((base * 256) % B) ++base;
     int ct = base >= 8 ? base : (8 / base) * base;
@@ -401,8 +401,8 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
             p->k5_lo.splits = 1; p->k5_lo.k_per_split = K;
         }
         p->k5_lo_tiles_n = cdiv(lower->I, 256);
-        p->chunk_done_lo = p->hdr->reserved + 20;
-        p->dx_done = p->hdr->reserved + 40;
+        p->chunk_done_lo = ws_chunk_counters(p->hdr, 1);
+        p->dx_done = ws_chunk_counters(p->hdr, 2);
     }
     p->k5 = GemmParams{};
     p->k5.A = d_ifgo; p->k5.B = e.Wx; p->k5.C = e.dx;
@@ -412,7 +412,7 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     p->k5_tiles_m = tiles_m; p->k5_tiles_n = tiles_n;
     p->k5_chunk_tiles = ct; p->k5_chunk_steps = ct * 256 / B; p->k5_chunks = cdiv(tiles_m, ct);
     p->n_active = n_active;
-    p->chunk_done = p->hdr->reserved;
+    p->chunk_done = ws_chunk_counters(p->hdr, 0);
     p->wg_tiles = 0;
     if (e.dWx && gemm16_eligible(dtype, K, I, M, K, I, true, true) && gemm16_eligible(dtype, K, H, M, K, H, true, true) &&
         H % 8 == 0) {

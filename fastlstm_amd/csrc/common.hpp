@@ -120,9 +120,15 @@ struct WsHeader {
 };
 static_assert(sizeof(WsHeader) == 256, "workspace header is 256 bytes");
 
+// Chunk counters of the launches that run GEMM tiles next to a recurrence: three arrays of
+// kMaxChunks device-scope counters behind the WsHeader, inside the 1 KiB header block (zero at launch).
+constexpr int kMaxChunks = 64;
+inline int *ws_chunk_counters(WsHeader *hdr, int which) { return reinterpret_cast<int *>(hdr + 1) + which * kMaxChunks; }
+
 // Recurrence workspace: header block (1 KiB, WsHeader in front) | 64 KiB of L2 barrier counters of
 // the XCD-local kernels (plans with a cross-CU barrier only) | flags | exchange slots.
 constexpr size_t kWsHeaderBytes = 1024;
+static_assert(sizeof(WsHeader) + 3 * kMaxChunks * sizeof(int) <= kWsHeaderBytes, "chunk counters fit the header block");
 constexpr size_t kWsCounterBytes = 65536;
 
 long long spin_limit_ticks();

@@ -45,7 +45,7 @@ struct BwdXcdParams {
     GemmParams k8, k9;  // M = 4H, N = I | H, K = T*B, A = d_ifgo (K-major), B = x | h (K-major), C = dWx | dWh
     int k8_tiles_n, k9_tiles_n, wg_tiles_m, wg_tiles;
     int n_active;       // workgroups of one layer's recurrence
-    int *chunk_done;    // [<= 32] device-scope counters, zero at launch
+    int *chunk_done;    // [<= kMaxChunks] device-scope counters, zero at launch
     // Two stacked layers in one launch (n_layers == 2, HELP instantiations).  The fields above describe
     // the UPPER layer, whose groups come first in the group numbering.  The lower layer's recurrence
     // reads the upper layer's dx (k5.C) as its dout: the helpers write it chunk by chunk, latest
@@ -60,8 +60,8 @@ struct BwdXcdParams {
     const void *Wh_lo;
     GemmParams k5_lo;   // M = T*B, N = I of the lower layer, K = 4H, A = d_ifgo_lo, B = Wx_lo (K-major), C = dx_lo
     int k5_lo_tiles_n;
-    int *chunk_done_lo; // [<= 20]
-    int *dx_done;       // [<= 20]
+    int *chunk_done_lo; // [<= kMaxChunks]
+    int *dx_done;       // [<= kMaxChunks]
     float *wg_scratch;  // stacked launches: 256 KiB per helper that owns a weight-gradient tile
     long long spin_limit;
 };

@@ -53,7 +53,7 @@ struct FwdXcdParams {
     GemmParams k1;        // M = T*B, N = 4H, K = I, A = x, B = Wx, C = ifgo, biases
     int k1_tiles_m, k1_tiles_n;
     int k1_chunk_tiles, k1_chunk_steps;
-    int *k1_done;         // [<= 32] device-scope counters, zero at launch
+    int *k1_done;         // [<= kMaxChunks] device-scope counters, zero at launch
     // Two stacked layers in one launch (n_layers == 2, HELP instantiations): the second layer's barrier
     // groups follow the first layer's in the group numbering (so they sit on other XCDs or CUs), its
     // input projection reads the first layer's out[1:] chunk by chunk as that layer produces it
@@ -64,7 +64,7 @@ struct FwdXcdParams {
     const void *Wh2;
     GemmParams k1b;       // M = T*B, N = 4H, K = H, A = out[1:] of the first layer, B = Wx2, C = ifgo2, biases
     int *k1_done2;        // chunk counters of the second projection
-    int *out_ready;       // [<= 20] device-scope counters, zero at launch
+    int *out_ready;       // [<= kMaxChunks] device-scope counters, zero at launch
     int n_active;         // workgroups of one layer's recurrence (groups * members)
     int keep;             // 1: store pre-activations and every cell state (training); 0: inference, only cell[T]
     long long spin_limit;
