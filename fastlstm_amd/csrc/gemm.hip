@@ -24,9 +24,10 @@ hipError_t launch_gemm_t(const GemmParams &p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (p.splits > 1) {
         const size_t total = (size_t)p.M * p.N;
-        const int blocks = (int)((total + 63) / 64);   // 64 outputs per block
+        const int slices = p.splits >= 16 ? 4 : 1;     // many splits: four threads per output
+        const int blocks = (int)((total * slices + 255) / 256);
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, p.Cpart,
-                           static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits);
+                           static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits, slices);
         e = hipGetLastError();
     }
     return e;
@@ -49,9 +50,10 @@ hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (p.splits > 1) {
         const size_t total = (size_t)p.M * p.N;
-        const int blocks = (int)((total + 63) / 64);   // 64 outputs per block
+        const int slices = p.splits >= 16 ? 4 : 1;     // many splits: four threads per output
+        const int blocks = (int)((total * slices + 255) / 256);
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, p.Cpart,
-                           static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits);
+                           static_cast<T *>(p.C), p.M, p.N, p.ldc, p.splits, slices);
         e = hipGetLastError();
     }
     return e;

@@ -218,29 +218,34 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmParams p) {
 
 // C[m][n] = sum_s part[s][m][n]  (deterministic split-K finish), cast to T.
 template <typename T>
-__global__ void splitk_reduce_kernel(const float *part, T *C, int M, int N, int ldc, int splits) {
-    // 256 threads = 64 outputs x 4 slices of the splits (k = slice, slice + 4, ...), eight loads in
-    // flight per thread, combined through LDS in a fixed order
+__global__ void splitk_reduce_kernel(const float *part, T *C, int M, int N, int ldc, int splits, int slices) {
+    // 256 threads = 256 / slices outputs x slices (1 or 4) of the splits (k = slice, slice + slices, ...),
+    // eight loads in flight per thread; four slices (many splits, few outputs) are combined through LDS in a
+    // fixed order
     __shared__ float red[4][64];
     const size_t total = (size_t)M * N;
-    const int ol = threadIdx.x & 63, slice = threadIdx.x >> 6;
-    const size_t i = (size_t)blockIdx.x * 64 + ol;
+    const int per_block = 256 / slices;
+    const int ol = threadIdx.x % per_block, slice = threadIdx.x / per_block;
+    const size_t i = (size_t)blockIdx.x * per_block + ol;
     float s = 0.f;
     if (i < total) {
         int k = slice;
-        for (; k + 28 < splits; k += 32) {
+        for (; k + 7 * slices < splits; k += 8 * slices) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(k + 4 * u) * total + i];
+            for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(k + slices * u) * total + i];
 #pragma unroll
             for (int u = 0; u < 8; ++u) s += v[u];
         }
-        for (; k < splits; k += 4) s += part[(size_t)k * total + i];
+        for (; k < splits; k += slices) s += part[(size_t)k * total + i];
     }
-    red[slice][ol] = s;
-    __syncthreads();
-    if (slice == 0 && i < total)
-        C[(i / N) * ldc + (i % N)] = Elem<T>::from_f32((red[0][ol] + red[1][ol]) + (red[2][ol] + red[3][ol]));
+    if (slices == 4) {
+        red[slice][ol] = s;
+        __syncthreads();
+        s = (red[0][ol] + red[1][ol]) + (red[2][ol] + red[3][ol]);
+        if (slice != 0) return;
+    }
+    if (i < total) C[(i / N) * ldc + (i % N)] = Elem<T>::from_f32(s);
 }
 
 // Column sums of in[R][C] (db = sum over time and batch of d_ifgo, lstm.py:497), two
