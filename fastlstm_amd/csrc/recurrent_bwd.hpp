@@ -280,6 +280,17 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     }
 
     int slot = 0;  // ring slot of this step's d_ifgo
+    // One hidden tile per workgroup: the lane's four units of the current step's tile rows (4 gates,
+    // c_{t-1}, dout), read a step ahead
+    using NxV = typename VecBytes<4 * E::BYTES>::type;
+    NxV nx[6];
+    auto load_items = [&](const unsigned char *gt_) __attribute__((always_inline)) {
+#pragma unroll
+        for (int gg = 0; gg < 4; ++gg) nx[gg] = *reinterpret_cast<const NxV *>(gt_ + goff[0] + gg * GSEG);
+        nx[4] = *reinterpret_cast<const NxV *>(gt_ + BT * GROW + soff[0]);
+        nx[5] = *reinterpret_cast<const NxV *>(gt_ + BT * GROW + BT * SROW + soff[0]);
+    };
+    if constexpr (SPLIT == 2 && VIO) load_items(tiles);
     // One reverse step; u = s % PD selects the prefetch ring entry at compile time.
     auto step = [&](const int s, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
@@ -300,16 +311,11 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
             using V = typename VecBytes<4 * E::BYTES>::type;
             constexpr int un_ = (u + 1) % PD;
             T xg[4][4], xc[4], xd[4], st_d[4][4];
-            if constexpr (VIO) {
+            if constexpr (VIO) {   // read behind the previous step's barrier (or in the prologue)
 #pragma unroll
-                for (int gg = 0; gg < 4; ++gg) {
-                    const V v = *reinterpret_cast<const V *>(gt + goff[0] + gg * GSEG);
-                    __builtin_memcpy(xg[gg], &v, sizeof(V));
-                }
-                const V vc = *reinterpret_cast<const V *>(gt + BT * GROW + soff[0]);
-                const V vd = *reinterpret_cast<const V *>(gt + BT * GROW + BT * SROW + soff[0]);
-                __builtin_memcpy(xc, &vc, sizeof(V));
-                __builtin_memcpy(xd, &vd, sizeof(V));
+                for (int gg = 0; gg < 4; ++gg) __builtin_memcpy(xg[gg], &nx[gg], 4 * E::BYTES);
+                __builtin_memcpy(xc, &nx[4], 4 * E::BYTES);
+                __builtin_memcpy(xd, &nx[5], 4 * E::BYTES);
             } else {
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
@@ -392,6 +398,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
 #pragma unroll
             for (int ks = 0; ks < KSB2; ++ks)   // past the end: any valid block (its weights are zero)
                 bq[ks] = xch.template load16<false>(xw + (unsigned)(min(ks, KSB - 1) * kWave + lane) * 16u);
+            if constexpr (VIO) {   // the next step's tile rows (in LDS since the barrier above)
+                if (s + 1 < T_) load_items(gt_next);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < KSB2; ++ks) acc = mfma_kstep<T>(wb2[ks], bq[ks], acc);

@@ -337,11 +337,16 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
             using V = typename VecBytes<MT * E::BYTES>::type;
             const unsigned xb = (unsigned)slot_r * xslot, xn = (unsigned)slot_w * xslot;
             f32x4 acc[MT];
+            V xv[4];
             {
                 u32x4 bq[KS2];
 #pragma unroll
                 for (int ks = 0; ks < KS2; ++ks)   // past the end: any valid block (its weights are zero)
                     bq[ks] = xch.template load16<false>(xb + (unsigned)(min(ks, KS - 1) * kWave + lane) * 16u);
+                if constexpr (VIO) {   // the lane's gates of this step: requested with the operand blocks
+#pragma unroll
+                    for (int gg = 0; gg < 4; ++gg) xv[gg] = *reinterpret_cast<const V *>(gt + goff[0] + gg * GSEG);
+                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int a = 0; a < MT; ++a) acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -354,8 +359,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
             for (int gg = 0; gg < 4; ++gg) {
                 if constexpr (VIO) {
-                    const V v = *reinterpret_cast<const V *>(gt + goff[0] + gg * GSEG);
-                    __builtin_memcpy(x4[gg], &v, sizeof(V));
+                    __builtin_memcpy(x4[gg], &xv[gg], sizeof(V));
                 } else {
 #pragma unroll
                     for (int m = 0; m < MT; ++m) x4[gg][m] = pre[u][m][gg];
