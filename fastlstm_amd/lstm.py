@@ -84,7 +84,8 @@ def _workspace(plan, T, H, code, backward, device):
 
 
 def _check_ws(ws, what):
-    if CHECK_STATUS:
+    # (reading the status word synchronises: not while the stream is being captured into a graph)
+    if CHECK_STATUS and not torch.cuda.is_current_stream_capturing():
         head = ws[:64].cpu().numpy().tobytes()  # synchronises
         _lib.check(_lib.load().fastlstm_ws_status(head), what)
 

@@ -1001,6 +1001,39 @@ def test_module_without_grad_takes_the_inference_path_same_bits(kw, T, B, I, H, 
     assert calls and all(calls) and y4.requires_grad
 
 
+@pytest.mark.parametrize("T,B,I,H,layers,dt", [(32, 64, 256, 1024, 1, torch.float16),   # XCD-local, projection in the launch
+                                               (40, 32, 128, 1024, 2, torch.float16),   # two layers in one launch
+                                               (16, 20, 24, 64, 1, torch.float16),      # one hidden tile per workgroup
+                                               (8, 16, 32, 256, 1, torch.float32)])
+def test_forward_replays_from_a_captured_graph(T, B, I, H, layers, dt):
+    """The module's forward captured into a HIP graph (the reference builds its version="graph" on
+    torch.cuda.graph too, fastlstm/lstm.py:149-233, one kernel node per timestep): every replay, with new input contents and other work on the device in
+    between, gives the eager result bit for bit.  The launches clear their workspaces with fill
+    kernels, never with memset nodes."""
+    torch.manual_seed(0)
+    m = FastLSTM(I, H, num_layers=layers).to("cuda", dt)
+    xs = [torch.randn(T, B, I, device="cuda").to(dt) for _ in range(3)]
+    static_x = xs[0].clone()
+    with torch.no_grad():
+        eager = [m(x)[0].clone() for x in xs]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                m(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y, _ = m(static_x)
+        for rep in range(2):
+            for i, x in enumerate(xs):
+                static_x.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(y, eager[i]), (rep, i)
+                (torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")).sum().item()
+
+
 # --------------------------------------------------------------------------------------
 # 4. BASELINE.json configurations at their real shapes
 # --------------------------------------------------------------------------------------
