@@ -368,11 +368,15 @@ struct LowerLayer {
     int I;
     void *scratch;          // device memory for the parked fp32 weight-gradient tiles (the wgrad workspace)
     size_t scratch_bytes;
+    const void *x, *h;      // the lower layer's input and its out (for its weight gradients; may be null)
+    void *dWx, *dWh;
 };
 
 bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, int T, int B, int H, int dtype,
-                      BwdXcdParams *p, bool *wgrad_fused, const LowerLayer *lower = nullptr) {
+                      BwdXcdParams *p, bool *wgrad_fused, const LowerLayer *lower = nullptr,
+                      bool *lower_wgrad_fused = nullptr) {
     *wgrad_fused = false;
+    if (lower_wgrad_fused) *lower_wgrad_fused = false;
     if (dtype == FASTLSTM_FP32 || !((c.mt == 2 && c.nkw == 16) || (c.mt == 1 && c.nkw == 8))) return false;
     const int layers = lower ? 2 : 1;
     if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
@@ -426,9 +430,26 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
         *wgrad_fused = true;
         if (lower) {   // the stacked helpers park their accumulators between chunks
             p->wg_scratch = static_cast<float *>(lower->scratch);
-            if ((size_t)std::min(p->wg_tiles, n_helpers) * 256 * 256 * sizeof(float) > lower->scratch_bytes) {
+            const size_t tile_bytes = (size_t)256 * 256 * sizeof(float);
+            const size_t upper_bytes = (size_t)std::min(p->wg_tiles, n_helpers) * tile_bytes;
+            if (upper_bytes > lower->scratch_bytes) {
                 p->wg_tiles = 0;
                 *wgrad_fused = false;
+            } else if (lower->dWx && lower->dWh && lower->x && lower->h && lower_wgrad_fused &&
+                       gemm16_eligible(dtype, K, lower->I, M, K, lower->I, true, true) && lower->I % 8 == 0) {
+                // the lower layer's weight gradients the same way, its tiles parked behind the upper layer's
+                GemmParams lo{};
+                lo.A = lower->d_ifgo; lo.M = K; lo.K = M; lo.lda = K; lo.splits = 1; lo.k_per_split = M;
+                p->k8_lo = lo; p->k8_lo.B = lower->x; p->k8_lo.C = lower->dWx; p->k8_lo.N = lower->I;
+                p->k8_lo.ldb = lower->I; p->k8_lo.ldc = lower->I;
+                p->k9_lo = lo; p->k9_lo.B = lower->h; p->k9_lo.C = lower->dWh; p->k9_lo.N = H; p->k9_lo.ldb = H; p->k9_lo.ldc = H;
+                p->k8_lo_tiles_n = cdiv(lower->I, 256);
+                const int lo_tiles = p->wg_tiles_m * (p->k8_lo_tiles_n + p->k9_tiles_n);
+                if (upper_bytes + (size_t)std::min(lo_tiles, n_helpers) * tile_bytes <= lower->scratch_bytes) {
+                    p->wg_lo_tiles = lo_tiles;
+                    p->wg_scratch_lo = p->wg_scratch + upper_bytes / sizeof(float);
+                    *lower_wgrad_fused = true;
+                }
             }
         }
     }
@@ -440,7 +461,8 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
 // to be computed.
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
-                const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false) {
+                const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false,
+                bool *lower_wgrad_fused = nullptr) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
     if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * 2 * c.xslot) return 2;
@@ -455,7 +477,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.n_layers = 1;
     if (extras) {
         bool wgrad_fused = false;
-        if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused, lower)) return 2;
+        if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused, lower, lower_wgrad_fused)) return 2;
         const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
         BwdXcdLauncher hl = dtype == FASTLSTM_FP16 ? launch_bwd_xcd_help_f16 : launch_bwd_xcd_help_bf16;
         int occ = 0;
@@ -888,7 +910,7 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
     if (int rc = check_dims(T, B, I, H)) return rc;
     unsigned char *fake = reinterpret_cast<unsigned char *>(static_cast<size_t>(4096));   // never dereferenced
     const BwdExtras e{fake, fake, fake, fake, fake, fake, H};
-    const LowerLayer lower{fake, fake, fake, fake, fake, fake, fake, fake, I, fake, (size_t)1 << 40};
+    const LowerLayer lower{fake, fake, fake, fake, fake, fake, fake, fake, I, fake, (size_t)1 << 40, fake, fake, fake, fake};
     const int rc = try_bwd_xcd(fake, fake, fake, fake, fake, fake, fake, fake, ws_bytes, T, B, H, dtype, nullptr, &e, &lower,
                                true);
     return (rc == FASTLSTM_OK || rc == 3) ? 1 : (rc < 0 ? rc : 0);
@@ -920,9 +942,10 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
     const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
     if (pl.wave_split != 2) {
         const BwdExtras e{Wx1, x1, out1, dx1, dWx1, dWh1, H};
-        const LowerLayer lower{dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, dx0, I, wgrad_ws, wgrad_ws_bytes};
+        const LowerLayer lower{dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, dx0, I, wgrad_ws, wgrad_ws_bytes, x, out0, dWx0, dWh0};
+        bool lower_wgrad_done = false;
         const int rc = try_bwd_xcd(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, static_cast<unsigned char *>(ws), ws_bytes, T, B,
-                                   H, dtype, s, &e, &lower);
+                                   H, dtype, s, &e, &lower, false, &lower_wgrad_done);
         if (rc < 0) return rc;
         if (rc == 0) {   // both recurrences, both dx and the upper weight gradients were one launch
             const int chunks = colsum_chunks(T * B);
@@ -933,6 +956,11 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
                                              stream))
                 return r2;
         }
+        if ((rc == 0 || rc == 3) && lower_wgrad_done)   // only the lower layer's bias gradient is left
+            return launch_colsum(dtype, d_ifgo0, db0, static_cast<float *>(wgrad_ws), T * B, 4 * H, colsum_chunks(T * B), s) ==
+                           hipSuccess
+                       ? FASTLSTM_OK
+                       : FASTLSTM_ERR_HIP;
         if (rc == 0 || rc == 3)
             return fastlstm_gemm_wgrad(d_ifgo0, x, out0, dWx0, dWh0, db0, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
     }

@@ -51,8 +51,10 @@ struct BwdXcdParams {
     // reads the upper layer's dx (k5.C) as its dout: the helpers write it chunk by chunk, latest
     // timesteps first (dx_done[c] counts the finished tiles of chunk c), and the lower recurrence
     // requests the dout of a timestep only when its chunk is complete.  The helpers also compute the
-    // lower layer's dx (k5_lo, when its C is not null) behind that recurrence; the lower layer's weight
-    // gradients are left to the caller.
+    // lower layer's dx (k5_lo, when its C is not null) behind that recurrence and, with wg_lo_tiles > 0,
+    // the lower layer's weight gradients (k8_lo, k9_lo: the same scheme as k8, k9, one tile per helper
+    // accumulated chunk by chunk as the lower recurrence finishes them); otherwise those are left to
+    // the caller.
     int n_layers;
     void *dh_lo, *dc_lo;
     const void *ifgo_lo, *cell_lo;
@@ -63,6 +65,9 @@ struct BwdXcdParams {
     int *chunk_done_lo; // [<= kMaxChunks]
     int *dx_done;       // [<= kMaxChunks]
     float *wg_scratch;  // stacked launches: 256 KiB per helper that owns a weight-gradient tile
+    GemmParams k8_lo, k9_lo;   // the lower layer's dWx, dWh (A = d_ifgo_lo, B = its x | h)
+    int k8_lo_tiles_n, wg_lo_tiles;
+    float *wg_scratch_lo;
     long long spin_limit;
 };
 
@@ -179,6 +184,19 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
                            p.k5_lo.C, p.k5_lo.M, p.k5_lo.N, p.k5_lo.K, p.k5_chunk_tiles, p.k5_lo_tiles_n, p.k5_tiles_m,
                            p.k5_chunks - 1 - k, k, h, n_helpers, (FASTLSTM_LDS_PTR unsigned char *)smem);
     };
+    // ... and the chunk's K range of this helper's weight-gradient tile of the lower layer
+    const int n8_lo = p.wg_tiles_m * p.k8_lo_tiles_n;
+    auto lower_wgrad = [&](int k) {
+        if (!stacked || h >= p.wg_lo_tiles) return;
+        const bool lo8 = h < n8_lo;
+        const GemmParams &q = lo8 ? p.k8_lo : p.k9_lo;
+        const int qi = lo8 ? h : h - n8_lo, qtn = lo8 ? p.k8_lo_tiles_n : p.k9_tiles_n;
+        const int c = p.k5_chunks - 1 - k;
+        const int kb = c * p.k5_chunk_tiles * 256, ke = min(q.K, kb + p.k5_chunk_tiles * 256);
+        helper_wgrad_chunk<T>(q.A, q.B, q.C, q.M, q.N, q.K, q.ldb, (qi / qtn) * 256, (qi % qtn) * 256, kb, ke,
+                              reinterpret_cast<f32x4 *>(p.wg_scratch_lo) + (size_t)h * (256 * 256 / 4), k == 0,
+                              k + 1 == p.k5_chunks, (FASTLSTM_LDS_PTR unsigned char *)smem);
+    };
     for (int k = 0; k < p.k5_chunks; ++k) {
         const int c = p.k5_chunks - 1 - k;   // chunk in forward time
         // d_ifgo of the chunk's timesteps is in memory once every recurrence workgroup said so
@@ -216,14 +234,20 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
                 if (threadIdx.x == 0) __hip_atomic_fetch_add(p.dx_done + c, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        if (stacked && k >= lag) lower_dx(k - lag);
+        if (stacked && k >= lag) {
+            lower_dx(k - lag);       // waits for the lower layer's chunk
+            lower_wgrad(k - lag);
+        }
     }
     if (own && !STACKED) {
         gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, 0, smem, acc);
         __syncthreads();
     }
     if (stacked)
-        for (int k = max(p.k5_chunks - lag, 0); k < p.k5_chunks; ++k) lower_dx(k);
+        for (int k = max(p.k5_chunks - lag, 0); k < p.k5_chunks; ++k) {
+            lower_dx(k);
+            lower_wgrad(k);
+        }
 #ifdef FASTLSTM_BWD_STAMPS
     if (threadIdx.x == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = waited; }
 #endif
@@ -235,6 +259,14 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
         gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
         __syncthreads();
     }
+    if (stacked)
+        for (int w = h + n_helpers; w < p.wg_lo_tiles; w += n_helpers) {
+            const bool w8 = w < n8_lo;
+            const GemmParams &q = w8 ? p.k8_lo : p.k9_lo;
+            const int qi = w8 ? w : w - n8_lo, qtn = w8 ? p.k8_lo_tiles_n : p.k9_tiles_n;
+            gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
+            __syncthreads();
+        }
 }
 
 // HELP: 0 = recurrence only; 1 = the workgroups without a role compute dx and the weight gradients;
@@ -397,12 +429,18 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 *reinterpret_cast<u32x4 *>(std_ + s_lds[i]) = dp[i];
             }
     };
+    // With helpers in the launch the d_ifgo tiles are written THROUGH to memory (sc1): the chunk
+    // hand-over below then needs no write-back of this XCD's L2, which stalled the releasing wave --
+    // and with it the whole group -- for several microseconds per chunk.
     auto tile_to_global = [&](int t) {
 #pragma unroll
         for (int i = 0; i < GPT; ++i)
-            if (g_ok[i])
-                *reinterpret_cast<u32x4 *>(d_ifgo + (size_t)t * B4H + g_glb[i]) =
-                    *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
+            if (g_ok[i]) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
+                T *dst = d_ifgo + (size_t)t * B4H + g_glb[i];
+                if (k5_live) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+                else *reinterpret_cast<u32x4 *>(dst) = v;
+            }
     };
     if (lower) {   // the latest chunk(s) of this layer's dout have to be there
         if (wave == 0) {
@@ -483,12 +521,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, vg, s);
         __syncthreads();
         // Every workgroup of the group has passed this step's publish point, where its stores of the
-        // previous steps (d_ifgo tiles included) were acknowledged by the L2.  When the previous step
-        // closed a chunk, ONE workgroup hands the group's share of it to the helpers: the release
-        // writes this XCD's L2 back (all of it, whichever CU wrote the lines), so that the other
-        // XCDs can read the chunk, and counts for all n_ht workgroups.
+        // previous steps (the written-through d_ifgo tiles included) were acknowledged: they are in
+        // memory.  When the previous step closed a chunk, ONE workgroup hands the group's share of it to
+        // the helpers on the other XCDs and counts for all n_ht workgroups.
         if (k5_live && j == 0 && tid == kWave && s > 0 && (t + 1) % p.k5_chunk_steps == 0)
-            __hip_atomic_fetch_add(chunk_done + (t + 1) / p.k5_chunk_steps, p.n_ht, __ATOMIC_RELEASE,
+            __hip_atomic_fetch_add(chunk_done + (t + 1) / p.k5_chunk_steps, p.n_ht, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps
@@ -544,7 +581,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     if (k5_live) {   // the last chunk (timesteps 0 ..)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == kWave) __hip_atomic_fetch_add(chunk_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == kWave) __hip_atomic_fetch_add(chunk_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 #ifdef FASTLSTM_BWD_STAMPS
     if (tid == 0) { stamps[1] = (long long)wall_clock64(); stamps[2] = -1; }

@@ -363,7 +363,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
             const int row = pc / PPSEG, k = pc % PPSEG;
             if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
                 const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
-                *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+                // a first layer that feeds a second one in the same launch writes its h THROUGH to memory
+                // (sc1): the chunk hand-over below then needs no write-back of this XCD's L2
+                const u32x4 hv = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+                if (feeds) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(out + go), "v"(hv) : "memory");
+                else *reinterpret_cast<u32x4 *>(out + go) = hv;
                 if (keep || t + 1 == T_)
                     *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
             }
@@ -393,10 +397,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         __syncthreads();
         FASTLSTM_TP(2);
         // Every workgroup of the group has published h_t, behind the acknowledgement of everything it
-        // stored before: out[t-1] (stored in step t-2) is in this XCD's L2.  When step t-2 closed a chunk,
-        // ONE workgroup writes the L2 back (release) and counts the chunk for the whole group.
+        // stored before: out[t-1] (stored in step t-2, written through) is in memory.  When step t-2
+        // closed a chunk, ONE workgroup counts the chunk for the whole group.
         if (feeds && j == 0 && tid == kWave && t >= 2 && (t - 1) % p.k1_chunk_steps == 0)
-            __hip_atomic_fetch_add(p.out_ready + (t - 1) / p.k1_chunk_steps - 1, p.n_ht, __ATOMIC_RELEASE,
+            __hip_atomic_fetch_add(p.out_ready + (t - 1) / p.k1_chunk_steps - 1, p.n_ht, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- acc[a][i] += Wslice(a) . h_{t-1}(i)^T over this wave's k-steps: all operand blocks
@@ -488,7 +492,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         const int counted = T_ >= 2 ? (T_ - 2) / p.k1_chunk_steps : 0;   // chunks 0 .. counted-1 are done
         if (tid == kWave)
             for (int c = counted; c < chunks; ++c)
-                __hip_atomic_fetch_add(p.out_ready + c, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(p.out_ready + c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 #ifdef FASTLSTM_TIMELINE
     __syncthreads();
