@@ -137,7 +137,16 @@ struct XcdCfg {
 
 // The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
 // and the workspace holds a ring with one slot per exchanged version.
-bool select_xcd(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c) {
+// Row range of the batch that the XCD-local launches of the calling thread cover (rows == 0: all of
+// it).  A batch with more tiles than one launch holds runs as several launches over row ranges.
+static thread_local int t_xcd_row0 = 0, t_xcd_rows = 0;
+struct XcdRowWindow {
+    XcdRowWindow(int row0, int rows) { t_xcd_row0 = row0; t_xcd_rows = rows; }
+    ~XcdRowWindow() { t_xcd_row0 = 0; t_xcd_rows = 0; }
+};
+
+bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c) {
+    const int B = t_xcd_rows ? t_xcd_rows : B_all;   // rows of this launch
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
     const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
@@ -249,6 +258,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
+    p.b_base = t_xcd_row0;
     p.spin_limit = spin_limit_ticks();
     p.keep = t_keep_activations;
     p.trace = g_rec_trace;
@@ -278,6 +288,32 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
 // callers may capture the stream into a graph).
 __global__ void zero_words_kernel(unsigned *p, size_t n) {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+// A batch with more 16-row tiles than one XCD-local launch holds (and no fit with 32-row tiles either):
+// rows per launch such that full launches use every XCD with 16-row tiles and the remainder fits
+// too, or 0.  The launches run one after the other on the stream and share the workspace.
+static int xcd_rows_per_launch(int T, int B, int H, int dtype, bool backward, size_t ws_bytes) {
+    const int candidates[4] = {512, 256, 128, 64};
+    for (int rows : candidates) {
+        if (rows >= B) continue;
+        XcdCfg c;
+        {
+            const XcdRowWindow w(0, rows);
+            if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c) || c.ntw != 1 || c.n_groups != kNumXcd * c.gpx) continue;
+        }
+        if (B % rows) {
+            const XcdRowWindow w(B - B % rows, B % rows);
+            if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c)) continue;
+        }
+        return rows;
+    }
+    return 0;
+}
+// the barrier counters of the XCD-local kernels start from zero in every launch
+static bool clear_xcd_counters(unsigned char *wsb, hipStream_t s) {
+    zero_words_kernel<<<64, 256, 0, s>>>(reinterpret_cast<unsigned *>(wsb + kWsHeaderBytes), kWsCounterBytes / 4);
+    return hipGetLastError() == hipSuccess;
 }
 
 // Shape of a launch of the register-resident kernels whose barrier groups span several XCDs
@@ -473,6 +509,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
+    p.b_base = t_xcd_row0;
     p.spin_limit = spin_limit_ticks();
     p.n_layers = 1;
     if (extras) {
@@ -635,6 +672,17 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     if (sync) {
         int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
         if (rc == 1) rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+        if (rc == 1) {   // too many batch tiles for one XCD-local launch: one launch per range of rows
+            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) {
+                for (int r0 = 0; r0 < B; r0 += rows) {
+                    if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
+                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const int r = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+                    if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
+                }
+                return FASTLSTM_OK;
+            }
+        }
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     FwdParams p{};
@@ -713,6 +761,18 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
         if (rc == 1)
             rc = try_bwd_wide(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
                               static_cast<hipStream_t>(stream));
+        if (rc == 1) {   // too many batch tiles for one XCD-local launch: one launch per range of rows
+            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, true, ws_bytes)) {
+                for (int r0 = 0; r0 < B; r0 += rows) {
+                    if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
+                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const int r = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
+                                              static_cast<hipStream_t>(stream));
+                    if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
+                }
+                return FASTLSTM_OK;
+            }
+        }
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     BwdParams p{};
@@ -981,7 +1041,8 @@ int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward,
     XcdCfg c;
     if (select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c)) return 1;
     WideCfg w;
-    return select_wide(T, B, H, dtype, backward != 0, ws_bytes, &w) ? 2 : 0;
+    if (select_wide(T, B, H, dtype, backward != 0, ws_bytes, &w)) return 2;
+    return xcd_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes) ? 1 : 0;
 }
 
 int fastlstm_ws_status(const void *ws_head) {

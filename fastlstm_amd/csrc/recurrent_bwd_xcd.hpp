@@ -31,6 +31,7 @@ struct BwdXcdParams {
     unsigned char *xbuf;   // ring: [T slots][groups][NT][KSB] operand blocks
     int T, B, H;
     int n_ht, gpx, n_groups;
+    int b_base;         // first batch row of this launch (a large batch runs as several launches over row ranges)
     int KSB;            // k-steps covering 4H
     // In-kernel dx = d_ifgo . Wx (HELP instantiations, k5_tiles_n > 0): the workgroups without a role
     // in the recurrence compute it in 256 x 256 tiles, latest timesteps first, as soon as the
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     }
     const bool lower = HELP == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
     const int g = lower ? vg - p.n_groups : vg;
-    const int u0 = j * HT, b0 = g * BT;
+    const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k5_live = HELP && p.k5_tiles_n > 0;
     int *chunk_done = lower ? p.chunk_done_lo : p.chunk_done;
     // chunk c of the upper layer's dx (this layer's dout) is complete when all its tiles were counted

@@ -45,6 +45,7 @@ struct FwdXcdParams {
     int n_ht;          // members of a barrier group (<= 32)
     int gpx;           // groups per XCD (32 / n_ht)
     int n_groups;      // batch tiles of this launch (<= 8 * gpx)
+    int b_base;        // first batch row of this launch (a large batch runs as several launches over row ranges)
     int KS;            // k-steps covering H
     // In-kernel input projection (HELP instantiations, k1_tiles_n > 0): the workgroups without a
     // role in the recurrence compute ifgo = x.Wx^T + b in 256 x 256 tiles, earliest timesteps first;
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         return;
     }
     const int layer = vg / p.n_groups, g = vg % p.n_groups;   // layer 1: the second of a stack
-    const int u0 = j * HT, b0 = g * BT;
+    const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k1_live = HELP && p.k1_tiles_n > 0;
     // chunk c of ifgo is complete when all its tiles were counted
     auto wait_chunk = [&](int c, int t) {
