@@ -670,19 +670,26 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (sync) {
+        // One launch per range of rows where the batch has too many 16-row tiles for one XCD-local launch;
+        // also instead of one launch with 32-row tiles of the 8-wave kernel (H = 1024, 16-bit), whose
+        // 32-row step costs 2.5 x its 16-row step (the 4-wave kernels of smaller H are faster in one
+        // launch with 32-row tiles).
+        auto by_row_ranges = [&](int rows) {
+            for (int r0 = 0; r0 < B; r0 += rows) {
+                if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return (int)FASTLSTM_ERR_HIP;
+                const XcdRowWindow w(r0, std::min(rows, B - r0));
+                const int r = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+                if (r != FASTLSTM_OK) return r < 0 ? r : (int)FASTLSTM_ERR_RESIDENCY;
+            }
+            return (int)FASTLSTM_OK;
+        };
+        XcdCfg whole;
+        if (select_xcd(T, B, H, dtype, false, ws_bytes, &whole) && whole.ntw == 2 && whole.nwv == 8)
+            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
         int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
         if (rc == 1) rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
-        if (rc == 1) {   // too many batch tiles for one XCD-local launch: one launch per range of rows
-            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) {
-                for (int r0 = 0; r0 < B; r0 += rows) {
-                    if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
-                    const XcdRowWindow w(r0, std::min(rows, B - r0));
-                    const int r = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
-                    if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
-                }
-                return FASTLSTM_OK;
-            }
-        }
+        if (rc == 1)
+            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     FwdParams p{};
