@@ -752,7 +752,8 @@ def test_xcd_local_barrier_timeout_is_reported_not_hung():
 
 
 @pytest.mark.parametrize("T,B,I,H,dt", [(70, 32, 256, 1024, torch.float16),     # two stacked layers per launch
-                                        (6, 128, 128, 2048, torch.bfloat16)])   # register-resident H = 2048 kernels
+                                        (6, 128, 128, 2048, torch.bfloat16),    # register-resident H = 2048 kernels
+                                        (4, 300, 64, 1024, torch.float16)])     # XCD-local launches over ranges of rows
 def test_stacked_and_wide_launches_drain_on_timeout(T, B, I, H, dt):
     """Host-forced failure path for the launches with chunk counters and multi-XCD flag barriers:
     with a spin limit of one poll every wait gives up, the grids drain, the status word reports the
