@@ -326,11 +326,11 @@ bool select_wide(int T, int B, int H, int dtype, bool backward, size_t ws_bytes,
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
     if (dtype == FASTLSTM_FP32) return false;
-    if (H % 256 || (H != 1536 && H != 2048)) return false;
+    if (H % 256 || H <= 1024 || H > 2048) return false;   // 1280, 1536, 1792, 2048
     c->nkw = backward ? H / 64 : H / 256;
     c->n_ht = H / 16;
-    if (c->n_ht % 32 || c->n_ht > kXcdGroupStride) return false;
-    c->xpg = c->n_ht / 32;
+    if (c->n_ht > kXcdGroupStride) return false;
+    c->xpg = cdiv(c->n_ht, 32);   // XCDs per group (the last one partly used when H is not a multiple of 512)
     c->n_groups = cdiv(B, 64);
     if (c->n_groups * c->xpg > kNumXcd) return false;
     c->ks = (backward ? 4 * H : H) / 32;

@@ -194,9 +194,9 @@ extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, 
                                    backward != 0, true, slots);
     // the XCD-local kernels lay their ring out for batch tiles of 16 or 32 rows, which covers at most
     // 16 rows (one operand block per k-step) more than the tiles of the plan
-    // (the kernels for H = 1536, 2048 use tiles of 64 rows: at most 48 rows more)
+    // (the kernels for H = 1280 ... 2048 use tiles of 64 rows: at most 48 rows more)
     const int KS = cdiv(backward ? 4 * H : H, kstep_of(dtype));
-    const int margin = (dtype != FASTLSTM_FP32 && (H == 1536 || H == 2048)) ? 3 : 1;
+    const int margin = (dtype != FASTLSTM_FP32 && H > 1024 && H <= 2048 && H % 256 == 0) ? 3 : 1;
     ws = std::max(ws, kWsHeaderBytes + kWsCounterBytes +
                           (size_t)slots * (plan->batch_chunks * slot + (size_t)margin * KS * kFragBytes));
     return ws;

@@ -21,7 +21,7 @@ namespace fastlstm {
 
 constexpr int kWideRing = 12;   // LDS blocks (1 KiB) per wave for operand blocks in flight (8 and 14: same step time)
 
-// number of k-steps per wave NKW = 4H / KSTEP / 8 (24 for H = 1536, 32 for H = 2048)
+// number of k-steps per wave NKW = 4H / KSTEP / 8 (20, 24, 28, 32 for H = 1280, 1536, 1792, 2048)
 template <typename T, int NKW>
 __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdParams p) {
     static_assert(sizeof(T) == 2, "16-bit element types");

@@ -19,7 +19,7 @@
 //    workgroup loads too); the 4 batch tiles of 16 rows are multiplied one after the other, the operand
 //    blocks of the next one in flight meanwhile: weights (128 registers), two sets of operand blocks
 //    (64) and accumulators (16) stay within 256 registers.
-// Requirements (host): 16-bit elements, H = 256 * NKW, H / 16 a multiple of 32, groups * xpg <= 8.
+// Requirements (host): 16-bit elements, H = 256 * NKW (1280 ... 2048), groups * xpg <= 8 with xpg = ceil(H / 512).
 #pragma once
 #include <type_traits>
 

@@ -212,7 +212,8 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
  * the current device for this shape and a workspace of ws_bytes: 0 = the general kernel
  * (exchange through device memory), 1 = the XCD-local kernel (barrier group on one XCD,
  * exchange through its L2; needs the ring workspace of fastlstm_recurrent_workspace_bytes and a
- * device that fastlstm_plan_device has probed), 2 = the register-resident kernel for H = 1536 and
+ * device that fastlstm_plan_device has probed; a batch with more tiles than one launch holds runs as
+ * several launches over ranges of rows), 2 = the register-resident kernel for H = 1280, 1536, 1792,
  * 2048 with 16-bit elements (barrier groups of H / 16 workgroups over several XCDs, 64 batch rows
  * each; same needs as 1).  Negative: fastlstm_status.  Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);

@@ -363,6 +363,8 @@ WIDE_CASES = [
     (5, 128, 2048, torch.bfloat16),   # config C's B and H: two groups of 128 workgroups
     (4, 100, 1536, torch.float16),    # 96 workgroups per group, ragged second group
     (3, 40, 2048, torch.float16),     # one partly filled group
+    (4, 128, 1280, torch.float16),    # 80 workgroups per group over three XCDs, the third partly used
+    (3, 70, 1792, torch.bfloat16),    # 112 workgroups per group over four XCDs
 ]
 
 
