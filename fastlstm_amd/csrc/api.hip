@@ -322,7 +322,8 @@ struct WideCfg {
     int nkw, n_ht, xpg, n_groups, ks, lds;
     size_t xslot;
 };
-bool select_wide(int T, int B, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c) {
+bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c) {
+    const int B = t_xcd_rows ? t_xcd_rows : B_all;   // rows of this launch
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
     if (dtype == FASTLSTM_FP32) return false;
@@ -341,6 +342,23 @@ bool select_wide(int T, int B, int H, int dtype, bool backward, size_t ws_bytes,
     return true;
 }
 
+// Rows per launch (see xcd_rows_per_launch) for the register-resident kernels of H > 1024: full launches of 64-row groups on all XCDs.
+static int wide_rows_per_launch(int T, int B, int H, int dtype, bool backward, size_t ws_bytes) {
+    const int xpg = cdiv(H / 16, 32);
+    const int rows = 64 * (kNumXcd / std::max(1, xpg));
+    if (H <= 1024 || rows >= B || rows <= 0) return 0;
+    WideCfg c;
+    {
+        const XcdRowWindow w(0, rows);
+        if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c)) return 0;
+    }
+    if (B % rows) {
+        const XcdRowWindow w(B - B % rows, B % rows);
+        if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c)) return 0;
+    }
+    return rows;
+}
+
 // Returns 1 when the kernel does not apply, else a fastlstm_status.
 int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
                  int H, int dtype, hipStream_t stream) {
@@ -353,6 +371,7 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KS = c.ks;
+    p.b_base = t_xcd_row0;
     p.spin_limit = spin_limit_ticks();
     p.keep = t_keep_activations;
     auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
@@ -374,6 +393,7 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KSB = c.ks;
+    p.b_base = t_xcd_row0;
     p.spin_limit = spin_limit_ticks();
     auto launch = dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16;
     int occ = 0;
@@ -690,6 +710,16 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         if (rc == 1) rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
         if (rc == 1)
             if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
+        if (rc == 1)
+            if (const int rows = wide_rows_per_launch(T, B, H, dtype, false, ws_bytes)) {
+                for (int r0 = 0; r0 < B; r0 += rows) {
+                    if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
+                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const int r = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+                    if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
+                }
+                return FASTLSTM_OK;
+            }
         if (rc != 1) return rc;   // launched (0) or failed (< 0); 1: not applicable, use the general kernels
     }
     FwdParams p{};
@@ -775,6 +805,16 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
                     const XcdRowWindow w(r0, std::min(rows, B - r0));
                     const int r = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
                                               static_cast<hipStream_t>(stream));
+                    if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
+                }
+                return FASTLSTM_OK;
+            }
+            if (const int rows = wide_rows_per_launch(T, B, H, dtype, true, ws_bytes)) {
+                for (int r0 = 0; r0 < B; r0 += rows) {
+                    if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
+                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const int r = try_bwd_wide(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
+                                               static_cast<hipStream_t>(stream));
                     if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
                 }
                 return FASTLSTM_OK;
@@ -1049,7 +1089,8 @@ int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward,
     if (select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c)) return 1;
     WideCfg w;
     if (select_wide(T, B, H, dtype, backward != 0, ws_bytes, &w)) return 2;
-    return xcd_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes) ? 1 : 0;
+    if (xcd_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes)) return 1;
+    return wide_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes) ? 2 : 0;
 }
 
 int fastlstm_ws_status(const void *ws_head) {

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int g = xcd / xpg, j = (xcd % xpg) * 32 + slot;
     if (g >= p.n_groups || j >= p.n_ht) return;
-    const int u0 = j * HT, b0 = g * BT;
+    const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                      // [8][NT][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * NT * kWave);   // gates, c, dout tiles

@@ -90,6 +90,7 @@ STAGE_CASES = [
     (3, 128, 128, 2048, torch.bfloat16),  # config C tiles (waves split the batch)
     (3, 300, 64, 1024, torch.float16),    # large batch: XCD-local launches over ranges of 128 rows (128 + 128 + 44)
     (4, 200, 64, 1024, torch.bfloat16),   # forward in two row ranges (128 + 72), reverse in one launch of 32-row tiles
+    (3, 200, 64, 2048, torch.float16),    # register-resident kernels over two row ranges (128 + 72)
     (3, 40, 64, 512, torch.float32),
 ]
 
