@@ -2,7 +2,7 @@
 //     C[m][n] = sum_k A(m,k) * B(n,k)   [+ bias0[n] + bias1[n]]
 // the same contraction as gemm.hpp's generic kernel, restricted to the aligned case
 // (K a multiple of 64, leading dimensions multiples of 8 elements, operands < 4 GiB)
-// that every BASELINE configuration of the LSTM hits.
+// that every benchmark configuration of the LSTM hits.
 //
 // Design for gfx950
 //  * BM x BN x 64 workgroup tile (256 x 256 for large problems), 4 waves in 2 x 2, each
