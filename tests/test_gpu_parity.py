@@ -132,10 +132,10 @@ def _random_shape(rng):
     if kind == "mid":
         return rng.randint(1, 24), rng.randint(1, 130), rng.randint(1, 300), rng.randint(65, 700), dt
     if kind == "tile":
-        H = rng.choice([128, 256, 384, 512, 768, 1024, 1024, 1536, 2048])
+        H = rng.choice([128, 256, 384, 512, 768, 1024, 1024, 1280, 1536, 1792, 2048])
         if dt == torch.float32:
             H = min(H, 1024)
-        return (rng.randint(1, 6), rng.choice([1, 8, 16, 31, 32, 33, 64, 65, 96, 128, 160, 256]),
+        return (rng.randint(1, 6), rng.choice([1, 8, 16, 31, 32, 33, 64, 65, 96, 128, 160, 200, 256, 300, 400]),
                 rng.choice([64, 100, 256, 1024]), H, dt)
     return rng.randint(1, 4), rng.randint(200, 700), rng.randint(8, 128), rng.choice([64, 200, 256, 512, 1024]), dt
 
