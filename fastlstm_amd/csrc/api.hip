@@ -608,22 +608,37 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
                : FASTLSTM_ERR_HIP;
 }
 
-int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
-                     void *stream) {
-    if (!d_ifgo || !Wx || !dx) return FASTLSTM_ERR_NULL;
-    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
-    if (int rc = check_dims(T, B, I, H)) return rc;
-    if (!aligned16(d_ifgo) || !aligned16(Wx) || !aligned16(dx)) return FASTLSTM_ERR_ALIGN;
+// dx = d_ifgo . Wx.  With a scratch buffer (fp32 partial sums) a product with few output tiles is
+// split along K so that it fills the device; without one it is a single pass.
+static int gemm_dx_impl(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
+                        void *scratch, size_t scratch_bytes, void *stream) {
     GemmParams p{};
     p.A = d_ifgo; p.B = Wx; p.C = dx;
     p.M = T * B; p.N = I; p.K = 4 * H;
     p.lda = 4 * H; p.ldb = I; p.ldc = I;
     p.splits = 1; p.k_per_split = 4 * H;
     int tile, splits;
-    gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, true, false, &tile, &splits);
+    gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, true, scratch != nullptr, &tile, &splits);
+    if (splits > 1) {
+        const int bk = tile ? 64 : gemm_bk(dtype);
+        const int kps = cdiv(cdiv(p.K, splits), bk) * bk;
+        splits = cdiv(p.K, kps);
+        if (splits > 1 && (size_t)splits * p.M * p.N * sizeof(float) <= scratch_bytes) {
+            p.splits = splits; p.k_per_split = kps; p.Cpart = static_cast<float *>(scratch);
+        }
+    }
     return launch_gemm_tiled(dtype, p, false, true, tile, static_cast<hipStream_t>(stream)) == hipSuccess
                ? FASTLSTM_OK
                : FASTLSTM_ERR_HIP;
+}
+
+int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
+                     void *stream) {
+    if (!d_ifgo || !Wx || !dx) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(d_ifgo) || !aligned16(Wx) || !aligned16(dx)) return FASTLSTM_ERR_ALIGN;
+    return gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, nullptr, 0, stream);
 }
 
 // tile and split-K factor of a weight-gradient product C[M,N] = A^T.B with reduction length K
@@ -1000,7 +1015,8 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
     if (rc != 3) {   // nothing was launched: recurrence, then dx
         if (int r2 = fastlstm_bwd_persistent(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
             return r2;
-        if (int r2 = fastlstm_gemm_dx(d_ifgo, Wx, dx, T, B, I, H, dtype, stream)) return r2;
+        // (the weight-gradient workspace is free until the next call: scratch for a split along K)
+        if (int r2 = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, wgrad_ws, wgrad_ws_bytes, stream)) return r2;
     }
     return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
 }
