@@ -38,7 +38,7 @@ PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MF
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the fused forward layer kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE,
 # scaled by a plain copy of known size (profiles/fwd_layer_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 1778.3e6}
+TRAFFIC_BYTES = {"B": 1778.3e6, "D": 336.1e6}   # D: the recurrence kernel alone (profiles/fwd_recurrence_D_pmc.md)
 
 
 def main():
@@ -280,7 +280,7 @@ def main():
         ach = nbytes / (t_rec * 1e-3) / 1e9
         roofline = {"kernel": "lstm_fwd_persistent_kernel<SPLIT=2> (one hidden tile per workgroup)", "bound": "hbm",
                     "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                    "traffic": None,
+                    "traffic": TRAFFIC_BYTES.get(args.workload),
                     "algorithmic": "s*(2*T*B*4H + 2*T*B*H + 4H*H) bytes per launch = %.1f MB" % (nbytes / 1e6),
                     "launch_ms": round(t_rec, 4),
                     "note": "latency-bound, not HBM-bound: %d independent workgroups (16 batch rows each) walk through "
