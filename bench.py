@@ -38,7 +38,7 @@ PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MF
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the fused forward layer kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE,
 # scaled by a plain copy of known size (profiles/fwd_layer_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 1778.3e6, "D": 336.1e6}   # D: the recurrence kernel alone (profiles/fwd_recurrence_D_pmc.md)
+TRAFFIC_BYTES = {"B": 1575.6e6, "D": 336.1e6}   # D: the recurrence kernel alone (profiles/fwd_recurrence_D_pmc.md)
 
 
 def main():

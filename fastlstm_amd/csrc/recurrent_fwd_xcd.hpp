@@ -148,13 +148,44 @@ template <typename T>
 __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *smem) {
     int n_helpers;
     const int h = helper_rank(p.n_ht, p.gpx, p.n_groups * p.n_layers, &n_helpers);
-    const int total = p.k1_tiles_m * p.k1_tiles_n;
-    int i0 = h, i1 = p.n_layers > 1 ? h : total;
+    int total = p.k1_tiles_m * p.k1_tiles_n;   // length of the tile list
     int *ready_flag = reinterpret_cast<int *>(smem);
+    // List position -> tile.  Plain: row-major over (row tile, column tile).  Where the helpers are whole
+    // XCDs and the column tiles divide among them, the tiles of a round (n_helpers of them: the same
+    // row tiles either way) are dealt so that an XCD keeps to its own column tiles: its panel of Wx
+    // (a few MiB) stays in that XCD's L2 for the whole launch instead of all of Wx streaming through
+    // every L2 once per pair of row tiles; x is then read by every helper XCD.
+    const int tn = p.k1_tiles_n, xcds = n_helpers / 32, cpx = xcds ? tn / xcds : 0;
+    const bool by_panel = n_helpers % 32 == 0 && xcds > 0 && tn % xcds == 0 && cpx > 0 && 32 % cpx == 0;
+    auto tile_of = [&](int idx, int *rt, int *ct) {
+        if (by_panel) {
+            const int round = idx / n_helpers, k = h / 32, sl = h % 32;
+            *rt = round * (32 / cpx) + sl / cpx;
+            *ct = k * cpx + sl % cpx;
+        } else {
+            *rt = idx / tn;
+            *ct = idx % tn;
+        }
+    };
+    if (by_panel) total = cdiv(p.k1_tiles_m, 32 / cpx) * n_helpers;   // whole rounds; positions past the last row tile are skipped
+    int i0 = h, i1 = p.n_layers > 1 ? h : total;
     while (i0 < total || i1 < total) {
+        {
+            int r_, c_;
+            if (i0 < total) {
+                tile_of(i0, &r_, &c_);
+                if (r_ >= p.k1_tiles_m) { i0 += n_helpers; continue; }
+            }
+            if (i1 < total) {
+                tile_of(i1, &r_, &c_);
+                if (r_ >= p.k1_tiles_m) { i1 += n_helpers; continue; }
+            }
+        }
         bool second = false;
         if (i1 < total) {
-            const int c1 = (i1 / p.k1_tiles_n) / p.k1_chunk_tiles;
+            int rt1, ct1;
+            tile_of(i1, &rt1, &ct1);
+            const int c1 = rt1 / p.k1_chunk_tiles;
             if (i0 < total) {   // one poll: is the chunk there?
                 if (threadIdx.x == 0)
                     *ready_flag = __hip_atomic_load(p.out_ready + c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= p.n_active;
@@ -169,8 +200,8 @@ __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *
             }
             if (second) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the first layer's h, written on other XCDs
         }
-        const int tile = second ? i1 : i0;
-        const int rt = tile / p.k1_tiles_n, ct = tile % p.k1_tiles_n;
+        int rt, ct;
+        tile_of(second ? i1 : i0, &rt, &ct);
         if (second) gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1b, rt * 256, ct * 256, 0, smem, 0);
         else gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
