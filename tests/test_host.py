@@ -47,6 +47,18 @@ def test_argument_validation_needs_no_gpu():
     assert lib.fastlstm_fwd_persistent(a, a, a, a, a, 1 << 20, 4, 4, 4, 7, None) == _lib.ERR_DTYPE
     assert lib.fastlstm_bwd_persistent(a, a, a, a, a, a, a, a + 8, 1 << 20, 4, 4, 4, 0, None) == _lib.ERR_ALIGN
     assert lib.fastlstm_bwd_persistent(a, a, a, None, a, a, a, a, 1 << 20, 4, 4, 4, 0, None) == _lib.ERR_NULL
+    # the layer entry points (training and inference form) and the stacked ones validate the same way
+    for name in ("fastlstm_fwd_layer", "fastlstm_fwd_layer_infer"):
+        fn = getattr(lib, name)
+        assert fn(a, a, a, a, a, a, a, None, a, 1 << 20, 4, 4, 4, 4, 0, None) == _lib.ERR_NULL
+        assert fn(a, a, a, a, a, a, a, a, a, 1 << 20, 4, 4, 0, 4, 0, None) == _lib.ERR_DIM
+        assert fn(a, a, a, a, a, a + 8, a, a, a, 1 << 20, 4, 4, 4, 4, 2, None) == _lib.ERR_ALIGN
+    for name in ("fastlstm_fwd_stack2", "fastlstm_fwd_stack2_infer"):
+        fn = getattr(lib, name)
+        assert fn(*([a] * 15), None, 1 << 20, 4, 4, 4, 4, 1, None) == _lib.ERR_NULL
+        assert fn(*([a] * 16), 1 << 20, 4, 4, 4, 4, 5, None) == _lib.ERR_DTYPE
+    assert lib.fastlstm_recurrent_kernel_kind(4, 4, 4, 9, 0, 1 << 20) == _lib.ERR_DTYPE
+    assert lib.fastlstm_recurrent_kernel_kind(0, 4, 4, 0, 0, 1 << 20) == _lib.ERR_DIM
     assert lib.fastlstm_plan_for(256, 163840, 4, 4, 0, 0, None) == _lib.ERR_NULL
     assert lib.fastlstm_ws_status(None) == _lib.ERR_NULL
     if not HAS_GPU:  # with valid arguments the first HIP call fails cleanly on a GPU-less host
