@@ -76,7 +76,7 @@ def forward(x, h0, c0, Wx, bx, Wh, bh, dtype=np.float64, round_mode=ROUND_NONE):
 
 
 def backward(dout, dh_n, dc_n, x, out, cell, ifgo, Wx, Wh, dtype=np.float64,
-             round_mode=ROUND_NONE, state_round=False):
+             round_mode=ROUND_NONE):
     """Returns dict(dx, dh0, dc0, dWx, dWh, db, d_ifgo) -- the quantities of
     fastlstm/lstm.py:236-334 (db is returned once; the reference hands the same
     tensor back for both biases, lstm.py:501)."""
@@ -97,8 +97,7 @@ def backward(dout, dh_n, dc_n, x, out, cell, ifgo, Wx, Wh, dtype=np.float64,
     fn(ctypes.c_int(T), ctypes.c_int(B), ctypes.c_int(I), ctypes.c_int(H), _ptr(dout), _ptr(dh_n),
        _ptr(dc_n), _ptr(x), _ptr(out), _ptr(cell), _ptr(ifgo), _ptr(Wx), _ptr(Wh),
        _ptr(res["dx"]), _ptr(res["dh0"]), _ptr(res["dc0"]), _ptr(res["dWx"]), _ptr(res["dWh"]),
-       _ptr(res["db"]), _ptr(res["d_ifgo"]), ctypes.c_int(round_mode),
-       ctypes.c_int(1 if state_round else 0))
+       _ptr(res["db"]), _ptr(res["d_ifgo"]), ctypes.c_int(round_mode))
     return res
 
 

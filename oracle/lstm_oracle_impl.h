@@ -23,7 +23,10 @@
  * Parity pinning (tests/test_oracle.py): every output of both functions is
  * checked against torch.nn.LSTM / torch.nn.LSTMCell autograd in float64 on
  * ragged shapes, against central finite differences on tiny inputs, and
- * against closed-form special cases (T=1, Wh=0, zero initial state).
+ * against closed-form special cases (T=1, Wh=0, zero initial state); the
+ * 16-bit round modes of both functions by representability of every stored
+ * value and, for the backward, by the matrix identities that tie dx, dWx,
+ * dWh and db to the rounded d_ifgo it returns.
  */
 
 #define CAT_(a, b) a##_##b
@@ -92,16 +95,15 @@ void FN(oracle_lstm_fwd)(int T, int B, int I, int H, const REAL *x, const REAL *
  * gradients flowing into the last hidden/cell state (NULL = zeros).
  * Outputs: dx [T,B,I], dh0, dc0 [B,H], dWx [4H,I], dWh [4H,H], db [4H],
  * d_ifgo [T,B,4H].  round_mode as above applies to the stored d_ifgo (which
- * is also what the recurrent product and the weight-gradient sums consume);
- * state_round != 0 additionally rounds the carried dc and dh_rec every step,
- * which is what the reference's default kernel does (kernels.py:1337-1342,
- * 1388-1390).
+ * is also what the recurrent product and the weight-gradient sums consume).
+ * The carried dc and dh_rec stay unrounded (the reference's default kernel
+ * rounds them through 16-bit buffers every step, kernels.py:1337-1342,
+ * 1388-1390; the HIP path keeps them in fp32 registers, so the checker does too).
  */
 void FN(oracle_lstm_bwd)(int T, int B, int I, int H, const REAL *dout, const REAL *dh_n,
                          const REAL *dc_n, const REAL *x, const REAL *out, const REAL *cell,
                          const REAL *ifgo, const REAL *Wx, const REAL *Wh, REAL *dx, REAL *dh0,
-                         REAL *dc0, REAL *dWx, REAL *dWh, REAL *db, REAL *d_ifgo, int round_mode,
-                         int state_round) {
+                         REAL *dc0, REAL *dWx, REAL *dWh, REAL *db, REAL *d_ifgo, int round_mode) {
     const size_t BH = (size_t)B * H, G = (size_t)4 * H;
     REAL *dh = (REAL *)malloc(BH * sizeof(REAL));
     REAL *dc = (REAL *)malloc(BH * sizeof(REAL));
@@ -137,7 +139,7 @@ void FN(oracle_lstm_bwd)(int T, int B, int I, int H, const REAL *dout, const REA
                 REAL d_i = dc1 * tg * si * ((REAL)1 - si);
                 REAL d_g = dc1 * si * ((REAL)1 - tg * tg);
                 REAL dcp = dc1 * sf;
-                dc[idx] = state_round ? (REAL)round_to((double)dcp, round_mode) : dcp;
+                dc[idx] = dcp;
                 dpb[u] = (REAL)round_to((double)d_i, round_mode);
                 dpb[H + u] = (REAL)round_to((double)d_f, round_mode);
                 dpb[2 * H + u] = (REAL)round_to((double)d_g, round_mode);
@@ -157,8 +159,6 @@ void FN(oracle_lstm_bwd)(int T, int B, int I, int H, const REAL *dout, const REA
 #pragma omp simd
                 for (int k = 0; k < I; ++k) dxb[k] += d * wx[k];
             }
-            if (state_round)
-                for (int k = 0; k < H; ++k) dhb[k] = (REAL)round_to((double)dhb[k], round_mode);
         }
         /* weight gradients: sums over batch (and, through the t loop, over time) */
 #pragma omp parallel for schedule(static)

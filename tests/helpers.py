@@ -62,3 +62,10 @@ def rel_err(a, b):
     """max |a - b| / max |b| (error max-norm relative to the reference's max-norm)"""
     a = _np64(a); b = _np64(b)
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def elementwise_ratio(got, want, rtol=1e-4, atol=1e-4):
+    """max over elements of |got - want| / (atol + rtol * |want|): <= 1 means every element is within
+    the allclose bound at these tolerances, with no scaling by the tensor's magnitude."""
+    a = _np64(got); b = _np64(want)
+    return float((np.abs(a - b) / (atol + rtol * np.abs(b))).max())

@@ -13,7 +13,7 @@ import torch
 
 import fastlstm_amd.lstm as L
 from fastlstm_amd import FastLSTM, PersistentLSTMfn, _lib
-from helpers import make_problem, nn_lstm_reference, rel_err, to_np
+from helpers import elementwise_ratio, make_problem, nn_lstm_reference, rel_err, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -47,6 +47,18 @@ def assert_close32(got, want, scale_atol=1.0):
                                atol=FP32_TOL * scale_atol)
 
 
+def assert_elementwise32(rows, what):
+    """rows: (name, got, want).  Prints the worst |got - want| / (1e-4 + 1e-4*|want|) of every tensor
+    and asserts that each ELEMENT is inside rtol = atol = 1e-4 (no scaling by the tensor's magnitude)."""
+    worst = 0.0
+    for name, got, want in rows:
+        r = elementwise_ratio(got, want, FP32_TOL, FP32_TOL)
+        print("    %s %-16s worst |err| / (atol + rtol*|ref|) = %.3f" % (what, name, r))
+        worst = max(worst, r)
+        assert r <= 1.0, (what, name, r)
+    return worst
+
+
 # --------------------------------------------------------------------------------------
 # 1. the reference's own integration grid (tests/test_lstm.py:160-220): 2 layers, I = 123,
 #    ragged B and H, fp32, module outputs and every parameter gradient vs nn.LSTM
@@ -69,10 +81,9 @@ def test_fastlstm_module_vs_nn_lstm(seq_size, batch_size, hidden_size):
     assert not hn1.requires_grad and not cn1.requires_grad  # nested tuple => no grad (lstm.py:522)
     y1.sum().backward()
     y2.sum().backward()
-    for n, p in m1.named_parameters():
-        ref = getattr(m2, n).grad
-        # gradients are sums over T*B terms: atol scales with their magnitude
-        assert_close32(p.grad, ref, scale_atol=max(1.0, float(ref.abs().max())))
+    rows = [("y", y1, y2), ("h_n", hn1, hn2), ("c_n", cn1, cn2)]
+    rows += [(n + ".grad", p.grad, getattr(m2, n).grad) for n, p in m1.named_parameters()]
+    assert_elementwise32(rows, "T%d B%d H%d" % (seq_size, batch_size, hidden_size))
 
 
 # --------------------------------------------------------------------------------------
@@ -217,6 +228,15 @@ def test_gpu_matches_golden_vectors():
         assert_close32(out, z[name + "/out/out"])
         assert_close32(hn, z[name + "/out/h_n"])
         assert_close32(cn, z[name + "/out/c_n"])
+        # the fixture's gradients belong to loss = sum(out*dout) + sum(h_n*dh_n) + sum(c_n*dc_n): the
+        # differentiable-state Function delivers dh_n / dc_n to the reverse kernel
+        out, hn, cn = L.PersistentLSTMStatefn.apply(x, h0, c0, *ws)
+        ((out * t("dout")).sum() + (hn * t("dh_n")).sum() + (cn * t("dc_n")).sum()).backward()
+        grads = [("dx", x), ("dWx", ws[0]), ("dbx", ws[1]), ("dWh", ws[2]), ("dbh", ws[3])]
+        if h0 is not None:
+            grads += [("dh0", h0), ("dc0", c0)]
+        for key, leaf in grads:
+            assert_close32(leaf.grad, z["%s/out/%s" % (name, key)])
 
 
 # --------------------------------------------------------------------------------------
@@ -1063,10 +1083,9 @@ def test_config_A_fp32_fwd_bwd_full_size():
     yr, (hr, cr) = ref(xr)
     assert_close32(y, yr); assert_close32(hn, hr); assert_close32(cn, cr)
     y.sum().backward(); yr.sum().backward()
-    assert_close32(xg.grad, xr.grad, scale_atol=max(1.0, float(xr.grad.abs().max())))
-    for n, prm in m.named_parameters():
-        rg = getattr(ref, n).grad
-        assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
+    rows = [("out", y, yr), ("h_n", hn, hr), ("c_n", cn, cr), ("dx", xg.grad, xr.grad)]
+    rows += [(n + ".grad", prm.grad, getattr(ref, n).grad) for n, prm in m.named_parameters()]
+    assert_elementwise32(rows, "config A")
 
 
 def test_config_B_fp16_forward_full_size():

@@ -196,3 +196,29 @@ def test_round_mode_stores_representable_values(oracle, mode, tdt):
     o0, c0, g0 = oracle.forward(*a, dtype=np.float32)
     eps = 2.0 ** -10 if mode == 1 else 2.0 ** -7
     np.testing.assert_allclose(o, o0, atol=T * eps)
+
+
+@pytest.mark.parametrize("mode,tdt", [(1, torch.float16), (2, torch.bfloat16)])
+def test_backward_round_mode_rounds_d_ifgo_and_everything_downstream_uses_it(oracle, mode, tdt):
+    """The 16-bit mode of the backward: the returned d_ifgo is representable in the 16-bit type, it is the
+    unrounded one to within half a unit in the last place per step, and dx, dW_x, dW_h, db are exactly
+    the matrix products / column sums of THAT rounded d_ifgo (a textbook matmul in float64)."""
+    T, B, I, H = 9, 5, 7, 12
+    p = make_problem(T, B, I, H, seed=21)
+    a = to_np(p, FWD_KEYS)
+    o, c, g = oracle.forward(*a, round_mode=mode)
+    dout, dh_n, dc_n = to_np(p, ["dout", "dh_n", "dc_n"])
+    r = oracle.backward(dout, dh_n, dc_n, a[0], o, c, g, a[3], a[5], round_mode=mode)
+    r0 = oracle.backward(dout, dh_n, dc_n, a[0], o, c, g, a[3], a[5])
+    d = torch.from_numpy(r["d_ifgo"])
+    assert torch.equal(d.to(tdt).double(), d)
+    eps = 2.0 ** -10 if mode == 1 else 2.0 ** -7
+    np.testing.assert_allclose(r["d_ifgo"], r0["d_ifgo"], atol=T * eps * np.abs(r0["d_ifgo"]).max())
+    assert np.abs(r["d_ifgo"] - r0["d_ifgo"]).max() > 0          # the mode does something
+    d2 = r["d_ifgo"].reshape(T * B, 4 * H)
+    np.testing.assert_allclose(r["dx"].reshape(T * B, I), d2 @ a[3], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(r["dWx"], d2.T @ a[0].reshape(T * B, I), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(r["dWh"], d2.T @ o[:-1].reshape(T * B, H), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(r["db"], d2.sum(0), rtol=1e-12, atol=1e-12)
+    # the state gradients are the recurrent product of the rounded d_ifgo of step 0 / the carried dc
+    np.testing.assert_allclose(r["dh0"], r["d_ifgo"][0] @ a[5], rtol=1e-12, atol=1e-12)
