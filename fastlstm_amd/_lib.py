@@ -51,6 +51,7 @@ SIGNATURES = {
     "fastlstm_gemm_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "fastlstm_ws_status": (_i, [_vp]),
+    "fastlstm_device_status": (_i, [_i, _i]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
     "fastlstm_set_gemm_trace": (None, [_vp]),
     "fastlstm_set_recurrent_trace": (None, [_vp]),

@@ -15,13 +15,12 @@ using namespace fastlstm;
 
 namespace fastlstm {
 
-// What the forward launches of the calling thread store besides out: 1 = gate pre-activations and
-// every cell state (the reverse pass reads them), 0 = inference.  Set for the duration of one of
-// the *_infer entry points.
-static thread_local int t_keep_activations = 1;
-struct InferenceScope {
-    InferenceScope() { t_keep_activations = 0; }
-    ~InferenceScope() { t_keep_activations = 1; }
+// What one recurrent launch covers and stores; handed down explicitly from the entry points.
+struct LaunchOpts {
+    int keep = 1;            // forward: 1 = store the gate pre-activations and every cell state (the reverse
+                             // pass reads them), 0 = inference (the *_infer entry points)
+    int row0 = 0, rows = 0;  // rows [row0, row0 + rows) of the batch; rows == 0: all of it.  A batch with more
+                             // tiles than one XCD-local launch holds runs as several launches over row ranges
 };
 
 static long long *g_rec_trace = nullptr;
@@ -39,7 +38,11 @@ int check_dims(int T, int B, int I, int H) {
 
 struct DeviceInfo {
     int num_cus = 0, lds = 0;
-    int xcd_round_robin = 0;   // 1: workgroup i of a launch runs on XCD i % 8 (probed once)
+    int xcd_round_robin = 0;   // 1: the workgroups of a launch are dealt to the 8 XCDs in turn (probed once)
+    // One pinned, device-visible word per device (allocated by the first planning call): a recurrent call
+    // whose launches ended with the abort flag raised sets it when that work completes on the device, and
+    // the next entry on the device reports it -- a failed barrier is never silent and costs no host sync.
+    int *status_host = nullptr, *status_dev = nullptr;
 };
 
 // Every workgroup reports the XCD it runs on (hardware register XCC_ID).
@@ -51,7 +54,8 @@ __global__ void xcc_probe_kernel(int *out) {
     }
 }
 
-// 1 when the device has 8 XCDs x 32 CUs and deals the workgroups of a launch to the XCDs in turn.
+// 1 when the device has 8 XCDs x 32 CUs and deals the workgroups of a launch to the XCDs in turn
+// (workgroup i on XCD (i + r) % 8 with one r for the whole dispatch; the kernels check r per launch).
 // Uses pinned host memory the kernel writes directly: no device allocation.
 int probe_xcd_round_robin(int num_cus) {
     if (num_cus != kNumXcd * 32) return 0;
@@ -64,9 +68,10 @@ int probe_xcd_round_robin(int num_cus) {
     if (hipHostGetDevicePointer(reinterpret_cast<void **>(&dptr), buf, 0) == hipSuccess) {
         hipLaunchKernelGGL(xcc_probe_kernel, dim3(n), dim3(64), 0, nullptr, dptr);
         if (hipGetLastError() == hipSuccess && hipDeviceSynchronize() == hipSuccess) {
-            ok = 1;
-            for (int i = 0; i < n; ++i)
-                if (buf[i] != i % kNumXcd) ok = 0;
+            // in turn, from whichever XCD the dispatch started at
+            ok = buf[0] >= 0 && buf[0] < kNumXcd;
+            for (int i = 0; i < n && ok; ++i)
+                if (buf[i] != (buf[0] + i) % kNumXcd) ok = 0;
         }
     }
     (void)hipHostFree(buf);
@@ -74,8 +79,17 @@ int probe_xcd_round_robin(int num_cus) {
 }
 
 DeviceInfo g_device_cache[64];
-void device_info_set_xcd(int device, int rr) {
-    if (device >= 0 && device < 64) g_device_cache[device].xcd_round_robin = rr;
+std::mutex g_device_mu;                       // guards g_device_cache
+std::atomic<int> g_status_words{0};           // devices that have a status word (0: no entry ever looks)
+void device_info_set_probe(int device, int rr, int *status_host, int *status_dev) {
+    std::lock_guard<std::mutex> lock(g_device_mu);
+    if (device < 0 || device >= 64) return;
+    g_device_cache[device].xcd_round_robin = rr;
+    if (status_host && !g_device_cache[device].status_host) {
+        g_device_cache[device].status_host = status_host;
+        g_device_cache[device].status_dev = status_dev;
+        g_status_words.fetch_add(1);
+    }
 }
 
 int device_info(int device, DeviceInfo *out) {
@@ -84,6 +98,7 @@ int device_info(int device, DeviceInfo *out) {
         if (hipGetDevice(&device) != hipSuccess) return FASTLSTM_ERR_HIP;
     }
     if (device >= 64) return FASTLSTM_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_device_mu);
     if (cache[device].num_cus == 0) {
         int cus = 0, lds = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
@@ -109,8 +124,41 @@ void probe_device(int device) {
     if (device < 0) device = cur;
     if (device != cur && hipSetDevice(device) != hipSuccess) return;
     const int rr = probe_xcd_round_robin(di.num_cus);
+    int *word = nullptr, *word_dev = nullptr;
+    if (hipHostMalloc(reinterpret_cast<void **>(&word), 64, hipHostMallocMapped) == hipSuccess) {
+        *word = 0;
+        if (hipHostGetDevicePointer(reinterpret_cast<void **>(&word_dev), word, 0) != hipSuccess) {
+            (void)hipHostFree(word);
+            word = word_dev = nullptr;
+        }
+    }
     if (device != cur) (void)hipSetDevice(cur);
-    device_info_set_xcd(device, rr);
+    device_info_set_probe(device, rr, word, word_dev);
+}
+
+// Behind the launches of a recurrent call: carries the abort flag of its workspace to the device's status word.
+__global__ void collect_status_kernel(const WsHeader *hdr, int *status_word) {
+    if (threadIdx.x == 0 && __hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        __hip_atomic_store(status_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// The status word of the current device says that an earlier recurrent call failed: report it once.
+int take_pending_status() {
+    if (g_status_words.load() == 0) return FASTLSTM_OK;   // no device was ever planned for: nothing to look at
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || !di.status_host) return FASTLSTM_OK;
+    if (__atomic_load_n(di.status_host, __ATOMIC_RELAXED) == 0) return FASTLSTM_OK;
+    __atomic_store_n(di.status_host, 0, __ATOMIC_RELAXED);
+    return FASTLSTM_ERR_TIMEOUT;
+}
+
+// Wraps a recurrent entry point: rc of its launches; on success the status collection is enqueued behind them.
+int finish_recurrent(int rc, void *ws, void *stream) {
+    if (rc != FASTLSTM_OK) return rc;
+    DeviceInfo di;
+    if (device_info(-1, &di) != FASTLSTM_OK || !di.status_dev) return rc;
+    collect_status_kernel<<<1, kWave, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const WsHeader *>(ws), di.status_dev);
+    return hipGetLastError() == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
 }
 
 typedef hipError_t (*FwdLauncher)(const FwdParams &, int, int, int, int, int, hipStream_t, int *);
@@ -137,16 +185,9 @@ struct XcdCfg {
 
 // The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
 // and the workspace holds a ring with one slot per exchanged version.
-// Row range of the batch that the XCD-local launches of the calling thread cover (rows == 0: all of
-// it).  A batch with more tiles than one launch holds runs as several launches over row ranges.
-static thread_local int t_xcd_row0 = 0, t_xcd_rows = 0;
-struct XcdRowWindow {
-    XcdRowWindow(int row0, int rows) { t_xcd_row0 = row0; t_xcd_rows = rows; }
-    ~XcdRowWindow() { t_xcd_row0 = 0; t_xcd_rows = 0; }
-};
-
-bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c) {
-    const int B = t_xcd_rows ? t_xcd_rows : B_all;   // rows of this launch
+// `launch_rows`: batch rows of this launch (0: all B_all of them).
+bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c, int launch_rows = 0) {
+    const int B = launch_rows ? launch_rows : B_all;
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
     const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
@@ -167,7 +208,8 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
         const int cand = hts[hi];
         const int frags = (cand / rows) * c->nkw;   // per wave (forward: halved again by the unit split of 8 waves)
         if (H % cand || H / cand > 32 || cand * s < 16 || frags > (backward ? 32 : 64)) continue;
-        const int groups_max = kNumXcd * (32 / (H / cand));
+        // groups per XCD: as many as its 32 CUs hold, and no more than the workspace has barrier counters for
+        const int groups_max = kNumXcd * std::min(32 / (H / cand), kXcdMaxGroups / kNumXcd);
         if (cdiv(B, 16) <= groups_max) { ht = cand; c->ntw = 1; }
         else if (cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
     }
@@ -175,9 +217,10 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
     c->mt = ht / rows;
     c->nwv = backward ? 8 : (c->mt * c->nkw > 32 ? 8 : 4);
     c->n_ht = H / ht;
-    c->gpx = 32 / c->n_ht;
+    c->gpx = std::min(32 / c->n_ht, kXcdMaxGroups / kNumXcd);
     const int bt = 16 * c->ntw;
     c->n_groups = cdiv(B, bt);
+    if (c->n_groups > kNumXcd * c->gpx) return false;   // (the tile loop above guarantees it; the kernels index counters by group)
     c->xslot = (size_t)c->n_groups * c->ntw * c->ks * kFragBytes;
     const size_t slots = backward ? (size_t)T : (size_t)T + 1;
     if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + slots * c->xslot) return false;
@@ -247,9 +290,9 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
 int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
                 int H, int dtype, hipStream_t stream, const void *x = nullptr, const void *Wx = nullptr,
                 const void *bx = nullptr, const void *bh = nullptr, int I = 0, const SecondLayer *second = nullptr,
-                bool dry_run = false) {
+                bool dry_run = false, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
-    if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c)) return 1;
+    if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c, o.rows)) return 1;
     if (second && ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + 1) * 2 * c.xslot) return 2;
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
@@ -258,9 +301,9 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KS = c.ks;
-    p.b_base = t_xcd_row0;
+    p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
-    p.keep = t_keep_activations;
+    p.keep = o.keep;
     p.trace = g_rec_trace;
     p.n_layers = 1;
     if (x) {
@@ -298,21 +341,21 @@ static int xcd_rows_per_launch(int T, int B, int H, int dtype, bool backward, si
     for (int rows : candidates) {
         if (rows >= B) continue;
         XcdCfg c;
-        {
-            const XcdRowWindow w(0, rows);
-            if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c) || c.ntw != 1 || c.n_groups != kNumXcd * c.gpx) continue;
-        }
-        if (B % rows) {
-            const XcdRowWindow w(B - B % rows, B % rows);
-            if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c)) continue;
-        }
+        if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c, rows) || c.ntw != 1 || c.n_groups != kNumXcd * c.gpx) continue;
+        if (B % rows && !select_xcd(T, B, H, dtype, backward, ws_bytes, &c, B % rows)) continue;
         return rows;
     }
     return 0;
 }
-// the barrier counters of the XCD-local kernels start from zero in every launch
+// Between two launches that share a workspace: the barrier counters of the XCD-local kernels start from
+// zero in every launch, and so does the XCD rotation its workgroups agree on (check_xcd_placement).
+__global__ void reset_xcd_state_kernel(WsHeader *hdr, unsigned *counters, size_t n) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) hdr->xcd_rotation = 0;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) counters[i] = 0u;
+}
 static bool clear_xcd_counters(unsigned char *wsb, hipStream_t s) {
-    zero_words_kernel<<<64, 256, 0, s>>>(reinterpret_cast<unsigned *>(wsb + kWsHeaderBytes), kWsCounterBytes / 4);
+    reset_xcd_state_kernel<<<64, 256, 0, s>>>(reinterpret_cast<WsHeader *>(wsb),
+                                              reinterpret_cast<unsigned *>(wsb + kWsHeaderBytes), kWsCounterBytes / 4);
     return hipGetLastError() == hipSuccess;
 }
 
@@ -322,8 +365,8 @@ struct WideCfg {
     int nkw, n_ht, xpg, n_groups, ks, lds;
     size_t xslot;
 };
-bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c) {
-    const int B = t_xcd_rows ? t_xcd_rows : B_all;   // rows of this launch
+bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0) {
+    const int B = rows ? rows : B_all;   // rows of this launch
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
     if (dtype == FASTLSTM_FP32) return false;
@@ -348,22 +391,16 @@ static int wide_rows_per_launch(int T, int B, int H, int dtype, bool backward, s
     const int rows = 64 * (kNumXcd / std::max(1, xpg));
     if (H <= 1024 || rows >= B || rows <= 0) return 0;
     WideCfg c;
-    {
-        const XcdRowWindow w(0, rows);
-        if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c)) return 0;
-    }
-    if (B % rows) {
-        const XcdRowWindow w(B - B % rows, B % rows);
-        if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c)) return 0;
-    }
+    if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c, rows)) return 0;
+    if (B % rows && !select_wide(T, B, H, dtype, backward, ws_bytes, &c, B % rows)) return 0;
     return rows;
 }
 
 // Returns 1 when the kernel does not apply, else a fastlstm_status.
 int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
-                 int H, int dtype, hipStream_t stream) {
+                 int H, int dtype, hipStream_t stream, const LaunchOpts &o = LaunchOpts()) {
     WideCfg c;
-    if (!select_wide(T, B, H, dtype, false, ws_bytes, &c)) return 1;
+    if (!select_wide(T, B, H, dtype, false, ws_bytes, &c, o.rows)) return 1;
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -371,9 +408,9 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KS = c.ks;
-    p.b_base = t_xcd_row0;
+    p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
-    p.keep = t_keep_activations;
+    p.keep = o.keep;
     auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
     int occ = 0;
     if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
@@ -383,9 +420,10 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
 }
 
 int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
-                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream) {
+                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
+                 const LaunchOpts &o = LaunchOpts()) {
     WideCfg c;
-    if (!select_wide(T, B, H, dtype, true, ws_bytes, &c)) return 1;
+    if (!select_wide(T, B, H, dtype, true, ws_bytes, &c, o.rows)) return 1;
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -393,7 +431,7 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KSB = c.ks;
-    p.b_base = t_xcd_row0;
+    p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
     auto launch = dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16;
     int occ = 0;
@@ -518,9 +556,9 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
                 const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false,
-                bool *lower_wgrad_fused = nullptr) {
+                bool *lower_wgrad_fused = nullptr, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
-    if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c)) return 1;
+    if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c, o.rows)) return 1;
     if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * 2 * c.xslot) return 2;
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
@@ -529,7 +567,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
     p.T = T; p.B = B; p.H = H;
     p.n_ht = c.n_ht; p.gpx = c.gpx; p.n_groups = c.n_groups; p.KSB = c.ks;
-    p.b_base = t_xcd_row0;
+    p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
     p.n_layers = 1;
     if (extras) {
@@ -691,8 +729,9 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
     return FASTLSTM_OK;
 }
 
-int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes,
-                            int T, int B, int H, int dtype, void *stream) {
+// keep: see LaunchOpts
+static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
+                               int H, int dtype, void *stream, int keep) {
     if (!ifgo || !out || !cell || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
@@ -709,11 +748,13 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         // also instead of one launch with 32-row tiles of the 8-wave kernel (H = 1024, 16-bit), whose
         // 32-row step costs 2.5 x its 16-row step (the 4-wave kernels of smaller H are faster in one
         // launch with 32-row tiles).
+        const LaunchOpts whole_batch{keep, 0, 0};
         auto by_row_ranges = [&](int rows) {
             for (int r0 = 0; r0 < B; r0 += rows) {
                 if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return (int)FASTLSTM_ERR_HIP;
-                const XcdRowWindow w(r0, std::min(rows, B - r0));
-                const int r = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+                const LaunchOpts o{keep, r0, std::min(rows, B - r0)};
+                const int r = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream),
+                                          nullptr, nullptr, nullptr, nullptr, 0, nullptr, false, o);
                 if (r != FASTLSTM_OK) return r < 0 ? r : (int)FASTLSTM_ERR_RESIDENCY;
             }
             return (int)FASTLSTM_OK;
@@ -721,16 +762,18 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
         XcdCfg whole;
         if (select_xcd(T, B, H, dtype, false, ws_bytes, &whole) && whole.ntw == 2 && whole.nwv == 8)
             if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
-        int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
-        if (rc == 1) rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+        int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream), nullptr,
+                             nullptr, nullptr, nullptr, 0, nullptr, false, whole_batch);
+        if (rc == 1)
+            rc = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream), whole_batch);
         if (rc == 1)
             if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
         if (rc == 1)
             if (const int rows = wide_rows_per_launch(T, B, H, dtype, false, ws_bytes)) {
                 for (int r0 = 0; r0 < B; r0 += rows) {
                     if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
-                    const XcdRowWindow w(r0, std::min(rows, B - r0));
-                    const int r = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream));
+                    const LaunchOpts o{keep, r0, std::min(rows, B - r0)};
+                    const int r = try_fwd_wide(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream), o);
                     if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
                 }
                 return FASTLSTM_OK;
@@ -745,7 +788,7 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
     p.KS = cdiv(H, kstep);
     p.spin_limit = spin_limit_ticks();
-    p.keep = t_keep_activations;
+    p.keep = keep;
     p.trace = g_rec_trace;
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
@@ -792,9 +835,15 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     return FASTLSTM_OK;
 }
 
-int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
-                            void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
-                            int dtype, void *stream) {
+int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
+                            int H, int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(fwd_persistent_impl(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream, 1), ws, stream);
+}
+
+static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
+                               void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
+                               int dtype, void *stream) {
     if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
@@ -817,9 +866,9 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
             if (const int rows = xcd_rows_per_launch(T, B, H, dtype, true, ws_bytes)) {
                 for (int r0 = 0; r0 < B; r0 += rows) {
                     if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
-                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const LaunchOpts o{1, r0, std::min(rows, B - r0)};
                     const int r = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
-                                              static_cast<hipStream_t>(stream));
+                                              static_cast<hipStream_t>(stream), nullptr, nullptr, false, nullptr, o);
                     if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
                 }
                 return FASTLSTM_OK;
@@ -827,9 +876,9 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
             if (const int rows = wide_rows_per_launch(T, B, H, dtype, true, ws_bytes)) {
                 for (int r0 = 0; r0 < B; r0 += rows) {
                     if (r0 && !clear_xcd_counters(wsb, static_cast<hipStream_t>(stream))) return FASTLSTM_ERR_HIP;
-                    const XcdRowWindow w(r0, std::min(rows, B - r0));
+                    const LaunchOpts o{1, r0, std::min(rows, B - r0)};
                     const int r = try_bwd_wide(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
-                                               static_cast<hipStream_t>(stream));
+                                               static_cast<hipStream_t>(stream), o);
                     if (r != FASTLSTM_OK) return r < 0 ? r : FASTLSTM_ERR_RESIDENCY;
                 }
                 return FASTLSTM_OK;
@@ -882,9 +931,17 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     return FASTLSTM_OK;
 }
 
-int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
-                       void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
-                       void *stream) {
+int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
+                            void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
+                            int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream),
+                            ws, stream);
+}
+
+static int fwd_layer_impl(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
+                          void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                          void *stream, int keep) {
     if (!x || !Wx || !bx || !bh || !Wh || !ifgo || !out || !cell || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
@@ -901,20 +958,30 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
         if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
         if (pl.wave_split != 2) {
             const int rc = try_fwd_xcd(ifgo, out, cell, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
-                                       static_cast<hipStream_t>(stream), x, Wx, bx, bh, I);
+                                       static_cast<hipStream_t>(stream), x, Wx, bx, bh, I, nullptr, false,
+                                       LaunchOpts{keep, 0, 0});
             if (rc <= 0) return rc;   // launched, or failed
         }
     }
 #endif
     if (int rc = fastlstm_gemm_ifgo(x, Wx, bx, bh, ifgo, T, B, I, H, dtype, stream)) return rc;
-    return fastlstm_fwd_persistent(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream);
+    return fwd_persistent_impl(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream, keep);
+}
+
+int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
+                       void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                       void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream, 1), ws,
+                            stream);
 }
 
 int fastlstm_fwd_layer_infer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
                              void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
                              void *stream) {
-    const InferenceScope scope;
-    return fastlstm_fwd_layer(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream);
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream, 0), ws,
+                            stream);
 }
 
 size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
@@ -934,10 +1001,10 @@ int fastlstm_fwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
     return rc == FASTLSTM_OK ? 1 : (rc < 0 ? rc : 0);
 }
 
-int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0, void *ifgo0,
-                        void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1, const void *Wh1,
-                        void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H,
-                        int dtype, void *stream) {
+static int fwd_stack2_impl(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0, void *ifgo0,
+                           void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1, const void *Wh1,
+                           void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H,
+                           int dtype, void *stream, int keep) {
     if (!x || !Wx0 || !bx0 || !bh0 || !Wh0 || !ifgo0 || !out0 || !cell0 || !Wx1 || !bx1 || !bh1 || !Wh1 || !ifgo1 ||
         !out1 || !cell1 || !ws)
         return FASTLSTM_ERR_NULL;
@@ -955,33 +1022,44 @@ int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const v
     if (pl.wave_split != 2) {
         const SecondLayer second{Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1};
         const int rc = try_fwd_xcd(ifgo0, out0, cell0, Wh0, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype, s, x,
-                                   Wx0, bx0, bh0, I, &second);
+                                   Wx0, bx0, bh0, I, &second, false, LaunchOpts{keep, 0, 0});
         if (rc <= 0) return rc;   // both layers in one launch, or failed
     }
 #endif
     // one layer after the other, the second on the first one's out[1:]; the workspace is cleared in between
-    if (int rc = fastlstm_fwd_layer(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, ws, ws_bytes, T, B, I, H, dtype, stream))
+    if (int rc = fwd_layer_impl(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, ws, ws_bytes, T, B, I, H, dtype, stream, keep))
         return rc;
     const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
     zero_words_kernel<<<256, 256, 0, s>>>(static_cast<unsigned *>(ws), zero / 4);
     if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
     const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
-    return fastlstm_fwd_layer(x1, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws, ws_bytes, T, B, H, H, dtype, stream);
+    return fwd_layer_impl(x1, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws, ws_bytes, T, B, H, H, dtype, stream, keep);
+}
+
+int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0, void *ifgo0,
+                        void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1, const void *Wh1,
+                        void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(fwd_stack2_impl(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1,
+                                            ws, ws_bytes, T, B, I, H, dtype, stream, 1),
+                            ws, stream);
 }
 
 int fastlstm_fwd_stack2_infer(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0,
                               void *ifgo0, void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1,
                               const void *Wh1, void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T,
                               int B, int I, int H, int dtype, void *stream) {
-    const InferenceScope scope;
-    return fastlstm_fwd_stack2(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1, ws,
-                               ws_bytes, T, B, I, H, dtype, stream);
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(fwd_stack2_impl(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1,
+                                            ws, ws_bytes, T, B, I, H, dtype, stream, 0),
+                            ws, stream);
 }
 
-int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
-                       const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
-                       void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
-                       int H, int dtype, void *stream) {
+static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
+                          const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
+                          void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
+                          int H, int dtype, void *stream) {
     if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !x || !h || !dx || !dWx || !dWh || !db ||
         !ws || !wgrad_ws)
         return FASTLSTM_ERR_NULL;
@@ -1013,12 +1091,22 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
                    : FASTLSTM_ERR_HIP;
     }
     if (rc != 3) {   // nothing was launched: recurrence, then dx
-        if (int r2 = fastlstm_bwd_persistent(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
+        if (int r2 = bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
             return r2;
         // (the weight-gradient workspace is free until the next call: scratch for a split along K)
         if (int r2 = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, wgrad_ws, wgrad_ws_bytes, stream)) return r2;
     }
     return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
+}
+
+int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
+                       const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
+                       void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
+                       int H, int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(bwd_layer_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, Wx, x, h, dx, dWx, dWh, db, ws, ws_bytes,
+                                           wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream),
+                            ws, stream);
 }
 
 size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
@@ -1039,12 +1127,12 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
     return (rc == FASTLSTM_OK || rc == 3) ? 1 : (rc < 0 ? rc : 0);
 }
 
-int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1, void *d_ifgo1,
-                        const void *Wh1, const void *Wx1, const void *out1, void *dWx1, void *dWh1, void *db1, void *dx1,
-                        void *dh0, void *dc0, const void *ifgo0, const void *cell0, void *d_ifgo0, const void *Wh0,
-                        const void *Wx0, const void *x, const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0,
-                        void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
-                        int dtype, void *stream) {
+static int bwd_stack2_impl(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1, void *d_ifgo1,
+                           const void *Wh1, const void *Wx1, const void *out1, void *dWx1, void *dWh1, void *db1, void *dx1,
+                           void *dh0, void *dc0, const void *ifgo0, const void *cell0, void *d_ifgo0, const void *Wh0,
+                           const void *Wx0, const void *x, const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0,
+                           void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
+                           int dtype, void *stream) {
     if (!dout || !dh1 || !dc1 || !ifgo1 || !cell1 || !d_ifgo1 || !Wh1 || !Wx1 || !out1 || !dWx1 || !dWh1 || !db1 || !dx1 ||
         !dh0 || !dc0 || !ifgo0 || !cell0 || !d_ifgo0 || !Wh0 || !Wx0 || !x || !out0 || !dx0 || !dWx0 || !dWh0 || !db0 ||
         !ws || !wgrad_ws)
@@ -1088,14 +1176,27 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
             return fastlstm_gemm_wgrad(d_ifgo0, x, out0, dWx0, dWh0, db0, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
     }
     // one layer after the other; the workspace is cleared in between
-    if (int rc = fastlstm_bwd_layer(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, x1, out1, dx1, dWx1, dWh1, db1, ws,
-                                    ws_bytes, wgrad_ws, wgrad_ws_bytes, T, B, H, H, dtype, stream))
+    if (int rc = bwd_layer_impl(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, x1, out1, dx1, dWx1, dWh1, db1, ws, ws_bytes,
+                                wgrad_ws, wgrad_ws_bytes, T, B, H, H, dtype, stream))
         return rc;
     const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
     zero_words_kernel<<<256, 256, 0, s>>>(static_cast<unsigned *>(ws), zero / 4);
     if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
-    return fastlstm_bwd_layer(dx1, dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, db0, ws, ws_bytes,
-                              wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
+    return bwd_layer_impl(dx1, dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, db0, ws, ws_bytes, wgrad_ws,
+                          wgrad_ws_bytes, T, B, I, H, dtype, stream);
+}
+
+int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1, void *d_ifgo1,
+                        const void *Wh1, const void *Wx1, const void *out1, void *dWx1, void *dWh1, void *db1, void *dx1,
+                        void *dh0, void *dc0, const void *ifgo0, const void *cell0, void *d_ifgo0, const void *Wh0,
+                        const void *Wx0, const void *x, const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0,
+                        void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
+                        int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    return finish_recurrent(bwd_stack2_impl(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, out1, dWx1, dWh1, db1, dx1, dh0, dc0,
+                                            ifgo0, cell0, d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, db0, ws, ws_bytes,
+                                            wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream),
+                            ws, stream);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
@@ -1115,6 +1216,15 @@ int fastlstm_ws_status(const void *ws_head) {
     return h->abort_flag ? FASTLSTM_ERR_TIMEOUT : FASTLSTM_OK;
 }
 
+int fastlstm_device_status(int device, int clear) {
+    if (fastlstm::g_status_words.load() == 0) return FASTLSTM_OK;
+    DeviceInfo di;
+    if (int rc = device_info(device, &di)) return rc;
+    if (!di.status_host || __atomic_load_n(di.status_host, __ATOMIC_RELAXED) == 0) return FASTLSTM_OK;
+    if (clear) __atomic_store_n(di.status_host, 0, __ATOMIC_RELAXED);
+    return FASTLSTM_ERR_TIMEOUT;
+}
+
 void fastlstm_set_spin_limit(long long ticks) {
     if (ticks > 0) fastlstm::g_spin_limit.store(ticks);
 }
@@ -1130,7 +1240,9 @@ const char *fastlstm_strerror(int status) {
             return "the W_h slice does not fit in LDS or the barrier group cannot be co-resident";
         case FASTLSTM_ERR_WORKSPACE: return "workspace is smaller than required";
         case FASTLSTM_ERR_HIP: return "a HIP runtime call failed";
-        case FASTLSTM_ERR_TIMEOUT: return "a barrier wait timed out (results are invalid)";
+        case FASTLSTM_ERR_TIMEOUT:
+            return "a recurrent launch on this device gave up a barrier wait or found a workgroup on the wrong XCD "
+                   "(the results of that call are invalid)";
         default: return "unknown status";
     }
 }

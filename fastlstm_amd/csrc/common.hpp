@@ -116,7 +116,8 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 struct WsHeader {
     int abort_flag;  // set to 1 by the first barrier wait that times out
     int timeout_group, timeout_step, timeout_seen;
-    int reserved[60];
+    int xcd_rotation;  // 1 + (XCD of a workgroup - its id) mod 8, agreed on by the workgroups of an XCD-placed launch
+    int reserved[59];
 };
 static_assert(sizeof(WsHeader) == 256, "workspace header is 256 bytes");
 

@@ -303,6 +303,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         }
         return;
     }
+    check_xcd_placement(p.hdr);
     const bool lower = HELP == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
     const int g = lower ? vg - p.n_groups : vg;
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch

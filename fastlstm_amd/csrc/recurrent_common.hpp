@@ -19,8 +19,6 @@
 //    (the data crosses the fabric once per XCD instead of once per CU);
 //  * coherent loads (sc1, miss the non-coherent cache levels): used when the workspace is
 //    too small for T+1 slots, or when two workgroups write parts of the same 128-byte line.
-// Setting kDeviceScopeExchange to false selects plain accesses bracketed by a
-// device-scope release/acquire fence pair instead (L2 write-back + invalidate per step).
 // Every wait is bounded: after `spin_limit` ticks of the 100 MHz clock it raises an
 // abort flag in the workspace header that ends every other wait as well, so the grid
 // always drains.
@@ -29,7 +27,6 @@
 
 namespace fastlstm {
 
-constexpr bool kDeviceScopeExchange = true;
 constexpr int kAuxDevice = 16;  // buffer-instruction cache policy: sc1 = device scope
 
 // Exchange buffer in global memory, addressed through a buffer resource so that the
@@ -41,26 +38,21 @@ struct XchgGlobal {
         : rsrc(__builtin_amdgcn_make_buffer_rsrc(b, 0, bytes, 0x00020000)), base(b) {}
     // COHERENT: device-scope load (sc1); otherwise an ordinary cached load
     template <bool COHERENT> __device__ __forceinline__ u32x4 load16(unsigned off) const {
-        if constexpr (!kDeviceScopeExchange) return *reinterpret_cast<const u32x4 *>(base + off);
-        else if constexpr (COHERENT) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAuxDevice);
+        if constexpr (COHERENT) return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAuxDevice);
         else return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
     }
     template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
-        if constexpr (!kDeviceScopeExchange) {
-            *reinterpret_cast<T *>(base + off) = v;
-        } else if constexpr (sizeof(T) == 2) {
+        if constexpr (sizeof(T) == 2) {
             __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rsrc, off, 0, kAuxDevice);
         } else {
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rsrc, off, 0, kAuxDevice);
         }
     }
     __device__ __forceinline__ void store8(unsigned off, u32x2 v) const {
-        if constexpr (kDeviceScopeExchange) __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, off, 0, kAuxDevice);
-        else *reinterpret_cast<u32x2 *>(base + off) = v;
+        __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, off, 0, kAuxDevice);
     }
     __device__ __forceinline__ void store16(unsigned off, u32x4 v) const {
-        if constexpr (kDeviceScopeExchange) __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, 0, kAuxDevice);
-        else *reinterpret_cast<u32x4 *>(base + off) = v;
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, 0, kAuxDevice);
     }
 };
 
@@ -119,8 +111,7 @@ __device__ __forceinline__ void wait_versions(const int *flags, int n, int targe
             }
         }
     }
-    if constexpr (kDeviceScopeExchange) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only
-    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only: the data is read at device scope
 }
 
 // Called by all threads of the workgroup after they stored the data of `version`.
@@ -129,9 +120,33 @@ __device__ __forceinline__ void publish_version(int *flag, int version) {
     // barrier, then one thread raises the flag
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(flag, version, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Members of a barrier group that is placed by XCD.  The hardware deals the workgroups of a dispatch to
+// the 8 XCDs in turn, but not always starting with XCD 0 (seen: a dispatch replayed from a HIP graph, and
+// eager dispatches after it, start at another XCD): workgroup i runs on XCD (i + r) % 8 with one r per
+// dispatch.  The grouping i % 8 == group % 8 puts a group on ONE XCD for every r, which is all the kernels
+// need.  What they cannot survive is a dispatch without a common r: a member on another XCD than its
+// peers would exchange through the wrong L2 and read stale lines without ever timing out.  So every
+// member checks: the first one to arrive records its r in the workspace header, every other one
+// compares, and a mismatch raises the abort flag (ends every wait of the launch; timeout_group = -3,
+// timeout_step = the workgroup id, timeout_seen = its XCD).  One register read and one atomic per workgroup
+// and launch.
+__device__ __forceinline__ void check_xcd_placement(WsHeader *hdr) {
     if (threadIdx.x == 0) {
-        if constexpr (kDeviceScopeExchange) __hip_atomic_store(flag, version, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else __hip_atomic_store(flag, version, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        const int mine = 1 + (int)(((xcc & 15u) + kNumXcd - blockIdx.x % kNumXcd) % kNumXcd);
+        int expected = 0;
+        if (!__hip_atomic_compare_exchange_strong(&hdr->xcd_rotation, &expected, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT) &&
+            expected != mine) {
+            hdr->timeout_group = -3;
+            hdr->timeout_step = (int)blockIdx.x;
+            hdr->timeout_seen = (int)(xcc & 15u);
+            __hip_atomic_store(&hdr->abort_flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int g = xcd / xpg, j = (xcd % xpg) * 32 + slot;
     if (g >= p.n_groups || j >= p.n_ht) return;
+    check_xcd_placement(p.hdr);
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                       // [8][TILES][64]

@@ -3,11 +3,12 @@
 //
 // Same mathematics and the same results as lstm_fwd_persistent_kernel (which replaces
 // fastlstm/kernels.py:414-663); what differs is where the data travels:
-//  * placement: the hardware deals workgroup i to XCD i % 8.  A barrier group takes its members
-//    from the workgroups of one XCD (i % 8 == group % 8); workgroups that are not needed return
-//    at once.  One workgroup fills the register file of a CU, so the up to 32 members of a group
-//    sit on the 32 CUs of their XCD.  The host verifies i % 8 == XCC_ID once per device before
-//    it selects this kernel;
+//  * placement: the hardware deals the workgroups of a dispatch to the XCDs in turn: workgroup i runs on
+//    XCD (i + r) % 8, with one rotation r per dispatch.  A barrier group takes its members from the
+//    workgroups with i % 8 == group % 8, which share an XCD whatever r is; workgroups that are not needed
+//    return at once.  One workgroup fills the register file of a CU, so the up to 32 members of a group
+//    sit on the 32 CUs of their XCD.  The host verifies the dealing once per device before it selects this
+//    kernel, and every launch verifies that its workgroups saw one common r (check_xcd_placement);
 //  * exchange data: ordinary stores (the vector L1 writes through to L2) and ordinary loads.  A
 //    load may hit in the CU's L1, which nobody keeps coherent, so every timestep writes a slot
 //    of its own (ring of T + 1 slots): an address is only read after its single write;
@@ -33,6 +34,7 @@ constexpr int kXcdCounterStride = 32;    // ints between replicas
 constexpr int kXcdGroupStride = kXcdReplicas * kXcdCounterStride;   // ints between groups (1 KiB)
 constexpr int kXcdMaxGroups = 64;
 static_assert((size_t)kXcdMaxGroups * kXcdGroupStride * sizeof(int) == kWsCounterBytes, "counter region of the workspace");
+static_assert(kXcdMaxGroups % kNumXcd == 0, "the same number of groups on every XCD");
 
 struct FwdXcdParams {
     void *ifgo;        // [T,B,4H] in: x.Wx^T+b, out: full pre-activations
@@ -255,6 +257,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         }
         return;
     }
+    check_xcd_placement(p.hdr);
     const int layer = vg / p.n_groups, g = vg % p.n_groups;   // layer 1: the second of a stack
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k1_live = HELP && p.k1_tiles_n > 0;

@@ -31,8 +31,9 @@ dtype_str = {  # fastlstm/lstm.py:24-28
 _DTYPE_CODE = {torch.float32: _lib.FP32, torch.float16: _lib.FP16, torch.bfloat16: _lib.BF16}
 
 # When set, every recurrent launch is followed by a device sync and a check of the
-# workspace status word (barrier time-out detection).  Off by default: the calls
-# are fully asynchronous, as in the reference.
+# workspace status word (barrier time-out detection at the failing call itself).  Off by
+# default: the calls are fully asynchronous, as in the reference, and a failed launch is
+# reported by the NEXT library call on the device (fastlstm_device_status, no sync).
 CHECK_STATUS = os.environ.get("FASTLSTM_CHECK_STATUS", "0") == "1"
 
 
@@ -87,7 +88,11 @@ def _check_ws(ws, what):
     # (reading the status word synchronises: not while the stream is being captured into a graph)
     if CHECK_STATUS and not torch.cuda.is_current_stream_capturing():
         head = ws[:64].cpu().numpy().tobytes()  # synchronises
-        _lib.check(_lib.load().fastlstm_ws_status(head), what)
+        status = _lib.load().fastlstm_ws_status(head)
+        if status != _lib.OK:
+            # reported here: the device's sticky status word need not report it again at the next call
+            _lib.load().fastlstm_device_status(ws.device.index, 1)
+        _lib.check(status, what)
 
 
 def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None, keep_activations=True):

@@ -224,6 +224,19 @@ int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward,
  * to completion, its results are invalid). */
 int fastlstm_ws_status(const void *ws_head);
 
+/* Failure reporting without a host synchronisation.  The first fastlstm_plan_device call for a device
+ * allocates one pinned, device-visible status word for it.  Every recurrent entry point
+ * (fastlstm_fwd_persistent, _fwd_layer[_infer], _fwd_stack2[_infer], _bwd_persistent, _bwd_layer,
+ * _bwd_stack2) enqueues, behind its launches, one tiny kernel that sets the word if the call's workspace
+ * ended with the abort flag raised (a barrier wait gave up, or a workgroup of an XCD-placed barrier group
+ * found itself on another XCD than the one the placement rule assumes).  The NEXT recurrent entry on that
+ * device then returns FASTLSTM_ERR_TIMEOUT before launching anything and clears the word: the results
+ * of the earlier call are invalid, and the caller learns it at most one call late instead of never.
+ * fastlstm_device_status reads the word of `device` (-1: current) at any time: FASTLSTM_OK or
+ * FASTLSTM_ERR_TIMEOUT; clear != 0 resets it.  It reflects the calls whose work has completed on the
+ * device by now.  No counterpart in the reference (its spin loops are unbounded, fastlstm/kernels.py:546-548). */
+int fastlstm_device_status(int device, int clear);
+
 /* Upper bound, in 100 MHz ticks, a barrier wait may spin before it gives up
  * (default 4e8 = 4 s).  Tests lower it to force the time-out path from the host. */
 void fastlstm_set_spin_limit(long long ticks);

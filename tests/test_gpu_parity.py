@@ -103,6 +103,8 @@ STAGE_CASES = [
     (4, 200, 64, 1024, torch.bfloat16),   # forward in two row ranges (128 + 72), reverse in one launch of 32-row tiles
     (3, 200, 64, 2048, torch.float16),    # register-resident kernels over two row ranges (128 + 72)
     (3, 40, 64, 512, torch.float32),
+    (2, 2100, 16, 96, torch.float16),     # 3 members per group: 10 groups would fit an XCD's CUs, the workspace has
+                                          # barrier counters for 8 per XCD -- 66 tiles of 32 rows must not run as one launch
 ]
 
 
@@ -375,7 +377,15 @@ def test_barrier_timeout_is_reported_not_hung():
         assert launch() == _lib.ERR_TIMEOUT
     finally:
         lib.fastlstm_set_spin_limit(400000000)
+    # the device's sticky status word saw it too (no sync needed to read it); the next entry point on the
+    # device reports the failure once, before launching anything, and the one after is healthy
+    assert lib.fastlstm_device_status(0, 0) == _lib.ERR_TIMEOUT
+    ws = torch.zeros(plan.ws_bytes, dtype=torch.uint8, device="cuda")
+    args = (ifgo.clone().data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(), ws.data_ptr(), ws.numel(), T, B, H, code, st)
+    assert lib.fastlstm_fwd_persistent(*args) == _lib.ERR_TIMEOUT
+    assert lib.fastlstm_device_status(0, 0) == _lib.OK
     assert launch() == _lib.OK  # and the next launch is healthy
+    assert lib.fastlstm_device_status(0, 0) == _lib.OK
     assert torch.isfinite(out.float()).all()
 
 
@@ -770,7 +780,9 @@ def test_xcd_local_barrier_timeout_is_reported_not_hung():
         assert launch() == _lib.ERR_TIMEOUT
     finally:
         lib.fastlstm_set_spin_limit(400000000)
+    assert lib.fastlstm_device_status(0, 1) == _lib.ERR_TIMEOUT   # read and cleared
     assert launch() == _lib.OK
+    assert lib.fastlstm_device_status(0, 0) == _lib.OK
     assert torch.isfinite(out.float()).all()
 
 
@@ -803,6 +815,7 @@ def test_stacked_and_wide_launches_drain_on_timeout(T, B, I, H, dt):
             run()
     finally:
         lib.fastlstm_set_spin_limit(400000000)
+    assert lib.fastlstm_device_status(0, 0) == _lib.OK   # the host mirror cleared the sticky word when it raised
     try:
         o, r = run()   # healthy again, still with status checks
     finally:
@@ -1057,6 +1070,61 @@ def test_forward_replays_from_a_captured_graph(T, B, I, H, layers, dt):
                 torch.cuda.synchronize()
                 assert torch.equal(y, eager[i]), (rep, i)
                 (torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")).sum().item()
+
+
+@pytest.mark.parametrize("T,B,I,H,layers,dt", [(16, 20, 24, 64, 1, torch.float16),      # one hidden tile per workgroup
+                                               (32, 64, 256, 1024, 1, torch.float16),   # XCD-local, GEMMs inside both launches
+                                               (40, 32, 128, 1024, 2, torch.float16)])  # two layers per launch, both directions
+def test_training_step_replays_from_a_captured_graph(T, B, I, H, layers, dt):
+    """Forward AND backward of the module captured into one HIP graph, the whole-network recipe of
+    PyTorch's CUDA-graph notes: warm-up on a side stream, gradients set to None, and no tensor of an earlier
+    autograd graph alive when the capture starts (an AccumulateGrad node kept alive from a step on another
+    stream makes the autograd engine add cross-stream event waits to the capture, which ends it with a
+    host crash inside hipStreamEndCapture -- a property of the capture, not of these kernels).  Every replay,
+    with new input contents, gives the eager step's output and parameter gradients bit for bit."""
+    import gc
+    torch.manual_seed(0)
+    m = FastLSTM(I, H, num_layers=layers).to("cuda", dt)
+    xs = [torch.randn(T, B, I, device="cuda").to(dt) for _ in range(3)]
+    ws = [torch.randn(T, B, H, device="cuda").to(dt) for _ in range(3)]
+    sx, sw = xs[0].clone(), ws[0].clone()
+
+    def step():
+        y, _ = m(sx)
+        (y * sw).sum().backward()
+        return y.detach()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            m.zero_grad(set_to_none=True)
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    m.zero_grad(set_to_none=True)
+    gc.collect()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sy = step()
+    replayed = []
+    for rep in range(2):
+        for i in range(3):
+            sx.copy_(xs[i]); sw.copy_(ws[i])
+            graph.replay()
+            torch.cuda.synchronize()
+            replayed.append((sy.clone(), [prm.grad.clone() for prm in m.parameters()]))
+            (torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")).sum().item()
+    for rep in range(2):
+        for i in range(3):
+            sx.copy_(xs[i]); sw.copy_(ws[i])
+            m.zero_grad(set_to_none=True)
+            y = step()
+            torch.cuda.synchronize()
+            gy, gp = replayed[rep * 3 + i]
+            assert torch.equal(gy, y), (rep, i)
+            for prm, gr in zip(m.parameters(), gp):
+                assert torch.equal(prm.grad, gr), (rep, i)
 
 
 # --------------------------------------------------------------------------------------

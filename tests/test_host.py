@@ -263,3 +263,11 @@ def test_oracle_matches_golden_vectors(oracle):
         if g("h0") is not None:
             np.testing.assert_allclose(r["dh0"], z[name + "/out/dh0"], rtol=1e-9, atol=1e-10)
             np.testing.assert_allclose(r["dc0"], z[name + "/out/dc0"], rtol=1e-9, atol=1e-10)
+
+
+def test_device_status_without_a_planned_device_is_ok():
+    """No planning call was made (there is no GPU here), so no status word exists: the query answers OK
+    without touching the HIP runtime, and so does the look every recurrent entry point takes first."""
+    lib = _lib.load()
+    assert lib.fastlstm_device_status(-1, 0) == _lib.OK
+    assert lib.fastlstm_device_status(0, 1) == _lib.OK
