@@ -45,6 +45,8 @@ SIGNATURES = {
     "fastlstm_fwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_layer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_layer_infer": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_fwd_layer_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_noalloc_scratch_bytes": (_sz, []),
     "fastlstm_bwd_layer": (_i, [_vp] * 15 + [_sz, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_gemm_dx": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -984,6 +984,55 @@ int fastlstm_fwd_layer_infer(const void *x, const void *Wx, const void *bx, cons
                             stream);
 }
 
+// ---- fastlstm_fwd_layer for callers that cannot allocate ---------------------------------------
+// The recurrence workspace lives in a file-scope device array instead of coming in as an argument.
+// In host code the array's NAME is only a stand-in (a kernel given it faults): its device address is
+// looked up once per device with hipGetSymbolAddress and kept; every use below goes through that pointer.
+constexpr size_t kNoAllocScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static unsigned char *g_scratch_ptr[64];   // per device, under g_scratch_mu
+static std::mutex g_scratch_mu;
+
+// Device address of this device's copy of `scratch` (each GPU holds its own copy at its own address).
+static int scratch_of_current_device(unsigned char **out) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return FASTLSTM_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return FASTLSTM_ERR_HIP;
+        g_scratch_ptr[device] = static_cast<unsigned char *>(ptr);
+    }
+    *out = g_scratch_ptr[device];
+    return FASTLSTM_OK;
+}
+
+size_t fastlstm_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+
+int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
+                               void *out, void *cell, int T, int B, int I, int H, int dtype, void *stream) {
+    if (!x || !Wx || !bx || !bh || !Wh || !ifgo || !out || !cell) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (int rc = take_pending_status()) return rc;
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
+    // the smallest workspace of this shape has to fit; beyond that the call uses as much of the array
+    // as a ring with one slot per timestep would take (more slots = the faster kernels, as with any workspace)
+    if (pl.ws_bytes > kNoAllocScratchBytes) return FASTLSTM_ERR_WORKSPACE;
+    const size_t ring = fastlstm_recurrent_workspace_bytes(&pl, T, H, dtype, 0);
+    const size_t use = std::min(kNoAllocScratchBytes, std::max(ring, pl.ws_bytes));
+    unsigned char *ptr = nullptr;
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    // the array keeps the last call's contents: clear what this call needs zeroed (a fill kernel, so the
+    // call can be captured into a graph)
+    const size_t zero = pl.ring_needs_zero ? use : std::min(use, pl.ws_zero_bytes);
+    zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(reinterpret_cast<unsigned *>(ptr), zero / 4);
+    if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+    return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ptr, use, T, B, I, H, dtype, stream, 1), ptr,
+                            stream);
+}
+
 size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
     const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 0);
     if (!plan || one == 0 || plan->wave_split == 2) return one;

@@ -115,6 +115,23 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
                        void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I,
                        int H, int dtype, void *stream);
 
+/* fastlstm_fwd_layer without a workspace argument and without any allocation.  No counterpart in the
+ * reference; it is for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The recurrence workspace is a static device array of
+ * fastlstm_noalloc_scratch_bytes() = 16 MiB inside the library (every GPU the library runs on holds its
+ * own copy until the process ends); the call clears the part it needs zeroed itself and calls no
+ * hipMalloc/hipFree.  Same results as fastlstm_fwd_layer with a zeroed workspace of
+ * min(16 MiB, fastlstm_recurrent_workspace_bytes(forward plan)) bytes -- the kernel choice follows the
+ * workspace size as it does there (XCD-local kernels while a slot per timestep fits, else the general
+ * ones).  FASTLSTM_ERR_WORKSPACE if the smallest workspace of the shape (plan.ws_bytes) exceeds the array.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; serialise them.  The XCD-local kernels are only chosen on a device that fastlstm_plan_device has
+ * seen (that call probes and may allocate; this one never does). */
+int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh,
+                               void *ifgo, void *out, void *cell, int T, int B, int I, int H, int dtype,
+                               void *stream);
+size_t fastlstm_noalloc_scratch_bytes(void);
+
 /* fastlstm_fwd_layer for a forward pass that no reverse pass follows (the reference decides this per
  * call from torch.is_grad_enabled / requires_grad and still stores everything, fastlstm/lstm.py:
  * 507-522): out[1..T] and cell[T] are the same bits as fastlstm_fwd_layer writes; the recurrence
