@@ -2,24 +2,33 @@
 """Benchmark of the LSTM hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload B|A|C|D|E] [--no-cpu] [--no-miopen]
+                    [--stage all|fwd_recurrence|gemms|fwd_layer|bwd_layer]
 
 A "step" is one pass of the workload's hot path over one batch of synthetic input
 (already resident in HBM).  The default workload is BASELINE.json's headline
 configuration B: single-layer fp16 FORWARD, batch 64, seq_len 512, input = hidden =
 1024 (x ~ N(0,1), h0,c0 ~ N(0,0.1), weights U(+-1/32), seeded).  Prints ONE JSON
 line: metric/value = batch*timesteps per second of that step, plus
-  roofline      for the dominant kernel (the persistent recurrence), measured with HIP
-                events on the launch stream,
+  roofline      for the dominant kernel (the launch that holds the persistent recurrence), timed with
+                HIP events on the launch stream: its algorithmic flops against the MFMA peak and, in
+                roofline.latency_bound, its time per timestep against the measured latency floor of a
+                step (barrier round trip + exchange of h_t, fastlstm_diag_step_probe),
   kernels       per-stage timings (input-projection GEMM, recurrence, and for the
                 forward+backward pass: reverse recurrence, dx GEMM, weight-gradient GEMMs),
-  fwd_bwd       the same workload timed forward+backward (loss = sum(out)),
+  fwd / fwd_bwd the workload timed forward and forward+backward (hot loop, mean of --steps calls),
+  do_bench      the same two with the protocol of the reference's scripts/benchmark.py:118-133
+                (triton.testing.do_bench: warm-up 40 ms, 160 ms of repetitions, the L2-sized buffer
+                cleared before each one, one event pair per repetition, median),
   nn_lstm_rocm  torch.nn.LSTM (MIOpen) on the same GPU, same shapes and dtype,
-  cpu_baseline  the CPU oracle (C, OpenMP) on a bounded sample of the same workload,
-  nn_lstm_cpu   torch.nn.LSTM on the host CPU cores on the same sample.
+  cpu_baseline  torch.nn.LSTM fp32 on the box's host cores (physical cores, stated) on the same workload,
+  cpu_oracle    the CPU oracle (C, OpenMP) on a bounded sample.
+The --stage values other than "all" launch a few repetitions of one group of kernels plus a plain
+copy of known size and print nothing: they are the targets of rocprofv3 counter runs (profiles/).
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -36,9 +45,30 @@ WORKLOADS = {
 }
 PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the fused forward layer kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE,
-# scaled by a plain copy of known size (profiles/fwd_layer_B_pmc.md); None = not measured
-TRAFFIC_BYTES = {"B": 1575.6e6, "D": 336.1e6}   # D: the recurrence kernel alone (profiles/fwd_recurrence_D_pmc.md)
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain
+# copy of known size.  Counters cannot be read from inside this process: the figures are copied from the
+# committed summaries named here (made by `rocprofv3 --pmc ... -- python3 bench.py --stage fwd_recurrence`).
+TRAFFIC = {"B": (1575.6e6, "profiles/fwd_layer_B_pmc.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
+
+
+def physical_cores():
+    """Physical cores this process may use: distinct (package, core) pairs of the CPUs in its affinity
+    mask, capped by OMP_NUM_THREADS (the box's CPU share)."""
+    allowed = os.sched_getaffinity(0)
+    seen = set()
+    try:
+        for cpu in allowed:
+            base = "/sys/devices/system/cpu/cpu%d/topology/" % cpu
+            with open(base + "physical_package_id") as f:
+                pkg = f.read().strip()
+            with open(base + "core_id") as f:
+                core = f.read().strip()
+            seen.add((pkg, core))
+        n = len(seen)
+    except OSError:
+        n = len(allowed)
+    cap = os.environ.get("OMP_NUM_THREADS")
+    return max(1, min(n, int(cap)) if cap else n)
 
 
 def main():
@@ -49,8 +79,8 @@ def main():
     ap.add_argument("--workload", default="B", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-miopen", action="store_true", help="skip the nn.LSTM-on-ROCm leg")
-    ap.add_argument("--stage", default="all", choices=["all", "fwd_recurrence"],
-                    help="fwd_recurrence: launch only the dominant kernel and a calibration copy (for counter runs)")
+    ap.add_argument("--stage", default="all", choices=["all", "fwd_recurrence", "gemms", "fwd_layer", "bwd_layer"],
+                    help="other than all: launch only that group of kernels and a calibration copy (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the LSTM recurrence is not sharded across "
@@ -121,14 +151,41 @@ def main():
                 total += s.elapsed_time(e)
         return total / reps
 
-    headline = step_fwd if mode == "fwd" else step_fwd_bwd
-    with torch.enable_grad():
-        ms = timed(headline, args.steps, args.warmup)
-        ms_fwd = ms if mode == "fwd" else timed(step_fwd, args.steps, args.warmup)
-        ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), 2)
-    value = B * T / (ms * 1e-3)
+    flush_buf = torch.empty(256 << 20, dtype=torch.uint8, device=dev)   # as triton's do_bench: 256 MB
 
-    # ---- per-stage device times through the C ABI (layer-0 shapes) -----------------------
+    def do_bench(fn, warmup_ms=40.0, rep_ms=160.0):
+        """triton.testing.do_bench(fn, warmup, rep, return_mode="median") restated: one untimed call,
+        estimate = mean of 5 calls, n = ms / estimate repetitions; before every repetition the cache-sized
+        buffer is cleared; one event pair per repetition, one synchronisation at the end; the median."""
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            flush_buf.zero_()
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        est = s.elapsed_time(e) / 5
+        if T < 128:            # the reference scales both for small problems (scripts/benchmark.py:118-131)
+            warmup_ms, rep_ms = warmup_ms * 1.5, rep_ms * 3
+        if H < 128:
+            warmup_ms, rep_ms = warmup_ms * 1.5, rep_ms * 3
+        if B < 32:
+            warmup_ms, rep_ms = warmup_ms * 1.5, rep_ms * 3
+        n_warm, n_rep = max(1, int(warmup_ms / est)), max(1, int(rep_ms / est))
+        for _ in range(n_warm):
+            fn()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_rep)]
+        for s, e in evs:
+            flush_buf.zero_()
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        return statistics.median(s.elapsed_time(e) for s, e in evs), n_rep
+
+    # ---- per-stage launches through the C ABI (layer-0 shapes) ---------------------------
     stream = torch.cuda.current_stream().cuda_stream
     Wx, Wh = model.weight_ih_l0.detach(), model.weight_hh_l0.detach()
     bx, bh = model.bias_ih_l0.detach(), model.bias_hh_l0.detach()
@@ -141,9 +198,8 @@ def main():
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
     # the workspaces lstm.py allocates per call (a one-slot-per-timestep exchange ring when it fits)
-    from fastlstm_amd import lstm as _host
-    ws_f = _host._workspace(plan_f, T, H, code, False, dev)
-    ws_b = _host._workspace(plan_b, T, H, code, True, dev)
+    ws_f = L._workspace(plan_f, T, H, code, False, dev)
+    ws_b = L._workspace(plan_b, T, H, code, True, dev)
 
     def zero_ws(ws, plan):  # the part a call needs zeroed: header, counters, flags
         n = ws.numel() if (plan.ring_needs_zero or ws.numel() == plan.ws_bytes) else plan.ws_zero_bytes
@@ -170,36 +226,6 @@ def main():
         _lib.check(lib.fastlstm_fwd_layer_infer(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
                                                 ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws_f.data_ptr(),
                                                 ws_f.numel(), T, B, I, H, code, stream), "fwd_layer_infer")
-
-    if args.stage == "fwd_recurrence":
-        # counter runs (rocprofv3 --pmc): the dominant kernel plus a plain copy of known size
-        # (2 x 256 MiB of traffic) that calibrates FETCH_SIZE / WRITE_SIZE
-        k1()
-        cal_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-        cal_dst = torch.empty_like(cal_src)
-        for _ in range(3):
-            rec_fwd_pre()
-            rec_fwd()            # the recurrence alone (ifgo complete at launch)
-            zero_ws(ws_f, plan_f)
-            layer_fwd()          # projection + recurrence in one launch where the library fuses them
-            zero_ws(ws_f, plan_f)
-            layer_fwd_infer()
-            cal_dst.copy_(cal_src)
-        torch.cuda.synchronize()
-        return
-
-    t_k1 = ev_time(k1)
-    t_rec = ev_time(rec_fwd, pre=rec_fwd_pre)
-    t_layer = ev_time(layer_fwd, pre=lambda: zero_ws(ws_f, plan_f))
-    t_infer = ev_time(layer_fwd_infer, pre=lambda: zero_ws(ws_f, plan_f))
-    kernels = {"gemm_ifgo_ms": round(t_k1, 4), "recurrent_fwd_ms": round(t_rec, 4),
-               "recurrent_fwd_us_per_step": round(t_rec * 1e3 / T, 3),
-               "fwd_layer_ms": round(t_layer, 4), "fwd_layer_infer_ms": round(t_infer, 4),
-               "gemm_ifgo_tflops": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12, 2),
-               "gemm_ifgo_frac_of_mfma_peak": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
-               "plan_fwd": plan_f.as_dict(), "plan_bwd": plan_b.as_dict()}
-    torch.cuda.synchronize()
-    _lib.check(lib.fastlstm_ws_status(ws_f[:64].cpu().numpy().tobytes()), "forward barrier status")
 
     # backward stages
     dout = torch.ones(T, B, H, device=dev, dtype=dt)
@@ -233,44 +259,106 @@ def main():
                                           db.data_ptr(), ws_b.data_ptr(), ws_b.numel(), ws_w.data_ptr(), ws_w.numel(),
                                           T, B, I, H, code, stream), "bwd_layer")
 
+    if args.stage != "all":
+        # counter runs (rocprofv3 --pmc / --kernel-trace): one group of kernels, three repetitions, plus a
+        # plain copy of known size (2 x 256 MiB of traffic) that calibrates FETCH_SIZE / WRITE_SIZE
+        k1()
+        zero_ws(ws_f, plan_f)
+        layer_fwd()             # valid ifgo / out / cell for the backward stages
+        cal_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        cal_dst = torch.empty_like(cal_src)
+        for _ in range(3):
+            if args.stage == "fwd_recurrence":
+                rec_fwd_pre()
+                rec_fwd()            # the recurrence alone (ifgo complete at launch)
+                zero_ws(ws_f, plan_f)
+                layer_fwd()          # projection + recurrence in one launch where the library fuses them
+                zero_ws(ws_f, plan_f)
+                layer_fwd_infer()
+            elif args.stage == "fwd_layer":
+                zero_ws(ws_f, plan_f)
+                layer_fwd()
+            elif args.stage == "bwd_layer":
+                rec_bwd_pre()
+                layer_bwd()
+            else:   # gemms: K1, K5, K8 + K9 (+ db) as stand-alone launches
+                rec_bwd_pre()
+                rec_bwd()            # a real d_ifgo
+                k1()
+                k5()
+                k89()
+            cal_dst.copy_(cal_src)
+        torch.cuda.synchronize()
+        return
+
+    headline = step_fwd if mode == "fwd" else step_fwd_bwd
+    with torch.enable_grad():
+        ms = timed(headline, args.steps, args.warmup)
+        ms_fwd = ms if mode == "fwd" else timed(step_fwd, args.steps, args.warmup)
+        ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), 2)
+        db_fwd, n_fwd = do_bench(step_fwd)
+        db_full, n_full = do_bench(step_fwd_bwd)
+    value = B * T / (ms * 1e-3)
+
+    t_k1 = ev_time(k1)
+    t_rec = ev_time(rec_fwd, pre=rec_fwd_pre)
+    t_layer = ev_time(layer_fwd, pre=lambda: zero_ws(ws_f, plan_f))
+    t_infer = ev_time(layer_fwd_infer, pre=lambda: zero_ws(ws_f, plan_f))
+    kernels = {"gemm_ifgo_ms": round(t_k1, 4), "recurrent_fwd_ms": round(t_rec, 4),
+               "recurrent_fwd_us_per_step": round(t_rec * 1e3 / T, 3),
+               "fwd_layer_ms": round(t_layer, 4), "fwd_layer_infer_ms": round(t_infer, 4),
+               "gemm_ifgo_tflops": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12, 2),
+               "gemm_ifgo_frac_of_mfma_peak": round(2.0 * T * B * I * 4 * H / (t_k1 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
+               "plan_fwd": plan_f.as_dict(), "plan_bwd": plan_b.as_dict()}
+    torch.cuda.synchronize()
+    _lib.check(lib.fastlstm_ws_status(ws_f[:64].cpu().numpy().tobytes()), "forward barrier status")
+
     t_rb = ev_time(rec_bwd, reps=5, pre=rec_bwd_pre)
     t_k5 = ev_time(k5, reps=5)
     t_k89 = ev_time(k89, reps=5)
     t_lb = ev_time(layer_bwd, reps=5, pre=rec_bwd_pre)
     torch.cuda.synchronize()
     _lib.check(lib.fastlstm_ws_status(ws_b[:64].cpu().numpy().tobytes()), "backward barrier status")
+    gf = 2.0 * T * B * I * 4 * H
+    gw = 2.0 * T * B * 4 * H * (I + H)
     kernels.update({
         "recurrent_bwd_ms": round(t_rb, 4), "recurrent_bwd_us_per_step": round(t_rb * 1e3 / T, 3),
         "gemm_dx_ms": round(t_k5, 4),
-        "gemm_dx_tflops": round(2.0 * T * B * I * 4 * H / (t_k5 * 1e-3) / 1e12, 2),
+        "gemm_dx_tflops": round(gf / (t_k5 * 1e-3) / 1e12, 2),
+        "gemm_dx_frac_of_mfma_peak": round(gf / (t_k5 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
         "gemm_wgrad_ms": round(t_k89, 4),
-        "gemm_wgrad_tflops": round(2.0 * T * B * 4 * H * (I + H) / (t_k89 * 1e-3) / 1e12, 2),
+        "gemm_wgrad_tflops": round(gw / (t_k89 * 1e-3) / 1e12, 2),
+        "gemm_wgrad_frac_of_mfma_peak": round(gw / (t_k89 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
         "bwd_layer_ms": round(t_lb, 4),
     })
 
     # ---- roofline of the dominant kernel of the headline (forward) path ------------------
     # XCD-local path with idle CUs: ONE launch does projection + recurrence (fastlstm_fwd_layer);
-    # otherwise the recurrence launch dominates.  Either way the bound is latency (T sequential
-    # steps), which the low MFMA fraction shows.
+    # otherwise the recurrence launch dominates.  The flops are priced against the MFMA peak; what bounds
+    # the launch is the latency of T sequential steps, measured below.
     rec_flops = 2.0 * B * H * 4 * H * T          # algorithmic flops of the recurrence
     k1_flops = 2.0 * T * B * I * 4 * H           # ... of the input projection
-    xcd_local = lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, ws_f.numel()) == 1
+    kind = lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, ws_f.numel())
+    xcd_local = kind == 1
     fused = xcd_local and t_layer < 0.9 * (t_k1 + t_rec)
+    traffic, traffic_src = TRAFFIC.get(args.workload, (None, None))
     if fused:
         flops, t_dom, kname = rec_flops + k1_flops, t_layer, "lstm_fwd_xcd_kernel<..., HELP=true> (projection + recurrence)"
         alg = "2*B*H*4H*T + 2*T*B*I*4H flop per launch = %.1f GFLOP" % (flops / 1e9)
     else:
         flops, t_dom = rec_flops, t_rec
-        kname = "lstm_fwd_xcd_kernel" if xcd_local else "lstm_fwd_persistent_kernel"
+        kname = {0: "lstm_fwd_persistent_kernel", 1: "lstm_fwd_xcd_kernel", 2: "lstm_fwd_wide_kernel"}[kind]
         alg = "2*B*H*4H*T flop per launch = %.1f GFLOP" % (flops / 1e9)
+        if args.workload == "B":
+            traffic, traffic_src = None, None
     ach = flops / (t_dom * 1e-3) / 1e12
     roofline = {"kernel": kname, "bound": "mfma", "achieved": round(ach, 2),
                 "peak": PEAK_TFLOPS[dname], "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS[dname], 4),
-                "traffic": TRAFFIC_BYTES.get(args.workload) if fused else None,
+                "traffic": traffic, "traffic_source": traffic_src,
                 "algorithmic": alg, "launch_ms": round(t_dom, 4),
-                "note": "latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange "
+                "note": "the launch is latency-bound, not MFMA-bound: T sequential steps, each a cross-CU exchange "
                         + ("through the L2 of one XCD" if xcd_local else "through device memory")
-                        + "; us/step of the recurrence alone is in kernels.recurrent_fwd_us_per_step"}
+                        + "; see latency_bound"}
 
     if plan_f.wave_split == 2:
         # one hidden tile per workgroup (H <= 64): no exchange between CUs at all; the kernel streams the
@@ -280,11 +368,45 @@ def main():
         ach = nbytes / (t_rec * 1e-3) / 1e9
         roofline = {"kernel": "lstm_fwd_persistent_kernel<SPLIT=2> (one hidden tile per workgroup)", "bound": "hbm",
                     "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                    "traffic": TRAFFIC_BYTES.get(args.workload),
+                    "traffic": traffic, "traffic_source": traffic_src,
                     "algorithmic": "s*(2*T*B*4H + 2*T*B*H + 4H*H) bytes per launch = %.1f MB" % (nbytes / 1e6),
                     "launch_ms": round(t_rec, 4),
                     "note": "latency-bound, not HBM-bound: %d independent workgroups (16 batch rows each) walk through "
                             "T sequential steps; us/step is in kernels.recurrent_fwd_us_per_step" % plan_f.n_btiles}
+    elif dname != "fp32" and H % 32 == 0 and H <= 2048:
+        # ---- the latency floor of a step, measured with the recurrence's own barrier and exchange code ----
+        # (fastlstm_diag_step_probe: 16-bit h tiles; one group is timed alone on an otherwise idle device)
+        if kind == 1:
+            pk, members, rows = 0, min(32, H // 8), 16   # the smallest unit tile that keeps a group on one XCD
+        elif kind == 2:
+            pk, members, rows = 1, H // 16, 64
+        else:
+            pk, members, rows = 1, plan_f.n_htiles, min(64, max(16, plan_f.bt // 16 * 16))
+        while H % members:
+            members -= 1
+        steps_p = 512
+        ws_p = torch.zeros(lib.fastlstm_diag_step_probe_bytes(steps_p, H, rows), dtype=torch.uint8, device=dev)
+        probe = {}
+        for pm, name in ((0, "empty_barrier_us"), (1, "barrier_plus_publish_us"), (2, "barrier_publish_fetch_us")):
+            def run(pm=pm):
+                _lib.check(lib.fastlstm_diag_step_probe(pk, pm, members, H, rows, steps_p, ws_p.data_ptr(), ws_p.numel(),
+                                                        stream), "step probe")
+            probe[name] = round(ev_time(run, reps=5, warmup=2, pre=lambda: ws_p[:70000].zero_()) * 1e3 / steps_p, 3)
+        torch.cuda.synchronize()
+        _lib.check(lib.fastlstm_ws_status(ws_p[:64].cpu().numpy().tobytes()), "step probe status")
+        mfma_us = 2.0 * B * H * 4 * H / (PEAK_TFLOPS[dname] * 1e12) * 1e6
+        bound = probe["barrier_publish_fetch_us"]
+        per_step = t_dom * 1e3 / T
+        roofline["latency_bound"] = {
+            "bound": "latency", "per_step_bound_us": bound, "achieved_us_per_step": round(per_step, 3),
+            "frac": round(bound / per_step, 4),
+            "recurrence_alone_us_per_step": round(t_rec * 1e3 / T, 3),
+            "frac_recurrence_alone": round(bound / (t_rec * 1e3 / T), 4),
+            "mfma_time_per_step_at_peak_us": round(mfma_us, 3),
+            "probe": dict(probe, group="XCD-local, L2 counters" if pk == 0 else "flag group over all XCDs",
+                          members=members, rows=rows, steps=steps_p),
+            "note": "per_step_bound_us = publish h_t + barrier round trip + fetch of the group's h_t, timed with the "
+                    "kernels' own code and no arithmetic (fastlstm_diag_step_probe mode 2); frac = bound / achieved"}
 
     res = {
         "metric": "lstm_%s_batch_timesteps_per_s" % mode, "value": round(value, 1), "unit": "batch*timesteps/s",
@@ -293,6 +415,10 @@ def main():
         "config": {"workload": "%s: %d-layer LSTM %s %s, B=%d T=%d I=%d H=%d" % (args.workload, layers, dname, mode, B, T, I, H)},
         "fwd": {"ms": round(ms_fwd, 4), "bt_per_s": round(B * T / (ms_fwd * 1e-3), 1)},
         "fwd_bwd": {"ms": round(ms_full, 4), "bt_per_s": round(B * T / (ms_full * 1e-3), 1)},
+        "do_bench": {"fwd_ms": round(db_fwd, 4), "fwd_reps": n_fwd, "fwd_bwd_ms": round(db_full, 4), "fwd_bwd_reps": n_full,
+                     "fwd_bt_per_s": round(B * T / (db_fwd * 1e-3), 1), "fwd_bwd_bt_per_s": round(B * T / (db_full * 1e-3), 1),
+                     "protocol": "median; warm-up 40 ms, 160 ms of repetitions, 256 MB buffer cleared before each, one "
+                                 "event pair per repetition (the reference's scripts/benchmark.py:118-133)"},
         "roofline": roofline, "kernels": kernels,
     }
 
@@ -320,16 +446,48 @@ def main():
         except Exception as exc:  # MIOpen may not support a configuration
             res["nn_lstm_rocm"] = {"error": str(exc)[:200]}
 
-    # ---- CPU baselines on a bounded sample (same B, I, H; fewer timesteps) ---------------
+    # ---- CPU baselines ---------------------------------------------------------------------
     if not args.no_cpu:
-        from oracle import lstm_oracle as orc
         import numpy as np
 
-        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cores = physical_cores()
         torch.set_num_threads(cores)
-        Wx_c, Wh_c = model.weight_ih_l0.detach().float().cpu(), model.weight_hh_l0.detach().float().cpu()
-        bx_c, bh_c = model.bias_ih_l0.detach().float().cpu(), model.bias_hh_l0.detach().float().cpu()
-        a = [t.numpy() for t in (Wx_c, bx_c, Wh_c, bh_c)]
+        cpu_model = torch.nn.LSTM(I, H, num_layers=layers)   # fp32, the module's parameters
+        with torch.no_grad():
+            for n, p in model.named_parameters():
+                getattr(cpu_model, n).copy_(p.float().cpu())
+
+        def cpu_pass(ts):
+            xs = x_cpu[:ts]
+            t0 = time.perf_counter()
+            if mode == "fwd":
+                with torch.no_grad():
+                    cpu_model(xs, (h0_cpu, c0_cpu))
+            else:
+                for p in cpu_model.parameters():
+                    p.grad = None
+                o, _ = cpu_model(xs, (h0_cpu, c0_cpu))
+                o.sum().backward()
+            return time.perf_counter() - t0
+
+        probe_t = min(T, 16)
+        per_step = cpu_pass(probe_t) / probe_t
+        per_step = min(per_step, cpu_pass(probe_t) / probe_t)
+        ts = int(max(probe_t, min(T, 4.0 / max(per_step, 1e-9))))      # a pass of at most ~4 s
+        passes = int(max(3, min(10, 12.0 / max(per_step * ts, 1e-9))))   # >= 3 passes, ~12 s in all
+        times = sorted(cpu_pass(ts) for _ in range(passes))
+        el = times[len(times) // 2]
+        res["cpu_baseline"] = {"value": round(B * ts / el, 1), "unit": "batch*timesteps/s", "cores": cores,
+                               "kind": "port",
+                               "sample": "torch.nn.LSTM fp32 (the parity target the reference's tests use) on the host, "
+                                         "%d physical cores = torch threads, same weights and inputs, all %d layer(s), "
+                                         "first %d of %d timesteps, %s; median of %d passes (%.3f s each)"
+                                         % (cores, layers, ts, T, mode, passes, el)}
+
+        from oracle import lstm_oracle as orc
+
+        a = [model.get_parameter(n).detach().float().cpu().numpy()
+             for n in ("weight_ih_l0", "bias_ih_l0", "weight_hh_l0", "bias_hh_l0")]
 
         def oracle_run(ts):
             t0 = time.perf_counter()
@@ -340,35 +498,14 @@ def main():
                              dtype=np.float32)
             return time.perf_counter() - t0
 
-        probe = min(T, 4)
-        per_step = oracle_run(probe) / probe
-        ts = int(max(probe, min(T, 12.0 / max(per_step, 1e-9))))
-        passes = int(max(1, min(20, 10.0 / max(per_step * ts, 1e-9))))   # ~10 s of CPU work
-        el = sum(oracle_run(ts) for _ in range(passes)) / passes
-        res["cpu_baseline"] = {"value": round(B * ts / el, 1), "unit": "batch*timesteps/s", "cores": cores,
-                               "kind": "port",
-                               "sample": "C/OpenMP fp32 oracle, layer 0, same B/I/H, first %d of %d timesteps, %s; "
-                                         "mean of %d passes of %.1f s" % (ts, T, mode, passes, el)}
-        ref_c = torch.nn.LSTM(I, H)
-        with torch.no_grad():
-            ref_c.weight_ih_l0.copy_(Wx_c); ref_c.weight_hh_l0.copy_(Wh_c)
-            ref_c.bias_ih_l0.copy_(bx_c); ref_c.bias_hh_l0.copy_(bh_c)
-        xs = x_cpu[:ts]
-
-        def cpu_ref():
-            t0 = time.perf_counter()
-            if mode == "fwd":
-                with torch.no_grad():
-                    ref_c(xs, (h0_cpu[:1], c0_cpu[:1]))
-            else:
-                o, _ = ref_c(xs, (h0_cpu[:1], c0_cpu[:1]))
-                o.sum().backward()
-            return time.perf_counter() - t0
-
-        cpu_ref()
-        el2 = min(cpu_ref() for _ in range(2))
-        res["nn_lstm_cpu"] = {"value": round(B * ts / el2, 1), "unit": "batch*timesteps/s", "cores": cores,
-                              "sample": "torch.nn.LSTM fp32 on the host, same sample (%d timesteps, %s)" % (ts, mode)}
+        probe_t = min(T, 4)
+        per_step = oracle_run(probe_t) / probe_t
+        ts = int(max(probe_t, min(T, 5.0 / max(per_step, 1e-9))))
+        el = oracle_run(ts)
+        res["cpu_oracle"] = {"value": round(B * ts / el, 1), "unit": "batch*timesteps/s",
+                             "threads": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)),
+                             "sample": "C/OpenMP fp32 oracle (the parity checker), layer 0, first %d of %d timesteps, %s; "
+                                       "one pass of %.1f s" % (ts, T, mode, el)}
 
     print(json.dumps(res))
 

@@ -52,6 +52,8 @@ SIGNATURES = {
     "fastlstm_gemm_dx": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_gemm_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "fastlstm_diag_step_probe": (_i, [_i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "fastlstm_diag_step_probe_bytes": (_sz, [_i, _i, _i]),
     "fastlstm_ws_status": (_i, [_vp]),
     "fastlstm_device_status": (_i, [_i, _i]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),

@@ -269,6 +269,21 @@ void fastlstm_set_gemm_trace(void *buf);
  * publish + stores, waiting for peers, operand fetch + MFMA + reduce. */
 void fastlstm_set_recurrent_trace(void *buf);
 
+/* Diagnostics: the latency bound of one recurrence step.  Runs `steps` rounds of the links of a timestep
+ * that no arithmetic throughput removes, with the recurrent kernels' own barrier and exchange code:
+ * mode 0 = the empty barrier (publish + wait), 1 = + every member stores its share of a `rows`-row fp16 h
+ * tile into the step's exchange slot, 2 = + every wave fetches its operand blocks of the step; 3, 4 (kind 0
+ * only) = the exchange without a barrier: consumers poll the data itself, unwritten values hold an all-ones
+ * sentinel, loads bypass the L1 (sc1 / sc0 sc1); the ring part of ws must then be filled with 0xFF bytes.
+ * kind 0 = an XCD-local group of `members` <= 32 workgroups (counters in that XCD's L2), kind 1 = a flag
+ * group of `members` <= 256 workgroups over all XCDs (device-scope flags).  H <= 2048, a multiple of 32 and of
+ * `members`; rows = 16, 32, 48 or 64 batch rows per group.  The caller times the launch (its duration /
+ * steps = microseconds per round); ws: zeroed device memory of fastlstm_diag_step_probe_bytes.  No
+ * counterpart in the reference. */
+int fastlstm_diag_step_probe(int kind, int mode, int members, int H, int rows, int steps, void *ws,
+                             size_t ws_bytes, void *stream);
+size_t fastlstm_diag_step_probe_bytes(int steps, int H, int rows);
+
 const char *fastlstm_strerror(int status);
 const char *fastlstm_version(void);
 
