@@ -47,8 +47,8 @@ PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}  # MI355X dense MF
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain
 # copy of known size.  Counters cannot be read from inside this process: the figures are copied from the
-# committed summaries named here (made by `rocprofv3 --pmc ... -- python3 bench.py --stage fwd_recurrence`).
-TRAFFIC = {"B": (1575.6e6, "profiles/fwd_layer_B_pmc.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
+# committed summaries named here (made by `rocprofv3 --pmc ... -- python3 bench.py --stage fwd_layer`).
+TRAFFIC = {"B": (1577.5e6, "profiles/recurrence_lds_l2_B.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
 
 
 def physical_cores():
