@@ -10,6 +10,7 @@
 #include "recurrent_bwd_xcd.hpp"
 #include "recurrent_bwd_wide.hpp"
 #include "recurrent_fwd_xcd.hpp"
+#include "recurrent_stream.hpp"
 
 using namespace fastlstm;
 
@@ -743,6 +744,36 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     const bool sync = pl.wave_split != 2;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
+    if (pl.wave_split == 3) {   // W_h does not fit on chip: pack it once, then stream it every step
+        const StreamLayout l = stream_layout(pl, H, dtype, false);
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        if (launch_pack_wh(dtype, false, Wh, wsb + l.wpack_off, H, l.KS, l.KSP, l.mt, pl.n_htiles, s) != hipSuccess)
+            return FASTLSTM_ERR_HIP;
+        FwdStreamParams p{};
+        p.ifgo = ifgo; p.out = out; p.cell = cell;
+        p.wpack = wsb + l.wpack_off;
+        p.hdr = reinterpret_cast<WsHeader *>(wsb);
+        p.T = T; p.B = B; p.H = H;
+        p.n_bt = pl.n_btiles; p.n_ht = pl.n_htiles;
+        p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
+        p.KS = l.KS; p.KSP = l.KSP;
+        p.keep = keep;
+        p.spin_limit = spin_limit_ticks();
+        const int n_bt_total = cdiv(B, pl.bt);
+        for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
+            const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+            unsigned char *chunk = wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * l.chunk_bytes;
+            p.flags = reinterpret_cast<int *>(chunk);
+            p.xbuf = chunk + l.flags_bytes;
+            p.b_base = bt0 * pl.bt;
+            const int grid = n_bt * pl.n_htiles;
+            int occ = 0;
+            if (launch_fwd_stream(dtype, p, l.mt, pl.bt / 16, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+            if ((long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
+            if (launch_fwd_stream(dtype, p, l.mt, pl.bt / 16, grid, pl.lds_bytes, s, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+        }
+        return FASTLSTM_OK;
+    }
     if (sync) {
         // One launch per range of rows where the batch has too many 16-row tiles for one XCD-local launch;
         // also instead of one launch with 32-row tiles of the 8-wave kernel (H = 1024, 16-bit), whose
@@ -856,6 +887,35 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
     const bool sync = pl.wave_split != 2;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
+    if (pl.wave_split == 3) {   // W_h does not fit on chip: pack Wh[:, units]^T once, then stream it every step
+        const StreamLayout l = stream_layout(pl, H, dtype, true);
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        if (launch_pack_wh(dtype, true, Wh, wsb + l.wpack_off, H, l.KS, l.KSP, l.mt, pl.n_htiles, s) != hipSuccess)
+            return FASTLSTM_ERR_HIP;
+        BwdStreamParams p{};
+        p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo;
+        p.wpack = wsb + l.wpack_off;
+        p.hdr = reinterpret_cast<WsHeader *>(wsb);
+        p.T = T; p.B = B; p.H = H;
+        p.n_bt = pl.n_btiles; p.n_ht = pl.n_htiles;
+        p.flag_stride = (int)align_up((size_t)pl.n_htiles, 64);
+        p.KSB = l.KS; p.KSBP = l.KSP;
+        p.spin_limit = spin_limit_ticks();
+        const int n_bt_total = cdiv(B, pl.bt);
+        for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
+            const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+            unsigned char *chunk = wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * l.chunk_bytes;
+            p.flags = reinterpret_cast<int *>(chunk);
+            p.xbuf = chunk + l.flags_bytes;
+            p.b_base = bt0 * pl.bt;
+            const int grid = n_bt * pl.n_htiles;
+            int occ = 0;
+            if (launch_bwd_stream(dtype, p, l.mt, pl.bt / 16, 0, pl.lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+            if ((long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
+            if (launch_bwd_stream(dtype, p, l.mt, pl.bt / 16, grid, pl.lds_bytes, s, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+        }
+        return FASTLSTM_OK;
+    }
     if (sync) {
         int rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, wsb, ws_bytes, T, B, H, dtype,
                              static_cast<hipStream_t>(stream));
@@ -1035,7 +1095,7 @@ int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, co
 
 size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
     const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 0);
-    if (!plan || one == 0 || plan->wave_split == 2) return one;
+    if (!plan || one == 0 || plan->wave_split >= 2) return one;
     const size_t head = kWsHeaderBytes + kWsCounterBytes;
     return one > head ? head + 2 * (one - head) : one;
 }
@@ -1160,7 +1220,7 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
 
 size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
     const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, 1);
-    if (!plan || one == 0 || plan->wave_split == 2) return one;
+    if (!plan || one == 0 || plan->wave_split >= 2) return one;
     const size_t head = kWsHeaderBytes + kWsCounterBytes;
     return one > head ? head + 2 * (one - head) : one;
 }
@@ -1251,6 +1311,10 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (T <= 0 || B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    {
+        fastlstm_plan pl;
+        if (plan_device(-1, B, H, dtype, backward, &pl, false) == FASTLSTM_OK && pl.wave_split == 3) return 3;
+    }
     XcdCfg c;
     if (select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c)) return 1;
     WideCfg w;
@@ -1286,7 +1350,8 @@ const char *fastlstm_strerror(int status) {
         case FASTLSTM_ERR_DTYPE: return "unsupported dtype (0 = fp32, 1 = fp16, 2 = bf16)";
         case FASTLSTM_ERR_ALIGN: return "a pointer is not 16-byte aligned";
         case FASTLSTM_ERR_RESIDENCY:
-            return "the W_h slice does not fit in LDS or the barrier group cannot be co-resident";
+            return "the barrier group cannot be co-resident on this device (hidden size beyond 64 units per compute unit, "
+                   "or fewer compute units than the plan assumes)";
         case FASTLSTM_ERR_WORKSPACE: return "workspace is smaller than required";
         case FASTLSTM_ERR_HIP: return "a HIP runtime call failed";
         case FASTLSTM_ERR_TIMEOUT:

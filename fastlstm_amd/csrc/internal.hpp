@@ -47,6 +47,23 @@ FASTLSTM_DECL_REC(f16)
 FASTLSTM_DECL_REC(bf16)
 #undef FASTLSTM_DECL_REC
 
+// streamed-weights kernels (recurrent_stream.hpp): plans with wave_split == 3
+struct FwdStreamParams;
+struct BwdStreamParams;
+hipError_t launch_fwd_stream(int dtype, const FwdStreamParams &p, int mt, int nt, int grid, int lds, hipStream_t s,
+                             int *max_blocks_per_cu);
+hipError_t launch_bwd_stream(int dtype, const BwdStreamParams &p, int mtb, int nt, int grid, int lds, hipStream_t s,
+                             int *max_blocks_per_cu);
+hipError_t launch_pack_wh(int dtype, bool backward, const void *Wh, unsigned char *wpack, int H, int KS, int KSP, int mt,
+                          int n_ht, hipStream_t s);
+// Workspace layout of a streamed-weights plan: header | counters | per batch chunk: flags, 2 exchange slots | packed W_h
+struct StreamLayout {
+    int KS, KSP;            // k-steps of the contraction, padded to the K loop's granule
+    int mt;                 // operand row tiles of a workgroup's weight slice (forward: ht / 4, reverse: ht / 16)
+    size_t flags_bytes, slot_bytes, chunk_bytes, wpack_off, wpack_bytes;
+};
+StreamLayout stream_layout(const fastlstm_plan &plan, int H, int dtype, bool backward);
+
 int fwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
 int bwd_lds_bytes(int H, int dtype, int ht, int bt, int split, bool sync);
 size_t recurrent_flags_bytes(int n_bt, int n_ht);

@@ -86,6 +86,22 @@ int recurrent_full_slots(int T, size_t slot_bytes, bool backward) {
     return (int)std::max<long long>(2, std::min(want, fit));
 }
 
+// k-steps are padded to the granule of the streamed K loop (4 waves x 2 chunks x 2 k-steps)
+constexpr int kStreamKPadHost = 16;
+
+StreamLayout stream_layout(const fastlstm_plan &plan, int H, int dtype, bool backward) {
+    StreamLayout l;
+    l.KS = cdiv(backward ? 4 * H : H, kstep_of(dtype));
+    l.KSP = cdiv(l.KS, kStreamKPadHost) * kStreamKPadHost;
+    l.mt = backward ? plan.ht / 16 : plan.ht / 4;
+    l.flags_bytes = recurrent_flags_bytes(plan.n_btiles, plan.n_htiles);
+    l.slot_bytes = (size_t)plan.n_btiles * (plan.bt / 16) * l.KSP * kFragBytes;
+    l.chunk_bytes = l.flags_bytes + 2 * l.slot_bytes;
+    l.wpack_off = align_up(kWsHeaderBytes + kWsCounterBytes + (size_t)plan.batch_chunks * l.chunk_bytes, 4096);
+    l.wpack_bytes = (size_t)plan.n_htiles * l.mt * l.KSP * kFragBytes;
+    return l;
+}
+
 }  // namespace fastlstm
 
 using namespace fastlstm;
@@ -171,7 +187,32 @@ extern "C" int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int d
             c.cost = step_ns * c.chunks;
             if (best.cost < 0 || c.cost < best.cost) best = c;
         }
-    if (best.cost < 0) return FASTLSTM_ERR_RESIDENCY;
+    if (best.cost < 0) {
+        // No tiling keeps the weight slices on chip: stream them every step (wave_split 3, recurrent_stream.hpp).
+        // One workgroup per slice of ht units and as many batch rows as its accumulators hold, so that the
+        // weights cross the memory system once per step; ht is the smallest slice that leaves the barrier group
+        // co-resident.
+        int ht = 0;
+        for (int cand : {16, 32, 64})
+            if (!ht && cdiv(H, cand) <= num_cus) ht = cand;
+        if (!ht) return FASTLSTM_ERR_RESIDENCY;   // H > 64 * num_cus
+        const int nt_max = 4 / (ht / 16);
+        int nt = 1;
+        while (nt < nt_max && nt * 16 < B) nt *= 2;
+        plan->ht = ht;
+        plan->bt = 16 * nt;
+        plan->n_htiles = cdiv(H, ht);
+        const int n_bt_total = cdiv(B, plan->bt);
+        plan->n_btiles = std::min(n_bt_total, std::max(1, num_cus / plan->n_htiles));
+        plan->batch_chunks = cdiv(n_bt_total, plan->n_btiles);
+        plan->wave_split = 3;
+        plan->lds_bytes = 4 * (backward ? ht / 16 : ht / 4) * nt * kFragBytes;   // the 4 waves' partial sums
+        const StreamLayout l = stream_layout(*plan, H, dtype, backward != 0);
+        plan->ws_bytes = l.wpack_off + l.wpack_bytes;
+        plan->ws_zero_bytes = l.wpack_off;   // header, counters, flags and the (small) exchange slots
+        plan->ring_needs_zero = 0;
+        return FASTLSTM_OK;
+    }
     plan->bt = best.bt;
     plan->ht = best.ht;
     plan->n_btiles = best.n_bt;
@@ -187,7 +228,7 @@ extern "C" int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int d
 
 extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype, int backward) {
     if (!plan || T <= 0 || H <= 0 || !dtype_ok(dtype)) return 0;
-    if (plan->wave_split == 2) return plan->ws_bytes;
+    if (plan->wave_split == 2 || plan->wave_split == 3) return plan->ws_bytes;
     const size_t slot = recurrent_slot_bytes(H, dtype, plan->bt, plan->n_btiles, backward != 0);
     const int slots = recurrent_full_slots(T, slot, backward != 0);
     size_t ws = recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks,

@@ -74,6 +74,10 @@ def _workspace(plan, T, H, code, backward, device):
     uses the XCD-local kernel where the shape allows (the barrier group on one XCD, exchange
     through its L2); the backward pass reads d_ifgo[t] once per XCD instead of once per CU.
     Without room for the ring (RING_MAX_BYTES) the two-slot workspace of the plan is used."""
+    if plan.wave_split == 3:   # streamed weights: flags and exchange slots zeroed, the packed-weights area is written by the call
+        ws = torch.empty(plan.ws_bytes, dtype=torch.uint8, device=device)
+        ws[:plan.ws_zero_bytes].zero_()
+        return ws
     if plan.wave_split != 2:
         ring = _lib.load().fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1 if backward else 0)
         if plan.ws_bytes < ring <= RING_MAX_BYTES:

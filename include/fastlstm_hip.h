@@ -42,7 +42,7 @@ typedef enum {
     FASTLSTM_ERR_DIM = -2,       /* non-positive or overflowing dimension */
     FASTLSTM_ERR_DTYPE = -3,     /* dtype not in fastlstm_dtype */
     FASTLSTM_ERR_ALIGN = -4,     /* pointer not 16-byte aligned */
-    FASTLSTM_ERR_RESIDENCY = -5, /* W_h slice does not fit on chip / grid cannot be co-resident */
+    FASTLSTM_ERR_RESIDENCY = -5, /* the barrier group cannot be co-resident (H > 64 units x compute units) */
     FASTLSTM_ERR_WORKSPACE = -6, /* workspace smaller than required */
     FASTLSTM_ERR_HIP = -7,       /* a HIP runtime call failed (no device, launch error) */
     FASTLSTM_ERR_TIMEOUT = -8    /* a workspace status word reports a barrier time-out */
@@ -62,9 +62,11 @@ typedef struct {
     int n_btiles;     /* batch tiles per launch */
     int n_htiles;     /* hidden tiles (= barrier group size); 1 => no cross-CU sync */
     int batch_chunks; /* sequential launches needed to cover B */
-    int wave_split;   /* 0: waves split K, 1: waves split batch tiles, 2: waves split W rows */
+    int wave_split;   /* 0: waves split K, 1: waves split batch tiles, 2: waves split W rows (H <= 64, no cross-CU sync),
+                         3: W_h does not fit on chip -- waves split K and the weight slice is streamed every step */
     int lds_bytes;    /* LDS the kernel will request */
-    size_t ws_bytes;  /* smallest workspace the recurrent call accepts (2 exchange slots) */
+    size_t ws_bytes;  /* smallest workspace the recurrent call accepts (2 exchange slots; wave_split 3: plus W_h once
+                         in operand order, which the call itself writes) */
     size_t ws_zero_bytes; /* leading bytes of the workspace that must be zero (header + counters + flags) */
     int ring_needs_zero;  /* 1: B or H leave padding in the exchange blocks -> zero the whole workspace */
 } fastlstm_plan;
@@ -232,7 +234,9 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
  * device that fastlstm_plan_device has probed; a batch with more tiles than one launch holds runs as
  * several launches over ranges of rows), 2 = the register-resident kernel for H = 1280, 1536, 1792,
  * 2048 with 16-bit elements (barrier groups of H / 16 workgroups over several XCDs, 64 batch rows
- * each; same needs as 1).  Negative: fastlstm_status.  Diagnostics; no counterpart in the reference. */
+ * each; same needs as 1), 3 = the streamed-weights kernel of a hidden size whose W_h does not fit on chip (more
+ * than 32 MiB: the reference's RELOAD_WEIGHTS case, fastlstm/lstm.py:70-72).  Negative: fastlstm_status.
+ * Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
 /* Reads the status word the recurrent kernels leave at the start of their

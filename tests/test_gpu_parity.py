@@ -133,6 +133,45 @@ def test_stages_vs_oracle(oracle, T, B, I, H, dt):
         assert rel_err(got, want) < tol, name
 
 
+STREAM_CASES = [
+    # T, B, I, H, dtype: hidden sizes whose W_h does not fit on chip -- the weight slices are streamed every step
+    # (the reference reloads its weights per step above H = 128, fastlstm/lstm.py:70-72)
+    (5, 20, 64, 2560, torch.float16),     # 160 slices of 16 units, 32-row batch tile
+    (4, 64, 32, 4096, torch.float16),     # 256 slices, one 64-row batch tile: every CU streams 512 KiB per step
+    (5, 24, 40, 1536, torch.float32),     # fp32 past 1024
+    (4, 70, 32, 2100, torch.bfloat16),    # ragged H (rows not 16-byte aligned, padded k-steps) and two batch chunks
+    (3, 150, 16, 2304, torch.float16),    # three sequential launches over the batch
+    (3, 16, 16, 5000, torch.float16),     # slices of 32 units
+]
+
+
+@pytest.mark.parametrize("T,B,I,H,dt", STREAM_CASES)
+def test_streamed_weights_vs_oracle(oracle, T, B, I, H, dt):
+    plan = _lib.Plan()
+    _lib.check(_lib.load().fastlstm_plan_device(0, B, H, RM[dt], 0, plan), "plan")
+    assert plan.wave_split == 3
+    assert _lib.load().fastlstm_recurrent_kernel_kind(T, B, H, RM[dt], 0, plan.ws_bytes) == 3
+    p = make_problem(T, B, I, H, seed=T * 1000 + H)
+    pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}
+    g = {k: dev(v, dt) for k, v in p.items()}
+    rm = RM[dt]
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    o_out, o_cell, o_ifgo = oracle.forward(*to_np(pr, FWD_KEYS), round_mode=rm)
+    out, cell, ifgo = L.lstm_persistent_fwd(g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"])
+    for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
+        assert rel_err(got, want) < tol, name
+    out_i, cell_i, _ = L.lstm_persistent_fwd(g["x"], g["h0"], g["c0"], g["Wx"], g["bx"], g["Wh"], g["bh"],
+                                             keep_activations=False)
+    assert torch.equal(out_i, out) and torch.equal(cell_i[-1], cell[-1])   # the inference form: same bits
+    dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
+    r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
+    d_x, dh0, dc0, dWx, dbx, dWh, dbh = L.lstm_persistent_bwd(g["dout"], g["dc_n"].clone(), g["dh_n"].clone(), g["x"], out,
+                                                             cell, ifgo, g["Wx"], g["Wh"])
+    for name, got, want in (("dx", d_x, r["dx"]), ("dh0", dh0, r["dh0"]), ("dc0", dc0, r["dc0"]),
+                            ("dWx", dWx, r["dWx"]), ("dWh", dWh, r["dWh"]), ("db", dbx, r["db"])):
+        assert rel_err(got, want) < tol, name
+
+
 def _random_shape(rng):
     """One (T, B, I, H, dtype) from four families: barrier-free sizes, ragged mid sizes, the tile
     multiples that select the XCD-local / register-resident kernels, and batches of many launches'

@@ -84,14 +84,10 @@ CUS, LDS = 256, 160 * 1024
 def test_tiling_rule_invariants(dtype, backward):
     lib = _lib.load()
     for B in (1, 4, 16, 44, 64, 100, 128, 256, 600, 2048):
-        for H in (1, 16, 33, 64, 65, 128, 257, 512, 768, 1024, 2048):
+        for H in (1, 16, 33, 64, 65, 128, 257, 512, 768, 1024, 2048, 2100, 3072, 4096, 9000, 16384):
             p = _lib.Plan()
             rc = lib.fastlstm_plan_for(CUS, LDS, B, H, dtype, backward, p)
-            if dtype == 0 and H > 1024:
-                assert rc in (_lib.OK, _lib.ERR_RESIDENCY)
-                if rc:
-                    continue
-            assert rc == _lib.OK, (B, H, dtype, backward)
+            assert rc == _lib.OK, (B, H, dtype, backward)   # no hidden size up to 64 units x CUs is refused
             assert p.lds_bytes <= LDS
             assert p.bt % 16 == 0 and p.bt * p.n_btiles * p.batch_chunks >= B
             if H <= 64:  # single hidden tile: barrier-free, any grid size
@@ -100,10 +96,22 @@ def test_tiling_rule_invariants(dtype, backward):
                 assert p.n_htiles * p.ht >= H and (p.n_htiles - 1) * p.ht < H
                 assert p.n_btiles * p.n_htiles <= CUS
                 assert (p.n_btiles - 1) * p.bt < B
-                assert p.wave_split in (0, 1)
+                assert p.wave_split in (0, 1, 3)
             kstep = 16 if dtype == 0 else 32
             ks = -(-(4 * H if backward else H) // kstep)
-            if p.n_htiles > 1:
+            if p.wave_split == 3:
+                # streamed weights (the slices do not fit on chip): at most 16 forward / 4 reverse output tiles per
+                # workgroup; workspace = header, counters, per batch chunk flags + 2 exchange slots, then all of
+                # W_h once in operand order with the k-steps padded to 16
+                assert (p.ht // 16) * (p.bt // 16) <= 4 and p.ht in (16, 32, 64)
+                ksp = -(-ks // 16) * 16
+                flags = -(-(p.n_btiles * (-(-p.n_htiles // 64) * 64) * 4) // 1024) * 1024
+                slots = 2 * p.n_btiles * (p.bt // 16) * ksp * 1024
+                head = -(-(1024 + 65536 + p.batch_chunks * (flags + slots)) // 4096) * 4096
+                assert p.ws_zero_bytes == head
+                rows = p.n_htiles * (p.ht // 16 if backward else p.ht // 4)
+                assert p.ws_bytes == head + rows * ksp * 1024
+            elif p.n_htiles > 1:
                 flags = -(-(p.n_btiles * (-(-p.n_htiles // 64) * 64) * 4) // 1024) * 1024
                 xbuf = 2 * p.n_btiles * (p.bt // 16) * ks * 1024
                 assert p.ws_bytes == 1024 + 65536 + p.batch_chunks * (flags + xbuf)
@@ -116,7 +124,9 @@ def test_tiling_rule_headline_configs():
     assert p.n_btiles * p.n_htiles == 256                                 # fills every CU
     assert lib.fastlstm_plan_for(CUS, LDS, 128, 2048, 2, 0, p) == 0     # config C: 32 MiB of W_h
     assert p.n_htiles == 256 and p.lds_bytes >= 128 * 1024
-    assert lib.fastlstm_plan_for(CUS, LDS, 64, 4096, 1, 0, p) == _lib.ERR_RESIDENCY
+    assert lib.fastlstm_plan_for(CUS, LDS, 64, 4096, 1, 0, p) == 0       # 128 MiB of W_h: streamed every step
+    assert p.wave_split == 3 and p.n_htiles == 256 and p.bt == 64 and p.ws_bytes > 128 << 20
+    assert lib.fastlstm_plan_for(CUS, LDS, 64, 64 * CUS + 1, 1, 0, p) == _lib.ERR_RESIDENCY   # more slices than CUs
     assert lib.fastlstm_plan_for(8, LDS, 64, 1024, 1, 0, p) == _lib.ERR_RESIDENCY  # too few CUs
     assert lib.fastlstm_plan_for(CUS, LDS, 64, 1024, 9, 0, p) == _lib.ERR_DTYPE
     assert lib.fastlstm_plan_for(CUS, LDS, 0, 1024, 1, 0, p) == _lib.ERR_DIM
