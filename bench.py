@@ -197,12 +197,12 @@ def main():
     plan_f, plan_b = _lib.Plan(), _lib.Plan()
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 0, plan_f), "plan")
     _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan_b), "plan")
-    # the workspaces lstm.py allocates per call (a one-slot-per-timestep exchange ring when it fits)
+    # the workspaces lstm.py allocates per call (header, barrier counters, two exchange slots)
     ws_f = L._workspace(plan_f, T, H, code, False, dev)
     ws_b = L._workspace(plan_b, T, H, code, True, dev)
 
     def zero_ws(ws, plan):  # the part a call needs zeroed: header, counters, flags
-        n = ws.numel() if (plan.ring_needs_zero or ws.numel() == plan.ws_bytes) else plan.ws_zero_bytes
+        n = ws.numel() if plan.ring_needs_zero else min(ws.numel(), plan.ws_zero_bytes)
         ws[:n].zero_()
 
     def k1():

@@ -57,6 +57,7 @@ SIGNATURES = {
     "fastlstm_ws_status": (_i, [_vp]),
     "fastlstm_device_status": (_i, [_i, _i]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
+    "fastlstm_set_kernel_families": (None, [_i]),
     "fastlstm_set_gemm_trace": (None, [_vp]),
     "fastlstm_set_recurrent_trace": (None, [_vp]),
     "fastlstm_strerror": (ctypes.c_char_p, [_i]),

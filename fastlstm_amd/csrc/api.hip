@@ -26,6 +26,7 @@ struct LaunchOpts {
 
 static long long *g_rec_trace = nullptr;
 static std::atomic<long long> g_spin_limit{400000000ll};  // 4 s of the 100 MHz clock
+static std::atomic<int> g_families{3};   // diagnostics: bit 0 = XCD-local kernels allowed, bit 1 = register-resident wide kernels
 long long spin_limit_ticks() { return g_spin_limit.load(); }
 
 namespace {
@@ -181,7 +182,7 @@ struct XcdCfg {
     int n_ht, gpx, n_groups;   // members of a group, groups per XCD, groups of the launch
     int ks;                    // k-steps of the contraction
     int lds;
-    size_t xslot;              // bytes of one ring slot
+    size_t xslot;              // bytes of one exchange slot (the kernels use two)
 };
 
 // The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
@@ -190,7 +191,7 @@ struct XcdCfg {
 bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c, int launch_rows = 0) {
     const int B = launch_rows ? launch_rows : B_all;
     DeviceInfo di;
-    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
+    if (!(g_families.load() & 1) || device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
     const int s = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     const int K = backward ? 4 * H : H;
     if (K % kstep || (H * s) % 16) return false;
@@ -223,8 +224,7 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
     c->n_groups = cdiv(B, bt);
     if (c->n_groups > kNumXcd * c->gpx) return false;   // (the tile loop above guarantees it; the kernels index counters by group)
     c->xslot = (size_t)c->n_groups * c->ntw * c->ks * kFragBytes;
-    const size_t slots = backward ? (size_t)T : (size_t)T + 1;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + slots * c->xslot) return false;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
     const int gseg = ht * s;
     const int red_blocks = backward ? 8 * c->mt * c->ntw : 4 * c->mt * c->ntw;
     c->lds = red_blocks * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
@@ -294,7 +294,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
                 bool dry_run = false, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c, o.rows)) return 1;
-    if (second && ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + 1) * 2 * c.xslot) return 2;
+    if (second && ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * 2 * c.xslot) return 2;   // both layers' slots side by side
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -369,7 +369,8 @@ struct WideCfg {
 bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0) {
     const int B = rows ? rows : B_all;   // rows of this launch
     DeviceInfo di;
-    if (device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32) return false;
+    if (!(g_families.load() & 2) || device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32)
+        return false;
     if (dtype == FASTLSTM_FP32) return false;
     if (H % 256 || H <= 1024 || H > 2048) return false;   // 1280, 1536, 1792, 2048
     c->nkw = backward ? H / 64 : H / 256;
@@ -380,7 +381,7 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     if (c->n_groups * c->xpg > kNumXcd) return false;
     c->ks = (backward ? 4 * H : H) / 32;
     c->xslot = (size_t)c->n_groups * 4 * c->ks * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + ((size_t)T + (backward ? 0 : 1)) * c->xslot) return false;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
     const int tiles = 64 * (4 * 32 + 16) + 2 * 64 * (32 + 16);   // gates + two state tiles of 64 rows x 16 units
     c->lds = backward ? 8 * 4 * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 16 * kFragBytes + tiles;
     return true;
@@ -560,7 +561,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
                 bool *lower_wgrad_fused = nullptr, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c, o.rows)) return 1;
-    if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + (size_t)T * 2 * c.xslot) return 2;
+    if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * 2 * c.xslot) return 2;   // both layers' slots side by side
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
@@ -824,14 +825,6 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, false);
-    if (sync) {  // as many ring slots as the workspace holds, up to one per version
-        const int full = recurrent_full_slots(T, slot_bytes, false);
-        const size_t avail = (ws_bytes - pl.ws_zero_bytes) / pl.batch_chunks / slot_bytes;
-        p.n_slots = (int)std::min<size_t>(full, avail);
-        // cached loads need a never-reused slot per version and 128-byte lines written by one
-        // workgroup only (16-bit tiles of 4 units share their lines with the neighbour tile)
-        p.coherent_loads = (p.n_slots < T + 1 || (dtype != FASTLSTM_FP32 && pl.ht == 4)) ? 1 : 0;
-    }
     // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
     int lds_bytes = pl.lds_bytes;
     {
@@ -852,7 +845,7 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
         p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
-        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
+        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
@@ -959,12 +952,6 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, true);
-    if (sync) {
-        const int full = recurrent_full_slots(T, slot_bytes, true);
-        const size_t avail = (ws_bytes - pl.ws_zero_bytes) / pl.batch_chunks / slot_bytes;
-        p.n_slots = (int)std::min<size_t>(full, avail);
-        p.coherent_loads = p.n_slots < T ? 1 : 0;
-    }
     // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
     int lds_bytes = pl.lds_bytes;
     {
@@ -977,7 +964,7 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
     for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
         const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
         p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
-        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * p.n_slots * slot_bytes;
+        p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;
         p.b_base = bt0 * pl.bt;
         const int grid = n_bt * pl.n_htiles;
@@ -1337,6 +1324,8 @@ int fastlstm_device_status(int device, int clear) {
     if (clear) __atomic_store_n(di.status_host, 0, __ATOMIC_RELAXED);
     return FASTLSTM_ERR_TIMEOUT;
 }
+
+void fastlstm_set_kernel_families(int mask) { fastlstm::g_families.store(mask & 3); }
 
 void fastlstm_set_spin_limit(long long ticks) {
     if (ticks > 0) fastlstm::g_spin_limit.store(ticks);

@@ -7,8 +7,9 @@
 // amount of arithmetic throughput removes; this kernel runs exactly those links (the functions the
 // real kernels call) for `steps` rounds so that the host can time them:
 //   mode 0  empty barrier: publish + wait only
-//   mode 1  + every member stores its share of a `rows`-row h tile into the step's exchange slot
-//   mode 2  + every wave fetches its operand blocks of the step (the loads the MFMAs would consume)
+//   mode 1  + every member stores its share of a `rows`-row h tile into the step's exchange slot (slot t % 2)
+//   mode 2  + every wave fetches its operand blocks of the step with the loads the real kernels use (they go
+//           past the L1 to the L2: a slot is rewritten every second step)
 //   mode 3, 4  (kind 0) the same exchange WITHOUT a barrier: a ring of 4 slots whose unwritten values hold
 //           a sentinel bit pattern (all ones: a NaN no gate output produces); a member stores its share
 //           of h_{t+1}, resets its share of the slot two versions back, and every wave polls its operand
@@ -27,13 +28,14 @@ namespace fastlstm {
 struct ProbeParams {
     WsHeader *hdr;
     int *counters;         // kind 0: [kXcdReplicas][kXcdCounterStride]; kind 1: one flag per member
-    unsigned char *xbuf;   // ring: [steps + 1][NT][KS] operand blocks of NT 16-row batch tiles
+    unsigned char *xbuf;   // modes 0-2: 2 slots, modes 3-4: 4 slots of [NT][KS] operand blocks of NT 16-row batch tiles
     int members, steps, KS, H, mode, kind, NT;
     long long spin_limit;
     unsigned *sink;        // one word per workgroup: keeps the loads alive
 };
 
 constexpr int kProbeWaves = 8;
+constexpr int kProbeSlots = 4;   // exchange slots behind the counters (modes 0-2 use two of them)
 
 __global__ __launch_bounds__(kWave *kProbeWaves) void step_probe_kernel(const ProbeParams p) {
     using T = _Float16;
@@ -115,12 +117,12 @@ __global__ __launch_bounds__(kWave *kProbeWaves) void step_probe_kernel(const Pr
         // ---- publish version t + 1 ----------------------------------------------------------
         if (p.mode >= 1) {
             if (p.kind == 0) {
-                const XchgL2 xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+                const XchgL2 xw(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
                 for (int it = tid; it < items; it += kWave * kProbeWaves)
                     xw.store_elem(((it >> 4) / HT) * p.KS * kFragBytes + frag_offset<T>(it & 15, j * HT + (it >> 4) % HT),
                                   E::from_f32((float)(t + it)));
             } else {
-                const XchgGlobal xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+                const XchgGlobal xw(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
                 for (int it = tid; it < items; it += kWave * kProbeWaves)
                     xw.store_elem(((it >> 4) / HT) * p.KS * kFragBytes + frag_offset<T>(it & 15, j * HT + (it >> 4) % HT),
                                   E::from_f32((float)(t + it)));
@@ -140,13 +142,14 @@ __global__ __launch_bounds__(kWave *kProbeWaves) void step_probe_kernel(const Pr
         // ---- fetch the group's h_{t+1}: wave w takes k-steps w % shares, + shares, ... of every batch tile
         // (the K-shares of the real kernels), 8 blocks in flight at a time
         if (p.mode >= 2) {
-            const XchgL2 xr(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+            const XchgL2 xr(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
             for (int nt = 0; nt < p.NT; ++nt) {
                 u32x4 v[8];
 #pragma unroll
                 for (int ki = 0; ki < 8; ++ki) {
                     const int ks = min(wave % shares + shares * ki, p.KS - 1);
-                    v[ki] = xr.load16((unsigned)((nt * p.KS + ks) * kWave + lane) * 16u);
+                    const unsigned off = (unsigned)((nt * p.KS + ks) * kWave + lane) * 16u;
+                    v[ki] = xr.load16_l2(off);
                 }
 #pragma unroll
                 for (int ki = 0; ki < 8; ++ki) acc ^= v[ki][0] ^ v[ki][1] ^ v[ki][2] ^ v[ki][3];
@@ -164,7 +167,7 @@ extern "C" {
 
 size_t fastlstm_diag_step_probe_bytes(int steps, int H, int rows) {
     if (steps <= 0 || H <= 0 || H % 32 || rows <= 0 || rows % 16) return 0;
-    return kWsHeaderBytes + kWsCounterBytes + ((size_t)steps + 1) * (rows / 16) * (H / 32) * kFragBytes + 4096;
+    return kWsHeaderBytes + kWsCounterBytes + (size_t)kProbeSlots * (rows / 16) * (H / 32) * kFragBytes + 4096;
 }
 
 int fastlstm_diag_step_probe(int kind, int mode, int members, int H, int rows, int steps, void *ws, size_t ws_bytes,
@@ -180,7 +183,7 @@ int fastlstm_diag_step_probe(int kind, int mode, int members, int H, int rows, i
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
     p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);
     p.xbuf = wsb + kWsHeaderBytes + kWsCounterBytes;
-    p.sink = reinterpret_cast<unsigned *>(p.xbuf + ((size_t)steps + 1) * (rows / 16) * (H / 32) * kFragBytes);
+    p.sink = reinterpret_cast<unsigned *>(p.xbuf + (size_t)kProbeSlots * (rows / 16) * (H / 32) * kFragBytes);
     p.members = members; p.steps = steps; p.KS = H / 32; p.H = H; p.mode = mode; p.kind = kind; p.NT = rows / 16;
     p.spin_limit = spin_limit_ticks();
     int occ = 0;

@@ -80,6 +80,16 @@ __device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t rsrc, u
 #endif
 }
 
+// The same with device scope (sc1): the load misses the non-coherent cache levels.
+__device__ __forceinline__ void load_block_to_lds_device(__amdgpu_buffer_rsrc_t rsrc, unsigned char *lds_block,
+                                                         unsigned voffset, unsigned soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (FASTLSTM_LDS_PTR void *)lds_block, 16, voffset, soffset, 0, 16);
+#else
+    (void)rsrc; (void)lds_block; (void)voffset; (void)soffset;
+#endif
+}
+
 // acc += a . b with the accumulator pinned to the accumulation registers (AGPRs).  With more
 // than 128 accumulators per lane the register allocator otherwise shuttles them between the two
 // halves of the register file around every MFMA.

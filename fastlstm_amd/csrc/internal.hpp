@@ -70,6 +70,5 @@ size_t recurrent_flags_bytes(int n_bt, int n_ht);
 size_t recurrent_slot_bytes(int H, int dtype, int bt, int n_bt, bool backward);
 size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chunks, bool backward, bool sync,
                           int slots);
-int recurrent_full_slots(int T, size_t slot_bytes, bool backward);
 
 }  // namespace fastlstm

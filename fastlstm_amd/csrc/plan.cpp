@@ -77,14 +77,6 @@ size_t recurrent_ws_bytes(int H, int dtype, int bt, int n_bt, int n_ht, int chun
     return kWsHeaderBytes + kWsCounterBytes + (size_t)chunks * (recurrent_flags_bytes(n_bt, n_ht) +
                                   (size_t)slots * recurrent_slot_bytes(H, dtype, bt, n_bt, backward));
 }
-// Slots of a full history ring (one per exchanged version), capped so that one launch's ring
-// stays addressable with 32-bit offsets and the workspace stays modest.
-int recurrent_full_slots(int T, size_t slot_bytes, bool backward) {
-    const size_t cap = (size_t)1 << 30;
-    const long long want = backward ? T : (long long)T + 1;
-    const long long fit = (long long)(cap / std::max<size_t>(slot_bytes, 1));
-    return (int)std::max<long long>(2, std::min(want, fit));
-}
 
 // k-steps are padded to the granule of the streamed K loop (4 waves x 2 chunks x 2 k-steps)
 constexpr int kStreamKPadHost = 16;
@@ -230,9 +222,8 @@ extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, 
     if (!plan || T <= 0 || H <= 0 || !dtype_ok(dtype)) return 0;
     if (plan->wave_split == 2 || plan->wave_split == 3) return plan->ws_bytes;
     const size_t slot = recurrent_slot_bytes(H, dtype, plan->bt, plan->n_btiles, backward != 0);
-    const int slots = recurrent_full_slots(T, slot, backward != 0);
-    size_t ws = recurrent_ws_bytes(H, dtype, plan->bt, plan->n_btiles, plan->n_htiles, plan->batch_chunks,
-                                   backward != 0, true, slots);
+    const int slots = 2;   // every kernel exchanges through two slots, whatever T is
+    size_t ws = plan->ws_bytes;
     // the XCD-local kernels lay their ring out for batch tiles of 16 or 32 rows, which covers at most
     // 16 rows (one operand block per k-step) more than the tiles of the plan
     // (the kernels for H = 1280 ... 2048 use tiles of 64 rows: at most 48 rows more)

@@ -36,14 +36,12 @@ struct BwdParams {
     const void *Wh;     // [4H,H]
     WsHeader *hdr;
     int *flags;
-    unsigned char *xbuf;   // [n_slots][n_bt][NT][KSB] operand blocks
+    unsigned char *xbuf;   // [2 slots][n_bt][NT][KSB] operand blocks
     int T, B, H;
     int b_base;
     int n_bt, n_ht, flag_stride;
     int KSB;            // k-steps covering 4H
     int ht;             // hidden units per workgroup (SPLIT 0/1: 4, 8 or 16)
-    int n_slots;        // exchange ring length (T: every step has its own slot)
-    int coherent_loads; // 1: read the exchange data with device-scope loads
     long long spin_limit;
     int vec_io;         // 1: the VIO instantiation is launched (complete, 16-byte aligned tile segments)
     long long *trace;   // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
@@ -180,8 +178,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
     const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KSB * kFragBytes : (unsigned)KSB * kFragBytes;
     const unsigned xgrp = SYNC ? (unsigned)g * NT * KSB * kFragBytes : 0u;
-    const int n_slots = SYNC ? p.n_slots : 2;
-    const bool coherent = SYNC && p.coherent_loads;
+    constexpr int n_slots = 2;   // reverse step s uses slot s % 2; the loads are device-scope (the address is reused)
     const Xchg xch(SYNC ? p.xbuf : xl, (unsigned)n_slots * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
@@ -559,8 +556,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                 }
             }
         };
-        if (coherent) kloop(std::true_type{});
-        else kloop(std::false_type{});
+        kloop(std::true_type{});
 #pragma unroll
         for (int i = 0; i < NTW; ++i) {
             const int pp = SPLIT == 0 ? wave : 0;

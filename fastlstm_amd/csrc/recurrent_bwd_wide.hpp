@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
     auto step = [&](const int s, auto par) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par)::value;
         const int t = T_ - 1 - s;
-        const XchgGlobal xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
+        const XchgGlobal xch(p.xbuf + (size_t)(s & 1) * xslot, (unsigned)xslot);
 
         // ---- point-wise gate backward for this thread's items --------------------------
 #pragma unroll
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
         for (int i = 0; i < NT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         const unsigned lane_off = (unsigned)lane * 16u;
         auto request = [&](int b) {
-            load_block_to_lds(xch.rsrc, ring + (b % S) * kFragBytes, lane_off, block_off(b));
+            load_block_to_lds_device(xch.rsrc, ring + (b % S) * kFragBytes, lane_off, block_off(b));   // (the slot's address is reused)
         };
 #pragma unroll
         for (int b = 0; b < S; ++b) request(b);

@@ -28,7 +28,7 @@ struct BwdXcdParams {
     const void *Wh;     // [4H,H]
     WsHeader *hdr;
     int *counters;         // [groups][kXcdReplicas][kXcdCounterStride], zero at launch
-    unsigned char *xbuf;   // ring: [T slots][groups][NT][KSB] operand blocks
+    unsigned char *xbuf;   // [2 slots][groups][NT][KSB] operand blocks; reverse step s uses slot s % 2
     int T, B, H;
     int n_ht, gpx, n_groups;
     int b_base;         // first batch row of this launch (a large batch runs as several launches over row ranges)
@@ -460,7 +460,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     auto step = [&](const int s, auto par) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par)::value;
         const int t = T_ - 1 - s;
-        const XchgL2 xch(p.xbuf + (size_t)s * xslot, (unsigned)xslot);
+        const XchgL2 xch(p.xbuf + (size_t)(s & 1) * xslot, (unsigned)xslot);
         // the dout of timestep t - 2 is requested behind this step's publish barrier: when it is the
         // latest timestep of a chunk, that chunk of the upper layer's dx must be complete
         if (lower && wave == 0 && t >= 2 && (t - 2) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - 2);
@@ -547,7 +547,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 const int ks = min(wave + NWV * (k0 + kk), KSB - 1);   // past the end: any valid block (its weights are zero)
 #pragma unroll
                 for (int i = 0; i < NTW; ++i)
-                    bq[kk][i] = xch.load16(xgrp + (unsigned)((i * KSB + ks) * kWave + lane) * 16u);
+                    bq[kk][i] = xch.load16_l2(xgrp + (unsigned)((i * KSB + ks) * kWave + lane) * 16u);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

@@ -34,13 +34,11 @@ struct FwdParams {
     const void *Wh;    // [4H,H]
     WsHeader *hdr;
     int *flags;        // [n_bt][flag_stride]
-    unsigned char *xbuf;  // [n_slots][n_bt][NT][KS] operand blocks
+    unsigned char *xbuf;  // [2 slots][n_bt][NT][KS] operand blocks
     int T, B, H;
     int b_base;        // first batch row covered by this launch
     int n_bt, n_ht, flag_stride;
     int KS;            // k-steps covering H
-    int n_slots;       // exchange ring length (T+1: every step has its own slot)
-    int coherent_loads;  // 1: read the exchange data with device-scope loads
     int vec_io;        // 1: move the ifgo / out / cell tiles through LDS with 16-byte accesses
     int w_regs;        // > 0: k-steps per wave of the W_h slice held in registers (NKW instantiation)
     int keep;          // 1: store the gate pre-activations and every cell state (what the reverse pass reads);
@@ -226,8 +224,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
     using Xchg = typename std::conditional<SYNC, XchgGlobal, XchgLds>::type;
     const unsigned xslot = SYNC ? (unsigned)p.n_bt * NT * KS * kFragBytes : (unsigned)KS * kFragBytes;
     const unsigned xgrp = SYNC ? (unsigned)g * NT * KS * kFragBytes : 0u;
-    const int n_slots = SYNC ? p.n_slots : 2;
-    const bool coherent = SYNC && p.coherent_loads;
+    constexpr int n_slots = 2;   // h_v lives in slot v % 2; the loads are device-scope (the address is reused)
     const Xchg xch(SYNC ? p.xbuf : xl, (unsigned)n_slots * xslot);
     int *my_flag = SYNC ? p.flags + (size_t)g * p.flag_stride + j : nullptr;
     const int *grp_flags = SYNC ? p.flags + (size_t)g * p.flag_stride : nullptr;
@@ -510,13 +507,8 @@ __global__ __launch_bounds__(kThreads) void lstm_fwd_persistent_kernel(const Fwd
 #pragma unroll
                     for (int i = 0; i < NTW; ++i) acc[a][i] = mfma_kstep<T>(wreg[a][ki], bq[ki][i], acc[a][i]);
         };
-        if constexpr (WREG) {
-            if (coherent) kloop_wreg(std::true_type{});
-            else kloop_wreg(std::false_type{});
-        } else {
-            if (coherent) kloop(std::true_type{});
-            else kloop(std::false_type{});
-        }
+        if constexpr (WREG) kloop_wreg(std::true_type{});
+        else kloop(std::true_type{});
 #ifdef FASTLSTM_TIMELINE
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 #endif

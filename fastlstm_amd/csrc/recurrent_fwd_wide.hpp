@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
     }
 
-    // exchange ring: slot s holds h_s, s = 0..T
+    // two exchange slots: h_s lives in slot s % 2
     const unsigned xgrp = (unsigned)g * NT * KS * kFragBytes;
     const size_t xslot = (size_t)p.n_groups * NT * KS * kFragBytes;
     int *grp_flags = p.counters + (size_t)g * kXcdGroupStride;   // n_ht <= kXcdGroupStride flags per group
@@ -179,13 +179,13 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         // ---- partial(a, i) = Wslice(a, this wave's k-steps) . h_{t-1}(i)^T, one batch tile i per pass.
         // The operand blocks of pass i + 1 are requested before pass i is multiplied (two register
         // sets): one exposed round trip per step, the others hide behind the MFMAs.
-        const XchgGlobal xr(p.xbuf + (size_t)t * xslot, (unsigned)xslot);
+        const XchgGlobal xr(p.xbuf + (size_t)(t & 1) * xslot, (unsigned)xslot);
         u32x4 bq[2][NKW];
         auto request = [&](auto ic) __attribute__((always_inline)) {
             constexpr int i = decltype(ic)::value;
 #pragma unroll
-            for (int ki = 0; ki < NKW; ++ki)
-                bq[i & 1][ki] = xr.template load16<false>(xgrp + (unsigned)((i * KS + wave + NWV * ki) * kWave + lane) * 16u);
+            for (int ki = 0; ki < NKW; ++ki)   // device-scope loads: the slot's address is reused every other step
+                bq[i & 1][ki] = xr.template load16<true>(xgrp + (unsigned)((i * KS + wave + NWV * ki) * kWave + lane) * 16u);
         };
         auto pass = [&](auto ic) __attribute__((always_inline)) {
             constexpr int i = decltype(ic)::value;
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         __syncthreads();
 
         // ---- every (tile, lane) item sums the 8 partials and applies the gates -------------------
-        const XchgGlobal xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+        const XchgGlobal xw(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const int tile = wave + NWV * m;

@@ -9,9 +9,11 @@
 //    return at once.  One workgroup fills the register file of a CU, so the up to 32 members of a group
 //    sit on the 32 CUs of their XCD.  The host verifies the dealing once per device before it selects this
 //    kernel, and every launch verifies that its workgroups saw one common r (check_xcd_placement);
-//  * exchange data: ordinary stores (the vector L1 writes through to L2) and ordinary loads.  A
-//    load may hit in the CU's L1, which nobody keeps coherent, so every timestep writes a slot
-//    of its own (ring of T + 1 slots): an address is only read after its single write;
+//  * exchange data: ordinary stores (the vector L1 writes through to L2) into one of TWO slots (h_v in slot
+//    v % 2: a slot is rewritten only after every member has published the version behind it, i.e. has read
+//    it), and loads that bypass the L1 and are served by the XCD's L2 (sc1): nobody keeps the L1s coherent,
+//    and a slot's address is reused every other step.  The exchange data never leaves the L2 (a ring with an
+//    address per timestep, read through the L1, was 10 - 25 % slower per step and cost O(T) workspace);
 //  * barrier: counters in L2.  Atomics execute in the L2, never in an L1: a member adds 1 to
 //    each of kXcdReplicas counters of its group after its stores were acknowledged, and polls
 //    one of them (its index % replicas) with scalar loads that bypass the scalar cache;
@@ -42,7 +44,7 @@ struct FwdXcdParams {
     const void *Wh;    // [4H,H]
     WsHeader *hdr;
     int *counters;        // [groups][kXcdReplicas][kXcdCounterStride], zero at launch
-    unsigned char *xbuf;  // ring: [T+1 slots][groups][NT][KS] operand blocks
+    unsigned char *xbuf;  // [2 slots][groups][NT][KS] operand blocks; h_v lives in slot v % 2
     int T, B, H;
     int n_ht;          // members of a barrier group (<= 32)
     int gpx;           // groups per XCD (32 / n_ht)
@@ -79,8 +81,13 @@ struct XchgL2 {
     __amdgpu_buffer_rsrc_t rsrc;
     __device__ __forceinline__ XchgL2(unsigned char *b, unsigned bytes)
         : rsrc(__builtin_amdgcn_make_buffer_rsrc(b, 0, bytes, 0x00020000)) {}
+    // ordinary load: may be served by the CU's L1 (only for addresses that are written once per launch)
     __device__ __forceinline__ u32x4 load16(unsigned off) const {
         return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+    }
+    // served by the L2: the L1, which may hold the line from the slot's previous use, is bypassed (sc1)
+    __device__ __forceinline__ u32x4 load16_l2(unsigned off) const {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 16);
     }
     template <typename T> __device__ __forceinline__ void store_elem(unsigned off, T v) const {
         if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rsrc, off, 0, 0);
@@ -440,7 +447,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
 
         // ---- acc[a][i] += Wslice(a) . h_{t-1}(i)^T over this wave's k-steps: all operand blocks
         // of the wave are requested at once, the weights come from registers
-        const XchgL2 xr(p.xbuf + (size_t)t * xslot, (unsigned)xslot);
+        const XchgL2 xr(p.xbuf + (size_t)(t & 1) * xslot, (unsigned)xslot);
         f32x4 acc[MTW][NTW];
 #pragma unroll
         for (int a = 0; a < MTW; ++a)
@@ -451,7 +458,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         for (int ki = 0; ki < NKW; ++ki) {
             const int ks = min(kq + 4 * ki, KS - 1);   // past the end: any valid block (its weights are zero)
 #pragma unroll
-            for (int i = 0; i < NTW; ++i) bq[ki][i] = xr.load16(xgrp + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
+            for (int i = 0; i < NTW; ++i) bq[ki][i] = xr.load16_l2(xgrp + (unsigned)((i * KS + ks) * kWave + lane) * 16u);
         }
         __builtin_amdgcn_sched_barrier(0);   // all loads are issued before the first MFMA: one round trip, not NKW
 #pragma unroll
@@ -475,7 +482,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         __syncthreads();
         FASTLSTM_TP(5);
 
-        const XchgL2 xw(p.xbuf + (size_t)(t + 1) * xslot, (unsigned)xslot);
+        const XchgL2 xw(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const int tile = wave + NWV * m;

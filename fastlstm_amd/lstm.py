@@ -61,31 +61,15 @@ def _plan(device, B, H, code, backward):
     return plan
 
 
-# Largest exchange ring (one slot per timestep) a recurrent call may allocate.
-RING_MAX_BYTES = 2 << 30
-
-
 def _workspace(plan, T, H, code, backward, device):
-    """Recurrence workspace, with the part the kernels need zeroed (header, counters, flags).
-
-    Plans whose workgroups synchronise across CUs get a ring with one exchange slot per timestep,
-    sized by fastlstm_recurrent_workspace_bytes(): no address of it is read before its only
-    write, so the kernels can read the exchange data through the caches.  The forward pass then
-    uses the XCD-local kernel where the shape allows (the barrier group on one XCD, exchange
-    through its L2); the backward pass reads d_ifgo[t] once per XCD instead of once per CU.
-    Without room for the ring (RING_MAX_BYTES) the two-slot workspace of the plan is used."""
-    if plan.wave_split == 3:   # streamed weights: flags and exchange slots zeroed, the packed-weights area is written by the call
-        ws = torch.empty(plan.ws_bytes, dtype=torch.uint8, device=device)
-        ws[:plan.ws_zero_bytes].zero_()
-        return ws
-    if plan.wave_split != 2:
-        ring = _lib.load().fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1 if backward else 0)
-        if plan.ws_bytes < ring <= RING_MAX_BYTES:
-            ws = torch.empty(ring, dtype=torch.uint8, device=device)
-            zero = ring if plan.ring_needs_zero else plan.ws_zero_bytes
-            ws[:zero].zero_()
-            return ws
-    return torch.zeros(plan.ws_bytes, dtype=torch.uint8, device=device)
+    """Recurrence workspace, with the part the kernels need zeroed (header, counters, flags; everything
+    when the exchange blocks have padding).  Its size does not depend on T: every kernel exchanges
+    h_t / d_ifgo[t] through two slots (a few hundred KiB; plans that stream W_h add one packed copy of it,
+    which the call itself writes)."""
+    n = _lib.load().fastlstm_recurrent_workspace_bytes(plan, T, H, code, 1 if backward else 0)
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
+    return ws
 
 
 def _check_ws(ws, what):
@@ -150,13 +134,11 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None, keep_activation
 
 
 def _stack2_workspace(plan, T, H, code, device):
-    """Workspace for fastlstm_fwd_stack2 (ring slots for both layers), or None if it would exceed
-    RING_MAX_BYTES; the part the kernels need zeroed is zeroed."""
+    """Workspace for fastlstm_fwd_stack2 (exchange slots for both layers); the part the kernels need
+    zeroed is zeroed."""
     n = _lib.load().fastlstm_stack2_workspace_bytes(plan, T, H, code)
-    if plan.wave_split == 2 or not plan.ws_bytes < n <= RING_MAX_BYTES:
-        return None
     ws = torch.empty(n, dtype=torch.uint8, device=device)
-    ws[:(n if plan.ring_needs_zero else plan.ws_zero_bytes)].zero_()
+    ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
     return ws
 
 
@@ -169,8 +151,6 @@ def stack2_runs_in_one_launch(T, B, I, H, dtype, device):
     with torch.cuda.device(device):
         plan = _plan(torch.device(device), B, H, code, False)
         n = lib.fastlstm_stack2_workspace_bytes(plan, T, H, code)
-        if plan.wave_split == 2 or not plan.ws_bytes < n <= RING_MAX_BYTES:
-            return False
         return lib.fastlstm_fwd_stack2_fused(T, B, I, H, code, n) == 1
 
 
@@ -215,8 +195,6 @@ def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, b
         (out0, cell0, ifgo0), (out1, cell1, ifgo1) = bufs
         plan = _plan(x.device, B, H, code, False)
         ws = _stack2_workspace(plan, T, H, code, x.device)
-        if ws is None:
-            ws = _workspace(plan, T, H, code, False, x.device)
         entry = lib.fastlstm_fwd_stack2 if keep_activations else lib.fastlstm_fwd_stack2_infer
         _lib.check(entry(x.data_ptr(), Wx0.data_ptr(), bx0.data_ptr(), bh0.data_ptr(), Wh0.data_ptr(),
                          ifgo0.data_ptr(), out0.data_ptr(), cell0.data_ptr(), Wx1.data_ptr(),
@@ -318,11 +296,8 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         dWx0, dWh0, db0 = new(G, I), new(G, H), new(G)
         plan = _plan(x.device, B, H, code, True)
         n = lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)
-        if plan.wave_split != 2 and plan.ws_bytes < n <= RING_MAX_BYTES:
-            ws = torch.empty(n, dtype=torch.uint8, device=x.device)
-            ws[:(n if plan.ring_needs_zero else plan.ws_zero_bytes)].zero_()
-        else:
-            ws = _workspace(plan, T, H, code, True, x.device)
+        ws = torch.empty(n, dtype=torch.uint8, device=x.device)
+        ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
         wws = torch.empty(max(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code),
                               lib.fastlstm_wgrad_workspace_bytes(T, B, H, H, code)), dtype=torch.uint8, device=x.device)
         p = lambda t: t.data_ptr()

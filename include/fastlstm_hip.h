@@ -84,13 +84,11 @@ int fastlstm_plan_for(int num_cus, int lds_limit, int B, int H, int dtype, int b
  * used on a device where that was seen.  The launch calls below never synchronise. */
 int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fastlstm_plan *plan);
 
-/* Workspace that gives every timestep its own exchange slot (a ring of T+1 forward / T backward
- * slots, capped at 1 GiB per launch).  With it no exchange address is read before its only
- * write, so the kernels read the exchange data through the caches, and where the shape allows
- * (fastlstm_recurrent_kernel_kind) the XCD-local kernels run: the workgroups that exchange data
- * sit on one XCD and exchange through its L2.  With less, down to plan->ws_bytes, the general
- * kernels exchange through device memory with cache-bypassing loads.  The first
- * plan->ws_zero_bytes bytes must be zero; the rest only if plan->ring_needs_zero. */
+/* Workspace of a recurrent call for this plan: header, barrier counters, flags and TWO exchange slots in the
+ * layout of whichever kernel family the call may choose (fastlstm_recurrent_kernel_kind) -- a few hundred KiB,
+ * independent of T (h_t / d_ifgo[t] of step t live in slot t % 2; plans that stream W_h add one packed copy of
+ * it).  At least plan->ws_bytes.  The first plan->ws_zero_bytes bytes must be zero; the rest only if
+ * plan->ring_needs_zero. */
 size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype, int backward);
 
 /* K1 -- ifgo[T*B,4H] = x[T*B,I] . Wx[4H,I]^T + (bx + bh).
@@ -239,6 +237,12 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
  * Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
+/* Diagnostics: which kernel families the recurrent entry points may choose besides the general kernels: bit 0 =
+ * the XCD-local kernels, bit 1 = the register-resident kernels of H = 1280 ... 2048 (default 3: both).  With 0
+ * every shape runs the general kernels, which lets a test or a measurement put two families side by side on
+ * the same inputs.  Process-wide; no counterpart in the reference. */
+void fastlstm_set_kernel_families(int mask);
+
 /* Reads the status word the recurrent kernels leave at the start of their
  * workspace; `ws_head` points to a HOST copy of the first 64 bytes.
  * 0 = ok, FASTLSTM_ERR_TIMEOUT = a barrier wait gave up (the kernel still ran
@@ -276,9 +280,10 @@ void fastlstm_set_recurrent_trace(void *buf);
 /* Diagnostics: the latency bound of one recurrence step.  Runs `steps` rounds of the links of a timestep
  * that no arithmetic throughput removes, with the recurrent kernels' own barrier and exchange code:
  * mode 0 = the empty barrier (publish + wait), 1 = + every member stores its share of a `rows`-row fp16 h
- * tile into the step's exchange slot, 2 = + every wave fetches its operand blocks of the step; 3, 4 (kind 0
- * only) = the exchange without a barrier: consumers poll the data itself, unwritten values hold an all-ones
- * sentinel, loads bypass the L1 (sc1 / sc0 sc1); the ring part of ws must then be filled with 0xFF bytes.
+ * tile into the step's exchange slot (slot t % 2), 2 = + every wave fetches its operand blocks of the step
+ * (loads that go past the L1, as in the kernels); 3, 4 (kind 0 only) = the exchange without a barrier:
+ * consumers poll the data itself, unwritten values hold an all-ones sentinel, loads bypass the L1 (sc1 /
+ * sc0 sc1); the exchange slots of ws (everything from byte 66560 on) must then hold 0xFF bytes.
  * kind 0 = an XCD-local group of `members` <= 32 workgroups (counters in that XCD's L2), kind 1 = a flag
  * group of `members` <= 256 workgroups over all XCDs (device-scope flags).  H <= 2048, a multiple of 32 and of
  * `members`; rows = 16, 32, 48 or 64 batch rows per group.  The caller times the launch (its duration /

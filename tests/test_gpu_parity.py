@@ -33,6 +33,12 @@ def _gpu_setup():
     L.CHECK_STATUS = old
 
 
+@pytest.fixture(autouse=True)
+def _all_kernel_families():
+    yield
+    _lib.load().fastlstm_set_kernel_families(3)   # whatever a test switched off is back on for the next one
+
+
 def npy(t):
     return t.detach().double().cpu().numpy()
 
@@ -440,8 +446,8 @@ WIDE_CASES = [
 
 @pytest.mark.parametrize("T,B,H,dt", WIDE_CASES)
 def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
-    """H = 1536 / 2048: with the ring workspace the C ABI runs the register-resident kernels whose
-    groups span several XCDs (kernel kind 2), without it the general kernels; both must meet the
+    """H = 1536 / 2048: the C ABI runs the register-resident kernels whose groups span several XCDs
+    (kernel kind 2), or -- with that family switched off -- the general kernels; both must meet the
     oracle on the same inputs."""
     lib = _lib.load()
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
@@ -459,8 +465,8 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
                                       ifgo0.data_ptr(), T, B, 64, H, code, st), "k1")
     results = {}
     for kind in ("general", "wide"):
-        sizes = [plans[bw].ws_bytes if kind == "general" else
-                 lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
+        lib.fastlstm_set_kernel_families(0 if kind == "general" else 3)
+        sizes = [lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
         assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (2 if kind == "wide" else 0)
         assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 1, sizes[1]) in ((0, 2) if kind == "wide" else (0,))
         ifgo = ifgo0.clone()
@@ -503,8 +509,8 @@ XCD_CASES = [
 
 @pytest.mark.parametrize("T,B,H,dt", XCD_CASES)
 def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
-    """The C ABI picks the XCD-local kernels when the workspace holds the exchange ring and the
-    general kernels when it does not; both must meet the oracle, on the same inputs."""
+    """The C ABI picks the XCD-local kernels where the shape allows, and the general kernels when that
+    family is switched off; both must meet the oracle, on the same inputs."""
     lib = _lib.load()
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
     rm = RM[dt]
@@ -522,8 +528,8 @@ def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H
                                       ifgo0.data_ptr(), T, B, H, H, code, st), "k1")
     results = {}
     for kind in ("general", "xcd"):
-        sizes = [plans[bw].ws_bytes if kind == "general" else
-                 lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
+        lib.fastlstm_set_kernel_families(0 if kind == "general" else 3)
+        sizes = [lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
         for bw in (0, 1):
             assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, bw, sizes[bw]) == (1 if kind == "xcd" else 0)
         ifgo = ifgo0.clone()
