@@ -139,7 +139,8 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     // tid_salt is zero.  A caller inside a loop passes one the compiler cannot see through, so that the
     // per-lane address arithmetic below is redone per call instead of being kept in registers (or
     // spilled and reloaded inside the k loop) across the caller's loop.
-    const int tid = threadIdx.x + tid_salt, lane = tid & 63, wave = tid >> 6;
+    // (the wave index as a scalar: the LDS destinations of the LDS-direct loads then need no v_readfirstlane)
+    const int tid = threadIdx.x + tid_salt, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave / WVN, wn = wave % WVN;
     const int nkt = (ke - kb) / BK;
@@ -192,15 +193,21 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     const unsigned a_kstep = A_KM ? (unsigned)BK * p.lda * 2 : BK * 2;  // byte advance per k-tile
     const unsigned b_kstep = B_KM ? (unsigned)BK * p.ldb * 2 : BK * 2;
 
-    // k-tile kt -> LDS stage; the k-tile advance never leaves the operand: scalar offset
-    auto gload = [&](int kt, int stage) {
+    // k-tile kt -> LDS stage, loads `part`, part + parts, ... of the wave's A_LOADS + B_LOADS (all of them:
+    // part 0 of 1); the k-tile advance never leaves the operand: scalar offset.  Inside the main loop the
+    // loads of a k-tile are dealt out among the multiplications, one or two at a time: eight waves that
+    // issue all 64 loads of a k-tile at once fill the vector-memory queue and stand in it instead of
+    // issuing MFMAs (K1 at T*B = 32768, 4H = 4096, K = 1024: 967 -> 1040 TFLOP/s).
+    auto gload = [&](int kt, int stage, int part, int parts) {
         unsigned char *sa = smem + stage * C::STAGE, *sb = sa + C::A_BYTES;
 #pragma unroll
         for (int i = 0; i < C::A_LOADS; ++i)
-            load_block_to_lds(ra_rsrc, sa + (wave + NWAVES * i) * kFragBytes, goff_a, kt * a_kstep + i * a_istep);
+            if (i % parts == part)
+                load_block_to_lds(ra_rsrc, sa + (wave + NWAVES * i) * kFragBytes, goff_a, kt * a_kstep + i * a_istep);
 #pragma unroll
         for (int i = 0; i < C::B_LOADS; ++i)
-            load_block_to_lds(rb_rsrc, sb + (wave + NWAVES * i) * kFragBytes, goff_b, kt * b_kstep + i * b_istep);
+            if ((i + C::A_LOADS) % parts == part)
+                load_block_to_lds(rb_rsrc, sb + (wave + NWAVES * i) * kFragBytes, goff_b, kt * b_kstep + i * b_istep);
     };
     // fragment of rows [tile16*16, +16) of the operand tile, k-step ks
     auto frag = [&](const unsigned char *tile, auto km_, auto ld_, int tile16, int ks) -> u32x4 {
@@ -232,11 +239,12 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     constexpr int D = NS - 1;                         // prefetch distance in k-tiles
     constexpr int LPT = C::A_LOADS + C::B_LOADS;      // loads per k-tile per wave
     static_assert(KSPT % 2 == 0, "fragment register sets alternate by k-step parity");
-    auto tile_ready = [&](int kt) {   // k-tile kt has landed in LDS; the stage of k-tile kt-1 is free
+    // k-tile kt has landed in LDS and the stage of k-tile kt-1 is free: the caller now issues the loads of
+    // k-tile kt-1+NS into it, before it calls tile_ready again
+    auto tile_ready = [&](int kt) {
         if (kt + D <= nkt) wait_vm_at_most<(D - 1) * LPT>();   // D-1 younger tiles may stay in flight
         else wait_vm_at_most<0>();                             // tail: fewer tiles behind this one
         __builtin_amdgcn_s_barrier();
-        if (kt + D < nkt) gload(kt + D, (kt + D) % NS);
     };
     if constexpr (A_KM || B_KM) {
         // Products with a K-major operand: all fragment reads are inline assembly (see
@@ -264,7 +272,7 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
         };
 #pragma unroll
         for (int d = 0; d < D; ++d)
-            if (d < nkt) gload(d, d);
+            if (d < nkt) gload(d, d, 0, 1);
         tile_ready(0);
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[0][j] = rd_b(0, 0, j);
@@ -274,6 +282,7 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
             auto step0 = [&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
                 constexpr bool rdb = i % EVERY == 0;
+                if (kt + D < nkt) gload(kt + D, (kt + D) % NS, i, TM);   // into the stage the last barrier freed
                 if constexpr (rdb) fb[1][i / EVERY] = rd_b(kt, 1, i / EVERY);
                 if constexpr (i + 1 < TM) fs[(i + 1) & 1] = rd_a(kt, 0, i + 1);
                 else fs[(i + 1) & 1] = rd_a(kt, 1, 0);
@@ -330,8 +339,9 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     };
 #pragma unroll
     for (int d = 0; d < D; ++d)
-        if (d < nkt) gload(d, d);
+        if (d < nkt) gload(d, d, 0, 1);
     tile_ready(0);
+    if (D < nkt) gload(D, D % NS, 0, 1);
 #pragma unroll
     for (int i = 0; i < TM; ++i) read_a(0, 0, i);
 #pragma unroll
@@ -346,6 +356,8 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
             // column j of the wave tile is multiplied while the next k-step's fragments stream in
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
+                // behind tile_ready(kt + 1): the stage of k-tile kt is free (its fragments are in registers)
+                if (last && kt + 1 + D < nkt) gload(kt + 1 + D, (kt + 1 + D) % NS, j, TN);
                 if (more) {
                     read_b(nkt_, nks, j);
 #pragma unroll
