@@ -51,10 +51,14 @@ struct BwdParams {
 // SPLIT 2: barrier-free small-H form, wave w owns unit tile w (up to 64 units), one n-tile.
 // VIO: the workgroup's tiles of ifgo[t], cell[t], dout[t] and d_ifgo[t] move between global memory
 // and LDS in 16-byte pieces (waves 1..3) instead of element by element; see the forward kernel.
+// SPLIT 2 with tile I/O runs 8 waves, as the forward kernel does: waves 0..3 compute, waves 4..7 move the tiles.
+template <int SPLIT, bool VIO> constexpr int bwd_threads() { return (SPLIT == 2 && VIO) ? 2 * kThreads : kThreads; }
+
 template <typename T, int NTW, int SPLIT, bool VIO>
-__global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const BwdParams p) {
+__global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persistent_kernel(const BwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
+    constexpr bool IOW = SPLIT == 2 && VIO;   // tile-moving waves 4..7 beside the computing waves 0..3
     constexpr bool ACC = (E::DT == FASTLSTM_FP32);
     constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;
     constexpr int P = SPLIT == 0 ? 4 : 1;
@@ -64,7 +68,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     constexpr int CH = 16 / NTW;                     // k-steps fetched per batch of loads (2 batches in flight)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const bool cw = !IOW || tid < kThreads;              // a computing wave
+    const int wave = IOW ? (tid >> 6) & 3 : tid >> 6;    // (a tile-moving wave mirrors the set-up of wave - 4 and never uses it)
     const int KSB = p.KSB, H = p.H, B = p.B, T_ = p.T;
     const int HT = SYNC ? p.ht : 16 * MTB;           // unit slots per workgroup
     const int RPT = SYNC ? p.ht : 16;                // weight rows stored per unit tile
@@ -93,13 +99,13 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     // [BT][HT] (c_{t-1} and dout[t]) with rows of SROW bytes.  HT is a run-time value here.
     constexpr int HTMAX = SYNC ? 16 : 64;
     constexpr int PPSEG_MAX = HTMAX * E::BYTES / 16 > 0 ? HTMAX * E::BYTES / 16 : 1;
-    constexpr int IOT = kThreads - kWave;   // wave 0 polls the flags and moves nothing
+    constexpr int IOT = IOW ? kThreads : kThreads - kWave;   // wave 0 polls the flags and moves nothing; IOW: waves 4..7
     constexpr int GPT = (BT * 4 * PPSEG_MAX + IOT - 1) / IOT, SPT = (BT * PPSEG_MAX + IOT - 1) / IOT;
     const int GSEG = HT * E::BYTES, GROW = 4 * GSEG + 16, SROW = GSEG + 16;
     const int PPSEG = GSEG / 16;            // 16-byte pieces per segment (>= 1 when VIO)
     const int TILE_BYTES = BT * GROW + 2 * BT * SROW;
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KSB * kFragBytes);   // SYNC: 1 set, else 2 (step parity)
-    const int io_tid = tid - kWave;         // < 0: not an I/O thread
+    const int io_tid = IOW ? tid - kThreads : tid - kWave;   // < 0: not an I/O thread
 
     const T *dout = static_cast<const T *>(p.dout);
     const T *ifgo = static_cast<const T *>(p.ifgo);
@@ -111,7 +117,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     {
         const int Kpad = KSB * E::KSTEP;
         const int total = Kpad * HT;
-        for (int idx = tid; idx < total; idx += kThreads) {
+        for (int idx = tid; cw && idx < total; idx += kThreads) {
             const int ul = idx % HT, k = idx / HT;
             const int uk = k >> 2, gate = k & 3;
             T v = E::from_f32(0.f);
@@ -125,7 +131,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         }
         if (tid < kWave) reinterpret_cast<u32x4 *>(Wl + zero_off)[tid] = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!SYNC) {
-            for (int idx = tid; idx < 2 * KSB * kWave; idx += kThreads)
+            for (int idx = tid; cw && idx < 2 * KSB * kWave; idx += kThreads)
                 reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
         }
     }
@@ -287,7 +293,9 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
         nx[4] = *reinterpret_cast<const NxV *>(gt_ + BT * GROW + soff[0]);
         nx[5] = *reinterpret_cast<const NxV *>(gt_ + BT * GROW + BT * SROW + soff[0]);
     };
-    if constexpr (SPLIT == 2 && VIO) load_items(tiles);
+    if constexpr (SPLIT == 2 && VIO) {
+        if (cw) load_items(tiles);
+    }
     // One reverse step; u = s % PD selects the prefetch ring entry at compile time.
     auto step = [&](const int s, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
@@ -307,6 +315,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
             // and the next step's input tiles are all in LDS.
             using V = typename VecBytes<4 * E::BYTES>::type;
             constexpr int un_ = (u + 1) % PD;
+            if (cw) {
             T xg[4][4], xc[4], xd[4], st_d[4][4];
             if constexpr (VIO) {   // read behind the previous step's barrier (or in the prologue)
 #pragma unroll
@@ -373,9 +382,6 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                     __builtin_memcpy(&v, pk, sizeof(V));
                     *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = v;
                 }
-                if (s + 1 < T_) tiles_to_lds(gpre[un_], cpre[un_], dpre[un_], gt_next);
-                __syncthreads();
-                tile_to_global(t, gt);
             } else {
 #pragma unroll
                 for (int m = 0; m < 4; ++m)
@@ -386,9 +392,19 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
                         dst[(size_t)2 * H] = st_d[m][2];
                         dst[(size_t)3 * H] = st_d[m][3];
                     }
+            }
+            }   // computing waves
+            // tile-moving waves: the next step's inputs into the other tile set before the barrier, this
+            // step's d_ifgo tile out of this one behind it
+            if constexpr (VIO) {
+                if (s + 1 < T_) tiles_to_lds(gpre[un_], cpre[un_], dpre[un_], gt_next);
+                __syncthreads();
+                tile_to_global(t, gt);
+            } else {
                 __syncthreads();
             }
             prefetch(s + PD, uc);
+            if (!cw) return;
             // dh_rec(units of this wave, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over K = 4H
             f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
             u32x4 bq[KSB2];
@@ -593,7 +609,7 @@ __global__ __launch_bounds__(kThreads) void lstm_bwd_persistent_kernel(const Bwd
     T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
 #pragma unroll
     for (int m = 0; m < IPT; ++m)
-        if (valid[m]) {
+        if (cw && valid[m]) {
             dh_out[off_h[m]] = E::from_f32(dh_rec[m]);
             dc_out[off_h[m]] = E::from_f32(dc_state[m]);
         }
