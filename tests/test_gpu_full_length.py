@@ -1,7 +1,8 @@
 """BASELINE.json's long configurations at their FULL sequence length against the fp32 CPU oracle
 (run with -m gpu on an MI355X).
 
-Config C (bf16, B=128, T=256, I=H=2048) and config E (fp16, two stacked layers, B=32, T=2048,
+Config B (fp16, B=64, T=512, I=H=1024: forward and backward) is the headline configuration.  Config C
+(bf16, B=128, T=256, I=H=2048) and config E (fp16, two stacked layers, B=32, T=2048,
 I=H=1024) are the two configurations whose time-dependent host code (exchange ring sizes, chunk
 hand-over between the stacked layers, which kernel a workspace size selects) only shows at the real
 T.  The 16-bit GPU results are compared with the oracle evaluated in fp32 WITHOUT any 16-bit
@@ -75,6 +76,34 @@ def test_config_C_bf16_full_length_vs_fp32_oracle(oracle):
     z = np.zeros((B, H), np.float32)
     o_out, o_cell, o_ifgo = oracle.forward(x.numpy(), z, z, w["weight_ih_l0"], w["bias_ih_l0"], w["weight_hh_l0"],
                                            w["bias_hh_l0"], dtype=np.float32)
+    r = oracle.backward(dout.numpy(), None, None, x.numpy(), o_out, o_cell, o_ifgo, w["weight_ih_l0"],
+                        w["weight_hh_l0"], dtype=np.float32)
+    _report([("out", rel_err(y, o_out[1:])), ("h_n", rel_err(hn[0], o_out[-1])), ("c_n", rel_err(cn[0], o_cell[-1])),
+             ("dx", rel_err(xg.grad, r["dx"])), ("dh0", rel_err(h0g.grad[0], r["dh0"])),
+             ("dc0", rel_err(c0g.grad[0], r["dc0"])), ("dW_x", rel_err(m.weight_ih_l0.grad, r["dWx"])),
+             ("dW_h", rel_err(m.weight_hh_l0.grad, r["dWh"])), ("db_x", rel_err(m.bias_ih_l0.grad, r["db"])),
+             ("db_h", rel_err(m.bias_hh_l0.grad, r["db"]))])
+
+
+def test_config_B_fp16_fwd_bwd_full_size_vs_fp32_oracle(oracle):
+    """The headline configuration, forward AND backward at full size (the GEMMs run inside both recurrent
+    launches), with a non-zero initial state and a random upstream gradient."""
+    T, B, I, H = 512, 64, 1024, 1024
+    dt = torch.float16
+    assert _kind(T, B, H, dt, False) == 1 and _kind(T, B, H, dt, True) == 1   # XCD-local kernels
+    m, w = _weights(I, H, 1, dt, 1235)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, B, I, generator=g).to(dt).float()
+    dout = torch.randn(T, B, H, generator=g).to(dt).float()
+    h0 = (torch.randn(1, B, H, generator=g) * 0.1).to(dt).float()
+    c0 = (torch.randn(1, B, H, generator=g) * 0.1).to(dt).float()
+    xg = x.cuda().to(dt).requires_grad_(True)
+    h0g, c0g = h0.cuda().to(dt).requires_grad_(True), c0.cuda().to(dt).requires_grad_(True)
+    y, (hn, cn) = m(xg, (h0g, c0g))
+    (y.float() * dout.cuda()).sum().backward()
+    torch.cuda.synchronize()
+    o_out, o_cell, o_ifgo = oracle.forward(x.numpy(), h0[0].numpy(), c0[0].numpy(), w["weight_ih_l0"], w["bias_ih_l0"],
+                                           w["weight_hh_l0"], w["bias_hh_l0"], dtype=np.float32)
     r = oracle.backward(dout.numpy(), None, None, x.numpy(), o_out, o_cell, o_ifgo, w["weight_ih_l0"],
                         w["weight_hh_l0"], dtype=np.float32)
     _report([("out", rel_err(y, o_out[1:])), ("h_n", rel_err(hn[0], o_out[-1])), ("c_n", rel_err(cn[0], o_cell[-1])),
