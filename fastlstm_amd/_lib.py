@@ -56,6 +56,7 @@ SIGNATURES = {
     "fastlstm_diag_step_probe_bytes": (_sz, [_i, _i, _i]),
     "fastlstm_ws_status": (_i, [_vp]),
     "fastlstm_device_status": (_i, [_i, _i]),
+    "fastlstm_prepare_forward": (_i, [_vp, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
     "fastlstm_set_kernel_families": (None, [_i]),
     "fastlstm_set_gemm_trace": (None, [_vp]),

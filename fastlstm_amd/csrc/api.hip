@@ -334,6 +334,29 @@ __global__ void zero_words_kernel(unsigned *p, size_t n) {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
+// One launch that gets a forward call ready: clears `zero_words` words of the workspace and writes the initial
+// state (h0, c0, or zeros when they are null) into slot 0 of out and cell, n elements of `esz` bytes each.
+__global__ void prepare_forward_kernel(unsigned *ws, size_t zero_words, unsigned char *out0, unsigned char *cell0,
+                                       const unsigned char *h0, const unsigned char *c0, size_t n, int esz) {
+    const size_t first = blockIdx.x * (size_t)blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = first; i < zero_words; i += stride) ws[i] = 0u;
+    if (esz == 2) {
+        unsigned short *o = reinterpret_cast<unsigned short *>(out0), *c = reinterpret_cast<unsigned short *>(cell0);
+        const unsigned short *h = reinterpret_cast<const unsigned short *>(h0), *cc = reinterpret_cast<const unsigned short *>(c0);
+        for (size_t i = first; i < n; i += stride) {
+            o[i] = h ? h[i] : (unsigned short)0;
+            c[i] = cc ? cc[i] : (unsigned short)0;
+        }
+    } else {
+        unsigned *o = reinterpret_cast<unsigned *>(out0), *c = reinterpret_cast<unsigned *>(cell0);
+        const unsigned *h = reinterpret_cast<const unsigned *>(h0), *cc = reinterpret_cast<const unsigned *>(c0);
+        for (size_t i = first; i < n; i += stride) {
+            o[i] = h ? h[i] : 0u;
+            c[i] = cc ? cc[i] : 0u;
+        }
+    }
+}
+
 // A batch with more 16-row tiles than one XCD-local launch holds (and no fit with 32-row tiles either):
 // rows per launch such that full launches use every XCD with 16-row tiles and the remainder fits
 // too, or 0.  The launches run one after the other on the stream and share the workspace.
@@ -1314,6 +1337,24 @@ int fastlstm_ws_status(const void *ws_head) {
     if (!ws_head) return FASTLSTM_ERR_NULL;
     const WsHeader *h = static_cast<const WsHeader *>(ws_head);
     return h->abort_flag ? FASTLSTM_ERR_TIMEOUT : FASTLSTM_OK;
+}
+
+int fastlstm_prepare_forward(void *ws, size_t zero_bytes, void *out0, void *cell0, const void *h0, const void *c0,
+                             int B, int H, int dtype, void *stream) {
+    if (!ws || !out0 || !cell0 || (h0 == nullptr) != (c0 == nullptr)) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    const int esz = elem_bytes(dtype);
+    const size_t align = (size_t)esz - 1;
+    if (!aligned16(ws) || zero_bytes % 4 || ((reinterpret_cast<size_t>(out0) | reinterpret_cast<size_t>(cell0) |
+                                             reinterpret_cast<size_t>(h0) | reinterpret_cast<size_t>(c0)) & align))
+        return FASTLSTM_ERR_ALIGN;
+    const size_t n = (size_t)B * H;
+    const int blocks = (int)std::min<size_t>(1024, (std::max(n, zero_bytes / 4) + 255) / 256);
+    prepare_forward_kernel<<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<unsigned *>(ws), zero_bytes / 4, static_cast<unsigned char *>(out0), static_cast<unsigned char *>(cell0),
+        static_cast<const unsigned char *>(h0), static_cast<const unsigned char *>(c0), n, esz);
+    return hipGetLastError() == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
 }
 
 int fastlstm_device_status(int device, int clear) {

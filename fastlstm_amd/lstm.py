@@ -72,6 +72,23 @@ def _workspace(plan, T, H, code, backward, device):
     return ws
 
 
+def _prepared_forward_workspace(plan, T, H, code, out, cell, h0, c0, stream):
+    """The workspace of a forward call, cleared where the kernels need zeros, and out[0] / cell[0] set to the
+    initial state (fastlstm/lstm.py:84-90) -- one launch (fastlstm_prepare_forward) instead of three."""
+    lib = _lib.load()
+    n = lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0)
+    ws = torch.empty(n, dtype=torch.uint8, device=out.device)
+    zero = n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes)
+    direct = h0 is None or all(s_.dtype == out.dtype and s_.shape == out[0].shape and s_.is_contiguous() for s_ in (h0, c0))
+    hp, cp = (h0.data_ptr(), c0.data_ptr()) if (direct and h0 is not None) else (None, None)
+    _lib.check(lib.fastlstm_prepare_forward(ws.data_ptr(), zero, out.data_ptr(), cell.data_ptr(), hp, cp,
+                                            out.shape[1], out.shape[2], code, stream), "fastlstm_prepare_forward")
+    if not direct:   # another dtype, a broadcast or a strided state: torch converts (the slots hold zeros)
+        out[0] = h0
+        cell[0] = c0
+    return ws
+
+
 def _check_ws(ws, what):
     # (reading the status word synchronises: not while the stream is being captured into a graph)
     if CHECK_STATUS and not torch.cuda.is_current_stream_capturing():
@@ -114,15 +131,9 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None, keep_activation
         # be 16-byte aligned for the vector loads of the weight-gradient GEMM
         out = torch.empty((seq_len + 1, batch_size, hidden_size), device=x.device, dtype=x.dtype)
         cell = torch.empty_like(out)
-        if h0 is not None:  # fastlstm/lstm.py:88-90
-            out[0] = h0
-            cell[0] = c0
-        else:
-            out[0].zero_()
-            cell[0].zero_()
         plan = _plan(x.device, batch_size, hidden_size, code, False)
-        ws = _workspace(plan, seq_len, hidden_size, code, False, x.device)
         stream = _stream()
+        ws = _prepared_forward_workspace(plan, seq_len, hidden_size, code, out, cell, h0, c0, stream)
         # input projection + time loop in one call (the library fuses the two where CUs would idle)
         entry = lib.fastlstm_fwd_layer if keep_activations else lib.fastlstm_fwd_layer_infer
         _lib.check(entry(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
@@ -607,6 +618,8 @@ class FastLSTM(nn.Module):
             layer += 1
         if self.batch_first:
             x = x.transpose(0, 1)
+        if len(h_n) == 1:   # one layer, one direction: views of the layer's last slots, no copy
+            return x, (h_n[0].unsqueeze(0), c_n[0].unsqueeze(0))
         return x, (torch.stack(h_n), torch.stack(c_n))
 
     def extra_repr(self):

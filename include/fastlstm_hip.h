@@ -237,6 +237,14 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
  * Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
+/* One launch that gets a forward call ready, instead of three fills/copies by the caller: clears the first
+ * `zero_bytes` bytes of the workspace (a multiple of 4; see fastlstm_recurrent_workspace_bytes for how many a
+ * call needs zeroed) and writes the initial state into slot 0 of out and cell: h0, c0 ([B,H] each, dense), or
+ * zeros when both are NULL.  Replaces `out[0] = h_0; cell[0] = c_0` / the zero initialisation of
+ * fastlstm/lstm.py:84-90.  A fill kernel, not a memset: the call can be captured into a graph. */
+int fastlstm_prepare_forward(void *ws, size_t zero_bytes, void *out0, void *cell0, const void *h0, const void *c0,
+                             int B, int H, int dtype, void *stream);
+
 /* Diagnostics: which kernel families the recurrent entry points may choose besides the general kernels: bit 0 =
  * the XCD-local kernels, bit 1 = the register-resident kernels of H = 1280 ... 2048 (default 3: both).  With 0
  * every shape runs the general kernels, which lets a test or a measurement put two families side by side on

@@ -317,6 +317,45 @@ def test_autograd_function_contract():
     assert_close32(h1, hr); assert_close32(c1, cr)
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+def test_prepare_forward_clears_the_workspace_and_sets_the_initial_state(dt):
+    """fastlstm_prepare_forward = `ws[:n].zero_(); out[0] = h0; cell[0] = c0` (or zeros) in one launch."""
+    lib = _lib.load()
+    B, H, code = 37, 72, RM[dt]
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for with_state in (True, False):
+        ws = torch.full((70000,), 0xAB, dtype=torch.uint8, device="cuda")
+        out = torch.randn(3, B, H, device="cuda", generator=g).to(dt)
+        cell = torch.randn(3, B, H, device="cuda", generator=g).to(dt)
+        out_before, cell_before = out.clone(), cell.clone()
+        h0 = torch.randn(B, H, device="cuda", generator=g).to(dt) if with_state else None
+        c0 = torch.randn(B, H, device="cuda", generator=g).to(dt) if with_state else None
+        _lib.check(lib.fastlstm_prepare_forward(ws.data_ptr(), 66560, out.data_ptr(), cell.data_ptr(),
+                                                h0.data_ptr() if with_state else None, c0.data_ptr() if with_state else None,
+                                                B, H, code, st), "prepare")
+        torch.cuda.synchronize()
+        assert int(ws[:66560].max()) == 0 and int(ws[66560:].min()) == 0xAB
+        assert torch.equal(out[0], h0 if with_state else torch.zeros_like(out[0]))
+        assert torch.equal(cell[0], c0 if with_state else torch.zeros_like(cell[0]))
+        assert torch.equal(out[1:], out_before[1:]) and torch.equal(cell[1:], cell_before[1:])
+    assert lib.fastlstm_prepare_forward(ws.data_ptr(), 64, out.data_ptr(), cell.data_ptr(), out.data_ptr(), None,
+                                        B, H, code, st) == _lib.ERR_NULL
+
+
+def test_module_takes_a_state_of_another_dtype_and_layout():
+    """An initial state that is not a dense tensor of the compute dtype goes through torch's conversion
+    (`out[0] = h_0`, fastlstm/lstm.py:88-90) instead of the one-launch preparation: same results."""
+    torch.manual_seed(11)
+    m = FastLSTM(24, 40).to("cuda", torch.float16)
+    x = torch.randn(6, 5, 24, device="cuda", dtype=torch.float16)
+    h0 = torch.randn(1, 5, 40, device="cuda") * 0.3
+    c0 = torch.randn(1, 40, 5, device="cuda").transpose(1, 2) * 0.3          # strided, fp32
+    y1, (h1, c1) = m(x, (h0, c0))
+    y2, (h2, c2) = m(x, (h0.half(), c0.half().contiguous()))
+    assert torch.equal(y1, y2) and torch.equal(h1, h2) and torch.equal(c1, c2)
+
+
 def test_recurrence_vanishes_with_zero_wh(oracle):
     T, B, I, H = 5, 20, 32, 96
     p = make_problem(T, B, I, H, seed=5, dtype=torch.float32)
