@@ -97,7 +97,7 @@ hipError_t launch_colsum_t(const void *in, void *out, float *part, int R, int C,
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(colsum_final_kernel<T>, dim3(cdiv(C, 64)), dim3(256), 0, s, part, static_cast<T *>(out),
+    hipLaunchKernelGGL(colsum_final_kernel<T>, dim3(cdiv(C, kColsumFinalCols)), dim3(256), 0, s, part, static_cast<T *>(out),
                        C, chunks);
     return hipGetLastError();
 }

@@ -305,16 +305,33 @@ __global__ void colsum_partial_kernel(const T *in, float *part, int R, int C, in
 
 // out[c] = sum over chunks of part[chunk][c].  A block of 256 threads covers 64 columns with 4
 // threads each (chunks k = slice, slice + 4, ...), summed through LDS in a fixed order.
+// 256 threads = 16 columns x 16 slices of the chunks; a thread sums chunks slice, slice + 16, ... with 8 loads in
+// flight (a chain of dependent loads over all chunks is pure latency), the slices meet in LDS in a fixed order.
+constexpr int kColsumFinalCols = 16;
 template <typename T> __global__ void colsum_final_kernel(const float *part, T *out, int C, int chunks) {
-    __shared__ float red[4][64];
-    const int cl = threadIdx.x & 63, slice = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + cl;
+    __shared__ float red[16][kColsumFinalCols];
+    const int cl = threadIdx.x & 15, slice = threadIdx.x >> 4;
+    const int c = blockIdx.x * kColsumFinalCols + cl;
     float s = 0.f;
-    if (c < C)
-        for (int k = slice; k < chunks; k += 4) s += part[(size_t)k * C + c];
+    if (c < C) {
+        int k = slice;
+        for (; k + 7 * 16 < chunks; k += 8 * 16) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(k + 16 * u) * C + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; k < chunks; k += 16) s += part[(size_t)k * C + c];
+    }
     red[slice][cl] = s;
     __syncthreads();
-    if (slice == 0 && c < C) out[c] = Elem<T>::from_f32((red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]));
+    if (slice == 0 && c < C) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t += red[i][cl];
+        out[c] = Elem<T>::from_f32(t);
+    }
 }
 
 }  // namespace fastlstm
