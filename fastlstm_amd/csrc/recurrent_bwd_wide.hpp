@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
     static_assert(NB % 4 == 0 && S > 4, "fragment registers rotate by 4; the ring is deeper than the read-ahead");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (uniform: in a scalar register)
     const int q = lane >> 4, r = lane & 15;
     const int KSB = p.KSB, H = p.H, B = p.B, T_ = p.T;
 

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (uniform: in a scalar register)
     const int q = lane >> 4, n = lane & 15;
     const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
     const bool keep = p.keep != 0;   // training: gate pre-activations and every cell state are stored
@@ -112,66 +112,77 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         publish(1);
     }
 
-    const size_t B4H = (size_t)B * 4 * H;
+    const size_t B4H = (size_t)B * 4 * H, BH = (size_t)B * H;
 
     // ---- coalesced tile I/O (see lstm_fwd_persistent_kernel) --------------------------------
-    constexpr int PD = 2;
-    u32x4 gpre[PD][GPT];
+    // The gates tile of a step (x_t.Wx^T + b, 64 rows x 4 gates x 16 units) travels global -> LDS tile with
+    // LDS-direct loads, a step ahead of its use, by waves 1..7: no register holds it meanwhile.  (Held in
+    // registers next to the 128 weight registers and two sets of operand blocks it was spilled right behind
+    // its load, and the spill waited for the load: a memory round trip on every step's critical path,
+    // 9.1 instead of 6.9 us per step at H = 2048.)  A tile row is GROW = 4 * GSEG + 16 bytes = 9 slots of 16
+    // bytes, so lane l of wave instruction i fills slot 64 i + l; the pad slot of a row and rows past B stay
+    // untouched (lanes switched off).
+    constexpr int SPR = GROW / 16, SLOTS = BT * SPR;       // slots per row, per tile
+    constexpr int DMA_N = (SLOTS + kWave - 1) / kWave;     // wave instructions per tile
+    constexpr int DPW = (DMA_N + NWV - 2) / (NWV - 1);     // per moving wave
     const size_t tile_org = (size_t)b0 * 4 * H + u0;
-    auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
-        if (io_tid < 0) return;
+    unsigned dma_off[DPW];
+    bool dma_ok[DPW];
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            const int seg = rem / PPSEG, k = rem % PPSEG;
-            const bool ok = pc < GPIECES && b0 + row < B;
-            const size_t off = ok ? (size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES) : 0;
-            dst[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + tile_org + off);
-        }
-    };
-    auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
+    for (int d = 0; d < DPW; ++d) {
+        const int i = (wave - 1) + (NWV - 1) * d, sl = i * kWave + lane;
+        const int row = sl / SPR, idx = sl % SPR;
+        dma_ok[d] = wave >= 1 && i < DMA_N && sl < SLOTS && idx < 4 * PPSEG && b0 + row < B;
+        dma_off[d] = dma_ok[d] ? (unsigned)(((size_t)row * 4 * H + (size_t)(idx / PPSEG) * H + (idx % PPSEG) * (16 / E::BYTES)) * E::BYTES) : 0u;
+    }
+    auto request_tile = [&](int t) {
+        if (t >= T_) return;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T *>(ifgo) + (size_t)t * B4H + tile_org, 0, (unsigned)((size_t)BT * 4 * H * E::BYTES), 0x00020000);
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            if (io_tid >= 0 && pc < GPIECES)
-                *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
-        }
+        for (int d = 0; d < DPW; ++d)
+            if (dma_ok[d]) load_block_to_lds(rs, tiles + (size_t)((wave - 1) + (NWV - 1) * d) * kFragBytes, dma_off[d], 0);
     };
+    // LDS tiles -> ifgo[t], out[t+1], cell[t+1]: buffer stores with a per-step base in scalar registers and per-lane
+    // byte offsets that never change (the gates tile slot by slot, as it came in; the state tiles in 16-byte pieces)
+    unsigned st_off[SPT];
+    int st_lds[SPT];
+    bool st_ok[SPT];
+#pragma unroll
+    for (int i = 0; i < SPT; ++i) {
+        const int pc = io_tid + IOT * i;
+        const int row = pc / PPSEG, k = pc % PPSEG;
+        st_ok[i] = io_tid >= 0 && pc < SPIECES && b0 + row < B;
+        st_off[i] = st_ok[i] ? (unsigned)(((size_t)row * H + k * (16 / E::BYTES)) * E::BYTES) : 0u;
+        st_lds[i] = st_ok[i] ? row * SROW + k * 16 : 0;
+    }
+    const size_t state_org = (size_t)b0 * H + u0;
     auto tiles_to_global = [&](int t, const unsigned char *gt) {
         const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+        if (keep) {
+            const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(
+                ifgo + (size_t)t * B4H + tile_org, 0, (unsigned)((size_t)BT * 4 * H * E::BYTES), 0x00020000);
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            const int seg = rem / PPSEG, k = rem % PPSEG;
-            if (keep && io_tid >= 0 && pc < GPIECES && b0 + row < B)
-                *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
-                                           k * (16 / E::BYTES)) =
-                    *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
+            for (int d = 0; d < DPW; ++d)
+                if (dma_ok[d])
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        *reinterpret_cast<const u32x4 *>(gt + (size_t)((wave - 1) + (NWV - 1) * d) * kFragBytes + lane * 16), rg,
+                        dma_off[d], 0, 0);
         }
+        const unsigned sbytes = (unsigned)((size_t)BT * H * E::BYTES);
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(out + (size_t)(t + 1) * BH + state_org, 0, sbytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(cell + (size_t)(t + 1) * BH + state_org, 0, sbytes, 0x00020000);
 #pragma unroll
-        for (int i = 0; i < SPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / PPSEG, k = pc % PPSEG;
-            if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
-                const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
-                *reinterpret_cast<u32x4 *>(out + go) = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
+        for (int i = 0; i < SPT; ++i)
+            if (st_ok[i]) {
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(sth + st_lds[i]), rh, st_off[i], 0, 0);
                 if (keep || t + 1 == T_)
-                    *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(stc + st_lds[i]), rc, st_off[i], 0, 0);
             }
-        }
     };
-    auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
-        if (t < T_) fetch_tile(t, gpre[u]);
-    };
-    prefetch(0, std::integral_constant<int, 0>{});
-    prefetch(1, std::integral_constant<int, 1>{});
+    request_tile(0);
 
-    auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
+    auto step = [&](const int t) __attribute__((always_inline)) {
         unsigned char *gt = tiles;
         if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
         __syncthreads();
@@ -205,8 +216,8 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         request(std::integral_constant<int, 0>{});
         pass(std::integral_constant<int, 0>{}); pass(std::integral_constant<int, 1>{});
         pass(std::integral_constant<int, 2>{}); pass(std::integral_constant<int, 3>{});
-        tile_to_lds(gpre[u], gt);
-        __syncthreads();
+        __syncthreads();   // (the gates tile of this step was requested a step ago: the compiler's wait for it, before
+                           // the first LDS access behind the request, fell in the first multiplication pass)
 
         // ---- every (tile, lane) item sums the 8 partials and applies the gates -------------------
         const XchgGlobal xw(p.xbuf + (size_t)((t + 1) & 1) * xslot, (unsigned)xslot);
@@ -252,12 +263,10 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         // requests below and the next step's operand requests then queue behind nothing (measured: 0.2-0.3 us
         // per step at H = 2048)
         if (keep) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        prefetch(t + PD, uc);
+        // the stores above have their data (the tile's rows were read out of LDS): the next step's gates may land there
+        request_tile(t + 1);
     };
-    for (int t0 = 0; t0 < T_; t0 += PD) {
-        step(t0, std::integral_constant<int, 0>{});
-        if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
-    }
+    for (int t = 0; t < T_; ++t) step(t);
 }
 
 }  // namespace fastlstm
