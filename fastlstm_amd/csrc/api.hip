@@ -814,9 +814,6 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
             }
             return (int)FASTLSTM_OK;
         };
-        XcdCfg whole;
-        if (select_xcd(T, B, H, dtype, false, ws_bytes, &whole) && whole.ntw == 2 && whole.nwv == 8)
-            if (const int rows = xcd_rows_per_launch(T, B, H, dtype, false, ws_bytes)) return by_row_ranges(rows);
         int rc = try_fwd_xcd(ifgo, out, cell, Wh, wsb, ws_bytes, T, B, H, dtype, static_cast<hipStream_t>(stream), nullptr,
                              nullptr, nullptr, nullptr, 0, nullptr, false, whole_batch);
         if (rc == 1)

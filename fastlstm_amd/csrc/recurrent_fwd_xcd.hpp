@@ -363,60 +363,97 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 
     // ---- coalesced tile I/O (see lstm_fwd_persistent_kernel) --------------------------------
-    constexpr int PD = 2;
-    u32x4 gpre[PD][GPT];
+    // The gates tile of a step is requested ahead of its use.  Groups of 16 rows hold it in registers for two
+    // steps (gpre) and copy it into the LDS tile when its step comes.  Groups of 32 rows have no registers to
+    // spare for that (it was spilled right behind its load, and the spill waited for the load: a memory round
+    // trip in every step): there the tile goes global -> LDS tile with LDS-direct loads, one step ahead, slot
+    // by slot (a padded tile row is SPR slots of 16 bytes; lane l of wave instruction i fills slot 64 i + l,
+    // the pad slot of a row and rows past B stay untouched), and leaves by the same slots.
+    constexpr bool DMA = NTW == 2 && NWV == 8;
+    constexpr int PD = DMA ? 1 : 2;
+    constexpr int SPR = GROW / 16, SLOTS = BT * SPR;
+    constexpr int DMA_N = (SLOTS + kWave - 1) / kWave, DPW = (DMA_N + NWV - 2) / (NWV - 1);
+    constexpr int GD = DMA ? DPW : GPT;   // gate pieces (or slots) per thread
+    u32x4 gpre[DMA ? 1 : PD][DMA ? 1 : GPT];
     const size_t tile_org = (size_t)b0 * 4 * H + u0;
-    auto fetch_tile = [&](int t, u32x4(&dst)[GPT]) {
-        if (io_tid < 0) return;
+    // Tile I/O goes through buffer loads / stores: the step's base address in scalar registers, per-lane byte offsets
+    // that never change (no 64-bit address arithmetic in vector registers per step)
+    unsigned g_off[GD], s_off[SPT];
+    int g_lds[GD], s_lds[SPT];
+    bool g_ok[GD], s_ok[SPT];
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            const int seg = rem / PPSEG, k = rem % PPSEG;
-            const bool ok = pc < GPIECES && b0 + row < B;
-            const size_t off = ok ? (size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES) : 0;
-            dst[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + tile_org + off);
+    for (int i = 0; i < GD; ++i) {
+        int row, seg, k;
+        if constexpr (DMA) {
+            const int wi = (wave - 1) + (NWV - 1) * i, sl = wi * kWave + lane, idx = sl % SPR;
+            row = sl / SPR; seg = idx / PPSEG; k = idx % PPSEG;
+            g_ok[i] = wave >= 1 && wi < DMA_N && sl < SLOTS && idx < 4 * PPSEG && b0 + row < B;
+            g_lds[i] = g_ok[i] ? sl * 16 : 0;
+        } else {
+            const int pc = io_tid + IOT * i, rem = pc % (4 * PPSEG);
+            row = pc / (4 * PPSEG); seg = rem / PPSEG; k = rem % PPSEG;
+            g_ok[i] = io_tid >= 0 && pc < GPIECES && b0 + row < B;
+            g_lds[i] = g_ok[i] ? row * GROW + seg * GSEG + k * 16 : 0;
+        }
+        g_off[i] = g_ok[i] ? (unsigned)(((size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES)) * E::BYTES) : 0u;
+    }
+#pragma unroll
+    for (int i = 0; i < SPT; ++i) {
+        const int pc = io_tid + IOT * i;
+        const int row = pc / PPSEG, k = pc % PPSEG;
+        s_ok[i] = io_tid >= 0 && pc < SPIECES && b0 + row < B;
+        s_off[i] = s_ok[i] ? (unsigned)(((size_t)row * H + k * (16 / E::BYTES)) * E::BYTES) : 0u;
+        s_lds[i] = s_ok[i] ? row * SROW + k * 16 : 0;
+    }
+    const size_t state_org = (size_t)b0 * H + u0;
+    const unsigned g_bytes = (unsigned)((size_t)BT * 4 * H * E::BYTES), s_bytes = (unsigned)((size_t)BT * H * E::BYTES);
+    auto fetch_tile = [&](int t, u32x4(&dst)[DMA ? 1 : GPT]) {
+        if (io_tid < 0) return;
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(ifgo + (size_t)t * B4H + tile_org, 0, g_bytes, 0x00020000);
+        if constexpr (DMA) {
+#pragma unroll
+            for (int i = 0; i < GD; ++i)
+                if (g_ok[i]) load_block_to_lds(rg, tiles + (size_t)((wave - 1) + (NWV - 1) * i) * kFragBytes, g_off[i], 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < GPT; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(rg, g_off[i], 0, 0);   // (pieces that do not exist read the tile's first bytes)
         }
     };
-    auto tile_to_lds = [&](const u32x4(&src)[GPT], unsigned char *gt) {
+    auto tile_to_lds = [&](const u32x4(&src)[DMA ? 1 : GPT], unsigned char *gt) {
+        if constexpr (!DMA) {
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            if (io_tid >= 0 && pc < GPIECES)
-                *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
+            for (int i = 0; i < GPT; ++i) {
+                const int pc = io_tid + IOT * i;
+                const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+                if (io_tid >= 0 && pc < GPIECES)
+                    *reinterpret_cast<u32x4 *>(gt + row * GROW + (rem / PPSEG) * GSEG + (rem % PPSEG) * 16) = src[i];
+            }
         }
     };
     auto tiles_to_global = [&](int t, const unsigned char *gt) {
         const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+        if (keep) {
+            const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(ifgo + (size_t)t * B4H + tile_org, 0, g_bytes, 0x00020000);
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-            const int seg = rem / PPSEG, k = rem % PPSEG;
-            if (keep && io_tid >= 0 && pc < GPIECES && b0 + row < B)
-                *reinterpret_cast<u32x4 *>(ifgo + ((size_t)t * B + b0 + row) * 4 * H + (size_t)seg * H + u0 +
-                                           k * (16 / E::BYTES)) =
-                    *reinterpret_cast<const u32x4 *>(gt + row * GROW + seg * GSEG + k * 16);
+            for (int i = 0; i < GD; ++i)
+                if (g_ok[i]) __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(gt + g_lds[i]), rg, g_off[i], 0, 0);
         }
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(out + (size_t)(t + 1) * BH + state_org, 0, s_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(cell + (size_t)(t + 1) * BH + state_org, 0, s_bytes, 0x00020000);
 #pragma unroll
-        for (int i = 0; i < SPT; ++i) {
-            const int pc = io_tid + IOT * i;
-            const int row = pc / PPSEG, k = pc % PPSEG;
-            if (io_tid >= 0 && pc < SPIECES && b0 + row < B) {
-                const size_t go = ((size_t)(t + 1) * B + b0 + row) * H + u0 + k * (16 / E::BYTES);
+        for (int i = 0; i < SPT; ++i)
+            if (s_ok[i]) {
                 // a first layer that feeds a second one in the same launch writes its h THROUGH to memory
                 // (sc1): the chunk hand-over below then needs no write-back of this XCD's L2
-                const u32x4 hv = *reinterpret_cast<const u32x4 *>(sth + row * SROW + k * 16);
-                if (feeds) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(out + go), "v"(hv) : "memory");
-                else *reinterpret_cast<u32x4 *>(out + go) = hv;
+                const u32x4 hv = *reinterpret_cast<const u32x4 *>(sth + s_lds[i]);
+                if (feeds) __builtin_amdgcn_raw_buffer_store_b128(hv, rh, s_off[i], 0, 16);
+                else __builtin_amdgcn_raw_buffer_store_b128(hv, rh, s_off[i], 0, 0);
                 if (keep || t + 1 == T_)
-                    *reinterpret_cast<u32x4 *>(cell + go) = *reinterpret_cast<const u32x4 *>(stc + row * SROW + k * 16);
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(stc + s_lds[i]), rc, s_off[i], 0, 0);
             }
-        }
     };
     auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
+        constexpr int u = DMA ? 0 : decltype(uc)::value;
         if (t < T_) fetch_tile(t, gpre[u]);
     };
     if (k1_live) {   // the first chunk of the input projection has to be there
@@ -424,10 +461,10 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
         __syncthreads();
     }
     prefetch(0, std::integral_constant<int, 0>{});
-    prefetch(1, std::integral_constant<int, 1>{});
+    if constexpr (PD > 1) prefetch(1, std::integral_constant<int, 1>{});
 
     auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
+        constexpr int u = DMA ? 0 : decltype(uc)::value;
         unsigned char *gt = tiles;
         FASTLSTM_TP(0);
         // the gates of step t + PD are requested at the end of this step: their chunk must have landed
@@ -524,7 +561,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     };
     for (int t0 = 0; t0 < T_; t0 += PD) {
         step(t0, std::integral_constant<int, 0>{});
-        if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
+        if constexpr (PD > 1)
+            if (t0 + 1 < T_) step(t0 + 1, std::integral_constant<int, 1>{});
     }
     if (feeds) {   // the chunks that no step has counted: every workgroup counts its own part
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
