@@ -383,87 +383,139 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     int *my_counter = grp_counters + (j % kXcdReplicas) * kXcdCounterStride;
 
     // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out --------------------
-    // two sets of tile pieces in flight: the tiles of step s + 2 are requested right after step s's
-    // tile went out (into the set that held step s's own tiles) and go to the LDS behind step s + 1's
-    // K loop -- almost two steps later, which also covers the memory latency while the workgroups
-    // without a role in the recurrence stream their GEMM operands
-    u32x4 gpre[2][GPT], cpre[2][SPT], dpre[2][SPT];
-    unsigned g_glb[GPT], s_glb[SPT];
-    int g_lds[GPT], s_lds[SPT];
-    bool g_ok[GPT], s_ok[SPT];
+    // Buffer loads / stores: the step's base addresses in scalar registers, per-lane byte offsets that never change.
+    // Groups of 16 rows keep two sets of tile pieces in flight in registers: the tiles of step s + 2 are requested
+    // right after step s's tile went out and go to the LDS behind step s + 1's K loop -- almost two steps later,
+    // which also covers the memory latency while the workgroups without a role in the recurrence stream their
+    // GEMM operands.  Groups of 32 rows have no registers for that (the pieces were spilled right behind their
+    // loads, and a spill waits for its load): there the three tiles go global -> LDS tiles with LDS-direct loads,
+    // one step ahead, slot by slot (a padded tile row is a whole number of 16-byte slots; lane l of wave
+    // instruction w fills slot 64 w + l of its tile; pad slots and rows past B stay untouched), and the d_ifgo tile
+    // leaves by the slots the same wave filled.
+    constexpr bool DMA = NTW == 2;
+    constexpr int DIST = DMA ? 1 : 2;                    // steps between the request of a tile and its use
+    constexpr int SPRG = GROW / 16, SPRS = SROW / 16;    // slots per padded row
+    constexpr int NG = (BT * SPRG + kWave - 1) / kWave, NS = (BT * SPRS + kWave - 1) / kWave;   // wave instructions per tile
+    constexpr int DT = (NG + 2 * NS + NWV - 2) / (NWV - 1);                                     // per moving wave
+    constexpr int GD = DMA ? DT : GPT, SD = DMA ? 1 : SPT;
+    u32x4 gpre[DMA ? 1 : 2][DMA ? 1 : GPT], cpre[DMA ? 1 : 2][DMA ? 1 : SPT], dpre[DMA ? 1 : 2][DMA ? 1 : SPT];
+    unsigned g_off[GD], s_off[SD];
+    int g_lds[GD], s_lds[SD], g_kind[GD];   // DMA: tile of item d (0 gates, 1 c, 2 dout; uniform), g_lds = byte inside that tile
+    bool g_ok[GD], s_ok[SD];
+    const size_t tile_org = (size_t)b0 * 4 * H + u0, state_org = (size_t)b0 * H + u0;
+    const unsigned g_bytes = (unsigned)((size_t)BT * 4 * H * E::BYTES), s_bytes = (unsigned)((size_t)BT * H * E::BYTES);
 #pragma unroll
-    for (int i = 0; i < GPT; ++i) {
-        const int pc = io_tid + IOT * i;
-        const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
-        const int seg = rem / PPSEG, k = rem % PPSEG;
-        g_ok[i] = io_tid >= 0 && pc < GPIECES && b0 + row < B;
-        g_lds[i] = g_ok[i] ? row * GROW + seg * GSEG + k * 16 : 0;
-        g_glb[i] = (unsigned)((size_t)b0 * 4 * H + u0) +
-                   (g_ok[i] ? (unsigned)(row * 4 * H + seg * H + k * (16 / E::BYTES)) : 0u);
+    for (int i = 0; i < GD; ++i) {
+        if constexpr (DMA) {
+            const int w = (wave - 1) + (NWV - 1) * i;
+            g_kind[i] = w < NG ? 0 : (w < NG + NS ? 1 : 2);
+            const int wi = w < NG ? w : (w < NG + NS ? w - NG : w - NG - NS), sl = wi * kWave + lane;
+            if (g_kind[i] == 0) {
+                const int row = sl / SPRG, idx = sl % SPRG;
+                g_ok[i] = wave >= 1 && sl < BT * SPRG && idx < 4 * PPSEG && b0 + row < B;
+                g_off[i] = g_ok[i] ? (unsigned)(((size_t)row * 4 * H + (size_t)(idx / PPSEG) * H + (idx % PPSEG) * (16 / E::BYTES)) * E::BYTES) : 0u;
+            } else {
+                const int row = sl / SPRS, idx = sl % SPRS;
+                g_ok[i] = wave >= 1 && w < NG + 2 * NS && sl < BT * SPRS && idx < PPSEG && b0 + row < B;
+                g_off[i] = g_ok[i] ? (unsigned)(((size_t)row * H + idx * (16 / E::BYTES)) * E::BYTES) : 0u;
+            }
+            g_lds[i] = sl * 16;
+        } else {
+            const int pc = io_tid + IOT * i;
+            const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG);
+            const int seg = rem / PPSEG, k = rem % PPSEG;
+            g_kind[i] = 0;
+            g_ok[i] = io_tid >= 0 && pc < GPIECES && b0 + row < B;
+            g_lds[i] = g_ok[i] ? row * GROW + seg * GSEG + k * 16 : 0;
+            g_off[i] = g_ok[i] ? (unsigned)(((size_t)row * 4 * H + (size_t)seg * H + k * (16 / E::BYTES)) * E::BYTES) : 0u;
+        }
     }
 #pragma unroll
-    for (int i = 0; i < SPT; ++i) {
+    for (int i = 0; i < SD; ++i) {
         const int pc = io_tid + IOT * i;
         const int row = pc / PPSEG, k = pc % PPSEG;
-        s_ok[i] = io_tid >= 0 && pc < SPIECES && b0 + row < B;
+        s_ok[i] = !DMA && io_tid >= 0 && pc < SPIECES && b0 + row < B;
         s_lds[i] = s_ok[i] ? row * SROW + k * 16 : 0;
-        s_glb[i] = (unsigned)((size_t)b0 * H + u0) + (s_ok[i] ? (unsigned)(row * H + k * (16 / E::BYTES)) : 0u);
+        s_off[i] = s_ok[i] ? (unsigned)(((size_t)row * H + k * (16 / E::BYTES)) * E::BYTES) : 0u;
     }
-    auto fetch_tiles = [&](int t, u32x4(&gp)[GPT], u32x4(&cp)[SPT], u32x4(&dp)[SPT]) {
+    auto fetch_tiles = [&](int t, u32x4(&gp)[DMA ? 1 : GPT], u32x4(&cp)[DMA ? 1 : SPT], u32x4(&dp)[DMA ? 1 : SPT]) {
         if (io_tid < 0) return;
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(ifgo) + (size_t)t * B4H + tile_org, 0, g_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(cell) + (size_t)t * BH + state_org, 0, s_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(dout) + (size_t)t * BH + state_org, 0, s_bytes, 0x00020000);
+        if constexpr (DMA) {
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) gp[i] = *reinterpret_cast<const u32x4 *>(ifgo + (size_t)t * B4H + g_glb[i]);
+            for (int i = 0; i < GD; ++i) {
+                const int w = (wave - 1) + (NWV - 1) * i;
+                if (g_kind[i] == 0) {
+                    if (g_ok[i]) load_block_to_lds(rg, tiles + (size_t)w * kFragBytes, g_off[i], 0);
+                } else if (g_kind[i] == 1) {
+                    if (g_ok[i]) load_block_to_lds(rc, tiles + BT * GROW + (size_t)(w - NG) * kFragBytes, g_off[i], 0);
+                } else {
+                    if (g_ok[i]) load_block_to_lds(rd, tiles + BT * GROW + BT * SROW + (size_t)(w - NG - NS) * kFragBytes, g_off[i], 0);
+                }
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < SPT; ++i) {
-            cp[i] = *reinterpret_cast<const u32x4 *>(cell + (size_t)t * BH + s_glb[i]);
-            dp[i] = *reinterpret_cast<const u32x4 *>(dout + (size_t)t * BH + s_glb[i]);
+            for (int i = 0; i < GPT; ++i) gp[i] = __builtin_amdgcn_raw_buffer_load_b128(rg, g_off[i], 0, 0);   // (pieces that do not exist read the tile's first bytes)
+#pragma unroll
+            for (int i = 0; i < SPT; ++i) {
+                cp[i] = __builtin_amdgcn_raw_buffer_load_b128(rc, s_off[i], 0, 0);
+                dp[i] = __builtin_amdgcn_raw_buffer_load_b128(rd, s_off[i], 0, 0);
+            }
         }
     };
-    auto tiles_to_lds = [&](const u32x4(&gp)[GPT], const u32x4(&cp)[SPT], const u32x4(&dp)[SPT]) {
-        unsigned char *stc = tiles + BT * GROW, *std_ = stc + BT * SROW;
+    auto tiles_to_lds = [&](const u32x4(&gp)[DMA ? 1 : GPT], const u32x4(&cp)[DMA ? 1 : SPT], const u32x4(&dp)[DMA ? 1 : SPT]) {
+        if constexpr (!DMA) {
+            unsigned char *stc = tiles + BT * GROW, *std_ = stc + BT * SROW;
 #pragma unroll
-        for (int i = 0; i < GPT; ++i)
-            if (g_ok[i]) *reinterpret_cast<u32x4 *>(tiles + g_lds[i]) = gp[i];
+            for (int i = 0; i < GPT; ++i)
+                if (g_ok[i]) *reinterpret_cast<u32x4 *>(tiles + g_lds[i]) = gp[i];
 #pragma unroll
-        for (int i = 0; i < SPT; ++i)
-            if (s_ok[i]) {
-                *reinterpret_cast<u32x4 *>(stc + s_lds[i]) = cp[i];
-                *reinterpret_cast<u32x4 *>(std_ + s_lds[i]) = dp[i];
-            }
+            for (int i = 0; i < SPT; ++i)
+                if (s_ok[i]) {
+                    *reinterpret_cast<u32x4 *>(stc + s_lds[i]) = cp[i];
+                    *reinterpret_cast<u32x4 *>(std_ + s_lds[i]) = dp[i];
+                }
+        }
     };
     // With helpers in the launch the d_ifgo tiles are written THROUGH to memory (sc1): the chunk
     // hand-over below then needs no write-back of this XCD's L2, which stalled the releasing wave --
     // and with it the whole group -- for several microseconds per chunk.
     auto tile_to_global = [&](int t) {
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(d_ifgo + (size_t)t * B4H + tile_org, 0, g_bytes, 0x00020000);
 #pragma unroll
-        for (int i = 0; i < GPT; ++i)
-            if (g_ok[i]) {
+        for (int i = 0; i < GD; ++i)
+            if (g_kind[i] == 0 && g_ok[i]) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(tiles + g_lds[i]);
-                T *dst = d_ifgo + (size_t)t * B4H + g_glb[i];
-                if (k5_live) asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
-                else *reinterpret_cast<u32x4 *>(dst) = v;
+                if (k5_live) __builtin_amdgcn_raw_buffer_store_b128(v, rg, g_off[i], 0, 16);
+                else __builtin_amdgcn_raw_buffer_store_b128(v, rg, g_off[i], 0, 0);
             }
     };
     if (lower) {   // the latest chunk(s) of this layer's dout have to be there
         if (wave == 0) {
             wait_dout(T_ - 1);
-            if (T_ > 1) wait_dout(T_ - 2);
+            if (DIST > 1 && T_ > 1) wait_dout(T_ - 2);
         }
         __syncthreads();
     }
     fetch_tiles(T_ - 1, gpre[0], cpre[0], dpre[0]);
-    if (T_ > 1) fetch_tiles(T_ - 2, gpre[1], cpre[1], dpre[1]);
-    tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
+    if constexpr (DMA) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's share of the tiles has landed before anyone reads them
+    } else {
+        if (T_ > 1) fetch_tiles(T_ - 2, gpre[1], cpre[1], dpre[1]);
+        tiles_to_lds(gpre[0], cpre[0], dpre[0]);   // step 0 works on the LDS tiles right away
+    }
     __syncthreads();
 
     // one reverse step; PAR = s % 2 picks the register sets at compile time
     auto step = [&](const int s, auto par) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par)::value;
+        constexpr int PAR = DMA ? 0 : decltype(par)::value, PARN = DMA ? 0 : (PAR ^ 1);
         const int t = T_ - 1 - s;
         const XchgL2 xch(p.xbuf + (size_t)(s & 1) * xslot, (unsigned)xslot);
-        // the dout of timestep t - 2 is requested behind this step's publish barrier: when it is the
+        // the dout of timestep t - DIST is requested behind this step's publish barrier: when it is the
         // latest timestep of a chunk, that chunk of the upper layer's dx must be complete
-        if (lower && wave == 0 && t >= 2 && (t - 2) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - 2);
+        if (lower && wave == 0 && t >= DIST && (t - DIST) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - DIST);
 
         // ---- point-wise gate backward for this thread's items --------------------------
 #pragma unroll
@@ -518,7 +570,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         if (tid < kXcdReplicas)
             __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         tile_to_global(t);
-        if (s + 2 < T_) fetch_tiles(t - 2, gpre[PAR], cpre[PAR], dpre[PAR]);
+        if (s + DIST < T_) fetch_tiles(t - DIST, gpre[PAR], cpre[PAR], dpre[PAR]);
 
         if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, vg, s);
         __syncthreads();
@@ -563,7 +615,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
 #pragma unroll
             for (int i = 0; i < NTW; ++i) red[((wave * MT + a) * NT + i) * kWave + lane] = acc[a][i];
         // the tile was drained before the barrier above: the next step's inputs take its place
-        if (s + 1 < T_) tiles_to_lds(gpre[PAR ^ 1], cpre[PAR ^ 1], dpre[PAR ^ 1]);
+        if (s + 1 < T_) tiles_to_lds(gpre[PARN], cpre[PARN], dpre[PARN]);
         __syncthreads();
         const float *redf = reinterpret_cast<const float *>(red);
 #pragma unroll
