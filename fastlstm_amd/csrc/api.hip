@@ -384,9 +384,10 @@ static bool clear_xcd_counters(unsigned char *wsb, hipStream_t s) {
 }
 
 // Shape of a launch of the register-resident kernels whose barrier groups span several XCDs
-// (recurrent_fwd_wide.hpp): 16 units x 64 batch rows per workgroup, H / 16 workgroups per group.
+// (recurrent_fwd_wide.hpp): 16 units x 16 nt batch rows per workgroup, H / 16 workgroups per group.
 struct WideCfg {
     int nkw, n_ht, xpg, n_groups, ks, lds;
+    int nt;   // batch tiles of 16 rows per group: the smallest of 1, 2, 4 with which the launch holds the batch
     size_t xslot;
 };
 bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0) {
@@ -400,13 +401,17 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     c->n_ht = H / 16;
     if (c->n_ht > kXcdGroupStride) return false;
     c->xpg = cdiv(c->n_ht, 32);   // XCDs per group (the last one partly used when H is not a multiple of 512)
-    c->n_groups = cdiv(B, 64);
+    // groups of 16 or 32 rows where they all fit the launch: more groups = more CUs for a small batch, and a
+    // CU then fetches a quarter or half of the operand bytes per step
+    c->nt = cdiv(B, 16) * c->xpg <= kNumXcd ? 1 : cdiv(B, 32) * c->xpg <= kNumXcd ? 2 : 4;
+    c->n_groups = cdiv(B, 16 * c->nt);
     if (c->n_groups * c->xpg > kNumXcd) return false;
     c->ks = (backward ? 4 * H : H) / 32;
-    c->xslot = (size_t)c->n_groups * 4 * c->ks * kFragBytes;
+    c->xslot = (size_t)c->n_groups * c->nt * c->ks * kFragBytes;
     if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
-    const int tiles = 64 * (4 * 32 + 16) + 2 * 64 * (32 + 16);   // gates + two state tiles of 64 rows x 16 units
-    c->lds = backward ? 8 * 4 * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 16 * kFragBytes + tiles;
+    const int gr = 16 * c->nt;
+    const int tiles = gr * (4 * 32 + 16) + 2 * gr * (32 + 16);   // gates + two state tiles of `gr` rows x 16 units
+    c->lds = backward ? 8 * c->nt * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 4 * c->nt * kFragBytes + tiles;
     return true;
 }
 
@@ -438,9 +443,9 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.keep = o.keep;
     auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
     int occ = 0;
-    if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, c.nt, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
-    if (launch(p, c.nkw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, c.nt, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
@@ -460,9 +465,9 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     p.spin_limit = spin_limit_ticks();
     auto launch = dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16;
     int occ = 0;
-    if (launch(p, c.nkw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, c.nt, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
-    if (launch(p, c.nkw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, c.nt, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 

@@ -38,9 +38,9 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_k
                                          int *max_blocks_per_cu);                                 \
     hipError_t launch_bwd_xcd_help_##SUF(const BwdXcdParams &p, int mt, int nkw, int ntw, int grid, int lds, \
                                          hipStream_t s, int *max_blocks_per_cu);                  \
-    hipError_t launch_fwd_wide_##SUF(const FwdXcdParams &p, int nkw, int grid, int lds, hipStream_t s, \
+    hipError_t launch_fwd_wide_##SUF(const FwdXcdParams &p, int nkw, int nt, int grid, int lds, hipStream_t s, \
                                      int *max_blocks_per_cu);                                    \
-    hipError_t launch_bwd_wide_##SUF(const BwdXcdParams &p, int nkw, int grid, int lds, hipStream_t s, \
+    hipError_t launch_bwd_wide_##SUF(const BwdXcdParams &p, int nkw, int nt, int grid, int lds, hipStream_t s, \
                                      int *max_blocks_per_cu);
 FASTLSTM_DECL_REC(f32)
 FASTLSTM_DECL_REC(f16)

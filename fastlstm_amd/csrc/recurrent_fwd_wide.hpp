@@ -8,15 +8,15 @@
 // of which has to read the h_t of ALL batch rows every step (512 KiB per CU and step for B = 128).
 // Here a workgroup of 8 waves holds 16 units x 4 gates x H (256 KiB for H = 2048) in registers, as
 // the XCD-local kernel does, so a group needs H / 16 workgroups (128) and the launch has room for two
-// groups of 64 batch rows: half the operand volume per CU.
+// groups of up to 64 batch rows: half the operand volume per CU.
 //  * placement: group g takes the workgroups of XCDs [g * xpg, (g + 1) * xpg), xpg = H / 16 / 32, so
 //    an XCD's L2 only ever holds the exchange data of one group;
-//  * exchange: device-scope (write-through) stores into a ring with one slot per timestep, ordinary
-//    cached loads (no address is read before its only write; the 32 CUs of an XCD share one fetch);
+//  * exchange: device-scope (write-through) stores into two slots (h_s lives in slot s % 2) and
+//    device-scope loads (past the CU's L1, served by the XCD's L2; the 32 CUs of an XCD share one fetch);
 //  * barrier: one flag per workgroup, raised with a device-scope store, polled by wave 0 of every
 //    member (wait_versions); h_t goes from the LDS tile to the exchange slot in whole 16-byte pieces;
 //  * the 8 waves split K eight ways (no wave loads an operand block that another wave of the
-//    workgroup loads too); the 4 batch tiles of 16 rows are multiplied one after the other, the operand
+//    workgroup loads too); the NT batch tiles of 16 rows are multiplied one after the other, the operand
 //    blocks of the next one in flight meanwhile: weights (128 registers), two sets of operand blocks
 //    (64) and accumulators (16) stay within 256 registers.
 // Requirements (host): 16-bit elements, H = 256 * NKW (1280 ... 2048), groups * xpg <= 8 with xpg = ceil(H / 512).
@@ -27,13 +27,25 @@
 
 namespace fastlstm {
 
-template <typename T, int NKW>
+// f(integral_constant<int, I>) for I = 0 .. N-1, each with its own compile-time index
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// NT batch tiles of 16 rows per group: 4 (64 rows; groups x XCDs-per-group <= 8 limits a launch to 128 rows at
+// H = 2048), or 2 or 1 where the batch fits the launch that way: a small batch then spreads over more groups,
+// i.e. more CUs, and a CU fetches a half or a quarter of the operand bytes per step (H = 2048, B = 16:
+// 3.3 instead of 5.8 us per step).
+template <typename T, int NKW, int NT>
 __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdParams p) {
     static_assert(sizeof(T) == 2, "16-bit element types");
     using E = Elem<T>;
     constexpr int NWV = 8, NTHR = kWave * NWV;
-    constexpr int MT = 4, NT = 4, TILES = MT * NT;           // unit tiles, batch tiles of 16 rows
-    constexpr int IPT = TILES / NWV;                         // (tile, lane) items per thread
+    constexpr int MT = 4, TILES = MT * NT;                   // unit tiles, batch tiles of 16 rows
+    constexpr int IPT = (TILES + NWV - 1) / NWV;             // (tile, lane) items per thread
     constexpr int HT = 4 * MT, BT = 16 * NT;
     constexpr int GSEG = HT * E::BYTES;                      // bytes of one gate segment of a row
     constexpr int GROW = 4 * GSEG + 16, SROW = GSEG + 16;
@@ -89,7 +101,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
         const int tile = wave + NWV * m;
         const int mt = tile / NT, nt = tile % NT;
         const int unit = u0 + mt * 4 + q, b = b0 + nt * 16 + n;
-        valid[m] = b < B;
+        valid[m] = tile < TILES && b < B;
         off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
         xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
         goff[m] = (nt * 16 + n) * GROW + (mt * 4 + q) * E::BYTES;
@@ -115,7 +127,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     const size_t B4H = (size_t)B * 4 * H, BH = (size_t)B * H;
 
     // ---- coalesced tile I/O (see lstm_fwd_persistent_kernel) --------------------------------
-    // The gates tile of a step (x_t.Wx^T + b, 64 rows x 4 gates x 16 units) travels global -> LDS tile with
+    // The gates tile of a step (x_t.Wx^T + b, BT rows x 4 gates x 16 units) travels global -> LDS tile with
     // LDS-direct loads, a step ahead of its use, by waves 1..7: no register holds it meanwhile.  (Held in
     // registers next to the 128 weight registers and two sets of operand blocks it was spilled right behind
     // its load, and the spill waited for the load: a memory round trip on every step's critical path,
@@ -214,8 +226,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
             __builtin_amdgcn_sched_barrier(0);
         };
         request(std::integral_constant<int, 0>{});
-        pass(std::integral_constant<int, 0>{}); pass(std::integral_constant<int, 1>{});
-        pass(std::integral_constant<int, 2>{}); pass(std::integral_constant<int, 3>{});
+        static_for<0, NT>(pass);
         __syncthreads();   // (the gates tile of this step was requested a step ago: the compiler's wait for it, before
                            // the first LDS access behind the request, fell in the first multiplication pass)
 
@@ -224,6 +235,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             const int tile = wave + NWV * m;
+            if (tile >= TILES) continue;   // (16-row groups: four tiles for eight waves)
             f32x4 s = red[tile * kWave + lane];
 #pragma unroll
             for (int pp = 1; pp < NWV; ++pp) s += red[(pp * TILES + tile) * kWave + lane];

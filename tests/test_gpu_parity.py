@@ -480,6 +480,14 @@ WIDE_CASES = [
     (3, 40, 2048, torch.float16),     # one partly filled group
     (4, 128, 1280, torch.float16),    # 80 workgroups per group over three XCDs, the third partly used
     (3, 70, 1792, torch.bfloat16),    # 112 workgroups per group over four XCDs
+    # batches that fit the launch as groups of 16 rows (one batch tile per workgroup)
+    (4, 32, 2048, torch.bfloat16),    # two 16-row groups of four XCDs each
+    (3, 20, 1536, torch.float16),     # ragged second group
+    (3, 9, 1792, torch.bfloat16),     # one partly filled group
+    (4, 32, 1280, torch.float16),     # three XCDs per group, the third partly used
+    # ... and as groups of 32 rows
+    (3, 64, 2048, torch.float16),
+    (4, 50, 1536, torch.bfloat16),    # ragged second group
 ]
 
 
