@@ -18,7 +18,8 @@ OBJDIR = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(LIBDIR, "libfastlstm_hip.so")
 SOURCES = ["api.hip", "gemm.hip", "diag.hip", "recurrent_stream.hip", "plan.cpp", "recurrent_f32.hip", "recurrent_f16.hip", "recurrent_bf16.hip",
            "recurrent_wreg_f32.hip", "recurrent_wreg_f16.hip", "recurrent_wreg_bf16.hip",
-           "recurrent_xcd_f32.hip", "recurrent_xcd_f16.hip", "recurrent_xcd_bf16.hip"]
+           "recurrent_xcd_f32.hip", "recurrent_xcd_f16.hip", "recurrent_xcd_bf16.hip",
+           "recurrent_wsplit_f16.hip", "recurrent_wsplit_bf16.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

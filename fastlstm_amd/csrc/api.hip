@@ -9,6 +9,7 @@
 #include "recurrent_fwd.hpp"
 #include "recurrent_bwd_xcd.hpp"
 #include "recurrent_bwd_wide.hpp"
+#include "recurrent_bwd_wide_split.hpp"
 #include "recurrent_fwd_xcd.hpp"
 #include "recurrent_stream.hpp"
 
@@ -26,7 +27,7 @@ struct LaunchOpts {
 
 static long long *g_rec_trace = nullptr;
 static std::atomic<long long> g_spin_limit{400000000ll};  // 4 s of the 100 MHz clock
-static std::atomic<int> g_families{3};   // diagnostics: bit 0 = XCD-local kernels allowed, bit 1 = register-resident wide kernels
+static std::atomic<int> g_families{7};   // diagnostics: bit 0 = XCD-local kernels allowed, bit 1 = register-resident wide kernels, bit 2 = their reverse form with teams
 long long spin_limit_ticks() { return g_spin_limit.load(); }
 
 namespace {
@@ -388,6 +389,7 @@ static bool clear_xcd_counters(unsigned char *wsb, hipStream_t s) {
 struct WideCfg {
     int nkw, n_ht, xpg, n_groups, ks, lds;
     int nt;   // batch tiles of 16 rows per group: the smallest of 1, 2, 4 with which the launch holds the batch
+    int v;    // reverse kernel, 64-row groups: members of a team that splits K (lstm_bwd_wide_split_kernel); 0 = no teams
     size_t xslot;
 };
 bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0) {
@@ -412,6 +414,15 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     const int gr = 16 * c->nt;
     const int tiles = gr * (4 * 32 + 16) + 2 * gr * (32 + 16);   // gates + two state tiles of `gr` rows x 16 units
     c->lds = backward ? 8 * c->nt * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 4 * c->nt * kFragBytes + tiles;
+    c->v = 0;
+    if (backward && c->nt == 4 && (g_families.load() & 4)) {
+        const int v = 4;   // divides the k-steps per wave (20 ... 32) and the workgroups of an XCD
+        const size_t partials = (size_t)c->n_groups * c->n_ht * v * 4 * kFragBytes;
+        if (c->n_ht % v == 0 && ws_bytes >= kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot + partials) {
+            c->v = v;
+            c->lds = 4 * kFragBytes + tiles + 8 * 4 * v * kFragBytes;   // the waves' sums take the place of their rings
+        }
+    }
     return true;
 }
 
@@ -463,11 +474,14 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     p.n_ht = c.n_ht; p.gpx = c.xpg; p.n_groups = c.n_groups; p.KSB = c.ks;
     p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
-    auto launch = dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16;
+    p.partials = p.xbuf + 2 * c.xslot;
+    auto launch = c.v ? (dtype == FASTLSTM_FP16 ? launch_bwd_wide_split_f16 : launch_bwd_wide_split_bf16)
+                      : (dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16);
+    const int form = c.v ? c.v : c.nt;
     int occ = 0;
-    if (launch(p, c.nkw, c.nt, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, form, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
-    if (launch(p, c.nkw, c.nt, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+    if (launch(p, c.nkw, form, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
@@ -1368,7 +1382,7 @@ int fastlstm_device_status(int device, int clear) {
     return FASTLSTM_ERR_TIMEOUT;
 }
 
-void fastlstm_set_kernel_families(int mask) { fastlstm::g_families.store(mask & 3); }
+void fastlstm_set_kernel_families(int mask) { fastlstm::g_families.store(mask & 7); }
 
 void fastlstm_set_spin_limit(long long ticks) {
     if (ticks > 0) fastlstm::g_spin_limit.store(ticks);

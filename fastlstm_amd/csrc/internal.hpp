@@ -41,7 +41,9 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_k
     hipError_t launch_fwd_wide_##SUF(const FwdXcdParams &p, int nkw, int nt, int grid, int lds, hipStream_t s, \
                                      int *max_blocks_per_cu);                                    \
     hipError_t launch_bwd_wide_##SUF(const BwdXcdParams &p, int nkw, int nt, int grid, int lds, hipStream_t s, \
-                                     int *max_blocks_per_cu);
+                                     int *max_blocks_per_cu);                                    \
+    hipError_t launch_bwd_wide_split_##SUF(const BwdXcdParams &p, int nkw, int v, int grid, int lds, hipStream_t s, \
+                                           int *max_blocks_per_cu);
 FASTLSTM_DECL_REC(f32)
 FASTLSTM_DECL_REC(f16)
 FASTLSTM_DECL_REC(bf16)

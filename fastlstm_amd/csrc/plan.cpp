@@ -231,5 +231,8 @@ extern "C" size_t fastlstm_recurrent_workspace_bytes(const fastlstm_plan *plan, 
     const int margin = (dtype != FASTLSTM_FP32 && H > 1024 && H <= 2048 && H % 256 == 0) ? 3 : 1;
     ws = std::max(ws, kWsHeaderBytes + kWsCounterBytes +
                           (size_t)slots * (plan->batch_chunks * slot + (size_t)margin * KS * kFragBytes));
+    // the reverse kernel of those hidden sizes exchanges partial sums among teams of up to 8 workgroups:
+    // 4 KiB per (receiver, sender), 256 workgroups
+    if (backward && margin == 3) ws += (size_t)256 * 8 * 4 * kFragBytes;
     return ws;
 }

@@ -70,6 +70,7 @@ struct BwdXcdParams {
     int k8_lo_tiles_n, wg_lo_tiles;
     float *wg_scratch_lo;
     long long spin_limit;
+    unsigned char *partials;   // lstm_bwd_wide_split_kernel: the teams' partial sums (see there)
 };
 
 // One 256 x 256 tile of dx = d_ifgo . Wx as a real function call.  The caller keeps the 128

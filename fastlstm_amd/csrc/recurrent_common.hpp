@@ -23,6 +23,8 @@
 // abort flag in the workspace header that ends every other wait as well, so the grid
 // always drains.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace fastlstm {
@@ -70,6 +72,14 @@ struct XchgLds {
     __device__ __forceinline__ void store16(unsigned off, u32x4 v) const { *reinterpret_cast<u32x4 *>(base + off) = v; }
 };
 
+
+// f(integral_constant<int, I>) for I = 0 .. N-1, each with its own compile-time index
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 // A value that is the same in all lanes, moved to scalar registers (the compiler cannot always tell).
 __device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }

@@ -27,14 +27,6 @@
 
 namespace fastlstm {
 
-// f(integral_constant<int, I>) for I = 0 .. N-1, each with its own compile-time index
-template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 // NT batch tiles of 16 rows per group: 4 (64 rows; groups x XCDs-per-group <= 8 limits a launch to 128 rows at
 // H = 2048), or 2 or 1 where the batch fits the launch that way: a small batch then spreads over more groups,
 // i.e. more CUs, and a CU fetches a half or a quarter of the operand bytes per step (H = 2048, B = 16:

@@ -246,7 +246,8 @@ int fastlstm_prepare_forward(void *ws, size_t zero_bytes, void *out0, void *cell
                              int B, int H, int dtype, void *stream);
 
 /* Diagnostics: which kernel families the recurrent entry points may choose besides the general kernels: bit 0 =
- * the XCD-local kernels, bit 1 = the register-resident kernels of H = 1280 ... 2048 (default 3: both).  With 0
+ * the XCD-local kernels, bit 1 = the register-resident kernels of H = 1280 ... 2048, bit 2 = the form of their
+ * reverse kernel in which teams of workgroups split the sums over K (default 7: all).  With 0
  * every shape runs the general kernels, which lets a test or a measurement put two families side by side on
  * the same inputs.  Process-wide; no counterpart in the reference. */
 void fastlstm_set_kernel_families(int mask);

@@ -480,6 +480,7 @@ WIDE_CASES = [
     (3, 40, 2048, torch.float16),     # one partly filled group
     (4, 128, 1280, torch.float16),    # 80 workgroups per group over three XCDs, the third partly used
     (3, 70, 1792, torch.bfloat16),    # 112 workgroups per group over four XCDs
+    (6, 128, 1536, torch.bfloat16),   # two full groups of three XCDs
     # batches that fit the launch as groups of 16 rows (one batch tile per workgroup)
     (4, 32, 2048, torch.bfloat16),    # two 16-row groups of four XCDs each
     (3, 20, 1536, torch.float16),     # ragged second group
@@ -495,7 +496,8 @@ WIDE_CASES = [
 def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
     """H = 1536 / 2048: the C ABI runs the register-resident kernels whose groups span several XCDs
     (kernel kind 2), or -- with that family switched off -- the general kernels; both must meet the
-    oracle on the same inputs."""
+    oracle on the same inputs.  So must both forms of the reverse kernel for groups of 64 rows: every
+    workgroup sums over all of K, or teams of workgroups split K and exchange partial sums."""
     lib = _lib.load()
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
     rm = RM[dt]
@@ -511,11 +513,11 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
     _lib.check(lib.fastlstm_gemm_ifgo(g["x"].data_ptr(), g["Wx"].data_ptr(), g["bx"].data_ptr(), g["bh"].data_ptr(),
                                       ifgo0.data_ptr(), T, B, 64, H, code, st), "k1")
     results = {}
-    for kind in ("general", "wide"):
-        lib.fastlstm_set_kernel_families(0 if kind == "general" else 3)
+    for kind in ("general", "wide", "teams"):
+        lib.fastlstm_set_kernel_families({"general": 0, "wide": 3, "teams": 7}[kind])
         sizes = [lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
-        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (2 if kind == "wide" else 0)
-        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 1, sizes[1]) in ((0, 2) if kind == "wide" else (0,))
+        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (0 if kind == "general" else 2)
+        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 1, sizes[1]) in ((0,) if kind == "general" else (0, 2))
         ifgo = ifgo0.clone()
         out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
         cell = torch.empty_like(out)
@@ -540,8 +542,9 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
         for name, got, want in (("d_ifgo", d_ifgo, r["d_ifgo"]), ("dh0", dh, r["dh0"]), ("dc0", dc, r["dc0"])):
             assert rel_err(got, want) < HALF_TOL, (kind, name)
         results[kind] = (out, cell, ifgo, d_ifgo, dh, dc)
-    for a, b in zip(results["general"], results["wide"]):   # two summation orders of the same sums
-        assert rel_err(a, b) < HALF_TOL
+    for other in ("wide", "teams"):
+        for a, b in zip(results["general"], results[other]):   # other summation orders of the same sums
+            assert rel_err(a, b) < HALF_TOL
 
 
 XCD_CASES = [
