@@ -331,6 +331,15 @@ def main():
         "gemm_wgrad_frac_of_mfma_peak": round(gw / (t_k89 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
         "bwd_layer_ms": round(t_lb, 4),
     })
+    # yardstick for the three GEMM stages: the vendor library (torch.matmul = hipBLASLt / rocBLAS) on the same
+    # operands and shapes, timed the same way; not part of any measured step
+    if dname != "f32":
+        x2, d2, h2 = x.reshape(T * B, I), d_ifgo.reshape(T * B, 4 * H), out[:T].reshape(T * B, H)
+        bias = torch.zeros(4 * H, dtype=x.dtype, device=dev)
+        t_l1 = ev_time(lambda: torch.addmm(bias, x2, Wx.t()), reps=5)
+        t_l5 = ev_time(lambda: torch.mm(d2, Wx), reps=5)
+        t_l89 = ev_time(lambda: (torch.mm(d2.t(), x2), torch.mm(d2.t(), h2), d2.sum(0)), reps=5)
+        kernels["library_gemm_ms"] = {"ifgo": round(t_l1, 4), "dx": round(t_l5, 4), "wgrad": round(t_l89, 4)}
 
     # ---- roofline of the dominant kernel of the headline (forward) path ------------------
     # XCD-local path with idle CUs: ONE launch does projection + recurrence (fastlstm_fwd_layer);

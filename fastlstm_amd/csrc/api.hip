@@ -397,22 +397,31 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     DeviceInfo di;
     if (!(g_families.load() & 2) || device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32)
         return false;
-    if (dtype == FASTLSTM_FP32) return false;
-    if (H % 256 || H <= 1024 || H > 2048) return false;   // 1280, 1536, 1792, 2048
-    c->nkw = backward ? H / 64 : H / 256;
+    // a weight row of 2.5 ... 4 KiB in steps of 512 bytes: H = 1280, 1536, 1792, 2048 with 16-bit elements,
+    // 640, 768, 896, 1024 with fp32
+    const int es = elem_bytes(dtype), kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
+    if ((H * es) % 512 || H * es <= 2048 || H * es > 4096) return false;
+    c->nkw = (backward ? 4 * H : H) / kstep / 8;
     c->n_ht = H / 16;
     if (c->n_ht > kXcdGroupStride) return false;
     c->xpg = cdiv(c->n_ht, 32);   // XCDs per group (the last one partly used when H is not a multiple of 512)
     // groups of 16 or 32 rows where they all fit the launch: more groups = more CUs for a small batch, and a
     // CU then fetches a quarter or half of the operand bytes per step
     c->nt = cdiv(B, 16) * c->xpg <= kNumXcd ? 1 : cdiv(B, 32) * c->xpg <= kNumXcd ? 2 : 4;
+    // fp32 multiplies at 1/16 of the 16-bit rate: 16 units x 64 rows per CU are more MFMA time than a step of the
+    // general kernels, which spread 4 units x all rows over every CU
+    if (dtype == FASTLSTM_FP32 && c->nt == 4) return false;
     c->n_groups = cdiv(B, 16 * c->nt);
     if (c->n_groups * c->xpg > kNumXcd) return false;
-    c->ks = (backward ? 4 * H : H) / 32;
+    // ... and a small fp32 batch leaves most CUs without a share of the forward product (B = 32, H = 1024: 6.0
+    // instead of 5.7 us per step; the reverse step, with four times the operand bytes, gains at every size)
+    if (dtype == FASTLSTM_FP32 && !backward && c->n_groups * c->xpg < 6) return false;
+    c->ks = (backward ? 4 * H : H) / kstep;
     c->xslot = (size_t)c->n_groups * c->nt * c->ks * kFragBytes;
     if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
     const int gr = 16 * c->nt;
-    const int tiles = gr * (4 * 32 + 16) + 2 * gr * (32 + 16);   // gates + two state tiles of `gr` rows x 16 units
+    const int gseg = 16 * es;
+    const int tiles = gr * (4 * gseg + 16) + 2 * gr * (gseg + 16);   // gates + two state tiles of `gr` rows x 16 units
     c->lds = backward ? 8 * c->nt * kFragBytes + tiles + 8 * kWideRing * kFragBytes : 8 * 4 * c->nt * kFragBytes + tiles;
     c->v = 0;
     if (backward && c->nt == 4 && (g_families.load() & 4)) {
@@ -452,7 +461,7 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
     p.keep = o.keep;
-    auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : launch_fwd_wide_bf16;
+    auto launch = dtype == FASTLSTM_FP16 ? launch_fwd_wide_f16 : dtype == FASTLSTM_BF16 ? launch_fwd_wide_bf16 : launch_fwd_wide_f32;
     int occ = 0;
     if (launch(p, c.nkw, c.nt, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
@@ -476,7 +485,7 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     p.spin_limit = spin_limit_ticks();
     p.partials = p.xbuf + 2 * c.xslot;
     auto launch = c.v ? (dtype == FASTLSTM_FP16 ? launch_bwd_wide_split_f16 : launch_bwd_wide_split_bf16)
-                      : (dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : launch_bwd_wide_bf16);
+                      : (dtype == FASTLSTM_FP16 ? launch_bwd_wide_f16 : dtype == FASTLSTM_BF16 ? launch_bwd_wide_bf16 : launch_bwd_wide_f32);
     const int form = c.v ? c.v : c.nt;
     int occ = 0;
     if (launch(p, c.nkw, form, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;

@@ -26,8 +26,8 @@ constexpr int kWideRing = 12;   // LDS blocks (1 KiB) per wave for operand block
 // 13.3 us per step)
 template <typename T, int NKW, int NT>
 __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdParams p) {
-    static_assert(sizeof(T) == 2, "16-bit element types");
     using E = Elem<T>;
+    constexpr bool ACC = E::BYTES == 4;                // fp32: library exp and IEEE division in the gates
     constexpr int NWV = 8, NTHR = kWave * NWV;
     constexpr int HT = 16, BT = 16 * NT;
     constexpr int IPT = (HT * BT + NTHR - 1) / NTHR;   // (unit, batch row) items per thread
@@ -184,11 +184,11 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
             T st_d[4];
             if (valid[m]) {
                 T *gl_ = reinterpret_cast<T *>(tiles + goff[m]);   // the item's 4 gates in the LDS tile
-                const float si = sigmoidf_<false>(E::to_f32(gl_[0]));
-                const float sf = sigmoidf_<false>(E::to_f32(gl_[HT]));
-                const float tg = tanhf_<false>(E::to_f32(gl_[2 * HT]));
-                const float so = sigmoidf_<false>(E::to_f32(gl_[3 * HT]));
-                const float tc = tanhf_<false>(c1v[m]);
+                const float si = sigmoidf_<ACC>(E::to_f32(gl_[0]));
+                const float sf = sigmoidf_<ACC>(E::to_f32(gl_[HT]));
+                const float tg = tanhf_<ACC>(E::to_f32(gl_[2 * HT]));
+                const float so = sigmoidf_<ACC>(E::to_f32(gl_[3 * HT]));
+                const float tc = tanhf_<ACC>(c1v[m]);
                 const float c0 = E::to_f32(*reinterpret_cast<const T *>(tiles + BT * GROW + soff[m]));
                 const float dh = dh_rec[m] + E::to_f32(*reinterpret_cast<const T *>(tiles + BT * GROW + BT * SROW + soff[m]));
                 const float dc1 = dc_state[m] + dh * so * (1.f - tc * tc);
@@ -210,13 +210,18 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) st_d[gt] = E::from_f32(0.f);
             }
-            // exchange copy: 4 consecutive k = (unit, gate 0..3); lanes l and l+16 own units u and u+1 of
-            // the same batch row, the even-unit lane writes both (16 bytes, write-through)
-            const u32x2 mine = *reinterpret_cast<u32x2 *>(st_d);
-            u32x2 other;
-            other[0] = (unsigned)__shfl_down((int)mine[0], 16);
-            other[1] = (unsigned)__shfl_down((int)mine[1], 16);
-            if (pair_lead[m]) xch.store16(xgrp + xoff[m], u32x4{mine[0], mine[1], other[0], other[1]});
+            // exchange copy: 4 consecutive k = (unit, gate 0..3), 16 bytes per unit with fp32; with 16-bit
+            // elements lanes l and l+16 own units u and u+1 of the same batch row and the even-unit lane
+            // writes both (16 bytes, write-through)
+            if constexpr (E::BYTES == 4) {
+                if (valid[m]) xch.store16(xgrp + xoff[m], *reinterpret_cast<u32x4 *>(st_d));
+            } else {
+                const u32x2 mine = *reinterpret_cast<u32x2 *>(st_d);
+                u32x2 other;
+                other[0] = (unsigned)__shfl_down((int)mine[0], 16);
+                other[1] = (unsigned)__shfl_down((int)mine[1], 16);
+                if (pair_lead[m]) xch.store16(xgrp + xoff[m], u32x4{mine[0], mine[1], other[0], other[1]});
+            }
         }
         publish_version(grp_flags + j, s + 1);   // waits for the stores, workgroup barrier, raises the flag
         tile_to_global(t);

@@ -33,8 +33,8 @@ namespace fastlstm {
 // 3.3 instead of 5.8 us per step).
 template <typename T, int NKW, int NT>
 __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdParams p) {
-    static_assert(sizeof(T) == 2, "16-bit element types");
     using E = Elem<T>;
+    constexpr bool ACC = E::BYTES == 4;                      // fp32: library exp and IEEE division in the gates
     constexpr int NWV = 8, NTHR = kWave * NWV;
     constexpr int MT = 4, TILES = MT * NT;                   // unit tiles, batch tiles of 16 rows
     constexpr int IPT = (TILES + NWV - 1) / NWV;             // (tile, lane) items per thread
@@ -237,8 +237,8 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
                 const float pf = E::to_f32(gl_[HT]) + s[1];
                 const float pg = E::to_f32(gl_[2 * HT]) + s[2];
                 const float po = E::to_f32(gl_[3 * HT]) + s[3];
-                const float c1 = sigmoidf_<false>(pf) * c_state[m] + sigmoidf_<false>(pi) * tanhf_<false>(pg);
-                const float h1 = sigmoidf_<false>(po) * tanhf_<false>(c1);
+                const float c1 = sigmoidf_<ACC>(pf) * c_state[m] + sigmoidf_<ACC>(pi) * tanhf_<ACC>(pg);
+                const float h1 = sigmoidf_<ACC>(po) * tanhf_<ACC>(c1);
                 c_state[m] = c1;
                 const T hv = E::from_f32(h1);
                 gl_[0] = E::from_f32(pi);

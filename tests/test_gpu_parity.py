@@ -489,18 +489,23 @@ WIDE_CASES = [
     # ... and as groups of 32 rows
     (3, 64, 2048, torch.float16),
     (4, 50, 1536, torch.bfloat16),    # ragged second group
+    # fp32 at H = 640 ... 1024 (the same bytes per weight row): groups of 16 or 32 rows on two XCDs
+    (4, 64, 1024, torch.float32),     # four 16-row groups
+    (3, 100, 768, torch.float32),     # 32-row groups, the last one ragged
+    (3, 20, 640, torch.float32),      # the second XCD of a group partly used
 ]
 
 
 @pytest.mark.parametrize("T,B,H,dt", WIDE_CASES)
 def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt):
-    """H = 1536 / 2048: the C ABI runs the register-resident kernels whose groups span several XCDs
+    """H = 1280 ... 2048 (fp32: 640 ... 1024): the C ABI runs the register-resident kernels whose groups span several XCDs
     (kernel kind 2), or -- with that family switched off -- the general kernels; both must meet the
     oracle on the same inputs.  So must both forms of the reverse kernel for groups of 64 rows: every
     workgroup sums over all of K, or teams of workgroups split K and exchange partial sums."""
     lib = _lib.load()
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
     rm = RM[dt]
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
     p = make_problem(T, B, 64, H, seed=5 + H + B)
     pr = {k: (v.to(dt).double() if v is not None else None) for k, v in p.items()}
     g = {k: dev(v, dt) for k, v in p.items()}
@@ -516,7 +521,8 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
     for kind in ("general", "wide", "teams"):
         lib.fastlstm_set_kernel_families({"general": 0, "wide": 3, "teams": 7}[kind])
         sizes = [lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
-        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (0 if kind == "general" else 2)
+        small32 = dt == torch.float32 and B <= 32   # (a small fp32 batch keeps the general forward kernel)
+        assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, sizes[0]) == (0 if kind == "general" or small32 else 2)
         assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 1, sizes[1]) in ((0,) if kind == "general" else (0, 2))
         ifgo = ifgo0.clone()
         out = torch.empty(T + 1, B, H, device="cuda", dtype=dt)
@@ -528,7 +534,7 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
         torch.cuda.synchronize()
         assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
         for name, got, want in (("out", out, o_out), ("cell", cell, o_cell), ("ifgo", ifgo, o_ifgo)):
-            assert rel_err(got, want) < HALF_TOL, (kind, name)
+            assert rel_err(got, want) < tol, (kind, name)
         d_ifgo = torch.empty_like(ifgo)
         dh, dc = g["dh_n"].clone(), g["dc_n"].clone()
         wsb = torch.zeros(sizes[1], dtype=torch.uint8, device="cuda")
@@ -540,11 +546,11 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
         dout, dh_n, dc_n, x, Wx, Wh = to_np(pr, ["dout", "dh_n", "dc_n", "x", "Wx", "Wh"])
         r = oracle.backward(dout, dh_n, dc_n, x, npy(out), npy(cell), npy(ifgo), Wx, Wh, round_mode=rm)
         for name, got, want in (("d_ifgo", d_ifgo, r["d_ifgo"]), ("dh0", dh, r["dh0"]), ("dc0", dc, r["dc0"])):
-            assert rel_err(got, want) < HALF_TOL, (kind, name)
+            assert rel_err(got, want) < tol, (kind, name)
         results[kind] = (out, cell, ifgo, d_ifgo, dh, dc)
     for other in ("wide", "teams"):
         for a, b in zip(results["general"], results[other]):   # other summation orders of the same sums
-            assert rel_err(a, b) < HALF_TOL
+            assert rel_err(a, b) < tol
 
 
 XCD_CASES = [
