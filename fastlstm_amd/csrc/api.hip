@@ -435,11 +435,12 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     return true;
 }
 
-// Rows per launch (see xcd_rows_per_launch) for the register-resident kernels of H > 1024: full launches of 64-row groups on all XCDs.
+// Rows per launch (see xcd_rows_per_launch) for the register-resident kernels: full launches of 64-row groups
+// (fp32: 32-row groups) on all XCDs.
 static int wide_rows_per_launch(int T, int B, int H, int dtype, bool backward, size_t ws_bytes) {
     const int xpg = cdiv(H / 16, 32);
-    const int rows = 64 * (kNumXcd / std::max(1, xpg));
-    if (H <= 1024 || rows >= B || rows <= 0) return 0;
+    const int rows = (dtype == FASTLSTM_FP32 ? 32 : 64) * (kNumXcd / std::max(1, xpg));
+    if (rows >= B || rows <= 0) return 0;
     WideCfg c;
     if (!select_wide(T, B, H, dtype, backward, ws_bytes, &c, rows)) return 0;
     if (B % rows && !select_wide(T, B, H, dtype, backward, ws_bytes, &c, B % rows)) return 0;

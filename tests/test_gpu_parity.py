@@ -109,6 +109,7 @@ STAGE_CASES = [
     (4, 200, 64, 1024, torch.bfloat16),   # forward in two row ranges (128 + 72), reverse in one launch of 32-row tiles
     (3, 200, 64, 2048, torch.float16),    # register-resident kernels over two row ranges (128 + 72)
     (3, 40, 64, 512, torch.float32),
+    (3, 200, 64, 1024, torch.float32),    # register-resident fp32 kernels over two row ranges (128 + 72)
     (2, 2100, 16, 96, torch.float16),     # 3 members per group: 10 groups would fit an XCD's CUs, the workspace has
                                           # barrier counters for 8 per XCD -- 66 tiles of 32 rows must not run as one launch
 ]
