@@ -90,6 +90,30 @@ __device__ __forceinline__ void load_block_to_lds_device(__amdgpu_buffer_rsrc_t 
 #endif
 }
 
+// 16 bytes per lane, global -> LDS at lds_addr + 16 * lane, with or without device scope; voff = the lane's byte offset,
+// soff = the block's byte offset (scalar).  Inline assembly, so that the compiler does not know of the load: it waits for every load it knows of before a workgroup barrier and for every LDS-direct load before an LDS access; the wave that uses this counts its own loads (s_waitcnt vmcnt(n)).  The s_nop: a scalar
+// operand may have been written by a vector instruction just before (v_readlane of a spilled scalar), and a
+// vector memory instruction may read such a register only 5 wait states later, which the compiler sees to for
+// its own instructions but not inside inline assembly (m0 needs 1 before the load).
+template <bool DEVICE_SCOPE>
+__device__ __forceinline__ void dma_block_asm(u32x4 rsrc, unsigned lds_addr, unsigned voff, unsigned soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // (m0 cannot be named as clobbered: a kernel that uses this sends every LDS-direct load through here, so that nothing else relies on m0)
+    if constexpr (DEVICE_SCOPE)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                     : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                     : "memory");
+#else
+    (void)rsrc; (void)lds_addr; (void)voff; (void)soff;
+#endif
+}
+
 // acc += a . b with the accumulator pinned to the accumulation registers (AGPRs).  With more
 // than 128 accumulators per lane the register allocator otherwise shuttles them between the two
 // halves of the register file around every MFMA.

@@ -27,30 +27,6 @@ namespace fastlstm {
 
 constexpr int kSplitRing = 8;   // LDS blocks (1 KiB) per wave for operand blocks in flight
 
-// 16 bytes per lane, global -> LDS at lds_addr + 16 * lane, with or without device scope; voff = the lane's byte offset,
-// soff = the block's byte offset (scalar).  See the note on inline assembly at the top.  The s_nop: a scalar
-// operand may have been written by a vector instruction just before (v_readlane of a spilled scalar), and a
-// vector memory instruction may read such a register only 5 wait states later, which the compiler sees to for
-// its own instructions but not inside inline assembly (m0 needs 1 before the load).
-template <bool DEVICE_SCOPE>
-__device__ __forceinline__ void dma_block_asm(u32x4 rsrc, unsigned lds_addr, unsigned voff, unsigned soff) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    // (m0 cannot be named as clobbered; nothing else in the kernel uses it: every LDS-direct load goes through here)
-    if constexpr (DEVICE_SCOPE)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
-                     :
-                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
-                     : "memory");
-    else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                     :
-                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
-                     : "memory");
-#else
-    (void)rsrc; (void)lds_addr; (void)voff; (void)soff;
-#endif
-}
-
 // number of k-steps per wave over the whole of K: NKW = 4H / KSTEP / 8 (20, 24, 28, 32 for H = 1280 ... 2048);
 // V members per team (divides NKW and 8; the 4 V accumulator tiles must fit the registers: V <= 4)
 template <typename T, int NKW, int V>
