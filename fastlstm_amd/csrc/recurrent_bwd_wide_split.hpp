@@ -304,7 +304,8 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_split_kernel(const Bw
             for (int w = 1; w < NWV; ++w) sum += red[(w * TILES + tl) * kWave + lane];
             // ... and go to their owner (this workgroup: through LDS)
             if (rv == mem) own[nt * kWave + lane] = sum;
-            else part.store16(part_to + (unsigned)nt * kFragBytes + lane_off, __builtin_bit_cast(u32x4, sum));
+            // (an ordinary store: the team shares one XCD, whose L2 the receivers' device-scope loads read)
+            else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), part.rsrc, part_to + (unsigned)nt * kFragBytes + lane_off, 0, 0);
         }
 
         // ---- the team's exchange: every member gets the others' sums for its 16 units ----
