@@ -36,7 +36,7 @@ def _gpu_setup():
 @pytest.fixture(autouse=True)
 def _all_kernel_families():
     yield
-    _lib.load().fastlstm_set_kernel_families(3)   # whatever a test switched off is back on for the next one
+    _lib.load().fastlstm_set_kernel_families(7)   # whatever a test switched off is back on for the next one
 
 
 def npy(t):
@@ -554,6 +554,53 @@ def test_wide_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H, dt)
             assert rel_err(a, b) < tol
 
 
+@pytest.mark.parametrize("H,dt", [(2048, torch.bfloat16), (1280, torch.float16), (1024, torch.float32), (640, torch.float32)])
+def test_register_resident_kernels_at_the_batch_sizes_where_their_form_changes(H, dt):
+    """Rows per group (16, 32, 64), launches over row ranges, the team form of the reverse kernel and the fp32
+    limits all switch on the batch size: around every threshold the C ABI's choice must agree with the general
+    kernels on the same inputs (outputs, states, stored activations, d_ifgo and the state gradients)."""
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    tol = 2 * FP32_TOL if dt == torch.float32 else HALF_TOL
+    st = torch.cuda.current_stream().cuda_stream
+    T = 3
+
+    def run(B, families):
+        lib.fastlstm_set_kernel_families(families)
+        gen = torch.Generator(device="cuda").manual_seed(B * 7 + H)
+        rnd = lambda *shape, s=1.0: (torch.randn(*shape, device="cuda", generator=gen) * s).to(dt)
+        ifgo, Wh = rnd(T, B, 4 * H, s=0.5), rnd(4 * H, H, s=H ** -0.5)
+        out = torch.zeros(T + 1, B, H, device="cuda", dtype=dt)
+        cell = torch.zeros_like(out)
+        out[0], cell[0] = rnd(B, H, s=0.1), rnd(B, H, s=0.1)
+        plans = [_lib.Plan(), _lib.Plan()]
+        ws = []
+        for bw in (0, 1):
+            _lib.check(lib.fastlstm_plan_device(0, B, H, code, bw, plans[bw]), "plan")
+            ws.append(torch.zeros(lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw), dtype=torch.uint8, device="cuda"))
+        kinds = tuple(lib.fastlstm_recurrent_kernel_kind(T, B, H, code, bw, ws[bw].numel()) for bw in (0, 1))
+        _lib.check(lib.fastlstm_fwd_persistent(ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), Wh.data_ptr(),
+                                               ws[0].data_ptr(), ws[0].numel(), T, B, H, code, st), "fwd")
+        dout, d_ifgo = rnd(T, B, H), torch.empty_like(ifgo)
+        dh, dc = rnd(B, H, s=0.1), rnd(B, H, s=0.1)
+        _lib.check(lib.fastlstm_bwd_persistent(dout.data_ptr(), dh.data_ptr(), dc.data_ptr(), ifgo.data_ptr(), cell.data_ptr(),
+                                               d_ifgo.data_ptr(), Wh.data_ptr(), ws[1].data_ptr(), ws[1].numel(), T, B, H, code, st), "bwd")
+        torch.cuda.synchronize()
+        for w in ws:
+            assert lib.fastlstm_ws_status(w[:64].cpu().numpy().tobytes()) == _lib.OK
+        return kinds, (out, cell, ifgo, d_ifgo, dh, dc)
+
+    seen = set()
+    for B in (1, 16, 17, 32, 33, 64, 65, 128, 129, 144, 260):
+        kinds0, want = run(B, 0)
+        kinds, got = run(B, 7)
+        assert kinds0 == (0, 0) and kinds[1] == 2, (B, kinds0, kinds)
+        seen.add(kinds)
+        for name, a, b in zip(("out", "cell", "ifgo", "d_ifgo", "dh0", "dc0"), got, want):
+            assert rel_err(a, npy(b)) < tol, (B, name)
+    assert (2, 2) in seen
+
+
 XCD_CASES = [
     # T, B, H, dtype          (hidden tile, members, batch tiles) of the XCD-local launch
     (20, 64, 1024, torch.float16),    # config B: 32 units x 32 members, 8 waves
@@ -585,7 +632,7 @@ def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H
                                       ifgo0.data_ptr(), T, B, H, H, code, st), "k1")
     results = {}
     for kind in ("general", "xcd"):
-        lib.fastlstm_set_kernel_families(0 if kind == "general" else 3)
+        lib.fastlstm_set_kernel_families(0 if kind == "general" else 7)
         sizes = [lib.fastlstm_recurrent_workspace_bytes(plans[bw], T, H, code, bw) for bw in (0, 1)]
         for bw in (0, 1):
             assert lib.fastlstm_recurrent_kernel_kind(T, B, H, code, bw, sizes[bw]) == (1 if kind == "xcd" else 0)
