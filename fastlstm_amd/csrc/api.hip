@@ -1261,6 +1261,17 @@ size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int
     return one > head ? head + 2 * (one - head) : one;
 }
 
+size_t fastlstm_stack2_bwd_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
+    const size_t need = std::max(fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype), fastlstm_wgrad_workspace_bytes(T, B, H, H, dtype));
+    if (need == 0 || dtype == FASTLSTM_FP32) return need;
+    // one parked 256 x 256 fp32 tile per helper and layer (see plan_bwd_helpers): with that much the one launch
+    // also computes the lower layer's weight gradients
+    const size_t tile_bytes = (size_t)256 * 256 * sizeof(float);
+    const int rows = cdiv(4 * H, 256), helpers = kNumXcd * 32;
+    const size_t upper = std::min(rows * 2 * cdiv(H, 256), helpers), lower = std::min(rows * (cdiv(I, 256) + cdiv(H, 256)), helpers);
+    return std::max(need, (upper + lower) * tile_bytes);
+}
+
 int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes) {
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;

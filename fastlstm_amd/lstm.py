@@ -309,8 +309,8 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         n = lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)
         ws = torch.empty(n, dtype=torch.uint8, device=x.device)
         ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
-        wws = torch.empty(max(lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code),
-                              lib.fastlstm_wgrad_workspace_bytes(T, B, H, H, code)), dtype=torch.uint8, device=x.device)
+        # (large enough for the one launch to take the lower layer's weight gradients too)
+        wws = torch.empty(lib.fastlstm_stack2_bwd_wgrad_workspace_bytes(T, B, I, H, code), dtype=torch.uint8, device=x.device)
         p = lambda t: t.data_ptr()
         _lib.check(lib.fastlstm_bwd_stack2(
             p(dh), p(dh1), p(dc1), p(ifgo1), p(cell1), p(d_ifgo1), p(Wh1), p(Wx1), p(out1), p(dWx1), p(dWh1), p(db1), p(dx1),

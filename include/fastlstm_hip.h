@@ -210,10 +210,12 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
  * layer (written, then read).  Where both XCD-local reverse recurrences fit the device side by side
  * and leave CUs without a role (fastlstm_bwd_stack2_fused returns 1), ONE launch runs both: the idle
  * workgroups compute dx1 chunk by chunk behind the upper recurrence, the lower recurrence follows
- * dx1 a few chunks behind, and the same workgroups accumulate dWx1, dWh1 and compute dx0; db1 and the
- * lower layer's weight gradients follow as separate launches.  ws:
- * fastlstm_stack2_bwd_workspace_bytes, zeroed like any recurrent workspace; wgrad_ws: the larger of
- * the two layers' fastlstm_wgrad_workspace_bytes.  Replaces two backward nodes of the layer loop at
+ * dx1 a few chunks behind, and the same workgroups accumulate dWx1, dWh1 and compute dx0; the bias
+ * gradients follow as separate launches, and so do the lower layer's weight gradients unless wgrad_ws is
+ * large enough to park their tiles between chunks.  ws: fastlstm_stack2_bwd_workspace_bytes, zeroed like
+ * any recurrent workspace; wgrad_ws: at least the larger of the two layers'
+ * fastlstm_wgrad_workspace_bytes; with fastlstm_stack2_bwd_wgrad_workspace_bytes (64 MiB at H = I = 1024)
+ * the launch takes the lower layer's dWx0, dWh0 too.  Replaces two backward nodes of the layer loop at
  * fastlstm/lstm.py:685-696 (each lstm.py:236-334 + 494-501). */
 int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1,
                         void *d_ifgo1, const void *Wh1, const void *Wx1, const void *out1, void *dWx1,
@@ -223,6 +225,7 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
                         size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
                         int dtype, void *stream);
 size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype);
+size_t fastlstm_stack2_bwd_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
 int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes);
 
 /* Which kernel fastlstm_fwd_persistent (backward = 0) / fastlstm_bwd_persistent (1) will launch on
