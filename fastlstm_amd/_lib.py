@@ -41,6 +41,9 @@ SIGNATURES = {
     "fastlstm_bwd_stack2": (_i, [_vp] * 27 + [_sz, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_stack2_bwd_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i]),
     "fastlstm_bwd_stack2_fused": (_i, [_i, _i, _i, _i, _i, _sz]),
+    "fastlstm_fwd_persistent_pair": (_i, [_vp] * 9 + [_sz, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_bwd_persistent_pair": (_i, [_vp] * 15 + [_sz, _i, _i, _i, _i, _vp]),
+    "fastlstm_pair_fused": (_i, [_i, _i, _i, _i, _i, _sz]),
     "fastlstm_stack2_bwd_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "fastlstm_gemm_ifgo": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),

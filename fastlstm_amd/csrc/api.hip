@@ -308,6 +308,11 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.keep = o.keep;
     p.trace = g_rec_trace;
     p.n_layers = 1;
+    if (second && !x) {   // two independent recurrences of this shape side by side (the second's projection is done)
+        if (2 * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
+        p.n_layers = 2;
+        p.ifgo2 = second->ifgo; p.out2 = second->out; p.cell2 = second->cell; p.Wh2 = second->Wh;
+    }
     if (x) {
         if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p, second)) return 2;
         const int lds = std::max(c.lds, Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES);
@@ -324,6 +329,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     int occ = 0;
     if (launch(p, c.mt, c.nkw, c.ntw, c.nwv, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
+    if (dry_run) return FASTLSTM_OK;
     // one workgroup per CU of the device; those without a role return at once
     if (launch(p, c.mt, c.nkw, c.ntw, c.nwv, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
@@ -518,6 +524,7 @@ struct LowerLayer {
     size_t scratch_bytes;
     const void *x, *h;      // the lower layer's input and its out (for its weight gradients; may be null)
     void *dWx, *dWh;
+    const void *dout = nullptr;   // two independent recurrences side by side (no extras): the second one's dout
 };
 
 bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, int T, int B, int H, int dtype,
@@ -624,6 +631,13 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
     p.n_layers = 1;
+    if (lower && !extras) {   // two independent recurrences of this shape side by side
+        if (2 * c.n_groups > kNumXcd * c.gpx) return 2;
+        p.n_layers = 2;
+        p.dh_lo = lower->dh; p.dc_lo = lower->dc; p.ifgo_lo = lower->ifgo; p.cell_lo = lower->cell;
+        p.d_ifgo_lo = lower->d_ifgo; p.Wh_lo = lower->Wh;
+        p.k5.C = const_cast<void *>(lower->dout);   // the kernel reads the second recurrence's dout from there
+    }
     if (extras) {
         bool wgrad_fused = false;
         if (!plan_bwd_helpers(c, d_ifgo, *extras, T, B, H, dtype, &p, &wgrad_fused, lower, lower_wgrad_fused)) return 2;
@@ -641,6 +655,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     int occ = 0;
     if (launch(p, c.mt, c.nkw, c.ntw, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
+    if (dry_run) return FASTLSTM_OK;
     if (launch(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
@@ -1033,6 +1048,97 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
     if (int rc = take_pending_status()) return rc;
     return finish_recurrent(bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream),
                             ws, stream);
+}
+
+// Two recurrences of one shape: side by side in one launch of the XCD-local kernels where both fit (returns 0), else
+// 1 (not launched).
+static int try_pair(bool backward, void *const a[7], void *const b[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                    void *stream, int keep, bool dry_run) {
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, backward ? 1 : 0, &pl, false)) return rc;
+    if (pl.wave_split == 2 || pl.wave_split == 3) return 1;
+    unsigned char *wsb = static_cast<unsigned char *>(ws);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc;
+    if (!backward) {
+        const SecondLayer second{nullptr, nullptr, nullptr, b[3], b[0], b[1], b[2]};
+        const LaunchOpts o{keep, 0, 0};
+        rc = try_fwd_xcd(a[0], a[1], a[2], a[3], wsb, ws_bytes, T, B, H, dtype, s, nullptr, nullptr, nullptr, nullptr, 0, &second,
+                         dry_run, o);
+    } else {
+        LowerLayer lower{b[1], b[2], b[3], b[4], b[5], b[6], nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr};
+        lower.dout = b[0];
+        rc = try_bwd_xcd(a[0], a[1], a[2], a[3], a[4], a[5], a[6], wsb, ws_bytes, T, B, H, dtype, s, nullptr, &lower, dry_run);
+    }
+    return rc == 2 ? 1 : rc;
+}
+
+int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    void *fake[7];
+    for (void *&q : fake) q = reinterpret_cast<void *>(static_cast<size_t>(4096));   // never dereferenced
+    const int rc = try_pair(backward != 0, fake, fake, fake[0], ws_bytes, T, B, H, dtype, nullptr, 1, true);
+    return rc == FASTLSTM_OK ? 1 : (rc < 0 ? rc : 0);
+}
+
+int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const void *Wh_a, void *ifgo_b, void *out_b,
+                                 void *cell_b, const void *Wh_b, void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                                 int keep_activations, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    if (!ifgo_a || !out_a || !cell_a || !Wh_a || !ifgo_b || !out_b || !cell_b || !Wh_b || !ws) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    void *const a[7] = {ifgo_a, out_a, cell_a, const_cast<void *>(Wh_a)}, *const b[7] = {ifgo_b, out_b, cell_b, const_cast<void *>(Wh_b)};
+    for (int i = 0; i < 4; ++i)
+        if (!aligned16(a[i]) || !aligned16(b[i])) return FASTLSTM_ERR_ALIGN;
+    if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
+    const int keep = keep_activations ? 1 : 0;
+    int rc = try_pair(false, a, b, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
+    if (rc == 1) {   // one after the other; the workspace is cleared in between
+        rc = fwd_persistent_impl(ifgo_a, out_a, cell_a, Wh_a, ws, ws_bytes, T, B, H, dtype, stream, keep);
+        if (rc == FASTLSTM_OK) {
+            fastlstm_plan pl;
+            if (int r2 = plan_device(-1, B, H, dtype, 0, &pl, false)) return r2;
+            const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
+            zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned *>(ws), zero / 4);
+            if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+            rc = fwd_persistent_impl(ifgo_b, out_b, cell_b, Wh_b, ws, ws_bytes, T, B, H, dtype, stream, keep);
+        }
+    }
+    return finish_recurrent(rc, ws, stream);
+}
+
+int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, const void *ifgo_a, const void *cell_a,
+                                 void *d_ifgo_a, const void *Wh_a, const void *dout_b, void *dh_b, void *dc_b,
+                                 const void *ifgo_b, const void *cell_b, void *d_ifgo_b, const void *Wh_b, void *ws,
+                                 size_t ws_bytes, int T, int B, int H, int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    void *const a[7] = {const_cast<void *>(dout_a), dh_a, dc_a, const_cast<void *>(ifgo_a), const_cast<void *>(cell_a), d_ifgo_a,
+                        const_cast<void *>(Wh_a)};
+    void *const b[7] = {const_cast<void *>(dout_b), dh_b, dc_b, const_cast<void *>(ifgo_b), const_cast<void *>(cell_b), d_ifgo_b,
+                        const_cast<void *>(Wh_b)};
+    for (int i = 0; i < 7; ++i) {
+        if (!a[i] || !b[i]) return FASTLSTM_ERR_NULL;
+        if (!aligned16(a[i]) || !aligned16(b[i])) return FASTLSTM_ERR_ALIGN;
+    }
+    if (!ws) return FASTLSTM_ERR_NULL;
+    if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    int rc = try_pair(true, a, b, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
+    if (rc == 1) {
+        rc = bwd_persistent_impl(dout_a, dh_a, dc_a, ifgo_a, cell_a, d_ifgo_a, Wh_a, ws, ws_bytes, T, B, H, dtype, stream);
+        if (rc == FASTLSTM_OK) {
+            fastlstm_plan pl;
+            if (int r2 = plan_device(-1, B, H, dtype, 1, &pl, false)) return r2;
+            const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
+            zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned *>(ws), zero / 4);
+            if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+            rc = bwd_persistent_impl(dout_b, dh_b, dc_b, ifgo_b, cell_b, d_ifgo_b, Wh_b, ws, ws_bytes, T, B, H, dtype, stream);
+        }
+    }
+    return finish_recurrent(rc, ws, stream);
 }
 
 static int fwd_layer_impl(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,

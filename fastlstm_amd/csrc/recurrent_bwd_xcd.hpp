@@ -56,7 +56,8 @@ struct BwdXcdParams {
     // the lower layer's weight gradients (k8_lo, k9_lo: the same scheme as k8, k9, one tile per helper
     // accumulated chunk by chunk as the lower recurrence finishes them); otherwise those are left to
     // the caller.
-    int n_layers;
+    int n_layers;       // (also 2, without helpers: two independent recurrences side by side, the second one described
+                        // by the *_lo fields and k5.C = its dout)
     void *dh_lo, *dc_lo;
     const void *ifgo_lo, *cell_lo;
     void *d_ifgo_lo;
@@ -297,7 +298,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
     const int vg = gl * kNumXcd + xcd;          // group index over the layers of the launch
-    constexpr int n_layers = HELP == 2 ? 2 : 1;
+    // two recurrences in the launch: a stack (HELP == 2), or two independent ones of the same shape side by side
+    // (HELP == 0 with n_layers == 2: the two directions of a bidirectional layer; `lower` is then simply the second)
+    const int n_layers = HELP == 2 ? 2 : (HELP == 0 && p.n_layers > 1 ? 2 : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP != 0) {
             if (p.k5_tiles_n > 0) bwd_helper<T, HELP == 2>(p, smem);
@@ -305,7 +308,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         return;
     }
     check_xcd_placement(p.hdr);
-    const bool lower = HELP == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
+    const bool lower = n_layers == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
+    const bool follows = HELP == 2 && lower;                // ... whose dout the helpers produce during the launch
     const int g = lower ? vg - p.n_groups : vg;
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k5_live = HELP && p.k5_tiles_n > 0;
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
                 else __builtin_amdgcn_raw_buffer_store_b128(v, rg, g_off[i], 0, 0);
             }
     };
-    if (lower) {   // the latest chunk(s) of this layer's dout have to be there
+    if (follows) {   // the latest chunk(s) of this layer's dout have to be there
         if (wave == 0) {
             wait_dout(T_ - 1);
             if (DIST > 1 && T_ > 1) wait_dout(T_ - 2);
@@ -516,7 +520,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         const XchgL2 xch(p.xbuf + (size_t)(s & 1) * xslot, (unsigned)xslot);
         // the dout of timestep t - DIST is requested behind this step's publish barrier: when it is the
         // latest timestep of a chunk, that chunk of the upper layer's dx must be complete
-        if (lower && wave == 0 && t >= DIST && (t - DIST) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - DIST);
+        if (follows && wave == 0 && t >= DIST && (t - DIST) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - DIST);
 
         // ---- point-wise gate backward for this thread's items --------------------------
 #pragma unroll

@@ -257,7 +257,9 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int gl = slot / p.n_ht, j = slot % p.n_ht;
     const int vg = gl * kNumXcd + xcd;          // group index over all layers of the launch
-    const int n_layers = HELP ? p.n_layers : 1;
+    // (without helpers n_layers == 2 means two independent recurrences of the same shape side by side: the two
+    // directions of a bidirectional layer; nothing links them)
+    const int n_layers = p.n_layers > 1 ? 2 : 1;
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
             if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);

@@ -320,6 +320,105 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
     return (dx0, dh0, dc0, dWx0, db0, dWh0, db0), (dx1, dh1, dc1, dWx1, db1, dWh1, db1)
 
 
+def pair_runs_in_one_launch(T, B, H, dtype, device, backward=False):
+    """True if two independent recurrences of this shape (the two directions of a bidirectional layer) run as
+    one launch (fastlstm_pair_fused)."""
+    if dtype not in _DTYPE_CODE or torch.device(device).type != "cuda":
+        return False
+    lib = _lib.load()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(device):
+        plan = _plan(torch.device(device), B, H, code, backward)
+        n = (lib.fastlstm_stack2_bwd_workspace_bytes if backward else lib.fastlstm_stack2_workspace_bytes)(plan, T, H, code)
+        return lib.fastlstm_pair_fused(T, B, H, code, int(backward), n) == 1
+
+
+def lstm_persistent_fwd_pair(xa, h0a, c0a, Wxa, bxa, Wha, bha, xb, h0b, c0b, Wxb, bxb, Whb, bhb, keep_activations=True):
+    """Two independent layers of one shape on their own inputs xa, xb [T,B,I] -- the two directions of a
+    bidirectional layer, xb being the time-reversed sequence: returns (out_a, cell_a, ifgo_a, out_b, cell_b,
+    ifgo_b) with the layouts and the results of two calls of lstm_persistent_fwd.  The two input projections are
+    two GEMM launches; the two time loops are one launch where the library can run them side by side."""
+    _require_gpu(xa, xb, Wxa, bxa, Wha, bha, Wxb, bxb, Whb, bhb, h0a, c0a, h0b, c0b)
+    code = _code(xa)
+    T, B, I = xa.shape
+    H = Wha.shape[1]
+    assert xb.shape == xa.shape and xb.dtype == xa.dtype and xa.is_contiguous() and xb.is_contiguous()
+    assert Wha.is_contiguous() and Whb.is_contiguous()
+    assert Wxa.shape == (4 * H, I) and Wxb.shape == (4 * H, I) and Wha.shape == (4 * H, H) and Whb.shape == (4 * H, H)
+    for w in (Wxa, bxa, Wha, bha, Wxb, bxb, Whb, bhb):
+        if w.dtype != xa.dtype:
+            raise TypeError("weights must have the dtype of x (%s), got %s" % (xa.dtype, w.dtype))
+    lib = _lib.load()
+    with torch.cuda.device(xa.device):
+        stream = _stream()
+        bufs = []
+        for x, h0, c0, Wx, bx, bh in ((xa, h0a, c0a, Wxa, bxa, bha), (xb, h0b, c0b, Wxb, bxb, bhb)):
+            x, Wx, bx, bh = _aligned(x), Wx.contiguous(), bx.contiguous(), bh.contiguous()
+            ifgo = torch.empty((T, B, 4 * H), device=x.device, dtype=x.dtype)
+            out = torch.empty((T + 1, B, H), device=x.device, dtype=x.dtype)
+            cell = torch.empty_like(out)
+            if h0 is not None:
+                out[0] = h0
+                cell[0] = c0
+            else:
+                out[0].zero_()
+                cell[0].zero_()
+            _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), ifgo.data_ptr(),
+                                              T, B, I, H, code, stream), "fastlstm_gemm_ifgo")
+            bufs.append((out, cell, ifgo))
+        (out_a, cell_a, ifgo_a), (out_b, cell_b, ifgo_b) = bufs
+        plan = _plan(xa.device, B, H, code, False)
+        ws = _stack2_workspace(plan, T, H, code, xa.device)
+        p = lambda t: t.data_ptr()
+        _lib.check(lib.fastlstm_fwd_persistent_pair(p(ifgo_a), p(out_a), p(cell_a), p(Wha), p(ifgo_b), p(out_b), p(cell_b), p(Whb),
+                                                    p(ws), ws.numel(), T, B, H, code, int(keep_activations), stream),
+                   "fastlstm_fwd_persistent_pair")
+        _check_ws(ws, "fastlstm_fwd_persistent_pair")
+    return out_a, cell_a, ifgo_a, out_b, cell_b, ifgo_b
+
+
+def lstm_persistent_bwd_pair(dh_a, d_state_a, xa, out_a, cell_a, ifgo_a, Wxa, Wha,
+                             dh_b, d_state_b, xb, out_b, cell_b, ifgo_b, Wxb, Whb):
+    """Reverse pass of lstm_persistent_fwd_pair: dh_* [T,B,H] are the gradients of out_*[1:], d_state_* optional
+    (dh_n, dc_n) pairs (zero when None).  The two reverse time loops are one launch where the library can run
+    them side by side; dx and the weight gradients follow per layer.  The same results as two calls of
+    lstm_persistent_bwd.  Returns two tuples (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)."""
+    _require_gpu(dh_a, dh_b, xa, xb, out_a, cell_a, ifgo_a, Wxa, Wha, out_b, cell_b, ifgo_b, Wxb, Whb)
+    code = _code(ifgo_a)
+    T, B, H = dh_a.shape
+    I = Wxa.shape[1]
+    lib = _lib.load()
+    with torch.cuda.device(xa.device):
+        stream = _stream()
+        p = lambda t: t.data_ptr()
+        sides = []
+        for dh, d_state, ifgo in ((dh_a, d_state_a, ifgo_a), (dh_b, d_state_b, ifgo_b)):
+            dh = dh.contiguous()
+            if dh.dtype != ifgo.dtype:
+                dh = dh.to(ifgo.dtype)
+            state = lambda k: (torch.zeros((B, H), device=ifgo.device, dtype=ifgo.dtype) if d_state is None
+                               else d_state[k].to(ifgo.dtype).reshape(B, H).clone())
+            sides.append((_aligned(dh), state(0), state(1), torch.empty_like(ifgo)))
+        (dha, dhn_a, dcn_a, d_ifgo_a), (dhb, dhn_b, dcn_b, d_ifgo_b) = sides
+        plan = _plan(xa.device, B, H, code, True)
+        n = lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)
+        ws = torch.empty(n, dtype=torch.uint8, device=xa.device)
+        ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
+        _lib.check(lib.fastlstm_bwd_persistent_pair(
+            p(dha), p(dhn_a), p(dcn_a), p(ifgo_a), p(cell_a), p(d_ifgo_a), p(Wha),
+            p(dhb), p(dhn_b), p(dcn_b), p(ifgo_b), p(cell_b), p(d_ifgo_b), p(Whb),
+            p(ws), ws.numel(), T, B, H, code, stream), "fastlstm_bwd_persistent_pair")
+        _check_ws(ws, "fastlstm_bwd_persistent_pair")
+        res = []
+        for x, out, d_ifgo, Wx, dhn, dcn in ((xa, out_a, d_ifgo_a, Wxa, dhn_a, dcn_a), (xb, out_b, d_ifgo_b, Wxb, dhn_b, dcn_b)):
+            x = _aligned(x.contiguous())
+            d_x = torch.empty_like(x)
+            _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo), p(Wx.contiguous()), p(d_x), T, B, I, H, code, stream), "fastlstm_gemm_dx")
+            dbx, dbh, dWx, dWh = Wgrad(d_ifgo, x, out)
+            res.append((d_x, dhn, dcn, dWx, dbx, dWh, dbh))
+    return res[0], res[1]
+
+
 def _autocast_operands(*tensors):
     """x and the parameters in the autocast dtype when autocast is on (fastlstm/lstm.py:509-515;
     the initial states are not cast)."""
@@ -418,6 +517,42 @@ class PersistentLSTMHistoryfn(torch.autograd.Function):
         if ctx.no_state:
             dh_0 = dc_0 = None
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
+
+
+class PersistentLSTMPairfn(torch.autograd.Function):
+    """Two independent layers of one shape as one autograd node (the two directions of a bidirectional layer):
+    forward through lstm_persistent_fwd_pair, backward through lstm_persistent_bwd_pair, one launch for both time
+    loops each way where the shapes allow.  apply(xa, h0a, c0a, Wxa, bxa, Wha, bha, xb, h0b, c0b, Wxb, bxb, Whb,
+    bhb, state_grads) -> (out_a, h_Ta, c_Ta, out_b, h_Tb, c_Tb); the final states carry a gradient only with
+    state_grads (as PersistentLSTMStatefn), else none (as PersistentLSTMfn)."""
+
+    @staticmethod
+    @custom_fwd(device_type="cuda")
+    def forward(ctx, xa, h0a, c0a, Wxa, bxa, Wha, bha, xb, h0b, c0b, Wxb, bxb, Whb, bhb, state_grads):
+        xa, Wxa, bxa, Wha, bha, xb, Wxb, bxb, Whb, bhb = _autocast_operands(xa, Wxa, bxa, Wha, bha, xb, Wxb, bxb, Whb, bhb)
+        out_a, cell_a, ifgo_a, out_b, cell_b, ifgo_b = lstm_persistent_fwd_pair(xa, h0a, c0a, Wxa, bxa, Wha, bha,
+                                                                                xb, h0b, c0b, Wxb, bxb, Whb, bhb)
+        ctx.no_state = (h0a is None, h0b is None)
+        ctx.save_for_backward(xa, out_a, cell_a, ifgo_a, Wxa, Wha, xb, out_b, cell_b, ifgo_b, Wxb, Whb)
+        finals = (out_a[-1].clone(), cell_a[-1].clone(), out_b[-1].clone(), cell_b[-1].clone())
+        if not state_grads:
+            ctx.mark_non_differentiable(*finals)
+        return out_a[1:], finals[0], finals[1], out_b[1:], finals[2], finals[3]
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, dh_a, dhn_a, dcn_a, dh_b, dhn_b, dcn_b):
+        xa, out_a, cell_a, ifgo_a, Wxa, Wha, xb, out_b, cell_b, ifgo_b, Wxb, Whb = ctx.saved_tensors
+        pair = lambda h, c: None if h is None and c is None else (
+            torch.zeros_like(cell_a[0]) if h is None else h, torch.zeros_like(cell_a[0]) if c is None else c)
+        ga, gb = lstm_persistent_bwd_pair(dh_a, pair(dhn_a, dcn_a), xa, out_a, cell_a, ifgo_a, Wxa, Wha,
+                                          dh_b, pair(dhn_b, dcn_b), xb, out_b, cell_b, ifgo_b, Wxb, Whb)
+        ga, gb = list(ga), list(gb)
+        if ctx.no_state[0]:
+            ga[1] = ga[2] = None
+        if ctx.no_state[1]:
+            gb[1] = gb[2] = None
+        return (*ga, *gb, None)
 
 
 class PersistentLSTMStack2fn(torch.autograd.Function):
@@ -604,6 +739,26 @@ class FastLSTM(nn.Module):
                 layer += 2
                 continue
             k = layer * directions
+            if (directions == 2 and x.dim() == 3 and x.is_cuda and pair_runs_in_one_launch(
+                    x.shape[0], x.shape[1], self.hidden_size,
+                    torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device)):
+                # both directions' time loops in one launch (the reverse direction: the same kernels over the
+                # time-reversed sequence; its final state belongs to t = 0)
+                wa, wb = self._layer_operands(layer), self._layer_operands(layer, "_reverse")
+                if inference:
+                    xa, *wa = _autocast_operands(x.contiguous(), *wa)
+                    xb, *wb = _autocast_operands(x.flip(0), *wb)
+                    oa, ca, _, ob, cb, _ = lstm_persistent_fwd_pair(xa, h_0[k], c_0[k], *wa, xb, h_0[k + 1], c_0[k + 1], *wb,
+                                                                    keep_activations=False)
+                    y, h_i, c_i, y_r, h_r, c_r = oa[1:], oa[-1], ca[-1], ob[1:], ob[-1], cb[-1]
+                else:
+                    y, h_i, c_i, y_r, h_r, c_r = PersistentLSTMPairfn.apply(
+                        x.contiguous(), h_0[k], c_0[k], *wa, x.flip(0), h_0[k + 1], c_0[k + 1], *wb, self.state_grads)
+                x = torch.cat((y, y_r.flip(0)), dim=-1)
+                h_n += [h_i, h_r]
+                c_n += [c_i, c_r]
+                layer += 1
+                continue
             y, (h_i, c_i) = fn(x, h_0[k], c_0[k], *self._layer_operands(layer))
             h_n += [h_i]
             c_n += [c_i]

@@ -177,6 +177,25 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
                             const void *cell, void *d_ifgo, const void *Wh, void *ws,
                             size_t ws_bytes, int T, int B, int H, int dtype, void *stream);
 
+/* Two independent recurrences of one shape -- the two directions of a bidirectional layer, whose reverse
+ * direction is the same time loop over the reversed sequence -- as ONE launch of the XCD-local kernels where
+ * both sets of barrier groups fit the device side by side, else one after the other.  Arguments of recurrence a,
+ * then b, as fastlstm_fwd_persistent / fastlstm_bwd_persistent take them; keep_activations = 0 is the inference
+ * form.  ws: fastlstm_stack2_workspace_bytes (forward) / fastlstm_stack2_bwd_workspace_bytes (the exchange slots
+ * of both recurrences), zeroed like any recurrent workspace.  fastlstm_pair_fused: 1 if the call is one launch
+ * for this shape and workspace size on the current device, 0 if not; negative: fastlstm_status.  The reference has
+ * no bidirectional layers (README.md:92-94): a host that adds them calls the time loop of
+ * fastlstm/lstm.py:102-112 / 277-290 once per direction; these two replace that pair of calls. */
+int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const void *Wh_a, void *ifgo_b,
+                                 void *out_b, void *cell_b, const void *Wh_b, void *ws, size_t ws_bytes, int T,
+                                 int B, int H, int dtype, int keep_activations, void *stream);
+int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, const void *ifgo_a,
+                                 const void *cell_a, void *d_ifgo_a, const void *Wh_a, const void *dout_b,
+                                 void *dh_b, void *dc_b, const void *ifgo_b, const void *cell_b, void *d_ifgo_b,
+                                 const void *Wh_b, void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                                 void *stream);
+int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
+
 /* K4 + K5 + K6..K9 for one layer in one call: the same results as fastlstm_bwd_persistent,
  * fastlstm_gemm_dx and fastlstm_gemm_wgrad one after the other (same arguments and workspace
  * contracts; dWx and dWh to the rounding of a different summation order).  Where the XCD-local

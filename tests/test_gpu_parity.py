@@ -601,6 +601,47 @@ def test_register_resident_kernels_at_the_batch_sizes_where_their_form_changes(H
     assert (2, 2) in seen
 
 
+PAIR_CASES = [
+    # T, B, I, H, dtype, one launch expected
+    (6, 32, 96, 512, torch.float16, True),
+    (5, 40, 64, 256, torch.float32, True),
+    (4, 64, 128, 1024, torch.bfloat16, True),     # config B's tiles: 4 + 4 groups on the 8 XCDs
+    (3, 200, 64, 1024, torch.float16, False),     # 7 + 7 groups of 32 rows do not fit: one after the other
+    (4, 24, 48, 72, torch.float16, False),        # general kernels: one after the other
+]
+
+
+@pytest.mark.parametrize("T,B,I,H,dt,fused", PAIR_CASES)
+def test_two_recurrences_side_by_side_equal_two_calls(T, B, I, H, dt, fused):
+    """fastlstm_fwd_persistent_pair / fastlstm_bwd_persistent_pair (the two directions of a bidirectional layer in
+    one launch) against two calls of the single-layer ops on the same operands: the same kernels do the same sums
+    in the same order, so the time loops' results are the same bits; dx and the weight gradients come from
+    stand-alone GEMM launches here and from the layer call there (another order of the same sums)."""
+    assert L.pair_runs_in_one_launch(T, B, H, dt, "cuda") == fused
+    assert L.pair_runs_in_one_launch(T, B, H, dt, "cuda", backward=True) == fused
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    sides = []
+    for seed in (11, 12):
+        p = make_problem(T, B, I, H, seed=seed + H)
+        sides.append({k: dev(v, dt) for k, v in p.items()})
+    a, b = sides
+    fwd_keys = ("x", "h0", "c0", "Wx", "bx", "Wh", "bh")
+    got = L.lstm_persistent_fwd_pair(*(a[k] for k in fwd_keys), *(b[k] for k in fwd_keys))
+    want = L.lstm_persistent_fwd(*(a[k] for k in fwd_keys)) + L.lstm_persistent_fwd(*(b[k] for k in fwd_keys))
+    for name, g_, w_ in zip(("out_a", "cell_a", "ifgo_a", "out_b", "cell_b", "ifgo_b"), got, want):
+        assert torch.equal(g_, w_), name
+    ga, gb = L.lstm_persistent_bwd_pair(a["dout"], (a["dh_n"], a["dc_n"]), a["x"], got[0], got[1], got[2], a["Wx"], a["Wh"],
+                                        b["dout"], (b["dh_n"], b["dc_n"]), b["x"], got[3], got[4], got[5], b["Wx"], b["Wh"])
+    for side, g_, (out, cell, ifgo) in ((a, ga, want[:3]), (b, gb, want[3:])):
+        w_ = L.lstm_persistent_bwd(side["dout"], side["dc_n"].clone(), side["dh_n"].clone(), side["x"], out, cell, ifgo,
+                                   side["Wx"], side["Wh"])
+        for name, x_, y_ in zip(("d_x", "dh_0", "dc_0", "dWx", "dbx", "dWh", "dbh"), g_, w_):
+            if name in ("dh_0", "dc_0"):
+                assert torch.equal(x_, y_), name
+            else:
+                assert rel_err(x_, npy(y_)) < tol, name
+
+
 XCD_CASES = [
     # T, B, H, dtype          (hidden tile, members, batch tiles) of the XCD-local launch
     (20, 64, 1024, torch.float16),    # config B: 32 units x 32 members, 8 waves
