@@ -19,6 +19,7 @@ import os
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 from torch.amp import custom_bwd, custom_fwd
 
 from . import _lib
@@ -609,7 +610,7 @@ class FastLSTM(nn.Module):
     states at each row's own last step, as nn.LSTM does."""
 
     def __init__(self, input_size, hidden_size, num_layers=1, version="persistent", device=None,
-                 dtype=None, *, bias=True, batch_first=False, bidirectional=False, state_grads=False):
+                 dtype=None, *, bias=True, batch_first=False, bidirectional=False, state_grads=False, dropout=0.0):
         super().__init__()
         self.input_size = input_size
         self.hidden_size = hidden_size
@@ -621,6 +622,9 @@ class FastLSTM(nn.Module):
         self.batch_first = batch_first
         self.bidirectional = bidirectional
         self.state_grads = state_grads
+        if not 0.0 <= dropout < 1.0:
+            raise ValueError("dropout should be a number in [0, 1), got %r" % (dropout,))
+        self.dropout = float(dropout)   # nn.LSTM's: on the outputs of every layer but the last, in training mode
         sqrt_k_inv = 1 / hidden_size**0.5
         directions = 2 if bidirectional else 1
         # same RNG consumption order as nn.LSTM: w_ih, w_hh, b_ih, b_hh per layer and direction
@@ -674,6 +678,8 @@ class FastLSTM(nn.Module):
                 c_n.append(cells.gather(0, last.expand(1, B, H))[0])
                 ys.append(y if d == 0 else y.gather(0, flip.expand(T, B, H)))
             x = ys[0] if directions == 1 else torch.cat(ys, dim=-1)
+            if self.training and self.dropout > 0.0 and layer + 1 < self.num_layers:
+                x = F.dropout(x, self.dropout, True)
         if packed.sorted_indices is not None:
             x, lengths = x.index_select(1, packed.sorted_indices), lengths[packed.sorted_indices.cpu()]
         data = pack_padded_sequence(x, lengths, enforce_sorted=True).data
@@ -710,10 +716,15 @@ class FastLSTM(nn.Module):
             fn = PersistentLSTMfn.apply
         h_n, c_n = [], []
         layer = 0
+        drop = self.dropout if self.training else 0.0
+
+        def between(y, done):   # dropout on what the next layer reads
+            return F.dropout(y, drop, True) if drop > 0.0 and done < self.num_layers else y
+
         while layer < self.num_layers:
             # two layers at a time where the library runs them as one launch (the second layer's
             # recurrence a chunk of timesteps behind the first); the results do not depend on it
-            if (directions == 1 and layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda
+            if (directions == 1 and drop == 0.0 and layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda
                     and stack2_runs_in_one_launch(
                         x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
                         torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device)):
@@ -754,7 +765,7 @@ class FastLSTM(nn.Module):
                 else:
                     y, h_i, c_i, y_r, h_r, c_r = PersistentLSTMPairfn.apply(
                         x.contiguous(), h_0[k], c_0[k], *wa, x.flip(0), h_0[k + 1], c_0[k + 1], *wb, self.state_grads)
-                x = torch.cat((y, y_r.flip(0)), dim=-1)
+                x = between(torch.cat((y, y_r.flip(0)), dim=-1), layer + 1)
                 h_n += [h_i, h_r]
                 c_n += [c_i, c_r]
                 layer += 1
@@ -769,7 +780,7 @@ class FastLSTM(nn.Module):
                 y = torch.cat((y, y_r.flip(0)), dim=-1)
                 h_n += [h_r]
                 c_n += [c_r]
-            x = y
+            x = between(y, layer + 1)
             layer += 1
         if self.batch_first:
             x = x.transpose(0, 1)
@@ -782,4 +793,6 @@ class FastLSTM(nn.Module):
         for name in ("bias", "batch_first", "bidirectional", "state_grads"):
             if getattr(self, name) != (name == "bias"):
                 s += ", %s=%s" % (name, getattr(self, name))
+        if self.dropout:
+            s += ", dropout=%g" % self.dropout
         return s

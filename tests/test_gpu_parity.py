@@ -601,6 +601,45 @@ def test_register_resident_kernels_at_the_batch_sizes_where_their_form_changes(H
     assert (2, 2) in seen
 
 
+@pytest.mark.parametrize("kw", [dict(num_layers=2), dict(num_layers=3, bidirectional=True)])
+def test_dropout_between_layers(kw):
+    """nn.LSTM's `dropout`: on the outputs of every layer but the last, in training mode only.  (MIOpen draws its
+    own mask, so the check is against the same layers composed by hand under the same seed.)"""
+    T, B, I, H, dt, p = 7, 16, 24, 128, torch.float16, 0.4
+    torch.manual_seed(3)
+    m = FastLSTM(I, H, dropout=p, **kw).to("cuda", dt)
+    plain = FastLSTM(I, H, **kw).to("cuda", dt)
+    plain.load_state_dict(m.state_dict())
+    x = torch.randn(T, B, I, device="cuda", dtype=dt)
+    m.eval()
+    plain.eval()
+    assert torch.equal(m(x)[0], plain(x)[0])            # no dropout outside training
+    m.train()
+    plain.train()
+    D = 2 if kw.get("bidirectional") else 1
+    singles = []
+    for layer in range(kw["num_layers"]):
+        one = FastLSTM(I if layer == 0 else D * H, H, bidirectional=D == 2).to("cuda", dt)
+        sd = {k.replace("_l%d" % layer, "_l0"): v for k, v in m.state_dict().items() if "_l%d" % layer in k}
+        one.load_state_dict(sd)
+        singles.append(one.train())
+    torch.manual_seed(17)
+    got, (h_n, _) = m(x)
+    torch.manual_seed(17)
+    y = x
+    for layer, one in enumerate(singles):
+        y = one(y)[0]
+        if layer + 1 < len(singles):
+            y = torch.nn.functional.dropout(y, p, True)
+    assert torch.equal(got, y)
+    assert not torch.equal(got, plain(x)[0])
+    assert h_n.shape == (kw["num_layers"] * D, B, H)
+    got.float().sum().backward()
+    assert all(q.grad is not None and torch.isfinite(q.grad.float()).all() for q in m.parameters())
+    with pytest.raises(ValueError):
+        FastLSTM(I, H, dropout=1.0)
+
+
 PAIR_CASES = [
     # T, B, I, H, dtype, one launch expected
     (6, 32, 96, 512, torch.float16, True),
