@@ -524,8 +524,9 @@ class PersistentLSTMPairfn(torch.autograd.Function):
     """Two independent layers of one shape as one autograd node (the two directions of a bidirectional layer):
     forward through lstm_persistent_fwd_pair, backward through lstm_persistent_bwd_pair, one launch for both time
     loops each way where the shapes allow.  apply(xa, h0a, c0a, Wxa, bxa, Wha, bha, xb, h0b, c0b, Wxb, bxb, Whb,
-    bhb, state_grads) -> (out_a, h_Ta, c_Ta, out_b, h_Tb, c_Tb); the final states carry a gradient only with
-    state_grads (as PersistentLSTMStatefn), else none (as PersistentLSTMfn)."""
+    bhb, state_grads) -> (out_a, h_Ta, c_Ta, out_b, h_Tb, c_Tb, cells_a, cells_b); the final states carry a gradient
+    only with state_grads (as PersistentLSTMStatefn), else none (as PersistentLSTMfn); cells_* [T,B,H] are the
+    cell-state histories, non-differentiable (as PersistentLSTMHistoryfn's)."""
 
     @staticmethod
     @custom_fwd(device_type="cuda")
@@ -536,13 +537,13 @@ class PersistentLSTMPairfn(torch.autograd.Function):
         ctx.no_state = (h0a is None, h0b is None)
         ctx.save_for_backward(xa, out_a, cell_a, ifgo_a, Wxa, Wha, xb, out_b, cell_b, ifgo_b, Wxb, Whb)
         finals = (out_a[-1].clone(), cell_a[-1].clone(), out_b[-1].clone(), cell_b[-1].clone())
-        if not state_grads:
-            ctx.mark_non_differentiable(*finals)
-        return out_a[1:], finals[0], finals[1], out_b[1:], finals[2], finals[3]
+        histories = (cell_a[1:], cell_b[1:])
+        ctx.mark_non_differentiable(*histories, *(() if state_grads else finals))
+        return out_a[1:], finals[0], finals[1], out_b[1:], finals[2], finals[3], histories[0], histories[1]
 
     @staticmethod
     @custom_bwd(device_type="cuda")
-    def backward(ctx, dh_a, dhn_a, dcn_a, dh_b, dhn_b, dcn_b):
+    def backward(ctx, dh_a, dhn_a, dcn_a, dh_b, dhn_b, dcn_b, _ha, _hb):
         xa, out_a, cell_a, ifgo_a, Wxa, Wha, xb, out_b, cell_b, ifgo_b, Wxb, Whb = ctx.saved_tensors
         pair = lambda h, c: None if h is None and c is None else (
             torch.zeros_like(cell_a[0]) if h is None else h, torch.zeros_like(cell_a[0]) if c is None else c)
@@ -666,14 +667,22 @@ class FastLSTM(nn.Module):
         # time index that reverses row b within its length and leaves its padding in place
         flip = torch.where(steps < lengths_dev[None, :], lengths_dev[None, :] - 1 - steps, steps)[:, :, None]
         h_n, c_n = [], []
+        H = self.hidden_size
         for layer in range(self.num_layers):
             ys = []
-            for d, suffix in enumerate(("", "_reverse")[:directions]):
-                k = layer * directions + d
-                xi = x if d == 0 else x.gather(0, flip.expand(T, B, x.shape[2]))
-                y, cells = PersistentLSTMHistoryfn.apply(xi.contiguous(), h_0[k], c_0[k],
-                                                         *self._layer_operands(layer, suffix))
-                H = self.hidden_size
+            xs = [x.contiguous()] + ([x.gather(0, flip.expand(T, B, x.shape[2]))] if directions == 2 else [])
+            k = layer * directions
+            if directions == 2 and pair_runs_in_one_launch(
+                    T, B, H, torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device):
+                # both directions' time loops in one launch
+                y_a, _, _, y_b, _, _, cells_a, cells_b = PersistentLSTMPairfn.apply(
+                    xs[0], h_0[k], c_0[k], *self._layer_operands(layer),
+                    xs[1], h_0[k + 1], c_0[k + 1], *self._layer_operands(layer, "_reverse"), False)
+                results = [(y_a, cells_a), (y_b, cells_b)]
+            else:
+                results = [PersistentLSTMHistoryfn.apply(xs[d], h_0[k + d], c_0[k + d], *self._layer_operands(layer, suffix))
+                           for d, suffix in enumerate(("", "_reverse")[:directions])]
+            for d, (y, cells) in enumerate(results):
                 h_n.append(y.gather(0, last.expand(1, B, H))[0])
                 c_n.append(cells.gather(0, last.expand(1, B, H))[0])
                 ys.append(y if d == 0 else y.gather(0, flip.expand(T, B, H)))
@@ -763,7 +772,7 @@ class FastLSTM(nn.Module):
                                                                     keep_activations=False)
                     y, h_i, c_i, y_r, h_r, c_r = oa[1:], oa[-1], ca[-1], ob[1:], ob[-1], cb[-1]
                 else:
-                    y, h_i, c_i, y_r, h_r, c_r = PersistentLSTMPairfn.apply(
+                    y, h_i, c_i, y_r, h_r, c_r, _, _ = PersistentLSTMPairfn.apply(
                         x.contiguous(), h_0[k], c_0[k], *wa, x.flip(0), h_0[k + 1], c_0[k + 1], *wb, self.state_grads)
                 x = between(torch.cat((y, y_r.flip(0)), dim=-1), layer + 1)
                 h_n += [h_i, h_r]
