@@ -15,6 +15,7 @@ gfx950 kernels) on the current HIP stream.  There is one code path, no Triton,
 no autotune warm-up run and no CPU fallback: tensors must live on the GPU and
 the library must be built, otherwise the calls raise.
 """
+import functools
 import os
 
 import torch
@@ -172,6 +173,152 @@ def _aligned(t):
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+@functools.lru_cache(maxsize=512)
+def _wavefront_chunks(T, B, H, dtype, device, backward):
+    # chunks of at least 64 timesteps: every launch costs about 50 us besides its steps (launch gaps, the prologue,
+    # the small GEMM in between), which a chunk of 32 steps does not win back (measured: no gain at T = 256 with
+    # 8 chunks); whole 16-byte units per timestep, so that every chunk's buffers start on a 16-byte boundary
+    if T < 256 or (B * H * torch.empty((), dtype=dtype).element_size()) % 16:
+        return 0
+    for n in (8, 6, 5, 4, 3, 2):
+        if T % n == 0 and T // n >= 64 and pair_runs_in_one_launch(T // n, B, H, dtype, device, backward):
+            return n
+    return 0
+
+
+def stack2_wavefront_chunks(T, B, H, dtype, device, backward=False):
+    """Into how many chunks of timesteps two stacked layers of this shape are cut so that the upper layer's chunk
+    k - 1 and the lower layer's chunk k run side by side in one launch (0: they are not).  For the shapes whose
+    two time loops fit the device side by side (pair_runs_in_one_launch) but which the library's own two-layer
+    launch (stack2_runs_in_one_launch) does not take."""
+    return _wavefront_chunks(int(T), int(B), int(H), dtype, str(torch.device(device)), bool(backward))
+
+
+def _small_projections(B, I, H):
+    """The library's own two-layer launch hides the GEMMs behind the time loops but fills its pipeline slowly; the
+    chunked wavefront leaves the GEMMs in the open and overlaps the time loops better.  Where the GEMMs are a few
+    per cent of a step anyway the wavefront wins (T = 256 ... 512, B = 16, I = H = 640: forward + backward 2.3 vs
+    2.6 and 3.7 vs 4.2 ms); B = 32, I = H = 1024 and B = 64, I = H = 768 are past the crossover."""
+    return B * I * H < 1.5e7
+
+
+def _chunk_workspaces(n_bytes, zero_bytes, count, device):
+    """`count` workspaces of n_bytes each, the first zero_bytes of every one cleared by ONE fill."""
+    stride = (n_bytes + 255) // 256 * 256
+    if zero_bytes >= n_bytes:
+        buf = torch.zeros(count * stride, dtype=torch.uint8, device=device)
+    else:
+        buf = torch.empty(count * stride, dtype=torch.uint8, device=device)
+        buf.view(count, stride)[:, :zero_bytes].zero_()
+    return [buf[k * stride:k * stride + n_bytes] for k in range(count)]
+
+
+def _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, n, keep_activations):
+    """lstm_persistent_fwd_stack2 as n + 1 launches: launch k runs chunk k of the lower layer's time loop and chunk
+    k - 1 of the upper layer's side by side (fastlstm_fwd_persistent_pair on sub-ranges of the buffers: a time
+    loop started at out[t0], cell[t0] continues the sequence); the upper layer's input projection of a chunk is a
+    GEMM launch in between.  (A chunk starts from the stored cell state, where the one-launch loop carries it in
+    fp32: with 16-bit elements the results differ from the layer-by-layer path by that rounding, once per chunk.)"""
+    lib = _lib.load()
+    code = _code(x)
+    T, B, I = x.shape
+    H = Wh0.shape[1]
+    Tc = T // n
+    dev_ = x.device
+    stream = _stream()
+    p = lambda t: t.data_ptr()
+    bufs = []
+    for h0, c0 in ((h0a, c0a), (h0b, c0b)):
+        ifgo = torch.empty((T, B, 4 * H), device=dev_, dtype=x.dtype)
+        out = torch.empty((T + 1, B, H), device=dev_, dtype=x.dtype)
+        cell = torch.empty_like(out)
+        if h0 is not None:
+            out[0] = h0
+            cell[0] = c0
+        else:
+            out[0].zero_()
+            cell[0].zero_()
+        bufs.append((out, cell, ifgo))
+    (out0, cell0, ifgo0), (out1, cell1, ifgo1) = bufs
+    _lib.check(lib.fastlstm_gemm_ifgo(p(x), p(Wx0), p(bx0), p(bh0), p(ifgo0), T, B, I, H, code, stream), "fastlstm_gemm_ifgo")
+    plan = _plan(dev_, B, H, code, False)
+    nb = lib.fastlstm_stack2_workspace_bytes(plan, Tc, H, code)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + 1, dev_)
+    keep = int(keep_activations)
+    # (addresses of the chunks by arithmetic: slicing tensors would cost the host more than a short chunk runs)
+    row = B * H * x.element_size()
+    g0, o0, c0_, g1, o1, c1_ = (p(t) for t in (ifgo0, out0, cell0, ifgo1, out1, cell1))
+    pWx1, pbx1, pbh1, pWh0, pWh1 = p(Wx1), p(bx1), p(bh1), p(Wh0), p(Wh1)
+    for k in range(n + 1):
+        ws, ta, tb = wss[k], k * Tc, (k - 1) * Tc
+        if k >= 1:   # the upper layer's projection of the chunk the lower layer has just finished
+            _lib.check(lib.fastlstm_gemm_ifgo(o0 + (1 + tb) * row, pWx1, pbx1, pbh1, g1 + tb * 4 * row, Tc, B, H, H, code, stream),
+                       "fastlstm_gemm_ifgo")
+        if 1 <= k < n:
+            _lib.check(lib.fastlstm_fwd_persistent_pair(g0 + ta * 4 * row, o0 + ta * row, c0_ + ta * row, pWh0, g1 + tb * 4 * row,
+                                                        o1 + tb * row, c1_ + tb * row, pWh1, p(ws), ws.numel(), Tc, B, H,
+                                                        code, keep, stream), "fastlstm_fwd_persistent_pair")
+        elif k == 0:
+            _lib.check(lib.fastlstm_fwd_persistent(g0, o0, c0_, pWh0, p(ws), ws.numel(), Tc, B, H, code, stream),
+                       "fastlstm_fwd_persistent")
+        else:
+            _lib.check(lib.fastlstm_fwd_persistent(g1 + tb * 4 * row, o1 + tb * row, c1_ + tb * row, pWh1, p(ws), ws.numel(),
+                                                   Tc, B, H, code, stream), "fastlstm_fwd_persistent")
+    for ws in wss:
+        _check_ws(ws, "fastlstm_fwd_persistent_pair")
+    return out0, cell0, ifgo0, out1, cell1, ifgo1
+
+
+def _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1, n):
+    """lstm_persistent_bwd_stack2 as n + 1 launches (see _fwd_stack2_wavefront): launch k runs the upper layer's
+    chunk n - 1 - k and the lower layer's chunk n - k of the reverse time loops side by side; the lower layer's dout
+    of a chunk (the upper layer's dx) is a GEMM launch in between; the weight gradients and the lower layer's dx
+    follow over the whole sequence."""
+    lib = _lib.load()
+    code = _code(ifgo1)
+    T, B, H = dh.shape
+    I = Wx0.shape[1]
+    Tc = T // n
+    dev_ = x.device
+    stream = _stream()
+    p = lambda t: t.data_ptr()
+    dh = dh.contiguous()
+    if dh.dtype != ifgo1.dtype:
+        dh = dh.to(ifgo1.dtype)
+    dh, x = _aligned(dh), _aligned(x.contiguous())
+    zeros = lambda: torch.zeros((B, H), device=dev_, dtype=x.dtype)
+    state = lambda d, k: zeros() if d is None else d[k].to(x.dtype).reshape(B, H).clone()
+    dh1, dc1, dh0, dc0 = state(d_state1, 0), state(d_state1, 1), state(d_state0, 0), state(d_state0, 1)
+    d_ifgo1, d_ifgo0 = torch.empty_like(ifgo1), torch.empty_like(ifgo0)
+    dx1 = torch.empty((T, B, H), device=dev_, dtype=x.dtype)
+    plan = _plan(dev_, B, H, code, True)
+    nb = lib.fastlstm_stack2_bwd_workspace_bytes(plan, Tc, H, code)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + 1, dev_)
+    Wx1c = Wx1.contiguous()
+    row = B * H * x.element_size()
+    pdh, pdx1, g1, c1_, dg1, g0, c0_, dg0 = (p(t) for t in (dh, dx1, ifgo1, cell1, d_ifgo1, ifgo0, cell0, d_ifgo0))
+    pdh1, pdc1, pdh0, pdc0, pWx1, pWh1, pWh0 = (p(t) for t in (dh1, dc1, dh0, dc0, Wx1c, Wh1, Wh0))
+    for k in range(n + 1):
+        ws, t1, t0 = wss[k], (n - 1 - k) * Tc, (n - k) * Tc
+        if k >= 1:   # the lower layer's dout of the chunk the upper layer has just finished
+            _lib.check(lib.fastlstm_gemm_dx(dg1 + t0 * 4 * row, pWx1, pdx1 + t0 * row, Tc, B, H, H, code, stream), "fastlstm_gemm_dx")
+        upper = (pdh + t1 * row, pdh1, pdc1, g1 + t1 * 4 * row, c1_ + t1 * row, dg1 + t1 * 4 * row, pWh1)
+        lower = (pdx1 + t0 * row, pdh0, pdc0, g0 + t0 * 4 * row, c0_ + t0 * row, dg0 + t0 * 4 * row, pWh0)
+        if 1 <= k < n:
+            _lib.check(lib.fastlstm_bwd_persistent_pair(*upper, *lower, p(ws), ws.numel(), Tc, B, H, code, stream),
+                       "fastlstm_bwd_persistent_pair")
+        else:
+            _lib.check(lib.fastlstm_bwd_persistent(*(upper if k == 0 else lower), p(ws), ws.numel(), Tc, B, H, code, stream),
+                       "fastlstm_bwd_persistent")
+    for ws in wss:
+        _check_ws(ws, "fastlstm_bwd_persistent_pair")
+    dx0 = torch.empty_like(x)
+    _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo0), p(Wx0.contiguous()), p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
+    db1, _, dWx1, dWh1 = Wgrad(d_ifgo1, out0[1:], out1)
+    db0, _, dWx0, dWh0 = Wgrad(d_ifgo0, x, out0)
+    return (dx0, dh0, dc0, dWx0, db0, dWh0, db0), (dx1, dh1, dc1, dWx1, db1, dWh1, db1)
+
+
 def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, keep_activations=True):
     """Two stacked layers (the second reads the first one's h): returns
     (out0, cell0, ifgo0, out1, cell1, ifgo1) with the layouts of lstm_persistent_fwd.  The same
@@ -192,6 +339,9 @@ def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, b
     x = _aligned(x)
     lib = _lib.load()
     with torch.cuda.device(x.device):
+        n = stack2_wavefront_chunks(T, B, H, x.dtype, x.device)
+        if n and (_small_projections(B, I, H) or not stack2_runs_in_one_launch(T, B, I, H, x.dtype, x.device)):
+            return _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, n, keep_activations)
         bufs = []
         for h0, c0 in ((h0a, c0a), (h0b, c0b)):
             ifgo = torch.empty((T, B, 4 * H), device=x.device, dtype=x.dtype)
@@ -293,6 +443,12 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
     I = Wx0.shape[1]
     lib = _lib.load()
     with torch.cuda.device(x.device):
+        plan = _plan(x.device, B, H, code, True)
+        n = stack2_wavefront_chunks(T, B, H, ifgo1.dtype, x.device, backward=True)
+        if n and (_small_projections(B, I, H) or lib.fastlstm_bwd_stack2_fused(
+                T, B, I, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) != 1):
+            return _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1,
+                                         d_state0, d_state1, n)
         dh = dh.contiguous()
         if dh.dtype != ifgo1.dtype:
             dh = dh.to(ifgo1.dtype)
@@ -643,6 +799,14 @@ class FastLSTM(nn.Module):
                     value = torch.rand(*shape, device=device, dtype=dtype) * 2 * sqrt_k_inv - sqrt_k_inv
                     setattr(self, name, nn.Parameter(value))
 
+    def _two_layers_at_once(self, x):
+        """Two stacked layers of this input's shape run overlapped: as one launch of the library, or as a wavefront
+        of chunked launches (stack2_wavefront_chunks)."""
+        dt = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
+        T, B, I = x.shape
+        return (stack2_runs_in_one_launch(T, B, I, self.hidden_size, dt, x.device)
+                or stack2_wavefront_chunks(T, B, self.hidden_size, dt, x.device) > 0)
+
     def _layer_operands(self, layer, suffix=""):
         """(Wx, bx, Wh, bh) of one layer and direction; zero biases when the module has none."""
         Wx = getattr(self, f"weight_ih_l{layer}{suffix}")
@@ -734,9 +898,7 @@ class FastLSTM(nn.Module):
             # two layers at a time where the library runs them as one launch (the second layer's
             # recurrence a chunk of timesteps behind the first); the results do not depend on it
             if (directions == 1 and drop == 0.0 and layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda
-                    and stack2_runs_in_one_launch(
-                        x.shape[0], x.shape[1], x.shape[2], self.hidden_size,
-                        torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype, x.device)):
+                    and self._two_layers_at_once(x)):
                 w = self._layer_operands(layer) + self._layer_operands(layer + 1)
                 if inference:
                     xi, *wc = _autocast_operands(x, *w)

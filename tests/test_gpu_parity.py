@@ -838,6 +838,59 @@ def test_fwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("T,B,I,H,dt", [(256, 16, 96, 640, torch.float16), (384, 32, 64, 256, torch.float32),
+                                        (320, 48, 128, 512, torch.bfloat16)])
+def test_two_layers_as_a_wavefront_of_chunked_pair_launches(T, B, I, H, dt):
+    """Shapes whose two time loops fit the device side by side but which the library's own two-layer launch does
+    not take: lstm_persistent_fwd_stack2 / lstm_persistent_bwd_stack2 cut the sequence into chunks and run the
+    upper layer's chunk k - 1 beside the lower layer's chunk k.  Against the layer-by-layer ops: the same bits with
+    fp32 (the weight gradients: another order of the same sums); with 16-bit elements a chunk starts from the
+    stored cell state where the one-launch loop carries it in fp32, hence a tolerance."""
+    assert not L.stack2_runs_in_one_launch(T, B, I, H, dt, "cuda")
+    assert L.stack2_wavefront_chunks(T, B, H, dt, "cuda") >= 2 and L.stack2_wavefront_chunks(T, B, H, dt, "cuda", backward=True) >= 2
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    g0 = {k: dev(v, dt) for k, v in make_problem(T, B, I, H, seed=41 + T).items()}
+    g1 = {k: dev(v, dt) for k, v in make_problem(T, B, H, H, seed=42 + T).items()}
+    keys = ("h0", "c0", "Wx", "bx", "Wh", "bh")
+    got = L.lstm_persistent_fwd_stack2(g0["x"], *(g0[k] for k in keys), *(g1[k] for k in keys))
+    ref0 = L.lstm_persistent_fwd(g0["x"], *(g0[k] for k in keys))
+    ref1 = L.lstm_persistent_fwd(ref0[0][1:], *(g1[k] for k in keys))
+    for name, a, b in zip(("out0", "cell0", "ifgo0", "out1", "cell1", "ifgo1"), got, ref0 + ref1):
+        if dt == torch.float32:
+            assert torch.equal(a, b), name
+        else:
+            assert rel_err(a, npy(b)) < tol, name
+    # the reverse pass on the layer-by-layer activations, both ways
+    out0, cell0, ifgo0, out1, cell1, ifgo1 = ref0 + ref1
+    r0, r1 = L.lstm_persistent_bwd_stack2(g1["dout"], g0["x"], out0, cell0, ifgo0, g0["Wx"], g0["Wh"], out1, cell1, ifgo1,
+                                          g1["Wx"], g1["Wh"], d_state0=(g0["dh_n"], g0["dc_n"]), d_state1=(g1["dh_n"], g1["dc_n"]))
+    w1 = L.lstm_persistent_bwd(g1["dout"], g1["dc_n"].clone(), g1["dh_n"].clone(), out0[1:], out1, cell1, ifgo1, g1["Wx"], g1["Wh"])
+    w0 = L.lstm_persistent_bwd(w1[0], g0["dc_n"].clone(), g0["dh_n"].clone(), g0["x"], out0, cell0, ifgo0, g0["Wx"], g0["Wh"])
+    for side, got_, want_ in (("upper", r1, w1), ("lower", r0, w0)):
+        for name, a, b in zip(("d_x", "dh_0", "dc_0", "dWx", "dbx", "dWh", "dbh"), got_, want_):
+            assert rel_err(a, npy(b)) < tol, (side, name)
+
+
+@pytest.mark.parametrize("layers,dt", [(2, torch.float16), (3, torch.bfloat16)])
+def test_stacked_module_through_the_wavefront_matches_nn_lstm(layers, dt):
+    T, B, I, H = 256, 16, 64, 384
+    assert L.stack2_wavefront_chunks(T, B, H, dt, "cuda") >= 2
+    torch.manual_seed(5)
+    m = FastLSTM(I, H, num_layers=layers).to("cuda", dt)
+    ref = torch.nn.LSTM(I, H, num_layers=layers).to("cuda", dt)
+    ref.load_state_dict(m.state_dict())
+    x = (torch.randn(T, B, I, device="cuda") * 0.5).to(dt).requires_grad_(True)
+    w = torch.randn(T, B, H, device="cuda").to(dt)
+    res = []
+    for mod in (m, ref):
+        x.grad = None
+        out, (h_n, c_n) = mod(x)
+        (out * w).sum().backward()
+        res.append([out.detach(), h_n.detach(), c_n.detach(), x.grad.clone()] + [q.grad.clone() for q in mod.parameters()])
+    for name, a, b in zip(["out", "h_n", "c_n", "dx"] + [n for n, _ in m.named_parameters()], *res):
+        assert rel_err(a, npy(b)) < 3 * HALF_TOL, name
+
+
 def test_two_layer_module_one_launch_matches_layer_by_layer():
     """FastLSTM with two layers of a shape that runs as one launch: outputs, final states and all
     gradients equal those of the layer-by-layer path (two PersistentLSTMfn nodes), bit for bit."""
