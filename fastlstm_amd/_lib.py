@@ -44,6 +44,10 @@ SIGNATURES = {
     "fastlstm_fwd_persistent_pair": (_i, [_vp] * 9 + [_sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_persistent_pair": (_i, [_vp] * 15 + [_sz, _i, _i, _i, _i, _vp]),
     "fastlstm_pair_fused": (_i, [_i, _i, _i, _i, _i, _sz]),
+    "fastlstm_fwd_persistent_multi": (_i, [_i] + [_vp] * 5 + [_sz, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_bwd_persistent_multi": (_i, [_i] + [_vp] * 8 + [_sz, _i, _i, _i, _i, _vp]),
+    "fastlstm_multi_fused": (_i, [_i, _i, _i, _i, _i, _i, _sz]),
+    "fastlstm_multi_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i, _i, _i]),
     "fastlstm_stack2_bwd_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "fastlstm_gemm_ifgo": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),

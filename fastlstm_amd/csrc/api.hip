@@ -23,6 +23,11 @@ struct LaunchOpts {
                              // pass reads them), 0 = inference (the *_infer entry points)
     int row0 = 0, rows = 0;  // rows [row0, row0 + rows) of the batch; rows == 0: all of it.  A batch with more
                              // tiles than one XCD-local launch holds runs as several launches over row ranges
+    // independent recurrences side by side beyond the first two (see try_multi): n_more of them, each its
+    // operand pointers in the order of the single entry point (forward: ifgo, out, cell, Wh; reverse: dout, dh, dc,
+    // ifgo, cell, d_ifgo, Wh)
+    int n_more = 0;
+    void *const (*more)[7] = nullptr;
 };
 
 static long long *g_rec_trace = nullptr;
@@ -308,10 +313,15 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.keep = o.keep;
     p.trace = g_rec_trace;
     p.n_layers = 1;
-    if (second && !x) {   // two independent recurrences of this shape side by side (the second's projection is done)
-        if (2 * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
-        p.n_layers = 2;
+    if (second && !x) {   // independent recurrences of this shape side by side (their projections are done)
+        const int n = 2 + o.n_more;
+        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
+        if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
+        p.n_layers = n;
         p.ifgo2 = second->ifgo; p.out2 = second->out; p.cell2 = second->cell; p.Wh2 = second->Wh;
+        for (int i = 0; i < o.n_more; ++i) {
+            p.ifgo_more[i] = o.more[i][0]; p.out_more[i] = o.more[i][1]; p.cell_more[i] = o.more[i][2]; p.Wh_more[i] = o.more[i][3];
+        }
     }
     if (x) {
         if (!plan_k1_helpers(c, x, Wx, bx, bh, ifgo, T, B, I, H, dtype, &p, second)) return 2;
@@ -631,9 +641,15 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.b_base = o.row0;
     p.spin_limit = spin_limit_ticks();
     p.n_layers = 1;
-    if (lower && !extras) {   // two independent recurrences of this shape side by side
-        if (2 * c.n_groups > kNumXcd * c.gpx) return 2;
-        p.n_layers = 2;
+    if (lower && !extras) {   // independent recurrences of this shape side by side
+        const int n = 2 + o.n_more;
+        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;
+        if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
+        p.n_layers = n;
+        for (int i = 0; i < o.n_more; ++i) {
+            p.dout_more[i] = o.more[i][0]; p.dh_more[i] = o.more[i][1]; p.dc_more[i] = o.more[i][2]; p.ifgo_more[i] = o.more[i][3];
+            p.cell_more[i] = o.more[i][4]; p.d_ifgo_more[i] = o.more[i][5]; p.Wh_more[i] = o.more[i][6];
+        }
         p.dh_lo = lower->dh; p.dc_lo = lower->dc; p.ifgo_lo = lower->ifgo; p.cell_lo = lower->cell;
         p.d_ifgo_lo = lower->d_ifgo; p.Wh_lo = lower->Wh;
         p.k5.C = const_cast<void *>(lower->dout);   // the kernel reads the second recurrence's dout from there
@@ -1050,27 +1066,122 @@ int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *if
                             ws, stream);
 }
 
-// Two recurrences of one shape: side by side in one launch of the XCD-local kernels where both fit (returns 0), else
+// n = 2 ... kMaxSideBySide recurrences of one shape (recs[r]: the operand pointers of recurrence r in the order of
+// the single entry point): side by side in one launch of the XCD-local kernels where they all fit (returns 0), else
 // 1 (not launched).
-static int try_pair(bool backward, void *const a[7], void *const b[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
-                    void *stream, int keep, bool dry_run) {
+static int try_multi(bool backward, int n, void *const (*recs)[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                     void *stream, int keep, bool dry_run) {
+    if (n < 2 || n > kMaxSideBySide) return 1;
     fastlstm_plan pl;
     if (int rc = plan_device(-1, B, H, dtype, backward ? 1 : 0, &pl, false)) return rc;
     if (pl.wave_split == 2 || pl.wave_split == 3) return 1;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    void *const *a = recs[0], *const *b = recs[1];
+    LaunchOpts o;
+    o.keep = keep;
+    o.n_more = n - 2;
+    o.more = recs + 2;
     int rc;
     if (!backward) {
         const SecondLayer second{nullptr, nullptr, nullptr, b[3], b[0], b[1], b[2]};
-        const LaunchOpts o{keep, 0, 0};
         rc = try_fwd_xcd(a[0], a[1], a[2], a[3], wsb, ws_bytes, T, B, H, dtype, s, nullptr, nullptr, nullptr, nullptr, 0, &second,
                          dry_run, o);
     } else {
         LowerLayer lower{b[1], b[2], b[3], b[4], b[5], b[6], nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr};
         lower.dout = b[0];
-        rc = try_bwd_xcd(a[0], a[1], a[2], a[3], a[4], a[5], a[6], wsb, ws_bytes, T, B, H, dtype, s, nullptr, &lower, dry_run);
+        rc = try_bwd_xcd(a[0], a[1], a[2], a[3], a[4], a[5], a[6], wsb, ws_bytes, T, B, H, dtype, s, nullptr, &lower, dry_run,
+                         nullptr, o);
     }
     return rc == 2 ? 1 : rc;
+}
+static int try_pair(bool backward, void *const a[7], void *const b[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                    void *stream, int keep, bool dry_run) {
+    void *recs[2][7];
+    for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
+    return try_multi(backward, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, dry_run);
+}
+
+size_t fastlstm_multi_workspace_bytes(const fastlstm_plan *plan, int n, int T, int H, int dtype, int backward) {
+    const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, backward);
+    if (!plan || one == 0 || n <= 1 || plan->wave_split >= 2) return one;
+    const size_t head = kWsHeaderBytes + kWsCounterBytes;
+    return one > head ? head + (size_t)n * (one - head) : one;
+}
+
+int fastlstm_multi_fused(int n, int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    if (n < 1 || n > kMaxSideBySide) return FASTLSTM_ERR_DIM;
+    void *fake[kMaxSideBySide][7];
+    for (auto &r : fake)
+        for (void *&q : r) q = reinterpret_cast<void *>(static_cast<size_t>(4096));   // never dereferenced
+    const int rc = try_multi(backward != 0, n, fake, fake[0][0], ws_bytes, T, B, H, dtype, nullptr, 1, true);
+    return rc == FASTLSTM_OK ? 1 : (rc < 0 ? rc : 0);
+}
+
+// n recurrences one after the other on one workspace, which is cleared in between
+static int multi_sequential(bool backward, int n, void *const (*r)[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
+                            void *stream, int keep) {
+    fastlstm_plan pl;
+    if (int rc = plan_device(-1, B, H, dtype, backward ? 1 : 0, &pl, false)) return rc;
+    const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
+    for (int i = 0; i < n; ++i) {
+        if (i) {
+            zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned *>(ws), zero / 4);
+            if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+        }
+        const int rc = backward ? bwd_persistent_impl(r[i][0], r[i][1], r[i][2], r[i][3], r[i][4], r[i][5], r[i][6], ws, ws_bytes, T, B,
+                                                      H, dtype, stream)
+                                : fwd_persistent_impl(r[i][0], r[i][1], r[i][2], r[i][3], ws, ws_bytes, T, B, H, dtype, stream, keep);
+        if (rc != FASTLSTM_OK) return rc;
+    }
+    return FASTLSTM_OK;
+}
+
+int fastlstm_fwd_persistent_multi(int n, void *const *ifgo, void *const *out, void *const *cell, const void *const *Wh, void *ws,
+                                  size_t ws_bytes, int T, int B, int H, int dtype, int keep_activations, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    if (!ifgo || !out || !cell || !Wh || !ws) return FASTLSTM_ERR_NULL;
+    if (n < 1 || n > kMaxSideBySide) return FASTLSTM_ERR_DIM;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    void *recs[kMaxSideBySide][7] = {};
+    for (int i = 0; i < n; ++i) {
+        recs[i][0] = ifgo[i]; recs[i][1] = out[i]; recs[i][2] = cell[i]; recs[i][3] = const_cast<void *>(Wh[i]);
+        for (int k = 0; k < 4; ++k) {
+            if (!recs[i][k]) return FASTLSTM_ERR_NULL;
+            if (!aligned16(recs[i][k])) return FASTLSTM_ERR_ALIGN;
+        }
+    }
+    if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
+    const int keep = keep_activations ? 1 : 0;
+    int rc = try_multi(false, n, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
+    if (rc == 1) rc = multi_sequential(false, n, recs, ws, ws_bytes, T, B, H, dtype, stream, keep);
+    return finish_recurrent(rc, ws, stream);
+}
+
+int fastlstm_bwd_persistent_multi(int n, const void *const *dout, void *const *dh, void *const *dc, const void *const *ifgo,
+                                  const void *const *cell, void *const *d_ifgo, const void *const *Wh, void *ws, size_t ws_bytes,
+                                  int T, int B, int H, int dtype, void *stream) {
+    if (int rc = take_pending_status()) return rc;
+    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !ws) return FASTLSTM_ERR_NULL;
+    if (n < 1 || n > kMaxSideBySide) return FASTLSTM_ERR_DIM;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, H, H)) return rc;
+    void *recs[kMaxSideBySide][7] = {};
+    for (int i = 0; i < n; ++i) {
+        recs[i][0] = const_cast<void *>(dout[i]); recs[i][1] = dh[i]; recs[i][2] = dc[i]; recs[i][3] = const_cast<void *>(ifgo[i]);
+        recs[i][4] = const_cast<void *>(cell[i]); recs[i][5] = d_ifgo[i]; recs[i][6] = const_cast<void *>(Wh[i]);
+        for (int k = 0; k < 7; ++k) {
+            if (!recs[i][k]) return FASTLSTM_ERR_NULL;
+            if (!aligned16(recs[i][k])) return FASTLSTM_ERR_ALIGN;
+        }
+    }
+    if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
+    int rc = try_multi(true, n, recs, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
+    if (rc == 1) rc = multi_sequential(true, n, recs, ws, ws_bytes, T, B, H, dtype, stream, 1);
+    return finish_recurrent(rc, ws, stream);
 }
 
 int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {

@@ -71,6 +71,9 @@ struct BwdXcdParams {
     int k8_lo_tiles_n, wg_lo_tiles;
     float *wg_scratch_lo;
     long long spin_limit;
+    // Without helpers, n_layers = 3 or 4 independent recurrences: recurrence r >= 2 is described by entry r - 2.
+    const void *dout_more[2], *ifgo_more[2], *cell_more[2], *Wh_more[2];
+    void *dh_more[2], *dc_more[2], *d_ifgo_more[2];
     unsigned char *partials;   // lstm_bwd_wide_split_kernel: the teams' partial sums (see there)
 };
 
@@ -300,7 +303,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over the layers of the launch
     // two recurrences in the launch: a stack (HELP == 2), or two independent ones of the same shape side by side
     // (HELP == 0 with n_layers == 2: the two directions of a bidirectional layer; `lower` is then simply the second)
-    const int n_layers = HELP == 2 ? 2 : (HELP == 0 && p.n_layers > 1 ? 2 : 1);
+    const int n_layers = HELP == 2 ? 2 : (HELP == 0 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP != 0) {
             if (p.k5_tiles_n > 0) bwd_helper<T, HELP == 2>(p, smem);
@@ -308,9 +311,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         return;
     }
     check_xcd_placement(p.hdr);
-    const bool lower = n_layers == 2 && vg >= p.n_groups;   // the lower layer of a stack (see BwdXcdParams::n_layers)
+    const int rec = vg / p.n_groups;                        // which recurrence of the launch
+    const bool lower = rec == 1;                            // the lower layer of a stack (see BwdXcdParams::n_layers)
     const bool follows = HELP == 2 && lower;                // ... whose dout the helpers produce during the launch
-    const int g = lower ? vg - p.n_groups : vg;
+    const int g = vg - rec * p.n_groups;
+    const int more = rec >= 2 ? rec - 2 : 0;
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k5_live = HELP && p.k5_tiles_n > 0;
     int *chunk_done = lower ? p.chunk_done_lo : p.chunk_done;
@@ -329,12 +334,13 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
     const int io_tid = tid - kWave;
 
-    const T *dout = static_cast<const T *>(lower ? p.k5.C : p.dout);
-    const T *ifgo = static_cast<const T *>(lower ? p.ifgo_lo : p.ifgo);
-    const T *cell = static_cast<const T *>(lower ? p.cell_lo : p.cell);
-    T *d_ifgo = static_cast<T *>(lower ? p.d_ifgo_lo : p.d_ifgo);
-    const T *Wh = static_cast<const T *>(lower ? p.Wh_lo : p.Wh);
-    T *dh_state = static_cast<T *>(lower ? p.dh_lo : p.dh), *dc_state_buf = static_cast<T *>(lower ? p.dc_lo : p.dc);
+    const T *dout = static_cast<const T *>(rec == 0 ? p.dout : lower ? p.k5.C : p.dout_more[more]);
+    const T *ifgo = static_cast<const T *>(rec == 0 ? p.ifgo : lower ? p.ifgo_lo : p.ifgo_more[more]);
+    const T *cell = static_cast<const T *>(rec == 0 ? p.cell : lower ? p.cell_lo : p.cell_more[more]);
+    T *d_ifgo = static_cast<T *>(rec == 0 ? p.d_ifgo : lower ? p.d_ifgo_lo : p.d_ifgo_more[more]);
+    const T *Wh = static_cast<const T *>(rec == 0 ? p.Wh : lower ? p.Wh_lo : p.Wh_more[more]);
+    T *dh_state = static_cast<T *>(rec == 0 ? p.dh : lower ? p.dh_lo : p.dh_more[more]);
+    T *dc_state_buf = static_cast<T *>(rec == 0 ? p.dc : lower ? p.dc_lo : p.dc_more[more]);
 
     // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
     // fragment (unit tile a, k-step ks): lane (q, r) holds row r = unit u0 + 16a + r and

@@ -30,6 +30,7 @@
 namespace fastlstm {
 
 constexpr int kAuxDevice = 16;  // buffer-instruction cache policy: sc1 = device scope
+constexpr int kMaxSideBySide = 4;   // independent recurrences of one shape in one launch of the XCD-local kernels
 
 // Exchange buffer in global memory, addressed through a buffer resource so that the
 // 16-byte operand loads can carry the device-scope cache policy.

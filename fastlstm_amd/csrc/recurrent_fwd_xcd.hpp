@@ -67,6 +67,11 @@ struct FwdXcdParams {
     int n_layers;
     void *ifgo2, *out2, *cell2;
     const void *Wh2;
+    // Without helpers n_layers = 2 ... kMaxSideBySide independent recurrences of one shape share the launch (the two
+    // directions of a bidirectional layer; the chunks of a wavefront over stacked layers): recurrence r >= 2 is
+    // described by the r - 2-th entries here.
+    void *ifgo_more[2], *out_more[2], *cell_more[2];
+    const void *Wh_more[2];
     GemmParams k1b;       // M = T*B, N = 4H, K = H, A = out[1:] of the first layer, B = Wx2, C = ifgo2, biases
     int *k1_done2;        // chunk counters of the second projection
     int *out_ready;       // [<= kMaxChunks] device-scope counters, zero at launch
@@ -259,7 +264,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over all layers of the launch
     // (without helpers n_layers == 2 means two independent recurrences of the same shape side by side: the two
     // directions of a bidirectional layer; nothing links them)
-    const int n_layers = p.n_layers > 1 ? 2 : 1;
+    const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : max(1, min(p.n_layers, kMaxSideBySide));
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
             if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);
@@ -282,10 +287,11 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + 4 * TILES * kWave);   // gates, h, c tiles
     const int io_tid = tid - kWave;
 
-    T *ifgo = static_cast<T *>(layer ? p.ifgo2 : p.ifgo);
-    T *out = static_cast<T *>(layer ? p.out2 : p.out);
-    T *cell = static_cast<T *>(layer ? p.cell2 : p.cell);
-    const T *Wh = static_cast<const T *>(layer ? p.Wh2 : p.Wh);
+    const int more = layer >= 2 ? layer - 2 : 0;
+    T *ifgo = static_cast<T *>(layer == 0 ? p.ifgo : layer == 1 ? p.ifgo2 : p.ifgo_more[more]);
+    T *out = static_cast<T *>(layer == 0 ? p.out : layer == 1 ? p.out2 : p.out_more[more]);
+    T *cell = static_cast<T *>(layer == 0 ? p.cell : layer == 1 ? p.cell2 : p.cell_more[more]);
+    const T *Wh = static_cast<const T *>(layer == 0 ? p.Wh : layer == 1 ? p.Wh2 : p.Wh_more[more]);
 
 #ifdef FASTLSTM_TIMELINE
     long long *tl = reinterpret_cast<long long *>(tiles + BT * GROW + 2 * BT * SROW + 64);

@@ -15,6 +15,7 @@ gfx950 kernels) on the current HIP stream.  There is one code path, no Triton,
 no autotune warm-up run and no CPU fallback: tensors must live on the GPU and
 the library must be built, otherwise the calls raise.
 """
+import ctypes
 import functools
 import os
 
@@ -173,25 +174,41 @@ def _aligned(t):
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+def multi_runs_in_one_launch(n, T, B, H, dtype, device, backward=False):
+    """True if n independent recurrences of this shape run as one launch (fastlstm_multi_fused)."""
+    if dtype not in _DTYPE_CODE or torch.device(device).type != "cuda":
+        return False
+    lib = _lib.load()
+    code = _DTYPE_CODE[dtype]
+    with torch.cuda.device(device):
+        plan = _plan(torch.device(device), B, H, code, backward)
+        nb = lib.fastlstm_multi_workspace_bytes(plan, n, T, H, code, int(backward))
+        return lib.fastlstm_multi_fused(n, T, B, H, code, int(backward), nb) == 1
+
+
 @functools.lru_cache(maxsize=512)
-def _wavefront_chunks(T, B, H, dtype, device, backward):
+def _wavefront_chunks(L, T, B, H, dtype, device, backward):
     # chunks of at least 64 timesteps: every launch costs about 50 us besides its steps (launch gaps, the prologue,
-    # the small GEMM in between), which a chunk of 32 steps does not win back (measured: no gain at T = 256 with
+    # the small GEMMs in between), which a chunk of 32 steps does not win back (measured: no gain at T = 256 with
     # 8 chunks); whole 16-byte units per timestep, so that every chunk's buffers start on a 16-byte boundary
     if T < 256 or (B * H * torch.empty((), dtype=dtype).element_size()) % 16:
         return 0
     for n in (8, 6, 5, 4, 3, 2):
-        if T % n == 0 and T // n >= 64 and pair_runs_in_one_launch(T // n, B, H, dtype, device, backward):
+        if T % n == 0 and T // n >= 64 and multi_runs_in_one_launch(L, T // n, B, H, dtype, device, backward):
             return n
     return 0
 
 
+def stack_wavefront_chunks(L, T, B, H, dtype, device, backward=False):
+    """Into how many chunks of timesteps L = 2 ... 4 stacked layers of this shape are cut so that layer l's chunk
+    k - l runs beside the other layers' in launch k (0: they are not): the shapes whose L time loops fit the device
+    side by side (multi_runs_in_one_launch)."""
+    return _wavefront_chunks(int(L), int(T), int(B), int(H), dtype, str(torch.device(device)), bool(backward))
+
+
 def stack2_wavefront_chunks(T, B, H, dtype, device, backward=False):
-    """Into how many chunks of timesteps two stacked layers of this shape are cut so that the upper layer's chunk
-    k - 1 and the lower layer's chunk k run side by side in one launch (0: they are not).  For the shapes whose
-    two time loops fit the device side by side (pair_runs_in_one_launch) but which the library's own two-layer
-    launch (stack2_runs_in_one_launch) does not take."""
-    return _wavefront_chunks(int(T), int(B), int(H), dtype, str(torch.device(device)), bool(backward))
+    """stack_wavefront_chunks for two layers."""
+    return stack_wavefront_chunks(2, T, B, H, dtype, device, backward)
 
 
 def _small_projections(B, I, H):
@@ -213,22 +230,28 @@ def _chunk_workspaces(n_bytes, zero_bytes, count, device):
     return [buf[k * stride:k * stride + n_bytes] for k in range(count)]
 
 
-def _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, n, keep_activations):
-    """lstm_persistent_fwd_stack2 as n + 1 launches: launch k runs chunk k of the lower layer's time loop and chunk
-    k - 1 of the upper layer's side by side (fastlstm_fwd_persistent_pair on sub-ranges of the buffers: a time
-    loop started at out[t0], cell[t0] continues the sequence); the upper layer's input projection of a chunk is a
-    GEMM launch in between.  (A chunk starts from the stored cell state, where the one-launch loop carries it in
-    fp32: with 16-bit elements the results differ from the layer-by-layer path by that rounding, once per chunk.)"""
+def _ptr_array(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+
+def _fwd_stack_wavefront(x, layers, n, keep_activations):
+    """L = len(layers) stacked layers, layers[l] = (h0, c0, Wx, bx, Wh, bh), as n + L - 1 launches: launch k runs
+    chunk k - l of layer l's time loop for every l side by side (fastlstm_fwd_persistent_multi on sub-ranges of the
+    buffers: a time loop started at out[t0], cell[t0] continues the sequence); the input projection of an upper
+    layer's chunk is a GEMM launch in between.  Returns [(out, cell, ifgo)] per layer.  (A chunk starts from the
+    stored cell state, where the one-launch loop carries it in fp32: with 16-bit elements the results differ from
+    the layer-by-layer path by that rounding, once per chunk.)"""
     lib = _lib.load()
     code = _code(x)
     T, B, I = x.shape
-    H = Wh0.shape[1]
+    H = layers[0][4].shape[1]
+    L = len(layers)
     Tc = T // n
     dev_ = x.device
     stream = _stream()
     p = lambda t: t.data_ptr()
     bufs = []
-    for h0, c0 in ((h0a, c0a), (h0b, c0b)):
+    for h0, c0, *_ in layers:
         ifgo = torch.empty((T, B, 4 * H), device=dev_, dtype=x.dtype)
         out = torch.empty((T + 1, B, H), device=dev_, dtype=x.dtype)
         cell = torch.empty_like(out)
@@ -239,84 +262,148 @@ def _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, W
             out[0].zero_()
             cell[0].zero_()
         bufs.append((out, cell, ifgo))
-    (out0, cell0, ifgo0), (out1, cell1, ifgo1) = bufs
-    _lib.check(lib.fastlstm_gemm_ifgo(p(x), p(Wx0), p(bx0), p(bh0), p(ifgo0), T, B, I, H, code, stream), "fastlstm_gemm_ifgo")
+    Wx0, bx0, bh0 = layers[0][2], layers[0][3], layers[0][5]
+    _lib.check(lib.fastlstm_gemm_ifgo(p(x), p(Wx0), p(bx0), p(bh0), p(bufs[0][2]), T, B, I, H, code, stream), "fastlstm_gemm_ifgo")
     plan = _plan(dev_, B, H, code, False)
-    nb = lib.fastlstm_stack2_workspace_bytes(plan, Tc, H, code)
-    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + 1, dev_)
+    nb = lib.fastlstm_multi_workspace_bytes(plan, L, Tc, H, code, 0)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1, dev_)
     keep = int(keep_activations)
     # (addresses of the chunks by arithmetic: slicing tensors would cost the host more than a short chunk runs)
     row = B * H * x.element_size()
-    g0, o0, c0_, g1, o1, c1_ = (p(t) for t in (ifgo0, out0, cell0, ifgo1, out1, cell1))
-    pWx1, pbx1, pbh1, pWh0, pWh1 = p(Wx1), p(bx1), p(bh1), p(Wh0), p(Wh1)
-    for k in range(n + 1):
-        ws, ta, tb = wss[k], k * Tc, (k - 1) * Tc
-        if k >= 1:   # the upper layer's projection of the chunk the lower layer has just finished
-            _lib.check(lib.fastlstm_gemm_ifgo(o0 + (1 + tb) * row, pWx1, pbx1, pbh1, g1 + tb * 4 * row, Tc, B, H, H, code, stream),
-                       "fastlstm_gemm_ifgo")
-        if 1 <= k < n:
-            _lib.check(lib.fastlstm_fwd_persistent_pair(g0 + ta * 4 * row, o0 + ta * row, c0_ + ta * row, pWh0, g1 + tb * 4 * row,
-                                                        o1 + tb * row, c1_ + tb * row, pWh1, p(ws), ws.numel(), Tc, B, H,
-                                                        code, keep, stream), "fastlstm_fwd_persistent_pair")
-        elif k == 0:
-            _lib.check(lib.fastlstm_fwd_persistent(g0, o0, c0_, pWh0, p(ws), ws.numel(), Tc, B, H, code, stream),
-                       "fastlstm_fwd_persistent")
-        else:
-            _lib.check(lib.fastlstm_fwd_persistent(g1 + tb * 4 * row, o1 + tb * row, c1_ + tb * row, pWh1, p(ws), ws.numel(),
-                                                   Tc, B, H, code, stream), "fastlstm_fwd_persistent")
+    po, pc, pg = [p(b[0]) for b in bufs], [p(b[1]) for b in bufs], [p(b[2]) for b in bufs]
+    pw = [(p(l[2]), p(l[3]), p(l[4]), p(l[5])) for l in layers]   # Wx, bx, Wh, bh
+    for k in range(n + L - 1):
+        active = [l for l in range(L) if 0 <= k - l < n]
+        for l in active:
+            if l >= 1:   # this layer's projection of the chunk the layer below has just finished
+                t = (k - l) * Tc
+                _lib.check(lib.fastlstm_gemm_ifgo(po[l - 1] + (1 + t) * row, pw[l][0], pw[l][1], pw[l][3], pg[l] + t * 4 * row,
+                                                  Tc, B, H, H, code, stream), "fastlstm_gemm_ifgo")
+        t_of = [(k - l) * Tc for l in active]
+        ws = wss[k]
+        _lib.check(lib.fastlstm_fwd_persistent_multi(
+            len(active), _ptr_array([pg[l] + t * 4 * row for l, t in zip(active, t_of)]),
+            _ptr_array([po[l] + t * row for l, t in zip(active, t_of)]), _ptr_array([pc[l] + t * row for l, t in zip(active, t_of)]),
+            _ptr_array([pw[l][2] for l in active]), p(ws), ws.numel(), Tc, B, H, code, keep, stream), "fastlstm_fwd_persistent_multi")
     for ws in wss:
-        _check_ws(ws, "fastlstm_fwd_persistent_pair")
+        _check_ws(ws, "fastlstm_fwd_persistent_multi")
+    return bufs
+
+
+def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
+    """Reverse pass of _fwd_stack_wavefront: acts[l] = (out, cell, ifgo), weights[l] = (Wx, Wh), d_states[l] = None or
+    (dh_n, dc_n).  Launch k runs chunk n - 1 - (k - u) of layer L - 1 - u for every u side by side; a lower layer's
+    dout of a chunk (the dx of the layer above) is a GEMM launch in between; the weight gradients and the lowest
+    layer's dx follow over the whole sequence.  Returns [(d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)] per layer."""
+    lib = _lib.load()
+    L = len(acts)
+    code = _code(acts[0][2])
+    T, B, H = dh.shape
+    I = weights[0][0].shape[1]
+    Tc = T // n
+    dev_ = x.device
+    dt = acts[0][2].dtype
+    stream = _stream()
+    p = lambda t: t.data_ptr()
+    dh = dh.contiguous()
+    if dh.dtype != dt:
+        dh = dh.to(dt)
+    dh, x = _aligned(dh), _aligned(x.contiguous())
+    state = lambda d, k: (torch.zeros((B, H), device=dev_, dtype=dt) if d is None else d[k].to(dt).reshape(B, H).clone())
+    dhs, dcs = [state(d, 0) for d in d_states], [state(d, 1) for d in d_states]
+    d_ifgo = [torch.empty_like(a[2]) for a in acts]
+    # douts[l]: gradient of layer l's out[1:]: dh for the top layer, the dx of layer l + 1 below it
+    douts = [torch.empty((T, B, H), device=dev_, dtype=dt) for _ in range(L - 1)] + [dh]
+    plan = _plan(dev_, B, H, code, True)
+    nb = lib.fastlstm_multi_workspace_bytes(plan, L, Tc, H, code, 1)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1, dev_)
+    row = B * H * dh.element_size()
+    pdo, pdg = [p(t) for t in douts], [p(t) for t in d_ifgo]
+    pg, pc = [p(a[2]) for a in acts], [p(a[1]) for a in acts]
+    Wxc = [w[0].contiguous() for w in weights]
+    pWx, pWh = [p(w) for w in Wxc], [p(w[1]) for w in weights]
+    pdh, pdc = [p(t) for t in dhs], [p(t) for t in dcs]
+    for k in range(n + L - 1):
+        active = [L - 1 - u for u in range(L) if 0 <= k - u < n]          # layers, top first
+        t_of = [(n - 1 - (k - (L - 1 - l))) * Tc for l in active]
+        for l, t in zip(active, t_of):
+            if l < L - 1:   # this layer's dout of the chunk the layer above has just finished
+                _lib.check(lib.fastlstm_gemm_dx(pdg[l + 1] + t * 4 * row, pWx[l + 1], pdo[l] + t * row, Tc, B, H, H, code, stream),
+                           "fastlstm_gemm_dx")
+        ws = wss[k]
+        _lib.check(lib.fastlstm_bwd_persistent_multi(
+            len(active), _ptr_array([pdo[l] + t * row for l, t in zip(active, t_of)]), _ptr_array([pdh[l] for l in active]),
+            _ptr_array([pdc[l] for l in active]), _ptr_array([pg[l] + t * 4 * row for l, t in zip(active, t_of)]),
+            _ptr_array([pc[l] + t * row for l, t in zip(active, t_of)]), _ptr_array([pdg[l] + t * 4 * row for l, t in zip(active, t_of)]),
+            _ptr_array([pWh[l] for l in active]), p(ws), ws.numel(), Tc, B, H, code, stream), "fastlstm_bwd_persistent_multi")
+    for ws in wss:
+        _check_ws(ws, "fastlstm_bwd_persistent_multi")
+    dx0 = torch.empty_like(x)
+    _lib.check(lib.fastlstm_gemm_dx(pdg[0], pWx[0], p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
+    res = []
+    for l in range(L):
+        xin = x if l == 0 else acts[l - 1][0][1:]
+        db, _, dWx, dWh = Wgrad(d_ifgo[l], xin, acts[l][0])
+        res.append((dx0 if l == 0 else douts[l - 1], dhs[l], dcs[l], dWx, db, dWh, db))
+    return res
+
+
+def _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, n, keep_activations):
+    (out0, cell0, ifgo0), (out1, cell1, ifgo1) = _fwd_stack_wavefront(
+        x, [(h0a, c0a, Wx0, bx0, Wh0, bh0), (h0b, c0b, Wx1, bx1, Wh1, bh1)], n, keep_activations)
     return out0, cell0, ifgo0, out1, cell1, ifgo1
 
 
 def _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1, n):
-    """lstm_persistent_bwd_stack2 as n + 1 launches (see _fwd_stack2_wavefront): launch k runs the upper layer's
-    chunk n - 1 - k and the lower layer's chunk n - k of the reverse time loops side by side; the lower layer's dout
-    of a chunk (the upper layer's dx) is a GEMM launch in between; the weight gradients and the lower layer's dx
-    follow over the whole sequence."""
-    lib = _lib.load()
-    code = _code(ifgo1)
+    r0, r1 = _bwd_stack_wavefront(dh, x, [(out0, cell0, ifgo0), (out1, cell1, ifgo1)], [(Wx0, Wh0), (Wx1, Wh1)],
+                                  [d_state0, d_state1], n)
+    return r0, r1
+
+
+def lstm_persistent_fwd_stack(x, layers, keep_activations=True):
+    """L = 2 ... 4 stacked layers, layers[l] = (h0 | None, c0 | None, Wx, bx, Wh, bh): [(out, cell, ifgo)] per layer,
+    the results of L calls of lstm_persistent_fwd in a row (16-bit elements: up to the rounding of the cell state at
+    chunk boundaries, see _fwd_stack_wavefront).  Needs stack_wavefront_chunks(L, ...) > 0."""
+    if x.dim() == 2:
+        x = x[None]
+    _require_gpu(x, *(t for l in layers for t in l))
+    T, B, I = x.shape
+    H = layers[0][4].shape[1]
+    assert x.is_contiguous()
+    for l, (_, _, Wx, bx, Wh, bh) in enumerate(layers):
+        assert Wx.shape == (4 * H, I if l == 0 else H) and Wh.shape == (4 * H, H) and Wh.is_contiguous()
+        for w in (Wx, bx, Wh, bh):
+            if w.dtype != x.dtype:
+                raise TypeError("weights must have the dtype of x (%s), got %s" % (x.dtype, w.dtype))
+    layers = [(h0, c0, Wx.contiguous(), bx.contiguous(), Wh, bh.contiguous()) for h0, c0, Wx, bx, Wh, bh in layers]
+    with torch.cuda.device(x.device):
+        n = stack_wavefront_chunks(len(layers), T, B, H, x.dtype, x.device)
+        if not n:
+            raise ValueError("no wavefront for %d layers of this shape" % len(layers))
+        return _fwd_stack_wavefront(_aligned(x), layers, n, keep_activations)
+
+
+def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
+    """Reverse pass of lstm_persistent_fwd_stack: acts[l] = (out, cell, ifgo), weights[l] = (Wx, Wh), d_states[l] = None
+    or (dh_n, dc_n).  [(d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)] per layer; falls back to one layer after the other where
+    the reverse time loops do not fit side by side."""
+    L = len(acts)
+    d_states = list(d_states) if d_states is not None else [None] * L
     T, B, H = dh.shape
-    I = Wx0.shape[1]
-    Tc = T // n
-    dev_ = x.device
-    stream = _stream()
-    p = lambda t: t.data_ptr()
-    dh = dh.contiguous()
-    if dh.dtype != ifgo1.dtype:
-        dh = dh.to(ifgo1.dtype)
-    dh, x = _aligned(dh), _aligned(x.contiguous())
-    zeros = lambda: torch.zeros((B, H), device=dev_, dtype=x.dtype)
-    state = lambda d, k: zeros() if d is None else d[k].to(x.dtype).reshape(B, H).clone()
-    dh1, dc1, dh0, dc0 = state(d_state1, 0), state(d_state1, 1), state(d_state0, 0), state(d_state0, 1)
-    d_ifgo1, d_ifgo0 = torch.empty_like(ifgo1), torch.empty_like(ifgo0)
-    dx1 = torch.empty((T, B, H), device=dev_, dtype=x.dtype)
-    plan = _plan(dev_, B, H, code, True)
-    nb = lib.fastlstm_stack2_bwd_workspace_bytes(plan, Tc, H, code)
-    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + 1, dev_)
-    Wx1c = Wx1.contiguous()
-    row = B * H * x.element_size()
-    pdh, pdx1, g1, c1_, dg1, g0, c0_, dg0 = (p(t) for t in (dh, dx1, ifgo1, cell1, d_ifgo1, ifgo0, cell0, d_ifgo0))
-    pdh1, pdc1, pdh0, pdc0, pWx1, pWh1, pWh0 = (p(t) for t in (dh1, dc1, dh0, dc0, Wx1c, Wh1, Wh0))
-    for k in range(n + 1):
-        ws, t1, t0 = wss[k], (n - 1 - k) * Tc, (n - k) * Tc
-        if k >= 1:   # the lower layer's dout of the chunk the upper layer has just finished
-            _lib.check(lib.fastlstm_gemm_dx(dg1 + t0 * 4 * row, pWx1, pdx1 + t0 * row, Tc, B, H, H, code, stream), "fastlstm_gemm_dx")
-        upper = (pdh + t1 * row, pdh1, pdc1, g1 + t1 * 4 * row, c1_ + t1 * row, dg1 + t1 * 4 * row, pWh1)
-        lower = (pdx1 + t0 * row, pdh0, pdc0, g0 + t0 * 4 * row, c0_ + t0 * row, dg0 + t0 * 4 * row, pWh0)
-        if 1 <= k < n:
-            _lib.check(lib.fastlstm_bwd_persistent_pair(*upper, *lower, p(ws), ws.numel(), Tc, B, H, code, stream),
-                       "fastlstm_bwd_persistent_pair")
-        else:
-            _lib.check(lib.fastlstm_bwd_persistent(*(upper if k == 0 else lower), p(ws), ws.numel(), Tc, B, H, code, stream),
-                       "fastlstm_bwd_persistent")
-    for ws in wss:
-        _check_ws(ws, "fastlstm_bwd_persistent_pair")
-    dx0 = torch.empty_like(x)
-    _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo0), p(Wx0.contiguous()), p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
-    db1, _, dWx1, dWh1 = Wgrad(d_ifgo1, out0[1:], out1)
-    db0, _, dWx0, dWh0 = Wgrad(d_ifgo0, x, out0)
-    return (dx0, dh0, dc0, dWx0, db0, dWh0, db0), (dx1, dh1, dc1, dWx1, db1, dWh1, db1)
+    with torch.cuda.device(x.device):
+        n = stack_wavefront_chunks(L, T, B, H, acts[0][2].dtype, x.device, backward=True)
+        if n:
+            return _bwd_stack_wavefront(dh, x, acts, weights, d_states, n)
+        res = [None] * L
+        for l in range(L - 1, -1, -1):
+            out, cell, ifgo = acts[l]
+            dt = ifgo.dtype
+            zeros = lambda: torch.zeros((B, H), device=x.device, dtype=dt)
+            dhn, dcn = (zeros(), zeros()) if d_states[l] is None else tuple(d.to(dt).reshape(B, H).clone() for d in d_states[l])
+            xin = x if l == 0 else acts[l - 1][0][1:]
+            res[l] = lstm_persistent_bwd(dh, dcn, dhn, xin, out, cell, ifgo, weights[l][0], weights[l][1])
+            dh = res[l][0]
+        return res
 
 
 def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, keep_activations=True):
@@ -713,6 +800,58 @@ class PersistentLSTMPairfn(torch.autograd.Function):
         return (*ga, *gb, None)
 
 
+class PersistentLSTMStackfn(torch.autograd.Function):
+    """L = 2 ... 4 stacked layers as one autograd node, run as a wavefront of chunked launches
+    (lstm_persistent_fwd_stack / lstm_persistent_bwd_stack).  apply(x, state_grads, L, *flat) with flat = (h_0, c_0,
+    Wx, bx, Wh, bh) per layer -> (out of the top layer, h_T, c_T of layer 0, h_T, c_T of layer 1, ...); the final
+    states carry a gradient only with state_grads."""
+
+    @staticmethod
+    @custom_fwd(device_type="cuda")
+    def forward(ctx, x, state_grads, L, *flat):
+        layers = []
+        for l in range(L):
+            h0, c0, Wx, bx, Wh, bh = flat[6 * l:6 * l + 6]
+            layers.append((h0, c0) + tuple(_autocast_operands(Wx, bx, Wh, bh)))
+        (x,) = _autocast_operands(x)
+        if x.dim() == 2:
+            x = x[None]
+        acts = lstm_persistent_fwd_stack(x, layers)
+        ctx.L = L
+        ctx.no_state = [l[0] is None for l in layers]
+        saved = [x]
+        for (out, cell, ifgo), (_, _, Wx, _, Wh, _) in zip(acts, layers):
+            saved += [out, cell, ifgo, Wx, Wh]
+        ctx.save_for_backward(*saved)
+        finals = []
+        for out, cell, _ in acts:
+            finals += [out[-1].clone(), cell[-1].clone()]
+        if not state_grads:
+            ctx.mark_non_differentiable(*finals)
+        return (acts[-1][0][1:], *finals)
+
+    @staticmethod
+    @custom_bwd(device_type="cuda")
+    def backward(ctx, dh, *d_finals):
+        L = ctx.L
+        x, rest = ctx.saved_tensors[0], ctx.saved_tensors[1:]
+        acts = [tuple(rest[5 * l:5 * l + 3]) for l in range(L)]
+        weights = [tuple(rest[5 * l + 3:5 * l + 5]) for l in range(L)]
+        zero = lambda: torch.zeros_like(acts[0][1][0])
+        d_states = []
+        for l in range(L):
+            h, c = d_finals[2 * l], d_finals[2 * l + 1]
+            d_states.append(None if h is None and c is None else (zero() if h is None else h, zero() if c is None else c))
+        res = lstm_persistent_bwd_stack(dh, x, acts, weights, d_states)
+        grads = [res[0][0], None, None]
+        for l in range(L):
+            _, dh0, dc0, dWx, dbx, dWh, dbh = res[l]
+            if ctx.no_state[l]:
+                dh0 = dc0 = None
+            grads += [dh0, dc0, dWx, dbx, dWh, dbh]
+        return tuple(grads)
+
+
 class PersistentLSTMStack2fn(torch.autograd.Function):
     """Two stacked layers as one autograd node: forward through lstm_persistent_fwd_stack2, backward
     through lstm_persistent_bwd_stack2 (one launch each where the shapes allow).  Same
@@ -895,6 +1034,30 @@ class FastLSTM(nn.Module):
             return F.dropout(y, drop, True) if drop > 0.0 and done < self.num_layers else y
 
         while layer < self.num_layers:
+            # three or four layers at a time as a wavefront of chunked launches where their time loops fit the
+            # device side by side
+            width = min(self.num_layers - layer, 4)
+            if directions == 1 and drop == 0.0 and width >= 3 and x.dim() == 3 and x.is_cuda:
+                dt_ = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
+                while width >= 3 and not stack_wavefront_chunks(width, x.shape[0], x.shape[1], self.hidden_size, dt_, x.device):
+                    width -= 1
+                if width >= 3:
+                    flat = []
+                    for l in range(layer, layer + width):
+                        flat += [h_0[l], c_0[l], *self._layer_operands(l)]
+                    if inference:
+                        xi, = _autocast_operands(x.contiguous())
+                        ls = [(flat[6 * i], flat[6 * i + 1]) + tuple(_autocast_operands(*flat[6 * i + 2:6 * i + 6])) for i in range(width)]
+                        acts = lstm_persistent_fwd_stack(xi, ls, keep_activations=False)
+                        x = acts[-1][0][1:]
+                        h_n += [a[0][-1] for a in acts]
+                        c_n += [a[1][-1] for a in acts]
+                    else:
+                        x, *finals = PersistentLSTMStackfn.apply(x.contiguous(), self.state_grads, width, *flat)
+                        h_n += finals[0::2]
+                        c_n += finals[1::2]
+                    layer += width
+                    continue
             # two layers at a time where the library runs them as one launch (the second layer's
             # recurrence a chunk of timesteps behind the first); the results do not depend on it
             if (directions == 1 and drop == 0.0 and layer + 1 < self.num_layers and x.dim() == 3 and x.is_cuda

@@ -196,6 +196,23 @@ int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, con
                                  void *stream);
 int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
+/* The same for n = 1 ... 4 independent recurrences of one shape, their operands as arrays of n pointers (entry r of
+ * each array belongs to recurrence r): the chunks of a wavefront over stacked layers -- launch k runs layer l's
+ * chunk k - l of timesteps for every layer l, a time loop started at out[t0] / cell[t0] continuing the sequence --
+ * which spreads the layer loop of fastlstm/lstm.py:685-696 (README.md:94: "doesn't exploit num_layer
+ * parallelisation") over the device.  One launch where n x the groups of one recurrence fit the XCDs
+ * (fastlstm_multi_fused), else one recurrence after the other.  ws: fastlstm_multi_workspace_bytes (the exchange
+ * slots of n recurrences), zeroed like any recurrent workspace. */
+int fastlstm_fwd_persistent_multi(int n, void *const *ifgo, void *const *out, void *const *cell,
+                                  const void *const *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
+                                  int dtype, int keep_activations, void *stream);
+int fastlstm_bwd_persistent_multi(int n, const void *const *dout, void *const *dh, void *const *dc,
+                                  const void *const *ifgo, const void *const *cell, void *const *d_ifgo,
+                                  const void *const *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
+                                  int dtype, void *stream);
+int fastlstm_multi_fused(int n, int T, int B, int H, int dtype, int backward, size_t ws_bytes);
+size_t fastlstm_multi_workspace_bytes(const fastlstm_plan *plan, int n, int T, int H, int dtype, int backward);
+
 /* K4 + K5 + K6..K9 for one layer in one call: the same results as fastlstm_bwd_persistent,
  * fastlstm_gemm_dx and fastlstm_gemm_wgrad one after the other (same arguments and workspace
  * contracts; dWx and dWh to the rounding of a different summation order).  Where the XCD-local

@@ -871,6 +871,62 @@ def test_two_layers_as_a_wavefront_of_chunked_pair_launches(T, B, I, H, dt):
             assert rel_err(a, npy(b)) < tol, (side, name)
 
 
+@pytest.mark.parametrize("L_,T,B,I,H,dt", [(4, 256, 16, 64, 256, torch.float32), (3, 256, 16, 96, 384, torch.float16),
+                                           (4, 320, 32, 64, 256, torch.bfloat16)])
+def test_three_and_four_layers_as_a_wavefront(L_, T, B, I, H, dt):
+    """lstm_persistent_fwd_stack / lstm_persistent_bwd_stack (launch k runs layer l's chunk k - l for every layer,
+    fastlstm_*_persistent_multi) against the layer-by-layer ops: the same bits with fp32 (weight gradients: another
+    order of the same sums), a tolerance with 16-bit elements (the cell state is rounded at chunk boundaries)."""
+    assert L.stack_wavefront_chunks(L_, T, B, H, dt, "cuda") >= 2 and L.stack_wavefront_chunks(L_, T, B, H, dt, "cuda", backward=True) >= 2
+    tol = FP32_TOL if dt == torch.float32 else HALF_TOL
+    gs = [{k: dev(v, dt) for k, v in make_problem(T, B, I if l == 0 else H, H, seed=51 + l + T).items()} for l in range(L_)]
+    keys = ("h0", "c0", "Wx", "bx", "Wh", "bh")
+    got = L.lstm_persistent_fwd_stack(gs[0]["x"], [tuple(g[k] for k in keys) for g in gs])
+    ref, xin = [], gs[0]["x"]
+    for g in gs:
+        ref.append(L.lstm_persistent_fwd(xin, *(g[k] for k in keys)))
+        xin = ref[-1][0][1:]
+    for l in range(L_):
+        for name, a, b in zip(("out", "cell", "ifgo"), got[l], ref[l]):
+            if dt == torch.float32:
+                assert torch.equal(a, b), (l, name)
+            else:
+                assert rel_err(a, npy(b)) < tol, (l, name)
+    # the reverse pass on the layer-by-layer activations, both ways
+    d_states = [(g["dh_n"], g["dc_n"]) for g in gs]
+    res = L.lstm_persistent_bwd_stack(gs[-1]["dout"], gs[0]["x"], ref, [(g["Wx"], g["Wh"]) for g in gs], d_states)
+    dh = gs[-1]["dout"]
+    for l in range(L_ - 1, -1, -1):
+        g = gs[l]
+        xin = gs[0]["x"] if l == 0 else ref[l - 1][0][1:]
+        want = L.lstm_persistent_bwd(dh, g["dc_n"].clone(), g["dh_n"].clone(), xin, *ref[l], g["Wx"], g["Wh"])
+        for name, a, b in zip(("d_x", "dh_0", "dc_0", "dWx", "dbx", "dWh", "dbh"), res[l], want):
+            assert rel_err(a, npy(b)) < tol, (l, name)
+        dh = want[0]
+
+
+def test_four_layer_module_through_the_wavefront_matches_nn_lstm():
+    T, B, I, H, dt = 256, 16, 48, 256, torch.float16
+    assert L.stack_wavefront_chunks(4, T, B, H, dt, "cuda") >= 2
+    torch.manual_seed(6)
+    m = FastLSTM(I, H, num_layers=5).to("cuda", dt)     # four layers as one wavefront, the fifth alone
+    ref = torch.nn.LSTM(I, H, num_layers=5).to("cuda", dt)
+    ref.load_state_dict(m.state_dict())
+    x = (torch.randn(T, B, I, device="cuda") * 0.5).to(dt).requires_grad_(True)
+    w = torch.randn(T, B, H, device="cuda").to(dt)
+    res = []
+    for mod in (m, ref):
+        x.grad = None
+        out, (h_n, c_n) = mod(x)
+        (out * w).sum().backward()
+        res.append([out.detach(), h_n.detach(), c_n.detach(), x.grad.clone()] + [q.grad.clone() for q in mod.parameters()])
+    for name, a, b in zip(["out", "h_n", "c_n", "dx"] + [n for n, _ in m.named_parameters()], *res):
+        assert rel_err(a, npy(b)) < 3 * HALF_TOL, name
+    with torch.no_grad():
+        out_i, (h_i, c_i) = m(x)
+    assert rel_err(out_i, npy(res[0][0])) < HALF_TOL and rel_err(h_i, npy(res[0][1])) < HALF_TOL
+
+
 @pytest.mark.parametrize("layers,dt", [(2, torch.float16), (3, torch.bfloat16)])
 def test_stacked_module_through_the_wavefront_matches_nn_lstm(layers, dt):
     T, B, I, H = 256, 16, 64, 384
