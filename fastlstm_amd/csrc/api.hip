@@ -315,7 +315,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.n_layers = 1;
     if (second && !x) {   // independent recurrences of this shape side by side (their projections are done)
         const int n = 2 + o.n_more;
-        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
+        if (c.ntw != 1 || n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
         if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
         p.n_layers = n;
         p.ifgo2 = second->ifgo; p.out2 = second->out; p.cell2 = second->cell; p.Wh2 = second->Wh;
@@ -643,7 +643,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.n_layers = 1;
     if (lower && !extras) {   // independent recurrences of this shape side by side
         const int n = 2 + o.n_more;
-        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;
+        if (c.ntw != 1 || n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;
         if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
         p.n_layers = n;
         for (int i = 0; i < o.n_more; ++i) {

@@ -303,7 +303,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over the layers of the launch
     // two recurrences in the launch: a stack (HELP == 2), or two independent ones of the same shape side by side
     // (HELP == 0 with n_layers == 2: the two directions of a bidirectional layer; `lower` is then simply the second)
-    const int n_layers = HELP == 2 ? 2 : (HELP == 0 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
+    // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
+    const int n_layers = HELP == 2 ? 2 : (HELP == 0 && NTW == 1 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP != 0) {
             if (p.k5_tiles_n > 0) bwd_helper<T, HELP == 2>(p, smem);
@@ -315,7 +316,13 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const bool lower = rec == 1;                            // the lower layer of a stack (see BwdXcdParams::n_layers)
     const bool follows = HELP == 2 && lower;                // ... whose dout the helpers produce during the launch
     const int g = vg - rec * p.n_groups;
-    const int more = rec >= 2 ? rec - 2 : 0;
+    // (constant indices only: a run-time index into the kernel's arguments would move them all to scratch memory;
+    // the helper instantiations never see more than two recurrences)
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
+        if constexpr (HELP != 0) return lower ? a1 : a0;
+        else if constexpr (NTW != 1) return a0;
+        else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
+    };
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
     const bool k5_live = HELP && p.k5_tiles_n > 0;
     int *chunk_done = lower ? p.chunk_done_lo : p.chunk_done;
@@ -334,13 +341,13 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * MT * NT * kWave);   // gates, c, dout tiles
     const int io_tid = tid - kWave;
 
-    const T *dout = static_cast<const T *>(rec == 0 ? p.dout : lower ? p.k5.C : p.dout_more[more]);
-    const T *ifgo = static_cast<const T *>(rec == 0 ? p.ifgo : lower ? p.ifgo_lo : p.ifgo_more[more]);
-    const T *cell = static_cast<const T *>(rec == 0 ? p.cell : lower ? p.cell_lo : p.cell_more[more]);
-    T *d_ifgo = static_cast<T *>(rec == 0 ? p.d_ifgo : lower ? p.d_ifgo_lo : p.d_ifgo_more[more]);
-    const T *Wh = static_cast<const T *>(rec == 0 ? p.Wh : lower ? p.Wh_lo : p.Wh_more[more]);
-    T *dh_state = static_cast<T *>(rec == 0 ? p.dh : lower ? p.dh_lo : p.dh_more[more]);
-    T *dc_state_buf = static_cast<T *>(rec == 0 ? p.dc : lower ? p.dc_lo : p.dc_more[more]);
+    const T *dout = static_cast<const T *>(pick(p.dout, static_cast<const void *>(p.k5.C), p.dout_more[0], p.dout_more[1]));
+    const T *ifgo = static_cast<const T *>(pick(p.ifgo, p.ifgo_lo, p.ifgo_more[0], p.ifgo_more[1]));
+    const T *cell = static_cast<const T *>(pick(p.cell, p.cell_lo, p.cell_more[0], p.cell_more[1]));
+    T *d_ifgo = static_cast<T *>(pick(p.d_ifgo, p.d_ifgo_lo, p.d_ifgo_more[0], p.d_ifgo_more[1]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh_lo, p.Wh_more[0], p.Wh_more[1]));
+    T *dh_state = static_cast<T *>(pick(p.dh, p.dh_lo, p.dh_more[0], p.dh_more[1]));
+    T *dc_state_buf = static_cast<T *>(pick(p.dc, p.dc_lo, p.dc_more[0], p.dc_more[1]));
 
     // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
     // fragment (unit tile a, k-step ks): lane (q, r) holds row r = unit u0 + 16a + r and

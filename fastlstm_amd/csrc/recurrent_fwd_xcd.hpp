@@ -264,7 +264,8 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over all layers of the launch
     // (without helpers n_layers == 2 means two independent recurrences of the same shape side by side: the two
     // directions of a bidirectional layer; nothing links them)
-    const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : max(1, min(p.n_layers, kMaxSideBySide));
+    // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
+    const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : (NTW == 1 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
             if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);
@@ -287,11 +288,17 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + 4 * TILES * kWave);   // gates, h, c tiles
     const int io_tid = tid - kWave;
 
-    const int more = layer >= 2 ? layer - 2 : 0;
-    T *ifgo = static_cast<T *>(layer == 0 ? p.ifgo : layer == 1 ? p.ifgo2 : p.ifgo_more[more]);
-    T *out = static_cast<T *>(layer == 0 ? p.out : layer == 1 ? p.out2 : p.out_more[more]);
-    T *cell = static_cast<T *>(layer == 0 ? p.cell : layer == 1 ? p.cell2 : p.cell_more[more]);
-    const T *Wh = static_cast<const T *>(layer == 0 ? p.Wh : layer == 1 ? p.Wh2 : p.Wh_more[more]);
+    // (constant indices only: a run-time index into the kernel's arguments would move them all to scratch memory;
+    // the helper instantiations never see more than two layers)
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
+        if constexpr (HELP) return layer ? a1 : a0;
+        else if constexpr (NTW != 1) return a0;
+        else return layer == 0 ? a0 : layer == 1 ? a1 : layer == 2 ? a2 : a3;
+    };
+    T *ifgo = static_cast<T *>(pick(p.ifgo, p.ifgo2, p.ifgo_more[0], p.ifgo_more[1]));
+    T *out = static_cast<T *>(pick(p.out, p.out2, p.out_more[0], p.out_more[1]));
+    T *cell = static_cast<T *>(pick(p.cell, p.cell2, p.cell_more[0], p.cell_more[1]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh2, p.Wh_more[0], p.Wh_more[1]));
 
 #ifdef FASTLSTM_TIMELINE
     long long *tl = reinterpret_cast<long long *>(tiles + BT * GROW + 2 * BT * SROW + 64);

@@ -1041,6 +1041,12 @@ class FastLSTM(nn.Module):
                 dt_ = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
                 while width >= 3 and not stack_wavefront_chunks(width, x.shape[0], x.shape[1], self.hidden_size, dt_, x.device):
                     width -= 1
+                # where the library runs PAIRS of these layers in one launch with the GEMMs hidden inside, and the
+                # GEMMs are large, pairs win over the whole pass (4 x (T = 1024, B = 32, I = H = 1024): forward +
+                # backward 13.3 ms in pairs, 14.2 four at a time; forward alone 5.3 vs 4.7)
+                if width >= 3 and not _small_projections(x.shape[1], self.hidden_size, self.hidden_size) and \
+                        stack2_runs_in_one_launch(x.shape[0], x.shape[1], x.shape[2], self.hidden_size, dt_, x.device):
+                    width = 0
                 if width >= 3:
                     flat = []
                     for l in range(layer, layer + width):
