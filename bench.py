@@ -48,7 +48,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain
 # copy of known size.  Counters cannot be read from inside this process: the figures are copied from the
 # committed summaries named here (made by `rocprofv3 --pmc ... -- python3 bench.py --stage fwd_layer`).
-TRAFFIC = {"B": (1409.9e6, "profiles/recurrence_lds_l2_B.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
+TRAFFIC = {"B": (1410.1e6, "profiles/recurrence_lds_l2_B.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
 
 
 def physical_cores():
@@ -84,7 +84,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the LSTM recurrence is not sharded across "
-              "GPUs; see DESIGN.md 'How it would shard'); --gpus %d is not supported" % args.gpus,
+              "GPUs: batch rows would be split, with one all-reduce of the weight gradients); "
+              "--gpus %d is not supported" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
 

@@ -1095,13 +1095,6 @@ static int try_multi(bool backward, int n, void *const (*recs)[7], void *ws, siz
     }
     return rc == 2 ? 1 : rc;
 }
-static int try_pair(bool backward, void *const a[7], void *const b[7], void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
-                    void *stream, int keep, bool dry_run) {
-    void *recs[2][7];
-    for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
-    return try_multi(backward, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, dry_run);
-}
-
 size_t fastlstm_multi_workspace_bytes(const fastlstm_plan *plan, int n, int T, int H, int dtype, int backward) {
     const size_t one = fastlstm_recurrent_workspace_bytes(plan, T, H, dtype, backward);
     if (!plan || one == 0 || n <= 1 || plan->wave_split >= 2) return one;
@@ -1185,12 +1178,7 @@ int fastlstm_bwd_persistent_multi(int n, const void *const *dout, void *const *d
 }
 
 int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
-    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
-    if (int rc = check_dims(T, B, H, H)) return rc;
-    void *fake[7];
-    for (void *&q : fake) q = reinterpret_cast<void *>(static_cast<size_t>(4096));   // never dereferenced
-    const int rc = try_pair(backward != 0, fake, fake, fake[0], ws_bytes, T, B, H, dtype, nullptr, 1, true);
-    return rc == FASTLSTM_OK ? 1 : (rc < 0 ? rc : 0);
+    return fastlstm_multi_fused(2, T, B, H, dtype, backward, ws_bytes);
 }
 
 int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const void *Wh_a, void *ifgo_b, void *out_b,
@@ -1205,18 +1193,10 @@ int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const 
         if (!aligned16(a[i]) || !aligned16(b[i])) return FASTLSTM_ERR_ALIGN;
     if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
     const int keep = keep_activations ? 1 : 0;
-    int rc = try_pair(false, a, b, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
-    if (rc == 1) {   // one after the other; the workspace is cleared in between
-        rc = fwd_persistent_impl(ifgo_a, out_a, cell_a, Wh_a, ws, ws_bytes, T, B, H, dtype, stream, keep);
-        if (rc == FASTLSTM_OK) {
-            fastlstm_plan pl;
-            if (int r2 = plan_device(-1, B, H, dtype, 0, &pl, false)) return r2;
-            const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
-            zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned *>(ws), zero / 4);
-            if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
-            rc = fwd_persistent_impl(ifgo_b, out_b, cell_b, Wh_b, ws, ws_bytes, T, B, H, dtype, stream, keep);
-        }
-    }
+    void *recs[2][7];
+    for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
+    int rc = try_multi(false, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
+    if (rc == 1) rc = multi_sequential(false, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep);
     return finish_recurrent(rc, ws, stream);
 }
 
@@ -1237,18 +1217,10 @@ int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, con
     if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
-    int rc = try_pair(true, a, b, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
-    if (rc == 1) {
-        rc = bwd_persistent_impl(dout_a, dh_a, dc_a, ifgo_a, cell_a, d_ifgo_a, Wh_a, ws, ws_bytes, T, B, H, dtype, stream);
-        if (rc == FASTLSTM_OK) {
-            fastlstm_plan pl;
-            if (int r2 = plan_device(-1, B, H, dtype, 1, &pl, false)) return r2;
-            const size_t zero = pl.ring_needs_zero ? ws_bytes : std::min(ws_bytes, pl.ws_zero_bytes);
-            zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned *>(ws), zero / 4);
-            if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
-            rc = bwd_persistent_impl(dout_b, dh_b, dc_b, ifgo_b, cell_b, d_ifgo_b, Wh_b, ws, ws_bytes, T, B, H, dtype, stream);
-        }
-    }
+    void *recs[2][7];
+    for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
+    int rc = try_multi(true, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
+    if (rc == 1) rc = multi_sequential(true, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, 1);
     return finish_recurrent(rc, ws, stream);
 }
 
