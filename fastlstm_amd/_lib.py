@@ -34,6 +34,7 @@ SIGNATURES = {
     "fastlstm_plan_device": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(Plan)]),
     "fastlstm_recurrent_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i, _i]),
     "fastlstm_recurrent_kernel_kind": (_i, [_i, _i, _i, _i, _i, _sz]),
+    "fastlstm_recurrent_rows_per_launch": (_i, [_i, _i, _i, _i, _i, _sz]),
     "fastlstm_fwd_stack2": (_i, [_vp] * 16 + [_sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_fwd_stack2_infer": (_i, [_vp] * 16 + [_sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_stack2_workspace_bytes": (_sz, [ctypes.POINTER(Plan), _i, _i, _i]),

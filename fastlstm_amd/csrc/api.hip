@@ -1559,6 +1559,20 @@ int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward,
     return wide_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes) ? 2 : 0;
 }
 
+int fastlstm_recurrent_rows_per_launch(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (T <= 0 || B <= 0 || H <= 0) return FASTLSTM_ERR_DIM;
+    {
+        fastlstm_plan pl;
+        if (plan_device(-1, B, H, dtype, backward, &pl, false) == FASTLSTM_OK && pl.wave_split == 3) return 0;
+    }
+    XcdCfg c;
+    WideCfg w;
+    if (select_xcd(T, B, H, dtype, backward != 0, ws_bytes, &c) || select_wide(T, B, H, dtype, backward != 0, ws_bytes, &w)) return 0;
+    if (const int rows = xcd_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes)) return rows;
+    return wide_rows_per_launch(T, B, H, dtype, backward != 0, ws_bytes);
+}
+
 int fastlstm_ws_status(const void *ws_head) {
     if (!ws_head) return FASTLSTM_ERR_NULL;
     const WsHeader *h = static_cast<const WsHeader *>(ws_head);

@@ -18,6 +18,7 @@ the library must be built, otherwise the calls raise.
 import ctypes
 import functools
 import os
+import threading
 
 import torch
 import torch.nn as nn
@@ -892,6 +893,61 @@ class PersistentLSTMStack2fn(torch.autograd.Function):
         return d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1, None
 
 
+_staging = threading.local()
+
+
+def _indices_to_device(dev, *tensors):
+    """int64 CPU tensors -> `dev` in one asynchronous copy through a pinned staging buffer kept per thread and
+    device (a pageable copy would stall the host until the stream has drained, and a fresh pinned allocation per
+    call costs milliseconds).  The buffer is reused only after the previous call's copy has run."""
+    if dev.type != "cuda":
+        return tuple(t.to(dev) for t in tensors)
+    n = sum(t.numel() for t in tensors)
+    stages = _staging.__dict__.setdefault("by_device", {})
+    with torch.cuda.device(dev):
+        key = torch.cuda.current_device()
+        stage = stages.get(key)
+        if stage is not None:
+            stage[1].synchronize()
+        if stage is None or stage[0].numel() < n:
+            stage = stages[key] = [torch.empty(max(n, 1 << 16), dtype=torch.int64).pin_memory(), None]
+        torch.cat([t.flatten() for t in tensors], out=stage[0][:n])
+        on_dev = stage[0][:n].to(dev, non_blocking=True)
+        stage[1] = torch.cuda.Event()
+        stage[1].record()
+    return on_dev.split([t.numel() for t in tensors])
+
+
+class _GatherRows(torch.autograd.Function):
+    """src[take]; the gradient of src is the rows `back` of the result's gradient -- for a gather in which every
+    row of src has one slot that counts (back[p]) and the other slots' gradients are zero by construction."""
+
+    @staticmethod
+    def forward(ctx, src, take, back):
+        ctx.save_for_backward(back)
+        return src.index_select(0, take)
+
+    @staticmethod
+    def backward(ctx, g):
+        back, = ctx.saved_tensors
+        return g.index_select(0, back), None, None
+
+
+class _TakeRows(torch.autograd.Function):
+    """src[idx] for distinct idx; the gradient is scattered back without atomics."""
+
+    @staticmethod
+    def forward(ctx, src, idx):
+        ctx.save_for_backward(idx)
+        ctx.n = src.shape[0]
+        return src.index_select(0, idx)
+
+    @staticmethod
+    def backward(ctx, g):
+        idx, = ctx.saved_tensors
+        return g.new_zeros(ctx.n, g.shape[1]).index_copy(0, idx, g), None
+
+
 class FastLSTM(nn.Module):
     """nn.LSTM-compatible parameters (names, shapes, order, seeded values) and the
     reference's forward contract (fastlstm/lstm.py:586-698): sequence-first input
@@ -959,12 +1015,82 @@ class FastLSTM(nn.Module):
         """PackedSequence input, nn.LSTM's contract: the sequences are padded to the longest, every layer
         runs over the padded batch (a row's steps behind its own end change nothing before it), the
         reverse direction runs over each row reversed within its own length, and the final states are
-        row b's out / cell at step len_b - 1.  The result is packed like the input."""
-        from torch.nn.utils.rnn import PackedSequence, pack_padded_sequence, pad_packed_sequence
-        x, lengths = pad_packed_sequence(packed)                 # [T,B,I], original batch order
+        row b's out / cell at step len_b - 1.  The result is packed like the input.
+
+        The padded batch keeps the packed order (rows sorted by length, longest first) and is made with ONE
+        gather, the packed result with one more (pad_packed_sequence / pack_padded_sequence copy timestep by
+        timestep, T launches each); slots behind a row's end hold some other row's data instead of zeros --
+        nothing reads what is computed from them, and their gradients are exactly zero.
+
+        A batch that the library runs as several launches over ranges of rows (more batch tiles than one
+        launch holds) is cut at those ranges here, and every range runs only to its own longest sequence: the
+        steps and GEMM rows behind it are not computed."""
+        from torch.nn.utils.rnn import PackedSequence
+        data, sizes = packed.data, packed.batch_sizes            # sizes [T] on the CPU: rows alive at step t
+        dev, N = data.device, data.shape[0]
+        T, B = int(sizes.numel()), int(sizes[0])
+        alive = sizes[:, None] > torch.arange(B)[None, :]        # [T,B]
+        lengths = alive.sum(0)                                   # per row, descending
+        offs = torch.cumsum(sizes, 0) - sizes                    # first packed row of step t
+        rows = self._packed_range_rows(T, B, lengths, data)
+        ranges = [(r0, min(B, r0 + rows), int(lengths[r0])) for r0 in range(0, B, rows)] if rows else [(0, B, T)]
+        # slot (t, j) of range r = row base_r + t*n_r + j of the ranges' padded tensors laid end to end
+        at = torch.zeros(T, B, dtype=torch.int64)
+        takes, base = [], 0
+        for r0, r1, Tr in ranges:
+            j = torch.arange(r0, r1)[None, :]
+            slot = base + torch.arange(Tr)[:, None] * (r1 - r0) + (j - r0)
+            takes.append(torch.where(j < sizes[:Tr, None], offs[:Tr, None] + j, slot % N).flatten())
+            at[:Tr, r0:r1] = slot
+            base += Tr * (r1 - r0)
+        take, at_packed, lengths_dev = _indices_to_device(dev, torch.cat(takes), at.flatten()[alive.flatten()], lengths)
+        x_all = _GatherRows.apply(data, take, at_packed)         # [sum Tr*n_r, I]
+        order = packed.sorted_indices
+        if order is not None:   # the states come in the caller's batch order
+            h_0 = [h if h is None else h.index_select(0, order) for h in h_0]
+            c_0 = [c if c is None else c.index_select(0, order) for c in c_0]
+        pieces, hs, cs, base = [], [], [], 0
+        for r0, r1, Tr in ranges:
+            n = Tr * (r1 - r0)
+            y, h_r, c_r = self._run_padded(x_all[base:base + n].view(Tr, r1 - r0, -1), lengths_dev[r0:r1],
+                                           [h if h is None else h[r0:r1] for h in h_0],
+                                           [c if c is None else c[r0:r1] for c in c_0])
+            pieces.append(y.reshape(n, -1))
+            hs.append(torch.stack(h_r))
+            cs.append(torch.stack(c_r))
+            base += n
+        y_all = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+        h_n, c_n = (hs[0], cs[0]) if len(hs) == 1 else (torch.cat(hs, dim=1), torch.cat(cs, dim=1))
+        out = PackedSequence(_TakeRows.apply(y_all, at_packed), packed.batch_sizes, packed.sorted_indices,
+                             packed.unsorted_indices)
+        if packed.unsorted_indices is not None:
+            h_n, c_n = h_n.index_select(1, packed.unsorted_indices), c_n.index_select(1, packed.unsorted_indices)
+        return out, (h_n, c_n)
+
+    def _packed_range_rows(self, T, B, lengths, data):
+        """Rows per range for a packed batch of B rows sorted by length (descending, lengths on the CPU): the rows
+        the library takes per launch where it runs this batch as several launches
+        (fastlstm_recurrent_rows_per_launch) and cutting there saves at least an eighth of the steps; else 0."""
+        dt = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else data.dtype
+        if not data.is_cuda or dt not in _DTYPE_CODE or B < 32:
+            return 0
+        lib = _lib.load()
+        code, H = _DTYPE_CODE[dt], self.hidden_size
+        with torch.cuda.device(data.device):
+            plan = _plan(data.device, B, H, code, False)
+            rows = lib.fastlstm_recurrent_rows_per_launch(T, B, H, code, 0,
+                                                          lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0))
+        if rows <= 0 or rows >= B:
+            return 0
+        saved = sum((T - int(lengths[r0])) * (min(B, r0 + rows) - r0) for r0 in range(0, B, rows))
+        return rows if saved * 8 >= T * B else 0
+
+    def _run_padded(self, x, lengths_dev, h_0, c_0):
+        """All layers over a padded batch x [T,B,I] with T = max(lengths); lengths_dev [B] on x's device; h_0, c_0:
+        per layer and direction [B,H] or None.  Returns (y [T,B,D*H], [h_n per layer and direction], [c_n ...])
+        with the final states taken at each row's own last step."""
         T, B = x.shape[0], x.shape[1]
         directions = 2 if self.bidirectional else 1
-        lengths_dev = lengths.to(x.device)
         steps = torch.arange(T, device=x.device)[:, None]
         last = (lengths_dev - 1)[None, :, None]                   # [1,B,1] index of a row's last step
         # time index that reverses row b within its length and leaves its padding in place
@@ -992,11 +1118,7 @@ class FastLSTM(nn.Module):
             x = ys[0] if directions == 1 else torch.cat(ys, dim=-1)
             if self.training and self.dropout > 0.0 and layer + 1 < self.num_layers:
                 x = F.dropout(x, self.dropout, True)
-        if packed.sorted_indices is not None:
-            x, lengths = x.index_select(1, packed.sorted_indices), lengths[packed.sorted_indices.cpu()]
-        data = pack_padded_sequence(x, lengths, enforce_sorted=True).data
-        out = PackedSequence(data, packed.batch_sizes, packed.sorted_indices, packed.unsorted_indices)
-        return out, (torch.stack(h_n), torch.stack(c_n))
+        return x, h_n, c_n
 
     def forward(self, x, h_c_0=None):
         directions = 2 if self.bidirectional else 1

@@ -276,6 +276,13 @@ int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_b
  * Diagnostics; no counterpart in the reference. */
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
 
+/* Rows of the batch that one launch of fastlstm_fwd_persistent / fastlstm_bwd_persistent takes when the
+ * batch has more tiles than a launch of kind 1 or 2 holds (the call then runs one launch per range of that
+ * many rows, one after the other); 0 when the whole batch is one launch.  A caller whose sequences differ in
+ * length (sorted by length, as in a PackedSequence) can cut its batch at these ranges and end each at its own
+ * longest sequence.  Negative: fastlstm_status.  Diagnostics; no counterpart in the reference. */
+int fastlstm_recurrent_rows_per_launch(int T, int B, int H, int dtype, int backward, size_t ws_bytes);
+
 /* One launch that gets a forward call ready, instead of three fills/copies by the caller: clears the first
  * `zero_bytes` bytes of the workspace (a multiple of 4; see fastlstm_recurrent_workspace_bytes for how many a
  * call needs zeroed) and writes the initial state into slot 0 of out and cell: h0, c0 ([B,H] each, dense), or

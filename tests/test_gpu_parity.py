@@ -1230,6 +1230,41 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
         assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
 
 
+@pytest.mark.parametrize("kw,B,H,dt", [(dict(), 272, 1024, torch.float16), (dict(bidirectional=True), 200, 1536, torch.bfloat16)])
+def test_packed_batch_larger_than_one_launch_is_cut_at_its_row_ranges(kw, B, H, dt):
+    """A packed batch that the library runs as several launches over ranges of rows is cut at those ranges in
+    the packed order, and every range stops at its own longest sequence: same contract, against nn.LSTM in
+    fp32 on the CPU (packed data, final states, every gradient; unsorted lengths, initial states given)."""
+    from torch.nn.utils.rnn import pack_sequence
+    import fastlstm_amd.lstm as L
+    I, layers, Tmax = 24, 2, 22
+    D = 2 if kw.get("bidirectional") else 1
+    m, ref = _option_pair(I, H, layers, dt, 43, **kw)
+    g = torch.Generator().manual_seed(10)
+    lengths = [int(v) for v in torch.randint(3, Tmax + 1, (B,), generator=g)]
+    lengths[5] = Tmax
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dt).float()
+    seqs = [rnd(n, I) for n in lengths]
+    h0, c0 = rnd(layers * D, B, H) * 0.3, rnd(layers * D, B, H) * 0.3
+    w, wh = rnd(sum(lengths), D * H), rnd(layers * D, B, H)
+    xr = pack_sequence(seqs, enforce_sorted=False)
+    xg = pack_sequence([t.cuda().to(dt) for t in seqs], enforce_sorted=False)
+    cuts = []
+    run_padded = m._run_padded
+    m._run_padded = lambda x, *a: (cuts.append(tuple(x.shape[:2])), run_padded(x, *a))[1]
+    y, (hn, cn) = m(xg, (h0.cuda().to(dt), c0.cuda().to(dt)))
+    # several ranges, the later ones shorter than the first
+    assert len(cuts) > 1 and sum(b for _, b in cuts) == B and cuts[0][0] == Tmax and cuts[-1][0] < Tmax, cuts
+    yr, (hr, cr) = ref(xr, (h0, c0))
+    assert torch.equal(y.batch_sizes, yr.batch_sizes) and torch.equal(y.unsorted_indices.cpu(), yr.unsorted_indices)
+    for got, want, name in ((y.data, yr.data, "y"), (hn, hr, "hn"), (cn, cr, "cn")):
+        assert rel_err(got, want) < HALF_TOL, name
+    ((y.data.float() * w.cuda()).sum() + (hn.float() * wh.cuda()).sum()).backward()
+    ((yr.data * w).sum() + (hr * wh).sum()).backward()
+    for n, prm in m.named_parameters():
+        assert rel_err(prm.grad, getattr(ref, n).grad) < HALF_TOL, n
+
+
 @pytest.mark.parametrize("T,B,I,H,layers,dt", [(9, 7, 11, 33, 1, torch.float32), (14, 5, 6, 65, 3, torch.float32),
                                                (70, 32, 256, 1024, 2, torch.float16)])   # one launch per pair
 def test_state_gradients_vs_nn_lstm(T, B, I, H, layers, dt):
