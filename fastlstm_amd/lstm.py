@@ -918,6 +918,27 @@ def _indices_to_device(dev, *tensors):
     return on_dev.split([t.numel() for t in tensors])
 
 
+@functools.lru_cache(maxsize=None)
+def _padded_hidden_size(T, B, H, code, device_index):
+    """The next hidden size above H (within a quarter, in steps of the MFMA k-step) that the XCD-local or the
+    register-resident kernels take, when H itself gets the general kernels; else 0."""
+    lib = _lib.load()
+    device = torch.device("cuda", device_index)
+
+    def kind(h):
+        with torch.cuda.device(device):
+            plan = _plan(device, B, h, code, False)
+            return lib.fastlstm_recurrent_kernel_kind(T, B, h, code, 0,
+                                                      lib.fastlstm_recurrent_workspace_bytes(plan, T, h, code, 0))
+    if kind(H) != 0:
+        return 0
+    step = 16 if code == _DTYPE_CODE[torch.float32] else 32
+    for Hp in range((H // step + 1) * step, H + H // 4 + step + 1, step):
+        if kind(Hp) in (1, 2):
+            return Hp
+    return 0
+
+
 class _GatherRows(torch.autograd.Function):
     """src[take]; the gradient of src is the rows `back` of the result's gradient -- for a gather in which every
     row of src has one slot that counts (back[p]) and the other slots' gradients are zero by construction."""
@@ -1129,6 +1150,9 @@ class FastLSTM(nn.Module):
         if self.version != "persistent":
             # the reference also offers "graph", "naive-pt" and "v1"; this build has one path
             raise ValueError(f"Not Implemnted: {self.version}")
+        Hp = self._hidden_padding(x)
+        if Hp:
+            return self._forward_hidden_padded(x, h_c_0, Hp)
         if isinstance(x, nn.utils.rnn.PackedSequence):
             return self._forward_packed(x, h_0, c_0)
         if self.batch_first and x.dim() == 3:
@@ -1250,6 +1274,41 @@ class FastLSTM(nn.Module):
             return x, (h_n[0].unsqueeze(0), c_n[0].unsqueeze(0))
         return x, (torch.stack(h_n), torch.stack(c_n))
 
+    def _hidden_padding(self, x):
+        """Hidden size to pad this call to, or 0.  A hidden size that only the general recurrent kernels take (not
+        a multiple of the MFMA k-step, or between the sizes the register-resident form covers) runs markedly
+        faster as the next size that the XCD-local or register-resident kernels take (T = 256, B = 32, 2 layers,
+        I = H = 650 as 672: forward 1.82 -> 1.15 ms), so the module pads W_x, W_h, the biases and the initial
+        states with zeros up to it: the added units' states stay exactly zero, nothing of them reaches the
+        others (their columns of W_h and of the next layer's W_x are zero), and their gradients are zero."""
+        packed = isinstance(x, nn.utils.rnn.PackedSequence)
+        data = x.data if packed else x
+        if not data.is_cuda or (not packed and data.dim() != 3):
+            return 0
+        dt = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else data.dtype
+        if dt not in _DTYPE_CODE:
+            return 0
+        if packed:
+            T, B = int(x.batch_sizes.numel()), int(x.batch_sizes[0])
+        else:
+            T, B = (data.shape[1], data.shape[0]) if self.batch_first else (data.shape[0], data.shape[1])
+        idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
+        return _padded_hidden_size(T, B, self.hidden_size, _DTYPE_CODE[dt], idx)
+
+    def _forward_hidden_padded(self, x, h_c_0, Hp):
+        H, D = self.hidden_size, 2 if self.bidirectional else 1
+        if h_c_0 is not None:
+            h_c_0 = tuple(F.pad(t, (0, Hp - H)) for t in h_c_0)
+        y, (h_n, c_n) = _HiddenPadded(self, Hp).forward(x, h_c_0)
+
+        def cut(t):   # [..., D*Hp] -> [..., D*H]
+            return t[..., :H].contiguous() if D == 1 else torch.cat((t[..., :H], t[..., Hp:Hp + H]), dim=-1)
+        if isinstance(y, nn.utils.rnn.PackedSequence):
+            y = nn.utils.rnn.PackedSequence(cut(y.data), y.batch_sizes, y.sorted_indices, y.unsorted_indices)
+        else:
+            y = cut(y)
+        return y, (h_n[..., :H].contiguous(), c_n[..., :H].contiguous())
+
     def extra_repr(self):
         s = "%d, %d, num_layers=%d" % (self.input_size, self.hidden_size, self.num_layers)
         for name in ("bias", "batch_first", "bidirectional", "state_grads"):
@@ -1258,3 +1317,43 @@ class FastLSTM(nn.Module):
         if self.dropout:
             s += ", dropout=%g" % self.dropout
         return s
+
+
+
+class _HiddenPadded:
+    """What FastLSTM.forward reads of a module, with the hidden size Hp and the module's parameters zero-padded to
+    it (FastLSTM._hidden_padding): W [4H, K] is four gate blocks of H rows, each padded to Hp rows; the K = H columns
+    of W_h, and the K = D*H columns of a deeper layer's W_x (D blocks of H, one per direction), are padded alike.
+    The pads are differentiable, so the gradients arrive at the module's own parameters."""
+
+    forward = FastLSTM.forward
+    _forward_packed = FastLSTM._forward_packed
+    _packed_range_rows = FastLSTM._packed_range_rows
+    _run_padded = FastLSTM._run_padded
+    _two_layers_at_once = FastLSTM._two_layers_at_once
+
+    def __init__(self, module, Hp):
+        self._module, self.hidden_size, self._operands = module, Hp, {}
+        for name in ("input_size", "num_layers", "version", "bias", "batch_first", "bidirectional", "state_grads",
+                     "dropout", "training"):
+            setattr(self, name, getattr(module, name))
+
+    def parameters(self):
+        return self._module.parameters()
+
+    def _hidden_padding(self, x):
+        return 0
+
+    def _layer_operands(self, layer, suffix=""):
+        if (layer, suffix) not in self._operands:
+            H, Hp, D = self._module.hidden_size, self.hidden_size, 2 if self.bidirectional else 1
+            Wx, bx, Wh, bh = self._module._layer_operands(layer, suffix)
+            p = Hp - H
+            if layer == 0:
+                Wx = F.pad(Wx.reshape(4, H, -1), (0, 0, 0, p))
+            else:
+                Wx = F.pad(Wx.reshape(4, H, D, H), (0, p, 0, 0, 0, p))
+            self._operands[(layer, suffix)] = (
+                Wx.reshape(4 * Hp, -1), F.pad(bx.reshape(4, H), (0, p)).reshape(-1),
+                F.pad(Wh.reshape(4, H, H), (0, p, 0, p)).reshape(4 * Hp, Hp), F.pad(bh.reshape(4, H), (0, p)).reshape(-1))
+        return self._operands[(layer, suffix)]

@@ -1230,6 +1230,39 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
         assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
 
 
+@pytest.mark.parametrize("kw,T,B,I,H,Hp,dt", [(dict(bidirectional=True), 20, 24, 50, 100, 112, torch.float32),
+                                              (dict(), 30, 16, 70, 650, 672, torch.float16),
+                                              (dict(bias=False, batch_first=True), 12, 8, 33, 1150, 1280, torch.bfloat16)])
+def test_hidden_sizes_that_only_the_general_kernels_take_run_zero_padded(kw, T, B, I, H, Hp, dt):
+    """The module pads such a hidden size to the next one the XCD-local / register-resident kernels take (zero
+    weights, biases and initial states for the added units): outputs, final states and every gradient against
+    nn.LSTM in fp32 on the CPU, two layers, initial states given, a loss on out, h_n and c_n."""
+    layers = 2
+    D = 2 if kw.get("bidirectional") else 1
+    m, ref = _option_pair(I, H, layers, dt, 47, state_grads=True, **kw)
+    g = torch.Generator().manual_seed(12)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dt).float()
+    x = rnd(B, T, I) if kw.get("batch_first") else rnd(T, B, I)
+    h0, c0 = rnd(layers * D, B, H) * 0.3, rnd(layers * D, B, H) * 0.3
+    wy, wh, wc = rnd(*x.shape[:2], D * H), rnd(layers * D, B, H), rnd(layers * D, B, H)
+    leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
+    leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
+    assert m._hidden_padding(leaves[0]) == Hp
+    y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
+    yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
+    assert y.shape == yr.shape and hn.shape == hr.shape and y.is_contiguous() and hn.is_contiguous()
+    ((y.float() * wy.cuda()).sum() + (hn.float() * wh.cuda()).sum() + (cn.float() * wc.cuda()).sum()).backward()
+    ((yr * wy).sum() + (hr * wh).sum() + (cr * wc).sum()).backward()
+    pairs = [(a.grad, b.grad, n) for a, b, n in zip(leaves, leaves_r, ("x", "h0", "c0"))]
+    pairs += [(prm.grad, getattr(ref, n).grad, n) for n, prm in m.named_parameters()]
+    for got, want, name in [(y, yr, "y"), (hn, hr, "hn"), (cn, cr, "cn")] + pairs:
+        assert got.shape == want.shape, name
+        if dt == torch.float32:
+            assert_close32(got, want, scale_atol=max(1.0, float(want.detach().abs().max())))
+        else:
+            assert rel_err(got, want) < HALF_TOL, name
+
+
 @pytest.mark.parametrize("kw,B,H,dt", [(dict(), 272, 1024, torch.float16), (dict(bidirectional=True), 200, 1536, torch.bfloat16)])
 def test_packed_batch_larger_than_one_launch_is_cut_at_its_row_ranges(kw, B, H, dt):
     """A packed batch that the library runs as several launches over ranges of rows is cut at those ranges in
