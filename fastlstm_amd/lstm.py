@@ -1150,9 +1150,9 @@ class FastLSTM(nn.Module):
         if self.version != "persistent":
             # the reference also offers "graph", "naive-pt" and "v1"; this build has one path
             raise ValueError(f"Not Implemnted: {self.version}")
-        Hp = self._hidden_padding(x)
-        if Hp:
-            return self._forward_hidden_padded(x, h_c_0, Hp)
+        padding = self._operand_padding(x)
+        if padding:
+            return self._forward_operands_padded(x, h_c_0, *padding)
         if isinstance(x, nn.utils.rnn.PackedSequence):
             return self._forward_packed(x, h_0, c_0)
         if self.batch_first and x.dim() == 3:
@@ -1274,34 +1274,48 @@ class FastLSTM(nn.Module):
             return x, (h_n[0].unsqueeze(0), c_n[0].unsqueeze(0))
         return x, (torch.stack(h_n), torch.stack(c_n))
 
-    def _hidden_padding(self, x):
-        """Hidden size to pad this call to, or 0.  A hidden size that only the general recurrent kernels take (not
-        a multiple of the MFMA k-step, or between the sizes the register-resident form covers) runs markedly
-        faster as the next size that the XCD-local or register-resident kernels take (T = 256, B = 32, 2 layers,
-        I = H = 650 as 672: forward 1.82 -> 1.15 ms), so the module pads W_x, W_h, the biases and the initial
-        states with zeros up to it: the added units' states stay exactly zero, nothing of them reaches the
-        others (their columns of W_h and of the next layer's W_x are zero), and their gradients are zero."""
+    def _operand_padding(self, x):
+        """(Hp, Ip): hidden and input size to zero-pad this call to, or None when it runs as it is.
+
+        A hidden size that only the general recurrent kernels take (not a multiple of the MFMA k-step, or between
+        the sizes the register-resident form covers) runs markedly faster as the next size that the XCD-local or
+        register-resident kernels take (T = 256, B = 32, 2 layers, I = H = 650 as 672: forward 1.82 -> 1.15 ms), so
+        the module pads W_x, W_h, the biases and the initial states with zeros up to it: the added units' states
+        stay exactly zero, nothing of them reaches the others (their columns of W_h and of the next layer's W_x are
+        zero), and their gradients are zero.  A 16-bit input size that is not a multiple of 64 keeps the first
+        layer's products off the MFMA tile kernel (T = 256, B = 32, H = 1024: I = 650 forward + backward 2.71 ms,
+        I = 704 1.64 ms): x and the columns of the first W_x get zero columns up to the next multiple."""
         packed = isinstance(x, nn.utils.rnn.PackedSequence)
         data = x.data if packed else x
         if not data.is_cuda or (not packed and data.dim() != 3):
-            return 0
+            return None
         dt = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else data.dtype
         if dt not in _DTYPE_CODE:
-            return 0
+            return None
         if packed:
             T, B = int(x.batch_sizes.numel()), int(x.batch_sizes[0])
         else:
             T, B = (data.shape[1], data.shape[0]) if self.batch_first else (data.shape[0], data.shape[1])
         idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
-        return _padded_hidden_size(T, B, self.hidden_size, _DTYPE_CODE[dt], idx)
+        H, I = self.hidden_size, self.input_size
+        Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx) or H
+        Ip = -(-I // 64) * 64 if dt != torch.float32 and I > 64 and data.shape[-1] == I else I
+        return (Hp, Ip) if (Hp, Ip) != (H, I) else None
 
-    def _forward_hidden_padded(self, x, h_c_0, Hp):
+    def _forward_operands_padded(self, x, h_c_0, Hp, Ip):
         H, D = self.hidden_size, 2 if self.bidirectional else 1
         if h_c_0 is not None:
             h_c_0 = tuple(F.pad(t, (0, Hp - H)) for t in h_c_0)
-        y, (h_n, c_n) = _HiddenPadded(self, Hp).forward(x, h_c_0)
+        if isinstance(x, nn.utils.rnn.PackedSequence):
+            x = nn.utils.rnn.PackedSequence(F.pad(x.data, (0, Ip - self.input_size)), x.batch_sizes, x.sorted_indices,
+                                            x.unsorted_indices)
+        else:
+            x = F.pad(x, (0, Ip - self.input_size))
+        y, (h_n, c_n) = _OperandsPadded(self, Hp, Ip).forward(x, h_c_0)
 
         def cut(t):   # [..., D*Hp] -> [..., D*H]
+            if Hp == H:
+                return t
             return t[..., :H].contiguous() if D == 1 else torch.cat((t[..., :H], t[..., Hp:Hp + H]), dim=-1)
         if isinstance(y, nn.utils.rnn.PackedSequence):
             y = nn.utils.rnn.PackedSequence(cut(y.data), y.batch_sizes, y.sorted_indices, y.unsorted_indices)
@@ -1320,11 +1334,12 @@ class FastLSTM(nn.Module):
 
 
 
-class _HiddenPadded:
-    """What FastLSTM.forward reads of a module, with the hidden size Hp and the module's parameters zero-padded to
-    it (FastLSTM._hidden_padding): W [4H, K] is four gate blocks of H rows, each padded to Hp rows; the K = H columns
-    of W_h, and the K = D*H columns of a deeper layer's W_x (D blocks of H, one per direction), are padded alike.
-    The pads are differentiable, so the gradients arrive at the module's own parameters."""
+class _OperandsPadded:
+    """What FastLSTM.forward reads of a module, with the hidden size Hp, the input size Ip and the module's parameters
+    zero-padded to them (FastLSTM._operand_padding): W [4H, K] is four gate blocks of H rows, each padded to Hp rows;
+    the K = H columns of W_h, and the K = D*H columns of a deeper layer's W_x (D blocks of H, one per direction), are
+    padded alike, the K = I columns of the first layer's W_x to Ip.  The pads are differentiable, so the gradients
+    arrive at the module's own parameters."""
 
     forward = FastLSTM.forward
     _forward_packed = FastLSTM._forward_packed
@@ -1332,17 +1347,16 @@ class _HiddenPadded:
     _run_padded = FastLSTM._run_padded
     _two_layers_at_once = FastLSTM._two_layers_at_once
 
-    def __init__(self, module, Hp):
-        self._module, self.hidden_size, self._operands = module, Hp, {}
-        for name in ("input_size", "num_layers", "version", "bias", "batch_first", "bidirectional", "state_grads",
-                     "dropout", "training"):
+    def __init__(self, module, Hp, Ip):
+        self._module, self.hidden_size, self.input_size, self._operands = module, Hp, Ip, {}
+        for name in ("num_layers", "version", "bias", "batch_first", "bidirectional", "state_grads", "dropout", "training"):
             setattr(self, name, getattr(module, name))
 
     def parameters(self):
         return self._module.parameters()
 
-    def _hidden_padding(self, x):
-        return 0
+    def _operand_padding(self, x):
+        return None
 
     def _layer_operands(self, layer, suffix=""):
         if (layer, suffix) not in self._operands:
@@ -1350,7 +1364,7 @@ class _HiddenPadded:
             Wx, bx, Wh, bh = self._module._layer_operands(layer, suffix)
             p = Hp - H
             if layer == 0:
-                Wx = F.pad(Wx.reshape(4, H, -1), (0, 0, 0, p))
+                Wx = F.pad(Wx.reshape(4, H, -1), (0, self.input_size - self._module.input_size, 0, p))
             else:
                 Wx = F.pad(Wx.reshape(4, H, D, H), (0, p, 0, 0, 0, p))
             self._operands[(layer, suffix)] = (

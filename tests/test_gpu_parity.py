@@ -1230,12 +1230,14 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
         assert_close32(prm.grad, rg, scale_atol=max(1.0, float(rg.abs().max())))
 
 
-@pytest.mark.parametrize("kw,T,B,I,H,Hp,dt", [(dict(bidirectional=True), 20, 24, 50, 100, 112, torch.float32),
-                                              (dict(), 30, 16, 70, 650, 672, torch.float16),
-                                              (dict(bias=False, batch_first=True), 12, 8, 33, 1150, 1280, torch.bfloat16)])
-def test_hidden_sizes_that_only_the_general_kernels_take_run_zero_padded(kw, T, B, I, H, Hp, dt):
-    """The module pads such a hidden size to the next one the XCD-local / register-resident kernels take (zero
-    weights, biases and initial states for the added units): outputs, final states and every gradient against
+@pytest.mark.parametrize("kw,T,B,I,H,Hp,Ip,dt", [(dict(bidirectional=True), 20, 24, 50, 100, 112, 50, torch.float32),
+                                                 (dict(), 30, 16, 70, 650, 672, 128, torch.float16),
+                                                 (dict(bidirectional=True), 24, 16, 300, 256, 256, 320, torch.float16),
+                                                 (dict(bias=False, batch_first=True), 12, 8, 33, 1150, 1280, 33, torch.bfloat16)])
+def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
+    """The module pads a hidden size that only the general kernels take to the next one the XCD-local /
+    register-resident kernels take (zero weights, biases and initial states for the added units), and a 16-bit
+    input size to a multiple of 64 (zero columns of x and W_x): outputs, final states and every gradient against
     nn.LSTM in fp32 on the CPU, two layers, initial states given, a loss on out, h_n and c_n."""
     layers = 2
     D = 2 if kw.get("bidirectional") else 1
@@ -1247,7 +1249,7 @@ def test_hidden_sizes_that_only_the_general_kernels_take_run_zero_padded(kw, T, 
     wy, wh, wc = rnd(*x.shape[:2], D * H), rnd(layers * D, B, H), rnd(layers * D, B, H)
     leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
     leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
-    assert m._hidden_padding(leaves[0]) == Hp
+    assert m._operand_padding(leaves[0]) == (Hp, Ip)
     y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
     yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
     assert y.shape == yr.shape and hn.shape == hr.shape and y.is_contiguous() and hn.is_contiguous()
