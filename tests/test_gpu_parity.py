@@ -1250,6 +1250,9 @@ def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I
     leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
     leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
     assert m._operand_padding(leaves[0]) == (Hp, Ip)
+    # sizes the fast kernels take run as they are; so does H <= 64 (the one-tile form of the general kernels)
+    for i_, h_ in ((64, 64), (128, 48), (256, 512), (1024, 2048)):
+        assert FastLSTM(i_, h_).to("cuda", torch.float16)._operand_padding(torch.empty(32, 256, i_, device="cuda", dtype=torch.float16)) is None
     y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
     yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
     assert y.shape == yr.shape and hn.shape == hr.shape and y.is_contiguous() and hn.is_contiguous()
