@@ -932,7 +932,7 @@ def _padded_hidden_size(T, B, H, code, device_index):
                                                       lib.fastlstm_recurrent_workspace_bytes(plan, T, h, code, 0))
     # (H <= 64 runs the general kernels' one-tile form, which has no exchange between workgroups at all and is the
     # fastest there is: T = 1024, B = 256, I = H = 64 forward + backward 2.1 ms as it is, 3.4 ms as H = 96)
-    if H <= 64 or kind(H) != 0:
+    if H <= 64 or T < 32 or kind(H) != 0:   # (a few steps do not repay the launches that pad and cut)
         return 0
     step = 16 if code == _DTYPE_CODE[torch.float32] else 32
     for Hp in range((H // step + 1) * step, H + H // 4 + step + 1, step):
@@ -1301,7 +1301,7 @@ class FastLSTM(nn.Module):
         idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
         H, I = self.hidden_size, self.input_size
         Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx) or H
-        Ip = -(-I // 64) * 64 if dt != torch.float32 and I > 64 and data.shape[-1] == I else I
+        Ip = -(-I // 64) * 64 if dt != torch.float32 and I > 64 and T * B >= 1024 and data.shape[-1] == I else I
         return (Hp, Ip) if (Hp, Ip) != (H, I) else None
 
     def _forward_operands_padded(self, x, h_c_0, Hp, Ip):
