@@ -1,0 +1,107 @@
+"""Seeded sweep of the module's option surface against torch.nn.LSTM (fp32, CPU, same weights).
+
+Every case draws its shape and options from its seed: sequence length, batch, input and hidden size
+(multiples of the MFMA k-step and odd sizes alike, so the padded and the unpadded dispatch both occur),
+1-4 layers, bidirectional, bias, batch_first, initial states given or not, dense or PackedSequence input,
+state_grads, dtype.  The module chooses among its forms by shape (general / XCD-local / register-resident
+kernels, pairs of layers in one launch, wavefronts of chunked launches, both directions side by side,
+zero-padded sizes, packed batches cut at row ranges); whichever it takes, outputs, final states and every
+gradient have to match nn.LSTM: fp32 rtol = atol = 1e-4 (atol scaled by the reference's magnitude for
+gradients), 16-bit <= 2e-2 of the reference's max-norm (reference evaluated with the rounded weights
+and inputs)."""
+import random
+
+import pytest
+import torch
+from torch.nn.utils.rnn import pack_sequence
+
+import fastlstm_amd.lstm as L
+from fastlstm_amd import FastLSTM
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL, HALF_TOL = 1e-4, 2e-2
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _check_every_launch():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    old = L.CHECK_STATUS
+    L.CHECK_STATUS = True
+    yield
+    L.CHECK_STATUS = old
+
+
+def draw(seed):
+    r = random.Random(1000 + seed)
+    dt = r.choice([torch.float32, torch.float16, torch.bfloat16])
+    kw = dict(bidirectional=r.random() < 0.4, bias=r.random() < 0.8, batch_first=r.random() < 0.3)
+    layers = r.choice([1, 1, 2, 2, 3, 4])
+    T = r.choice([1, 3, 17, 33, 64, 70, 130, 260])
+    B = r.choice([1, 2, 5, 16, 24, 33, 64, 70])
+    I = r.choice([1, 7, 32, 50, 64, 100, 128, 200, 300])
+    H = r.choice([8, 20, 32, 48, 64, 65, 96, 100, 128, 200, 256, 300, 384, 512, 650])
+    if T * B * H * layers > 260 * 33 * 512 * 2:   # keep the CPU reference to seconds
+        T = min(T, 70)
+    return dict(dt=dt, kw=kw, layers=layers, T=T, B=B, I=I, H=H, states=r.random() < 0.5, packed=r.random() < 0.3,
+                state_grads=r.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_module_against_nn_lstm(seed):
+    c = draw(seed)
+    dt, kw, layers, T, B, I, H = c["dt"], c["kw"], c["layers"], c["T"], c["B"], c["I"], c["H"]
+    D = 2 if kw["bidirectional"] else 1
+    torch.manual_seed(seed)
+    m = FastLSTM(I, H, num_layers=layers, state_grads=c["state_grads"], **kw)
+    ref = torch.nn.LSTM(I, H, num_layers=layers, **kw)
+    with torch.no_grad():
+        for n, prm in m.named_parameters():
+            prm.copy_(prm.to(dt).float())
+            getattr(ref, n).copy_(prm)
+    m = m.to("cuda", dt)
+    g = torch.Generator().manual_seed(seed)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dt).float()
+    h0, c0 = rnd(layers * D, B, H) * 0.3, rnd(layers * D, B, H) * 0.3
+    wh, wc = rnd(layers * D, B, H), rnd(layers * D, B, H)
+    state = (lambda *ts: tuple(ts)) if c["states"] else (lambda *ts: None)
+    leaves = [t.cuda().to(dt).requires_grad_(True) for t in (h0, c0)]
+    leaves_r = [t.clone().requires_grad_(True) for t in (h0, c0)]
+    if c["packed"]:
+        lengths = [int(v) for v in torch.randint(1, T + 1, (B,), generator=g)]
+        seqs = [rnd(n, I) for n in lengths]
+        xs = [s.cuda().to(dt).requires_grad_(True) for s in seqs]
+        xr = [s.clone().requires_grad_(True) for s in seqs]
+        y, (hn, cn) = m(pack_sequence(xs, enforce_sorted=False), state(*leaves))
+        yr, (hr, cr) = ref(pack_sequence(xr, enforce_sorted=False), state(*leaves_r))
+        assert torch.equal(y.batch_sizes, yr.batch_sizes)
+        y, yr = y.data, yr.data
+    else:
+        x = rnd(B, T, I) if kw["batch_first"] else rnd(T, B, I)
+        xs, xr = [x.cuda().to(dt).requires_grad_(True)], [x.clone().requires_grad_(True)]
+        y, (hn, cn) = m(xs[0], state(*leaves))
+        yr, (hr, cr) = ref(xr[0], state(*leaves_r))
+    assert y.shape == yr.shape and hn.shape == hr.shape and cn.shape == cr.shape, c
+    wy = rnd(*yr.shape)
+    loss, loss_r = (y.float() * wy.cuda()).sum(), (yr * wy).sum()
+    if c["state_grads"] or c["packed"]:   # final states that carry a gradient
+        loss, loss_r = loss + (hn.float() * wh.cuda()).sum(), loss_r + (hr * wh).sum()
+    if c["state_grads"] and not c["packed"]:
+        loss, loss_r = loss + (cn.float() * wc.cuda()).sum(), loss_r + (cr * wc).sum()
+    loss.backward()
+    loss_r.backward()
+    rows = [(y, yr, "y"), (hn, hr, "hn"), (cn, cr, "cn")]
+    # (the sequences of a packed batch as one tensor: the max-norm of a one-element gradient is no yardstick)
+    rows += [(torch.cat([a.grad for a in xs]), torch.cat([b.grad for b in xr]), "dx")]
+    if c["states"]:
+        rows += [(a.grad, b.grad, n) for a, b, n in zip(leaves, leaves_r, ("dh0", "dc0"))]
+    rows += [(prm.grad, getattr(ref, n).grad, n) for n, prm in m.named_parameters()]
+    for got, want, name in rows:
+        assert got is not None and got.shape == want.shape, (name, c)
+        if dt == torch.float32:
+            scale = max(1.0, float(want.detach().abs().max()))
+            torch.testing.assert_close(got.detach().cpu().double(), want.detach().double(), rtol=FP32_TOL,
+                                       atol=FP32_TOL * scale, msg=lambda s: "%s %s: %s" % (name, c, s))
+        else:
+            assert rel_err(got, want) < HALF_TOL, (name, c, rel_err(got, want))
