@@ -374,15 +374,16 @@ __global__ void prepare_forward_kernel(unsigned *ws, size_t zero_words, unsigned
     }
 }
 
-// A batch with more 16-row tiles than one XCD-local launch holds (and no fit with 32-row tiles either):
-// rows per launch such that full launches use every XCD with 16-row tiles and the remainder fits
-// too, or 0.  The launches run one after the other on the stream and share the workspace.
+// A batch with more tiles than one XCD-local launch holds, even with 32-row tiles: rows per launch such that
+// full launches use every XCD (with 32-row tiles where they fit: twice the rows of a launch for 1.1 ... 1.65
+// times its step; T = 256, B = 1024, H = 512 fp16 forward 4.4 -> 2.6 ms) and the remainder fits too, or 0.
+// The launches run one after the other on the stream and share the workspace.
 static int xcd_rows_per_launch(int T, int B, int H, int dtype, bool backward, size_t ws_bytes) {
     const int candidates[4] = {512, 256, 128, 64};
     for (int rows : candidates) {
         if (rows >= B) continue;
         XcdCfg c;
-        if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c, rows) || c.ntw != 1 || c.n_groups != kNumXcd * c.gpx) continue;
+        if (!select_xcd(T, B, H, dtype, backward, ws_bytes, &c, rows) || c.n_groups != kNumXcd * c.gpx) continue;
         if (B % rows && !select_xcd(T, B, H, dtype, backward, ws_bytes, &c, B % rows)) continue;
         return rows;
     }
