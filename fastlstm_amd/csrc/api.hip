@@ -240,6 +240,14 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
     return true;
 }
 
+// GEMM work of `flop` on `n_helpers` CUs inside a recurrent launch of about rec_ms: worth while when the launch, which
+// lasts as long as the longer of the two, beats the recurrence followed by the same work on the whole device.  A CU
+// inside the launch sustains about 3.5 TFLOP/s on the 256 x 256 16-bit tiles.
+static bool helpers_keep_up(double flop, int n_helpers, double rec_ms) {
+    const double helper_ms = flop / (n_helpers * 3.5e9);
+    return std::max(helper_ms, rec_ms) <= rec_ms + helper_ms * n_helpers / 256.0;
+}
+
 // In-kernel input projection: possible when the XCD-local forward kernel is the 8-wave one, at
 // least a quarter of the CUs have no role in the recurrence, and K1 suits the 256 x 256 16-bit
 // tile kernel.  Fills the k1 fields of *p (chunking by time) and returns true.
@@ -259,6 +267,7 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     const int max_chunks = kMaxChunks;
     const int M = T * B, N = 4 * H;
     if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;
+    if (!second && !helpers_keep_up(2.0 * M * N * I, n_helpers, T * (c.ntw == 1 ? 2.3e-3 : 3.8e-3))) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
     // a chunk: whole timesteps, about one round of the helpers, at most kMaxChunks chunks
     int base = 1;
@@ -551,6 +560,24 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     const int max_chunks = kMaxChunks;
     const int I = e.I, M = T * B, K = 4 * H;
     if (!gemm16_eligible(dtype, M, I, K, K, I, false, true) || I % 8) return false;
+    // The helpers have to keep up with the recurrence: with few of them (8 idle CUs per XCD at H = 768) the launch
+    // lasts as long as their share of dx, dW_x and dW_h, and launches of their own on the whole device behind the
+    // recurrence are faster (T = 256, B = 128, I = H = 768: layer backward 2.3 ms inside, 1.3 ms behind).
+    // A weight-gradient tile is one helper's from the first timestep to the last (2 * 256 * 256 * T * B flop), so with
+    // fewer tiles than helpers (H = 384: 24 tiles) most helpers have none and the launch lasts as long as one tile.
+    // Of {dx and the weight gradients inside, dx inside, nothing inside} the fastest by this estimate is taken.
+    bool wgrad_inside = true;
+    if (!lower) {
+        const double per_cu = 3.5e9, rec_ms = T * (c.ntw == 1 ? 3.0e-3 : 5.4e-3);   // flop per ms and CU inside a launch
+        const double dx_flop = 2.0 * M * K * I, wg_flop = 2.0 * M * K * (I + H);
+        const int wg_tiles = cdiv(K, 256) * (cdiv(I, 256) + cdiv(H, 256));
+        const double tile_ms = cdiv(wg_tiles, n_helpers) * 2.0 * 256 * 256 * M / per_cu;
+        const double all_ms = std::max(rec_ms, std::max((dx_flop + wg_flop) / (n_helpers * per_cu), tile_ms));
+        const double dx_ms = std::max(rec_ms, dx_flop / (n_helpers * per_cu)) + wg_flop / (256 * per_cu);
+        const double none_ms = rec_ms + (dx_flop + wg_flop) / (256 * per_cu);
+        if (none_ms < std::min(all_ms, dx_ms)) return false;
+        wgrad_inside = all_ms <= dx_ms;
+    }
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(I, 256);
     // a chunk: whole timesteps, about 8 row tiles (a short tail behind the recurrence), at most kMaxChunks chunks
     int base = 1;
@@ -584,8 +611,8 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     p->n_active = n_active;
     p->chunk_done = ws_chunk_counters(p->hdr, 0);
     p->wg_tiles = 0;
-    if (e.dWx && gemm16_eligible(dtype, K, I, M, K, I, true, true) && gemm16_eligible(dtype, K, H, M, K, H, true, true) &&
-        H % 8 == 0) {
+    if (wgrad_inside && e.dWx && gemm16_eligible(dtype, K, I, M, K, I, true, true) &&
+        gemm16_eligible(dtype, K, H, M, K, H, true, true) && H % 8 == 0) {
         GemmParams g{};
         g.A = d_ifgo; g.M = K; g.K = M; g.lda = K; g.splits = 1; g.k_per_split = M;
         p->k8 = g; p->k8.B = e.x; p->k8.C = e.dWx; p->k8.N = I; p->k8.ldb = I; p->k8.ldc = I;
