@@ -441,7 +441,8 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     if (c->n_groups * c->xpg > kNumXcd) return false;
     // ... and a small fp32 batch leaves most CUs without a share of the forward product (B = 32, H = 1024: 6.0
     // instead of 5.7 us per step; the reverse step, with four times the operand bytes, gains at every size)
-    if (dtype == FASTLSTM_FP32 && !backward && c->n_groups * c->xpg < 6) return false;
+    // (a remainder of rows behind full launches still runs here: the general kernel would take the whole batch)
+    if (dtype == FASTLSTM_FP32 && !backward && c->n_groups * c->xpg < 6 && B == B_all) return false;
     c->ks = (backward ? 4 * H : H) / kstep;
     c->xslot = (size_t)c->n_groups * c->nt * c->ks * kFragBytes;
     if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;

@@ -930,11 +930,23 @@ def _padded_hidden_size(T, B, H, code, device_index):
             plan = _plan(device, B, h, code, False)
             return lib.fastlstm_recurrent_kernel_kind(T, B, h, code, 0,
                                                       lib.fastlstm_recurrent_workspace_bytes(plan, T, h, code, 0))
-    # (H <= 64 runs the general kernels' one-tile form, which has no exchange between workgroups at all and is the
-    # fastest there is: T = 1024, B = 256, I = H = 64 forward + backward 2.1 ms as it is, 3.4 ms as H = 96)
-    if H <= 64 or T < 32 or kind(H) != 0:   # (a few steps do not repay the launches that pad and cut)
+    fp32 = code == _DTYPE_CODE[torch.float32]
+    if T < 32:   # a few steps do not repay the launches that pad and cut
         return 0
-    step = 16 if code == _DTYPE_CODE[torch.float32] else 32
+    if H <= 64:
+        # The general kernels' one-tile form (no exchange between workgroups at all).  In 16 bits it is the fastest
+        # there is at H = 64 (T = 1024, B = 256, I = H = 64 forward + backward 2.1 ms as it is, 3.4 ms as H = 96), and
+        # at 16 and 32, but sizes in between lose the 16-byte tile moves (T = 256, B = 64, forward / forward +
+        # backward: H = 48 0.91 / 1.83 ms, H = 64 0.25 / 0.58).  In fp32 it is bound by the true-fp32 MFMA rate and the
+        # XCD-local kernels win from H = 80 on (H = 64 0.73 / 1.57, H = 48 1.34 / 2.73, as H = 80 0.60 / 1.22).
+        if H <= 16 or H == 32:
+            return 0
+        if fp32:
+            return 80 if kind(80) == 1 else 0
+        return 64 if H < 64 else 0
+    if kind(H) != 0:
+        return 0
+    step = 16 if fp32 else 32
     for Hp in range((H // step + 1) * step, H + H // 4 + step + 1, step):
         if kind(Hp) in (1, 2):
             return Hp

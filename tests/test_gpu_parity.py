@@ -1251,7 +1251,7 @@ def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I
     leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
     assert m._operand_padding(leaves[0]) == (Hp, Ip)
     # sizes the fast kernels take run as they are; so does H <= 64 (the one-tile form of the general kernels)
-    for i_, h_ in ((64, 64), (128, 48), (256, 512), (1024, 2048)):
+    for i_, h_ in ((64, 64), (128, 32), (256, 512), (1024, 2048)):
         assert FastLSTM(i_, h_).to("cuda", torch.float16)._operand_padding(torch.empty(32, 256, i_, device="cuda", dtype=torch.float16)) is None
     # ... and a few timesteps do not repay the padding
     assert m._operand_padding(leaves[0][:, :4] if kw.get("batch_first") else leaves[0][:4]) is None
