@@ -268,11 +268,17 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     const int M = T * B, N = 4 * H;
     if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;
     if (!second && !helpers_keep_up(2.0 * M * N * I, n_helpers, T * (c.ntw == 1 ? 2.3e-3 : 3.8e-3))) return false;
+    // two layers: both projections on the helpers; past 1.25 x the time of the two time loops side by side the layers
+    // are better run one by one, each with more helpers (config E: 1.0)
+    if (second && 2.0 * M * N * (I + H) / (n_helpers * 3.5e9) > 1.25 * T * 2.4e-3) return false;
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256);
     // a chunk: whole timesteps, about one round of the helpers, at most kMaxChunks chunks
     int base = 1;
     while ((base * 256) % B) ++base;                       // row tiles that hold whole timesteps
     int ct = std::max(1, n_helpers / tiles_n / base) * base;
+    // the second layer starts a chunk behind the first: no more than 64 timesteps per chunk (B = 16: a round of the
+    // helpers would be 192)
+    if (second) ct = std::min(ct, std::max(1, 64 * B / 256 / base) * base);
     while (cdiv(tiles_m, ct) > max_chunks) ct += base;
     const int steps = ct * 256 / B;
     if (steps < 2) return false;
@@ -584,6 +590,13 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     int base = 1;
     while ((base * 256) % B) ++base;
     int ct = base >= 8 ? base : (8 / base) * base;
+    if (lower) {
+        // the lower layer runs two chunks behind the upper one: no more than 64 timesteps per chunk
+        ct = std::min(ct, std::max(1, 64 * B / 256 / base) * base);
+        // dx, dW_x and dW_h of both layers on the helpers: see plan_k1_helpers (config E: 1.0)
+        const double flop = 2.0 * M * K * (2.0 * I + H) + 2.0 * M * K * ((lower->dx ? 2.0 : 1.0) * lower->I + H);
+        if (flop / (n_helpers * 3.5e9) > 1.25 * T * 3.6e-3) return false;
+    }
     while (cdiv(tiles_m, ct) > max_chunks) ct += base;
     p->n_layers = layers;
     if (lower) {
