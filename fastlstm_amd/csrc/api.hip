@@ -194,7 +194,10 @@ struct XcdCfg {
 // The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
 // and the workspace holds a ring with one slot per exchanged version.
 // `launch_rows`: batch rows of this launch (0: all B_all of them).
-bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c, int launch_rows = 0) {
+// copies > 1: that many recurrences of this shape share the launch (16-row groups only), so the unit tile has to leave
+// room for all their groups.
+bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c, int launch_rows = 0,
+                int copies = 1) {
     const int B = launch_rows ? launch_rows : B_all;
     DeviceInfo di;
     if (!(g_families.load() & 1) || device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1) return false;
@@ -218,8 +221,8 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
         if (H % cand || H / cand > 32 || cand * s < 16 || frags > (backward ? 32 : 64)) continue;
         // groups per XCD: as many as its 32 CUs hold, and no more than the workspace has barrier counters for
         const int groups_max = kNumXcd * std::min(32 / (H / cand), kXcdMaxGroups / kNumXcd);
-        if (cdiv(B, 16) <= groups_max) { ht = cand; c->ntw = 1; }
-        else if (cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
+        if (copies * cdiv(B, 16) <= groups_max) { ht = cand; c->ntw = 1; }
+        else if (copies == 1 && cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
     }
     if (!ht) return false;
     c->mt = ht / rows;
@@ -228,9 +231,9 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
     c->gpx = std::min(32 / c->n_ht, kXcdMaxGroups / kNumXcd);
     const int bt = 16 * c->ntw;
     c->n_groups = cdiv(B, bt);
-    if (c->n_groups > kNumXcd * c->gpx) return false;   // (the tile loop above guarantees it; the kernels index counters by group)
+    if (copies * c->n_groups > kNumXcd * c->gpx) return false;   // (the tile loop above guarantees it; the kernels index counters by group)
     c->xslot = (size_t)c->n_groups * c->ntw * c->ks * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)copies * c->xslot) return false;
     const int gseg = ht * s;
     const int red_blocks = backward ? 8 * c->mt * c->ntw : 4 * c->mt * c->ntw;
     c->lds = red_blocks * kFragBytes + bt * (4 * gseg + 16) + 2 * bt * (gseg + 16);
@@ -314,7 +317,8 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
                 const void *bx = nullptr, const void *bh = nullptr, int I = 0, const SecondLayer *second = nullptr,
                 bool dry_run = false, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
-    if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c, o.rows)) return 1;
+    const int copies = (second && !x) ? 2 + o.n_more : 1;   // independent recurrences side by side
+    if (!select_xcd(T, B, H, dtype, false, ws_bytes, &c, o.rows, copies)) return copies > 1 ? 2 : 1;
     if (second && ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * 2 * c.xslot) return 2;   // both layers' slots side by side
     FwdXcdParams p{};
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
@@ -671,7 +675,8 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
                 const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false,
                 bool *lower_wgrad_fused = nullptr, const LaunchOpts &o = LaunchOpts()) {
     XcdCfg c;
-    if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c, o.rows)) return 1;
+    const int copies = (lower && !extras) ? 2 + o.n_more : 1;   // independent recurrences side by side
+    if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c, o.rows, copies)) return copies > 1 ? 2 : 1;
     if (lower && ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * 2 * c.xslot) return 2;   // both layers' slots side by side
     BwdXcdParams p{};
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
