@@ -48,9 +48,34 @@ def draw(seed):
                 state_grads=r.random() < 0.5)
 
 
+# Shapes at which the dispatch changes form: both directions side by side with a larger unit tile; two stacked
+# layers in one launch at a small batch (chunks of 64 timesteps); reverse launches that keep all, only dx, or none
+# of their GEMMs inside; row ranges of 32-row groups; a remainder of rows behind full fp32 register-resident
+# launches; small hidden sizes that run as 64 / 80.
+FORMS = [
+    dict(dt=torch.float16, kw=dict(bidirectional=True, bias=True, batch_first=False), layers=1, T=64, B=128, I=256, H=256),
+    dict(dt=torch.float16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=2, T=256, B=16, I=1024, H=1024),
+    dict(dt=torch.float16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=1, T=64, B=128, I=768, H=768),
+    dict(dt=torch.bfloat16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=1, T=64, B=256, I=384, H=384),
+    dict(dt=torch.bfloat16, kw=dict(bidirectional=False, bias=False, batch_first=True), layers=1, T=40, B=1024, I=512, H=512),
+    dict(dt=torch.float32, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=1, T=20, B=144, I=64, H=1024),
+    dict(dt=torch.float16, kw=dict(bidirectional=True, bias=True, batch_first=False), layers=2, T=40, B=24, I=48, H=48),
+    dict(dt=torch.float32, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=2, T=40, B=24, I=48, H=48),
+]
+
+
+@pytest.mark.parametrize("form", range(len(FORMS)))
+def test_module_against_nn_lstm_where_the_dispatch_changes_form(form):
+    c = dict(FORMS[form], states=form % 2 == 0, packed=False, state_grads=form % 3 == 0)
+    _check(c, 100 + form)
+
+
 @pytest.mark.parametrize("seed", range(48))
 def test_module_against_nn_lstm(seed):
-    c = draw(seed)
+    _check(draw(seed), seed)
+
+
+def _check(c, seed):
     dt, kw, layers, T, B, I, H = c["dt"], c["kw"], c["layers"], c["T"], c["B"], c["I"], c["H"]
     D = 2 if kw["bidirectional"] else 1
     torch.manual_seed(seed)
