@@ -1313,7 +1313,7 @@ class FastLSTM(nn.Module):
         idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
         H, I = self.hidden_size, self.input_size
         Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx) or H
-        Ip = -(-I // 64) * 64 if dt != torch.float32 and I > 64 and T * B >= 1024 and data.shape[-1] == I else I
+        Ip = -(-I // 64) * 64 if dt != torch.float32 and T * B >= 1024 and data.shape[-1] == I else I
         return (Hp, Ip) if (Hp, Ip) != (H, I) else None
 
     def _forward_operands_padded(self, x, h_c_0, Hp, Ip):
