@@ -1271,7 +1271,7 @@ def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I
 
 
 @pytest.mark.parametrize("kw,B,H,dt", [(dict(), 400, 1024, torch.float16), (dict(bidirectional=True), 200, 1536, torch.bfloat16)])
-def test_packed_batch_larger_than_one_launch_is_cut_at_its_row_ranges(kw, B, H, dt):
+def test_packed_batch_larger_than_one_launch_is_cut_at_its_row_ranges(kw, B, H, dt, monkeypatch):
     """A packed batch that the library runs as several launches over ranges of rows is cut at those ranges in
     the packed order, and every range stops at its own longest sequence: same contract, against nn.LSTM in
     fp32 on the CPU (packed data, final states, every gradient; unsorted lengths, initial states given)."""
@@ -1290,8 +1290,9 @@ def test_packed_batch_larger_than_one_launch_is_cut_at_its_row_ranges(kw, B, H, 
     xr = pack_sequence(seqs, enforce_sorted=False)
     xg = pack_sequence([t.cuda().to(dt) for t in seqs], enforce_sorted=False)
     cuts = []
-    run_padded = m._run_padded
-    m._run_padded = lambda x, *a: (cuts.append(tuple(x.shape[:2])), run_padded(x, *a))[1]
+    run_padded = L.FastLSTM._run_padded
+    for cls in (L.FastLSTM, L._OperandsPadded):   # (the module itself, and its view with zero-padded sizes)
+        monkeypatch.setattr(cls, "_run_padded", lambda self, x, *a: (cuts.append(tuple(x.shape[:2])), run_padded(self, x, *a))[1])
     y, (hn, cn) = m(xg, (h0.cuda().to(dt), c0.cuda().to(dt)))
     # several ranges, the later ones shorter than the first
     assert len(cuts) > 1 and sum(b for _, b in cuts) == B and cuts[0][0] == Tmax and cuts[-1][0] < Tmax, cuts
