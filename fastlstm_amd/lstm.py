@@ -192,7 +192,7 @@ def _wavefront_chunks(L, T, B, H, dtype, device, backward):
     # chunks of at least 64 timesteps: every launch costs about 50 us besides its steps (launch gaps, the prologue,
     # the small GEMMs in between), which a chunk of 32 steps does not win back (measured: no gain at T = 256 with
     # 8 chunks); whole 16-byte units per timestep, so that every chunk's buffers start on a 16-byte boundary
-    if T < 256 or (B * H * torch.empty((), dtype=dtype).element_size()) % 16:
+    if T < 128 or (B * H * torch.empty((), dtype=dtype).element_size()) % 16:
         return 0
     for n in (8, 6, 5, 4, 3, 2):
         if T % n == 0 and T // n >= 64 and multi_runs_in_one_launch(L, T // n, B, H, dtype, device, backward):
