@@ -1204,7 +1204,8 @@ class FastLSTM(nn.Module):
                 # where the library runs PAIRS of these layers in one launch with the GEMMs hidden inside, and the
                 # GEMMs are large, pairs win over the whole pass (4 x (T = 1024, B = 32, I = H = 1024): forward +
                 # backward 13.3 ms in pairs, 14.2 four at a time; forward alone 5.3 vs 4.7)
-                if width >= 3 and not _small_projections(x.shape[1], self.hidden_size, self.hidden_size) and \
+                # (a forward pass that no backward pass follows goes four at a time)
+                if width >= 3 and not inference and not _small_projections(x.shape[1], self.hidden_size, self.hidden_size) and \
                         stack2_runs_in_one_launch(x.shape[0], x.shape[1], x.shape[2], self.hidden_size, dt_, x.device):
                     width = 0
                 if width >= 3:
