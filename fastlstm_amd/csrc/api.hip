@@ -428,7 +428,8 @@ struct WideCfg {
     int v;    // reverse kernel, 64-row groups: members of a team that splits K (lstm_bwd_wide_split_kernel); 0 = no teams
     size_t xslot;
 };
-bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0) {
+// copies > 1: that many recurrences of this shape share the launch (groups of 16 or 32 rows only).
+bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, WideCfg *c, int rows = 0, int copies = 1) {
     const int B = rows ? rows : B_all;   // rows of this launch
     DeviceInfo di;
     if (!(g_families.load() & 2) || device_info(-1, &di) != FASTLSTM_OK || di.xcd_round_robin != 1 || di.num_cus < kNumXcd * 32)
@@ -443,19 +444,20 @@ bool select_wide(int T, int B_all, int H, int dtype, bool backward, size_t ws_by
     c->xpg = cdiv(c->n_ht, 32);   // XCDs per group (the last one partly used when H is not a multiple of 512)
     // groups of 16 or 32 rows where they all fit the launch: more groups = more CUs for a small batch, and a
     // CU then fetches a quarter or half of the operand bytes per step
-    c->nt = cdiv(B, 16) * c->xpg <= kNumXcd ? 1 : cdiv(B, 32) * c->xpg <= kNumXcd ? 2 : 4;
+    c->nt = copies * cdiv(B, 16) * c->xpg <= kNumXcd ? 1 : copies * cdiv(B, 32) * c->xpg <= kNumXcd ? 2 : 4;
+    if (copies > 1 && c->nt == 4) return false;
     // fp32 multiplies at 1/16 of the 16-bit rate: 16 units x 64 rows per CU are more MFMA time than a step of the
     // general kernels, which spread 4 units x all rows over every CU
     if (dtype == FASTLSTM_FP32 && c->nt == 4) return false;
     c->n_groups = cdiv(B, 16 * c->nt);
-    if (c->n_groups * c->xpg > kNumXcd) return false;
+    if (copies * c->n_groups * c->xpg > kNumXcd) return false;
     // ... and a small fp32 batch leaves most CUs without a share of the forward product (B = 32, H = 1024: 6.0
     // instead of 5.7 us per step; the reverse step, with four times the operand bytes, gains at every size)
     // (a remainder of rows behind full launches still runs here: the general kernel would take the whole batch)
-    if (dtype == FASTLSTM_FP32 && !backward && c->n_groups * c->xpg < 6 && B == B_all) return false;
+    if (dtype == FASTLSTM_FP32 && !backward && copies * c->n_groups * c->xpg < 6 && B == B_all) return false;
     c->ks = (backward ? 4 * H : H) / kstep;
     c->xslot = (size_t)c->n_groups * c->nt * c->ks * kFragBytes;
-    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * c->xslot) return false;
+    if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)copies * c->xslot) return false;
     const int gr = 16 * c->nt;
     const int gseg = 16 * es;
     const int tiles = gr * (4 * gseg + 16) + 2 * gr * (gseg + 16);   // gates + two state tiles of `gr` rows x 16 units
@@ -485,11 +487,21 @@ static int wide_rows_per_launch(int T, int B, int H, int dtype, bool backward, s
 }
 
 // Returns 1 when the kernel does not apply, else a fastlstm_status.
+// `second` (+ o.more): independent recurrences of the same shape side by side in the launch, as try_fwd_xcd takes them.
 int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned char *wsb, size_t ws_bytes, int T, int B,
-                 int H, int dtype, hipStream_t stream, const LaunchOpts &o = LaunchOpts()) {
+                 int H, int dtype, hipStream_t stream, const LaunchOpts &o = LaunchOpts(), const SecondLayer *second = nullptr,
+                 bool dry_run = false) {
     WideCfg c;
-    if (!select_wide(T, B, H, dtype, false, ws_bytes, &c, o.rows)) return 1;
+    const int copies = second ? 2 + o.n_more : 1;
+    if (copies > kMaxSideBySide || !select_wide(T, B, H, dtype, false, ws_bytes, &c, o.rows, copies)) return 1;
     FwdXcdParams p{};
+    p.n_layers = copies;
+    if (second) {
+        p.ifgo2 = second->ifgo; p.out2 = second->out; p.cell2 = second->cell; p.Wh2 = second->Wh;
+        for (int i = 0; i < o.n_more; ++i) {
+            p.ifgo_more[i] = o.more[i][0]; p.out_more[i] = o.more[i][1]; p.cell_more[i] = o.more[i][2]; p.Wh_more[i] = o.more[i][3];
+        }
+    }
     p.ifgo = ifgo; p.out = out; p.cell = cell; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
     p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);   // here: one flag per workgroup
@@ -503,16 +515,31 @@ int try_fwd_wide(void *ifgo, void *out, void *cell, const void *Wh, unsigned cha
     int occ = 0;
     if (launch(p, c.nkw, c.nt, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
+    if (dry_run) return FASTLSTM_OK;
     if (launch(p, c.nkw, c.nt, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
 
+// `second` (7 operand pointers in the order of this call's own; + o.more): independent recurrences of the same shape
+// side by side in the launch.
 int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                  unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
-                 const LaunchOpts &o = LaunchOpts()) {
+                 const LaunchOpts &o = LaunchOpts(), void *const *second = nullptr, bool dry_run = false) {
     WideCfg c;
-    if (!select_wide(T, B, H, dtype, true, ws_bytes, &c, o.rows)) return 1;
+    const int copies = second ? 2 + o.n_more : 1;
+    if (copies > kMaxSideBySide || !select_wide(T, B, H, dtype, true, ws_bytes, &c, o.rows, copies)) return 1;
+    if (copies > 1) c.v = 0;   // (never set: the team form is for 64-row groups)
     BwdXcdParams p{};
+    p.n_layers = copies;
+    if (second) {
+        p.k5.C = second[0];   // the kernels read the second recurrence's dout from there
+        p.dh_lo = second[1]; p.dc_lo = second[2]; p.ifgo_lo = second[3]; p.cell_lo = second[4];
+        p.d_ifgo_lo = second[5]; p.Wh_lo = second[6];
+        for (int i = 0; i < o.n_more; ++i) {
+            p.dout_more[i] = o.more[i][0]; p.dh_more[i] = o.more[i][1]; p.dc_more[i] = o.more[i][2]; p.ifgo_more[i] = o.more[i][3];
+            p.cell_more[i] = o.more[i][4]; p.d_ifgo_more[i] = o.more[i][5]; p.Wh_more[i] = o.more[i][6];
+        }
+    }
     p.dout = dout; p.dh = dh; p.dc = dc; p.ifgo = ifgo; p.cell = cell; p.d_ifgo = d_ifgo; p.Wh = Wh;
     p.hdr = reinterpret_cast<WsHeader *>(wsb);
     p.counters = reinterpret_cast<int *>(wsb + kWsHeaderBytes);   // here: one flag per workgroup
@@ -528,6 +555,7 @@ int try_bwd_wide(const void *dout, void *dh, void *dc, const void *ifgo, const v
     int occ = 0;
     if (launch(p, c.nkw, form, 0, c.lds, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
     if (occ < 1) return 1;
+    if (dry_run) return FASTLSTM_OK;
     if (launch(p, c.nkw, form, kNumXcd * 32, c.lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
     return FASTLSTM_OK;
 }
@@ -1134,11 +1162,13 @@ static int try_multi(bool backward, int n, void *const (*recs)[7], void *ws, siz
         const SecondLayer second{nullptr, nullptr, nullptr, b[3], b[0], b[1], b[2]};
         rc = try_fwd_xcd(a[0], a[1], a[2], a[3], wsb, ws_bytes, T, B, H, dtype, s, nullptr, nullptr, nullptr, nullptr, 0, &second,
                          dry_run, o);
+        if (rc == 1 || rc == 2) rc = try_fwd_wide(a[0], a[1], a[2], a[3], wsb, ws_bytes, T, B, H, dtype, s, o, &second, dry_run);
     } else {
         LowerLayer lower{b[1], b[2], b[3], b[4], b[5], b[6], nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr};
         lower.dout = b[0];
         rc = try_bwd_xcd(a[0], a[1], a[2], a[3], a[4], a[5], a[6], wsb, ws_bytes, T, B, H, dtype, s, nullptr, &lower, dry_run,
                          nullptr, o);
+        if (rc == 1 || rc == 2) rc = try_bwd_wide(a[0], a[1], a[2], a[3], a[4], a[5], a[6], wsb, ws_bytes, T, B, H, dtype, s, o, b, dry_run);
     }
     return rc == 2 ? 1 : rc;
 }

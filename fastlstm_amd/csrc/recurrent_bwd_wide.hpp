@@ -48,8 +48,15 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
     // ---- placement: group g on XCDs g*xpg .. (hardware deals workgroup i to XCD i % 8) --------
     const int xpg = p.gpx;
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
-    const int g = xcd / xpg, j = (xcd % xpg) * 32 + slot;
-    if (g >= p.n_groups || j >= p.n_ht) return;
+    // several independent recurrences of one shape may share the launch (p.n_layers; NT <= 2), as in the forward kernel
+    const int n_rec = NT <= 2 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1;
+    const int vg = xcd / xpg, j = (xcd % xpg) * 32 + slot;
+    if (vg >= n_rec * p.n_groups || j >= p.n_ht) return;
+    const int rec = vg / p.n_groups, g = vg - rec * p.n_groups;
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {   // (constant indices only, see the forward kernel)
+        if constexpr (NT > 2) return a0;
+        else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
+    };
     check_xcd_placement(p.hdr);
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
 
@@ -58,11 +65,13 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
     unsigned char *ring = tiles + BT * GROW + 2 * BT * SROW + (size_t)wave * S * kFragBytes;   // this wave's blocks
     const int io_tid = tid - kWave;
 
-    const T *dout = static_cast<const T *>(p.dout);
-    const T *ifgo = static_cast<const T *>(p.ifgo);
-    const T *cell = static_cast<const T *>(p.cell);
-    T *d_ifgo = static_cast<T *>(p.d_ifgo);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    const T *dout = static_cast<const T *>(pick(p.dout, static_cast<const void *>(p.k5.C), p.dout_more[0], p.dout_more[1]));
+    const T *ifgo = static_cast<const T *>(pick(p.ifgo, p.ifgo_lo, p.ifgo_more[0], p.ifgo_more[1]));
+    const T *cell = static_cast<const T *>(pick(p.cell, p.cell_lo, p.cell_more[0], p.cell_more[1]));
+    T *d_ifgo = static_cast<T *>(pick(p.d_ifgo, p.d_ifgo_lo, p.d_ifgo_more[0], p.d_ifgo_more[1]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh_lo, p.Wh_more[0], p.Wh_more[1]));
+    T *dh_state = static_cast<T *>(pick(p.dh, p.dh_lo, p.dh_more[0], p.dh_more[1]));
+    T *dc_state_buf = static_cast<T *>(pick(p.dc, p.dc_lo, p.dc_more[0], p.dc_more[1]));
 
     // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
     // fragment k-step ks = wave + 8 ki: lane (q, r) holds row r = unit u0 + r and
@@ -99,14 +108,14 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
         roff[m] = ((nt < NT ? nt : 0) * kWave + (ul >> 2) * 16 + n) * 4 + (ul & 3);
         goff[m] = (nt * 16 + n) * GROW + ul * E::BYTES;
         soff[m] = (nt * 16 + n) * SROW + ul * E::BYTES;
-        dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
-        dc_state[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dc)[off_h[m]]) : 0.f;
+        dh_rec[m] = valid[m] ? E::to_f32(dh_state[off_h[m]]) : 0.f;
+        dc_state[m] = valid[m] ? E::to_f32(dc_state_buf[off_h[m]]) : 0.f;
         c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
     }
 
-    const unsigned xgrp = (unsigned)g * NT * KSB * kFragBytes;
-    const size_t xslot = (size_t)p.n_groups * NT * KSB * kFragBytes;
-    int *grp_flags = p.counters + (size_t)g * kXcdGroupStride;   // one flag per workgroup of the group
+    const unsigned xgrp = (unsigned)vg * NT * KSB * kFragBytes;
+    const size_t xslot = (size_t)n_rec * p.n_groups * NT * KSB * kFragBytes;
+    int *grp_flags = p.counters + (size_t)vg * kXcdGroupStride;   // one flag per workgroup of the group
 
     // ---- coalesced tile I/O: ifgo[t], cell[t], dout[t] in, d_ifgo[t] out (two sets in flight) ----
     u32x4 gpre[2][GPT], cpre[2][SPT], dpre[2][SPT];
@@ -227,7 +236,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
         tile_to_global(t);
         if (s + 2 < T_) fetch_tiles(t - 2, gpre[PAR], cpre[PAR], dpre[PAR]);
 
-        if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, g, s);
+        if (wave == 0) wait_versions(grp_flags, p.n_ht, s + 1, p.hdr, p.spin_limit, vg, s);
         __syncthreads();
 
         // ---- dh_rec(units, rows) = Wh[:, units]^T . d_ifgo[t](rows, :)^T over this wave's k-steps ----
@@ -278,7 +287,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdPa
         if (s + 1 < T_) step(s + 1, std::integral_constant<int, 1>{});
     }
 
-    T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
+    T *dh_out = dh_state, *dc_out = dc_state_buf;
 #pragma unroll
     for (int m = 0; m < IPT; ++m)
         if (valid[m]) {

@@ -55,19 +55,28 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     // ---- placement: group g on XCDs g*xpg .. (hardware deals workgroup i to XCD i % 8) --------
     const int xpg = p.gpx;   // XCDs per group
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
-    const int g = xcd / xpg, j = (xcd % xpg) * 32 + slot;
-    if (g >= p.n_groups || j >= p.n_ht) return;
+    // several independent recurrences of one shape may share the launch (p.n_layers; NT <= 2): recurrence r takes the
+    // groups r * n_groups ... of the launch, with its own operands, flags and exchange blocks
+    const int n_rec = NT <= 2 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1;
+    const int vg = xcd / xpg, j = (xcd % xpg) * 32 + slot;
+    if (vg >= n_rec * p.n_groups || j >= p.n_ht) return;
     check_xcd_placement(p.hdr);
+    const int rec = vg / p.n_groups, g = vg - rec * p.n_groups;
+    // (constant indices only: a run-time index into the kernel's arguments would move them all to scratch memory)
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
+        if constexpr (NT > 2) return a0;
+        else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
+    };
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch
 
     f32x4 *red = reinterpret_cast<f32x4 *>(smem);                                       // [8][TILES][64]
     unsigned char *tiles = reinterpret_cast<unsigned char *>(red + NWV * TILES * kWave);   // gates, h, c tiles
     const int io_tid = tid - kWave;
 
-    T *ifgo = static_cast<T *>(p.ifgo);
-    T *out = static_cast<T *>(p.out);
-    T *cell = static_cast<T *>(p.cell);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    T *ifgo = static_cast<T *>(pick(p.ifgo, p.ifgo2, p.ifgo_more[0], p.ifgo_more[1]));
+    T *out = static_cast<T *>(pick(p.out, p.out2, p.out_more[0], p.out_more[1]));
+    T *cell = static_cast<T *>(pick(p.cell, p.cell2, p.cell_more[0], p.cell_more[1]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh2, p.Wh_more[0], p.Wh_more[1]));
 
     // ---- prologue 1: this wave's fragments of the W_h slice, global -> registers ---------
     // fragment (m-tile a, k-step ks = wave + 8 ki): lane (q, r) holds row r = (unit a*4 + r/4, gate r%4),
@@ -102,9 +111,9 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
     }
 
     // two exchange slots: h_s lives in slot s % 2
-    const unsigned xgrp = (unsigned)g * NT * KS * kFragBytes;
-    const size_t xslot = (size_t)p.n_groups * NT * KS * kFragBytes;
-    int *grp_flags = p.counters + (size_t)g * kXcdGroupStride;   // n_ht <= kXcdGroupStride flags per group
+    const unsigned xgrp = (unsigned)vg * NT * KS * kFragBytes;
+    const size_t xslot = (size_t)n_rec * p.n_groups * NT * KS * kFragBytes;
+    int *grp_flags = p.counters + (size_t)vg * kXcdGroupStride;   // n_ht <= kXcdGroupStride flags per group
     auto publish = [&](int version) { publish_version(grp_flags + j, version); };
 
     // ---- prologue 2: publish h_0 (slot 0) as version 1 -------------------------------------
@@ -188,7 +197,7 @@ __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdPa
 
     auto step = [&](const int t) __attribute__((always_inline)) {
         unsigned char *gt = tiles;
-        if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, g, t);
+        if (wave == 0) wait_versions(grp_flags, p.n_ht, t + 1, p.hdr, p.spin_limit, vg, t);
         __syncthreads();
 
         // ---- partial(a, i) = Wslice(a, this wave's k-steps) . h_{t-1}(i)^T, one batch tile i per pass.

@@ -647,6 +647,10 @@ PAIR_CASES = [
     (4, 64, 128, 1024, torch.bfloat16, True),     # config B's tiles: 4 + 4 groups on the 8 XCDs
     (3, 200, 64, 1024, torch.float16, False),     # 7 + 7 groups of 32 rows do not fit: one after the other
     (4, 24, 48, 72, torch.float16, False),        # general kernels: one after the other
+    (5, 16, 64, 2048, torch.bfloat16, True),      # register-resident kernels: one 16-row group each, 4 XCDs per group
+    (4, 32, 64, 1536, torch.float16, True),       # ... one 32-row group each on 3 XCDs (alone: two 16-row groups)
+    (3, 24, 64, 1024, torch.float32, True),       # ... fp32
+    (3, 64, 64, 2048, torch.float16, False),      # 64-row groups: one after the other
 ]
 
 
@@ -667,8 +671,11 @@ def test_two_recurrences_side_by_side_equal_two_calls(T, B, I, H, dt, fused):
     fwd_keys = ("x", "h0", "c0", "Wx", "bx", "Wh", "bh")
     got = L.lstm_persistent_fwd_pair(*(a[k] for k in fwd_keys), *(b[k] for k in fwd_keys))
     want = L.lstm_persistent_fwd(*(a[k] for k in fwd_keys)) + L.lstm_persistent_fwd(*(b[k] for k in fwd_keys))
+    # (the register-resident kernels take 32-row groups for two recurrences where one alone gets 16-row groups: the
+    # eight partial sums of a tile are then added starting from another wave's -- fp32 results agree to rounding)
+    same_bits = lambda x_, y_: torch.equal(x_, y_) if not (dt == torch.float32 and H >= 640) else rel_err(x_, npy(y_)) < 1e-6
     for name, g_, w_ in zip(("out_a", "cell_a", "ifgo_a", "out_b", "cell_b", "ifgo_b"), got, want):
-        assert torch.equal(g_, w_), name
+        assert same_bits(g_, w_), name
     ga, gb = L.lstm_persistent_bwd_pair(a["dout"], (a["dh_n"], a["dc_n"]), a["x"], got[0], got[1], got[2], a["Wx"], a["Wh"],
                                         b["dout"], (b["dh_n"], b["dc_n"]), b["x"], got[3], got[4], got[5], b["Wx"], b["Wh"])
     for side, g_, (out, cell, ifgo) in ((a, ga, want[:3]), (b, gb, want[3:])):
@@ -676,7 +683,7 @@ def test_two_recurrences_side_by_side_equal_two_calls(T, B, I, H, dt, fused):
                                    side["Wx"], side["Wh"])
         for name, x_, y_ in zip(("d_x", "dh_0", "dc_0", "dWx", "dbx", "dWh", "dbh"), g_, w_):
             if name in ("dh_0", "dc_0"):
-                assert torch.equal(x_, y_), name
+                assert same_bits(x_, y_), name
             else:
                 assert rel_err(x_, npy(y_)) < tol, name
 
