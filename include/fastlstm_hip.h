@@ -107,9 +107,9 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
 
 /* K1 + K2/K3 for one layer in one call: the same results as fastlstm_gemm_ifgo followed by
  * fastlstm_fwd_persistent (same arguments, same workspace contract).  Where the XCD-local
- * recurrence leaves CUs without a role (few batch tiles), the workgroups on those CUs compute the
- * input projection inside the same launch, earliest timesteps first, and the recurrence follows
- * them chunk by chunk; otherwise the two stages are launched back to back.  Replaces
+ * recurrence leaves CUs without a role (few batch tiles) and those CUs keep up with the recurrence, the
+ * workgroups on them compute the input projection inside the same launch, earliest timesteps first, and
+ * the recurrence follows them chunk by chunk; otherwise the two stages are launched back to back.  Replaces
  * fastlstm/lstm.py:66-68 together with 131-142. */
 int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh,
                        void *ifgo, void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I,
@@ -217,8 +217,9 @@ size_t fastlstm_multi_workspace_bytes(const fastlstm_plan *plan, int n, int T, i
  * fastlstm_gemm_dx and fastlstm_gemm_wgrad one after the other (same arguments and workspace
  * contracts; dWx and dWh to the rounding of a different summation order).  Where the XCD-local
  * reverse recurrence leaves CUs without a role, the workgroups on those CUs compute dx and the
- * weight gradients inside the same launch, chunk of timesteps by chunk behind the recurrence;
- * otherwise the stages are launched back to back.  Replaces fastlstm/lstm.py:277-290, 294 and
+ * weight gradients (or dx alone, whichever an estimate of their throughput makes the shorter call) inside
+ * the same launch, chunk of timesteps by chunk behind the recurrence; otherwise the stages are launched
+ * back to back.  Replaces fastlstm/lstm.py:277-290, 294 and
  * 494-501 together. */
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
                        void *d_ifgo, const void *Wh, const void *Wx, const void *x, const void *h,
