@@ -213,10 +213,9 @@ def stack2_wavefront_chunks(T, B, H, dtype, device, backward=False):
 
 
 def _small_projections(B, I, H):
-    """The library's own two-layer launch hides the GEMMs behind the time loops but fills its pipeline slowly; the
-    chunked wavefront leaves the GEMMs in the open and overlaps the time loops better.  Where the GEMMs are a few
-    per cent of a step anyway the wavefront wins (T = 256 ... 512, B = 16, I = H = 640: forward + backward 2.3 vs
-    2.6 and 3.7 vs 4.2 ms); B = 32, I = H = 1024 and B = 64, I = H = 768 are past the crossover."""
+    """Three or four stacked layers: the wavefront of chunked launches leaves the GEMMs in the open, the library's
+    two-layer launches (pair by pair) hide them behind the time loops.  Where the GEMMs are a few per cent of a step
+    the wavefront wins; B = 32, I = H = 1024 and B = 64, I = H = 768 are past the crossover for a training pass."""
     return B * I * H < 1.5e7
 
 
@@ -428,7 +427,8 @@ def lstm_persistent_fwd_stack2(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, b
     lib = _lib.load()
     with torch.cuda.device(x.device):
         n = stack2_wavefront_chunks(T, B, H, x.dtype, x.device)
-        if n and (_small_projections(B, I, H) or not stack2_runs_in_one_launch(T, B, I, H, x.dtype, x.device)):
+        # (the library's own two-layer launch, with the GEMMs inside, wins wherever it applies)
+        if n and not stack2_runs_in_one_launch(T, B, I, H, x.dtype, x.device):
             return _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, Wh1, bh1, n, keep_activations)
         bufs = []
         for h0, c0 in ((h0a, c0a), (h0b, c0b)):
@@ -533,8 +533,7 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
     with torch.cuda.device(x.device):
         plan = _plan(x.device, B, H, code, True)
         n = stack2_wavefront_chunks(T, B, H, ifgo1.dtype, x.device, backward=True)
-        if n and (_small_projections(B, I, H) or lib.fastlstm_bwd_stack2_fused(
-                T, B, I, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) != 1):
+        if n and lib.fastlstm_bwd_stack2_fused(T, B, I, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) != 1:
             return _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1,
                                          d_state0, d_state1, n)
         dh = dh.contiguous()
