@@ -890,8 +890,11 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
 }
 
 // keep: see LaunchOpts
+// others / n_others: further independent recurrences of this shape (operands in the order ifgo, out, cell, Wh) that
+// share every launch -- only where the plan is the one-tile form (wave_split 2: no exchange between workgroups).
 static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
-                               int H, int dtype, void *stream, int keep) {
+                               int H, int dtype, void *stream, int keep, void *const (*others)[7] = nullptr,
+                               int n_others = 0) {
     if (!ifgo || !out || !cell || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
@@ -901,6 +904,7 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     const bool sync = pl.wave_split != 2;
+    if (n_others && (sync || n_others > 3)) return FASTLSTM_ERR_DIM;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (pl.wave_split == 3) {   // W_h does not fit on chip: pack it once, then stream it every step
@@ -977,6 +981,10 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     p.spin_limit = spin_limit_ticks();
     p.keep = keep;
     p.trace = g_rec_trace;
+    p.n_rec = 1 + n_others;
+    for (int i = 0; i < n_others; ++i) {
+        p.ifgo_x[i] = others[i][0]; p.out_x[i] = others[i][1]; p.cell_x[i] = others[i][2]; p.Wh_x[i] = others[i][3];
+    }
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, false);
@@ -1003,7 +1011,8 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
         p.b_base = bt0 * pl.bt;
-        const int grid = n_bt * pl.n_htiles;
+        p.n_bt_launch = n_bt;
+        const int grid = p.n_rec * n_bt * pl.n_htiles;
         int occ = 0;
         if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
@@ -1020,9 +1029,10 @@ int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, v
     return finish_recurrent(fwd_persistent_impl(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream, 1), ws, stream);
 }
 
+// others / n_others: see fwd_persistent_impl (operands in the order of this call's own seven).
 static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
                                void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
-                               int dtype, void *stream) {
+                               int dtype, void *stream, void *const (*others)[7] = nullptr, int n_others = 0) {
     if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
@@ -1033,6 +1043,7 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
     if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     const bool sync = pl.wave_split != 2;
+    if (n_others && (sync || n_others > 3)) return FASTLSTM_ERR_DIM;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (pl.wave_split == 3) {   // W_h does not fit on chip: pack Wh[:, units]^T once, then stream it every step
@@ -1104,6 +1115,11 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
     p.ht = pl.ht;
     p.spin_limit = spin_limit_ticks();
     p.trace = g_rec_trace;
+    p.n_rec = 1 + n_others;
+    for (int i = 0; i < n_others; ++i) {
+        p.dout_x[i] = others[i][0]; p.dh_x[i] = others[i][1]; p.dc_x[i] = others[i][2]; p.ifgo_x[i] = others[i][3];
+        p.cell_x[i] = others[i][4]; p.d_ifgo_x[i] = others[i][5]; p.Wh_x[i] = others[i][6];
+    }
     const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, true);
@@ -1122,7 +1138,8 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;
         p.b_base = bt0 * pl.bt;
-        const int grid = n_bt * pl.n_htiles;
+        p.n_bt_launch = n_bt;
+        const int grid = p.n_rec * n_bt * pl.n_htiles;
         int occ = 0;
         if (launch(p, pl.ht, pl.bt, pl.wave_split, 0, lds_bytes, nullptr, &occ) != hipSuccess) return FASTLSTM_ERR_HIP;
         if (sync && (long long)occ * pl.num_cus < grid) return FASTLSTM_ERR_RESIDENCY;
@@ -1149,10 +1166,16 @@ static int try_multi(bool backward, int n, void *const (*recs)[7], void *ws, siz
     if (n < 2 || n > kMaxSideBySide) return 1;
     fastlstm_plan pl;
     if (int rc = plan_device(-1, B, H, dtype, backward ? 1 : 0, &pl, false)) return rc;
-    if (pl.wave_split == 2 || pl.wave_split == 3) return 1;
+    if (pl.wave_split == 3) return 1;
+    void *const *a = recs[0], *const *b = recs[1];
+    if (pl.wave_split == 2) {   // the one-tile form: no exchange between workgroups, any number of them side by side
+        if (dry_run) return FASTLSTM_OK;
+        return backward ? bwd_persistent_impl(a[0], a[1], a[2], a[3], a[4], a[5], a[6], ws, ws_bytes, T, B, H, dtype, stream,
+                                              recs + 1, n - 1)
+                        : fwd_persistent_impl(a[0], a[1], a[2], a[3], ws, ws_bytes, T, B, H, dtype, stream, keep, recs + 1, n - 1);
+    }
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    void *const *a = recs[0], *const *b = recs[1];
     LaunchOpts o;
     o.keep = keep;
     o.n_more = n - 2;

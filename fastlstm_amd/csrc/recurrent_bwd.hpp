@@ -45,6 +45,10 @@ struct BwdParams {
     long long spin_limit;
     int vec_io;         // 1: the VIO instantiation is launched (complete, 16-byte aligned tile segments)
     long long *trace;   // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
+    // SPLIT 2 only: n_rec > 1 independent recurrences of this shape share the launch (see FwdParams)
+    int n_rec, n_bt_launch;
+    const void *dout_x[3], *ifgo_x[3], *cell_x[3], *Wh_x[3];
+    void *dh_x[3], *dc_x[3], *d_ifgo_x[3];
 };
 
 // SPLIT 0: waves split K (NTW n-tiles per WG); SPLIT 1: waves split N (NTW n-tiles per wave);
@@ -85,6 +89,17 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
         g = blockIdx.x;
         j = 0;
     }
+    int rec = 0;   // which recurrence of the launch
+    if constexpr (!SYNC) {
+        if (p.n_rec > 1) {
+            rec = blockIdx.x / p.n_bt_launch;
+            g = blockIdx.x - rec * p.n_bt_launch;
+        }
+    }
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {   // (constant indices only, see the forward kernel)
+        if constexpr (SYNC) return a0;
+        else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
+    };
     const int u0 = j * HT;
     const int b0 = p.b_base + g * BT;
 
@@ -107,11 +122,13 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KSB * kFragBytes);   // SYNC: 1 set, else 2 (step parity)
     const int io_tid = IOW ? tid - kThreads : tid - kWave;   // < 0: not an I/O thread
 
-    const T *dout = static_cast<const T *>(p.dout);
-    const T *ifgo = static_cast<const T *>(p.ifgo);
-    const T *cell = static_cast<const T *>(p.cell);
-    T *d_ifgo = static_cast<T *>(p.d_ifgo);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    const T *dout = static_cast<const T *>(pick(p.dout, p.dout_x[0], p.dout_x[1], p.dout_x[2]));
+    const T *ifgo = static_cast<const T *>(pick(p.ifgo, p.ifgo_x[0], p.ifgo_x[1], p.ifgo_x[2]));
+    const T *cell = static_cast<const T *>(pick(p.cell, p.cell_x[0], p.cell_x[1], p.cell_x[2]));
+    T *d_ifgo = static_cast<T *>(pick(p.d_ifgo, p.d_ifgo_x[0], p.d_ifgo_x[1], p.d_ifgo_x[2]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh_x[0], p.Wh_x[1], p.Wh_x[2]));
+    T *dh_io = static_cast<T *>(pick(p.dh, p.dh_x[0], p.dh_x[1], p.dh_x[2]));
+    T *dc_io = static_cast<T *>(pick(p.dc, p.dc_x[0], p.dc_x[1], p.dc_x[2]));
 
     // ---- prologue: Wh[:, units] -> LDS, transposed into operand order ------------------
     {
@@ -176,8 +193,8 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
         soff[m] = (nt * 16 + n) * SROW + ul * E::BYTES;
         const int mtile = ul >> 4, ur = ul & 15;
         roff[m] = ((mtile * NT + (nt < NT ? nt : 0)) * kWave + (ur >> 2) * 16 + n) * 4 + (ur & 3);
-        dh_rec[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dh)[off_h[m]]) : 0.f;
-        dc_state[m] = valid[m] ? E::to_f32(static_cast<const T *>(p.dc)[off_h[m]]) : 0.f;
+        dh_rec[m] = valid[m] ? E::to_f32(dh_io[off_h[m]]) : 0.f;
+        dc_state[m] = valid[m] ? E::to_f32(dc_io[off_h[m]]) : 0.f;
         c1v[m] = valid[m] ? E::to_f32(cell[(size_t)T_ * BH + off_h[m]]) : 0.f;
     }
 
@@ -606,7 +623,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
         }
     }
 
-    T *dh_out = static_cast<T *>(p.dh), *dc_out = static_cast<T *>(p.dc);
+    T *dh_out = dh_io, *dc_out = dc_io;
 #pragma unroll
     for (int m = 0; m < IPT; ++m)
         if (cw && valid[m]) {

@@ -45,6 +45,11 @@ struct FwdParams {
                        // 0: inference, ifgo stays the input projection and only cell[T] is written
     long long spin_limit;
     long long *trace;  // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
+    // SPLIT 2 only (no exchange between workgroups): n_rec > 1 independent recurrences of this shape share the launch,
+    // recurrence r on the workgroups r * n_bt_launch ...; operands of recurrences 1 ... in the arrays
+    int n_rec, n_bt_launch;
+    void *ifgo_x[3], *out_x[3], *cell_x[3];
+    const void *Wh_x[3];
 };
 
 // SPLIT 0: waves split K   (MT m-tiles, NTW n-tiles per WG, 4 partial sums)
@@ -92,6 +97,18 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
         g = blockIdx.x;
         j = 0;
     }
+    int rec = 0;   // which recurrence of the launch
+    if constexpr (!SYNC) {
+        if (p.n_rec > 1) {
+            rec = blockIdx.x / p.n_bt_launch;
+            g = blockIdx.x - rec * p.n_bt_launch;
+        }
+    }
+    // (constant indices only: a run-time index into the kernel's arguments would move them all to scratch memory)
+    auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
+        if constexpr (SYNC) return a0;
+        else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
+    };
     const int u0 = j * HT;                  // first hidden unit of this workgroup
     const int b0 = p.b_base + g * BT;       // first batch row
 
@@ -139,10 +156,10 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
 #else
 #define FASTLSTM_TP(ev) do {} while (0)
 #endif
-    T *ifgo = static_cast<T *>(p.ifgo);
-    T *out = static_cast<T *>(p.out);
-    T *cell = static_cast<T *>(p.cell);
-    const T *Wh = static_cast<const T *>(p.Wh);
+    T *ifgo = static_cast<T *>(pick(p.ifgo, p.ifgo_x[0], p.ifgo_x[1], p.ifgo_x[2]));
+    T *out = static_cast<T *>(pick(p.out, p.out_x[0], p.out_x[1], p.out_x[2]));
+    T *cell = static_cast<T *>(pick(p.cell, p.cell_x[0], p.cell_x[1], p.cell_x[2]));
+    const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh_x[0], p.Wh_x[1], p.Wh_x[2]));
 
     // ---- prologue 1: W_h slice -> LDS in operand order (zero padded) ----------------
     {

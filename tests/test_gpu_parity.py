@@ -651,6 +651,8 @@ PAIR_CASES = [
     (4, 32, 64, 1536, torch.float16, True),       # ... one 32-row group each on 3 XCDs (alone: two 16-row groups)
     (3, 24, 64, 1024, torch.float32, True),       # ... fp32
     (3, 64, 64, 2048, torch.float16, False),      # 64-row groups: one after the other
+    (6, 200, 48, 64, torch.float16, True),        # one hidden tile per workgroup: both recurrences' workgroups in one grid
+    (5, 33, 16, 32, torch.float32, True),
 ]
 
 
@@ -1441,7 +1443,7 @@ def test_module_without_grad_takes_the_inference_path_same_bits(kw, T, B, I, H, 
     m = FastLSTM(I, H, **kw).to("cuda", torch.float16)
     x = torch.randn(T, B, I, device="cuda").half()
     calls = []
-    for name in ("lstm_persistent_fwd", "lstm_persistent_fwd_stack2"):
+    for name in ("lstm_persistent_fwd", "lstm_persistent_fwd_stack2", "lstm_persistent_fwd_pair"):
         orig = getattr(L, name)
         monkeypatch.setattr(L, name, lambda *a, _o=orig, **k: (calls.append(k.get("keep_activations", True)), _o(*a, **k))[1])
     y, (hn, cn) = m(x)
