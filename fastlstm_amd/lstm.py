@@ -197,6 +197,10 @@ def _wavefront_chunks(L, T, B, H, dtype, device, backward):
     for n in (8, 6, 5, 4, 3, 2):
         if T % n == 0 and T // n >= 64 and multi_runs_in_one_launch(L, T // n, B, H, dtype, device, backward):
             return n
+    # no even cut: n equal chunks behind a prefix of T % n < n timesteps, which every layer runs on its own first
+    for n in (8, 6, 5, 4, 3, 2):
+        if T // n >= 64 and multi_runs_in_one_launch(L, T // n, B, H, dtype, device, backward):
+            return n
     return 0
 
 
@@ -265,21 +269,30 @@ def _fwd_stack_wavefront(x, layers, n, keep_activations):
     Wx0, bx0, bh0 = layers[0][2], layers[0][3], layers[0][5]
     _lib.check(lib.fastlstm_gemm_ifgo(p(x), p(Wx0), p(bx0), p(bh0), p(bufs[0][2]), T, B, I, H, code, stream), "fastlstm_gemm_ifgo")
     plan = _plan(dev_, B, H, code, False)
+    r = T - n * Tc   # timesteps in front of the n equal chunks (T not a multiple of n): layer by layer
     nb = lib.fastlstm_multi_workspace_bytes(plan, L, Tc, H, code, 0)
-    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1, dev_)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1 + (L if r else 0), dev_)
     keep = int(keep_activations)
     # (addresses of the chunks by arithmetic: slicing tensors would cost the host more than a short chunk runs)
     row = B * H * x.element_size()
     po, pc, pg = [p(b[0]) for b in bufs], [p(b[1]) for b in bufs], [p(b[2]) for b in bufs]
     pw = [(p(l[2]), p(l[3]), p(l[4]), p(l[5])) for l in layers]   # Wx, bx, Wh, bh
+    for l in range(L if r else 0):
+        if l >= 1:
+            _lib.check(lib.fastlstm_gemm_ifgo(po[l - 1] + row, pw[l][0], pw[l][1], pw[l][3], pg[l], r, B, H, H, code, stream),
+                       "fastlstm_gemm_ifgo")
+        ws = wss[n + L - 1 + l]
+        _lib.check(lib.fastlstm_fwd_persistent_multi(1, _ptr_array([pg[l]]), _ptr_array([po[l]]), _ptr_array([pc[l]]),
+                                                     _ptr_array([pw[l][2]]), p(ws), ws.numel(), r, B, H, code, keep, stream),
+                   "fastlstm_fwd_persistent_multi")
     for k in range(n + L - 1):
         active = [l for l in range(L) if 0 <= k - l < n]
         for l in active:
             if l >= 1:   # this layer's projection of the chunk the layer below has just finished
-                t = (k - l) * Tc
+                t = r + (k - l) * Tc
                 _lib.check(lib.fastlstm_gemm_ifgo(po[l - 1] + (1 + t) * row, pw[l][0], pw[l][1], pw[l][3], pg[l] + t * 4 * row,
                                                   Tc, B, H, H, code, stream), "fastlstm_gemm_ifgo")
-        t_of = [(k - l) * Tc for l in active]
+        t_of = [r + (k - l) * Tc for l in active]
         ws = wss[k]
         _lib.check(lib.fastlstm_fwd_persistent_multi(
             len(active), _ptr_array([pg[l] + t * 4 * row for l, t in zip(active, t_of)]),
@@ -315,8 +328,9 @@ def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
     # douts[l]: gradient of layer l's out[1:]: dh for the top layer, the dx of layer l + 1 below it
     douts = [torch.empty((T, B, H), device=dev_, dtype=dt) for _ in range(L - 1)] + [dh]
     plan = _plan(dev_, B, H, code, True)
+    r = T - n * Tc   # the prefix of the forward pass: here behind the chunks, layer by layer from the top
     nb = lib.fastlstm_multi_workspace_bytes(plan, L, Tc, H, code, 1)
-    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1, dev_)
+    wss = _chunk_workspaces(nb, nb if plan.ring_needs_zero else min(nb, plan.ws_zero_bytes), n + L - 1 + (L if r else 0), dev_)
     row = B * H * dh.element_size()
     pdo, pdg = [p(t) for t in douts], [p(t) for t in d_ifgo]
     pg, pc = [p(a[2]) for a in acts], [p(a[1]) for a in acts]
@@ -325,7 +339,7 @@ def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
     pdh, pdc = [p(t) for t in dhs], [p(t) for t in dcs]
     for k in range(n + L - 1):
         active = [L - 1 - u for u in range(L) if 0 <= k - u < n]          # layers, top first
-        t_of = [(n - 1 - (k - (L - 1 - l))) * Tc for l in active]
+        t_of = [r + (n - 1 - (k - (L - 1 - l))) * Tc for l in active]
         for l, t in zip(active, t_of):
             if l < L - 1:   # this layer's dout of the chunk the layer above has just finished
                 _lib.check(lib.fastlstm_gemm_dx(pdg[l + 1] + t * 4 * row, pWx[l + 1], pdo[l] + t * row, Tc, B, H, H, code, stream),
@@ -336,6 +350,13 @@ def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
             _ptr_array([pdc[l] for l in active]), _ptr_array([pg[l] + t * 4 * row for l, t in zip(active, t_of)]),
             _ptr_array([pc[l] + t * row for l, t in zip(active, t_of)]), _ptr_array([pdg[l] + t * 4 * row for l, t in zip(active, t_of)]),
             _ptr_array([pWh[l] for l in active]), p(ws), ws.numel(), Tc, B, H, code, stream), "fastlstm_bwd_persistent_multi")
+    for l in range(L - 1, -1, -1) if r else ():
+        if l < L - 1:
+            _lib.check(lib.fastlstm_gemm_dx(pdg[l + 1], pWx[l + 1], pdo[l], r, B, H, H, code, stream), "fastlstm_gemm_dx")
+        ws = wss[n + L - 1 + l]
+        _lib.check(lib.fastlstm_bwd_persistent_multi(
+            1, _ptr_array([pdo[l]]), _ptr_array([pdh[l]]), _ptr_array([pdc[l]]), _ptr_array([pg[l]]), _ptr_array([pc[l]]),
+            _ptr_array([pdg[l]]), _ptr_array([pWh[l]]), p(ws), ws.numel(), r, B, H, code, stream), "fastlstm_bwd_persistent_multi")
     for ws in wss:
         _check_ws(ws, "fastlstm_bwd_persistent_multi")
     dx0 = torch.empty_like(x)

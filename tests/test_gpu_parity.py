@@ -848,7 +848,9 @@ def test_fwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
 
 
 @pytest.mark.parametrize("T,B,I,H,dt", [(256, 16, 96, 640, torch.float16), (384, 32, 64, 256, torch.float32),
-                                        (320, 48, 128, 512, torch.bfloat16)])
+                                        (320, 48, 128, 512, torch.bfloat16),
+                                        (389, 32, 64, 256, torch.float32),      # 6 chunks of 64 behind a prefix of 5 timesteps
+                                        (263, 16, 96, 640, torch.float16)])     # 4 chunks of 65 behind 3
 def test_two_layers_as_a_wavefront_of_chunked_pair_launches(T, B, I, H, dt):
     """Shapes whose two time loops fit the device side by side but which the library's own two-layer launch does
     not take: lstm_persistent_fwd_stack2 / lstm_persistent_bwd_stack2 cut the sequence into chunks and run the
@@ -881,7 +883,8 @@ def test_two_layers_as_a_wavefront_of_chunked_pair_launches(T, B, I, H, dt):
 
 
 @pytest.mark.parametrize("L_,T,B,I,H,dt", [(4, 256, 16, 64, 256, torch.float32), (3, 256, 16, 96, 384, torch.float16),
-                                           (4, 320, 32, 64, 256, torch.bfloat16)])
+                                           (4, 320, 32, 64, 256, torch.bfloat16),
+                                           (3, 197, 16, 64, 256, torch.float32)])   # 3 chunks of 65 behind a prefix of 2
 def test_three_and_four_layers_as_a_wavefront(L_, T, B, I, H, dt):
     """lstm_persistent_fwd_stack / lstm_persistent_bwd_stack (launch k runs layer l's chunk k - l for every layer,
     fastlstm_*_persistent_multi) against the layer-by-layer ops: the same bits with fp32 (weight gradients: another
