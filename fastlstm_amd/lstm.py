@@ -412,10 +412,28 @@ def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
     d_states = list(d_states) if d_states is not None else [None] * L
     T, B, H = dh.shape
     with torch.cuda.device(x.device):
-        n = stack_wavefront_chunks(L, T, B, H, acts[0][2].dtype, x.device, backward=True)
-        if n:
-            return _bwd_stack_wavefront(dh, x, acts, weights, d_states, n)
+        lib = _lib.load()
+        code = _code(acts[0][2])
         res = [None] * L
+        # Where the GEMMs are large, the reverse pass is faster as the library's two-layer launches from the top down
+        # (the GEMMs inside them) than as one wavefront with the GEMMs in the open (4 x (T = 512, B = 16, I = H = 1024):
+        # reverse pass 4.2 against 5.2 ms), whichever way the forward pass went.
+        plan = _plan(x.device, B, H, code, True)
+        if L >= 3 and not _small_projections(B, H, H) and lib.fastlstm_bwd_stack2_fused(
+                T, B, H, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1:
+            l = L - 1
+            while l >= 1:
+                xin = x if l == 1 else acts[l - 2][0][1:]
+                res[l - 1], res[l] = lstm_persistent_bwd_stack2(dh, xin, *acts[l - 1], weights[l - 1][0], weights[l - 1][1],
+                                                                *acts[l], weights[l][0], weights[l][1],
+                                                                d_state0=d_states[l - 1], d_state1=d_states[l])
+                dh = res[l - 1][0]
+                l -= 2
+            L = l + 1   # a lowest layer without a partner follows below
+        else:
+            n = stack_wavefront_chunks(L, T, B, H, acts[0][2].dtype, x.device, backward=True)
+            if n:
+                return _bwd_stack_wavefront(dh, x, acts, weights, d_states, n)
         for l in range(L - 1, -1, -1):
             out, cell, ifgo = acts[l]
             dt = ifgo.dtype
@@ -1221,13 +1239,8 @@ class FastLSTM(nn.Module):
                 dt_ = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else x.dtype
                 while width >= 3 and not stack_wavefront_chunks(width, x.shape[0], x.shape[1], self.hidden_size, dt_, x.device):
                     width -= 1
-                # where the library runs PAIRS of these layers in one launch with the GEMMs hidden inside, and the
-                # GEMMs are large, pairs win over the whole pass (4 x (T = 1024, B = 32, I = H = 1024): forward +
-                # backward 13.3 ms in pairs, 14.2 four at a time; forward alone 5.3 vs 4.7)
-                # (a forward pass that no backward pass follows goes four at a time)
-                if width >= 3 and not inference and not _small_projections(x.shape[1], self.hidden_size, self.hidden_size) and \
-                        stack2_runs_in_one_launch(x.shape[0], x.shape[1], x.shape[2], self.hidden_size, dt_, x.device):
-                    width = 0
+                # (the reverse pass of such a block chooses by itself between one wavefront and the library's two-layer
+                # launches, lstm_persistent_bwd_stack)
                 if width >= 3:
                     flat = []
                     for l in range(layer, layer + width):
