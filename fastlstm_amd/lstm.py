@@ -216,13 +216,6 @@ def stack2_wavefront_chunks(T, B, H, dtype, device, backward=False):
     return stack_wavefront_chunks(2, T, B, H, dtype, device, backward)
 
 
-def _small_projections(B, I, H):
-    """Three or four stacked layers: the wavefront of chunked launches leaves the GEMMs in the open, the library's
-    two-layer launches (pair by pair) hide them behind the time loops.  Where the GEMMs are a few per cent of a step
-    the wavefront wins; B = 32, I = H = 1024 and B = 64, I = H = 768 are past the crossover for a training pass."""
-    return B * I * H < 1.5e7
-
-
 def _chunk_workspaces(n_bytes, zero_bytes, count, device):
     """`count` workspaces of n_bytes each, the first zero_bytes of every one cleared by ONE fill."""
     stride = (n_bytes + 255) // 256 * 256
@@ -415,11 +408,12 @@ def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
         lib = _lib.load()
         code = _code(acts[0][2])
         res = [None] * L
-        # Where the GEMMs are large, the reverse pass is faster as the library's two-layer launches from the top down
-        # (the GEMMs inside them) than as one wavefront with the GEMMs in the open (4 x (T = 512, B = 16, I = H = 1024):
-        # reverse pass 4.2 against 5.2 ms), whichever way the forward pass went.
+        # From H = 768 on, the reverse pass is faster as the library's two-layer launches from the top down (the GEMMs
+        # inside them) than as one wavefront with the GEMMs in the open, whichever way the forward pass went
+        # (4 x (T = 512, I = H): forward + backward H = 1024, B = 16 6.60 against 7.59 ms, H = 768, B = 16 6.16 / 6.82,
+        # H = 1024, B = 8 6.52 / 7.21; level at H = 512; H = 384 7.68 / 6.90).
         plan = _plan(x.device, B, H, code, True)
-        if L >= 3 and not _small_projections(B, H, H) and lib.fastlstm_bwd_stack2_fused(
+        if L >= 3 and H >= 768 and lib.fastlstm_bwd_stack2_fused(
                 T, B, H, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1:
             l = L - 1
             while l >= 1:
