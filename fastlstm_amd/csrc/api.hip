@@ -194,8 +194,8 @@ struct XcdCfg {
 // The XCD-local kernels apply when the device deals workgroups to XCDs in turn, the shape fits
 // and the workspace holds a ring with one slot per exchanged version.
 // `launch_rows`: batch rows of this launch (0: all B_all of them).
-// copies > 1: that many recurrences of this shape share the launch (16-row groups only), so the unit tile has to leave
-// room for all their groups.
+// copies > 1: that many recurrences of this shape share the launch, so the unit tile has to leave room for all their
+// groups.
 bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_bytes, XcdCfg *c, int launch_rows = 0,
                 int copies = 1) {
     const int B = launch_rows ? launch_rows : B_all;
@@ -222,7 +222,7 @@ bool select_xcd(int T, int B_all, int H, int dtype, bool backward, size_t ws_byt
         // groups per XCD: as many as its 32 CUs hold, and no more than the workspace has barrier counters for
         const int groups_max = kNumXcd * std::min(32 / (H / cand), kXcdMaxGroups / kNumXcd);
         if (copies * cdiv(B, 16) <= groups_max) { ht = cand; c->ntw = 1; }
-        else if (copies == 1 && cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
+        else if (copies * cdiv(B, 32) <= groups_max) { ht = cand; c->ntw = 2; }
     }
     if (!ht) return false;
     c->mt = ht / rows;
@@ -334,7 +334,7 @@ int try_fwd_xcd(void *ifgo, void *out, void *cell, const void *Wh, unsigned char
     p.n_layers = 1;
     if (second && !x) {   // independent recurrences of this shape side by side (their projections are done)
         const int n = 2 + o.n_more;
-        if (c.ntw != 1 || n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
+        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;   // every group needs its CUs on one XCD
         if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
         p.n_layers = n;
         p.ifgo2 = second->ifgo; p.out2 = second->out; p.cell2 = second->cell; p.Wh2 = second->Wh;
@@ -718,7 +718,8 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
     p.n_layers = 1;
     if (lower && !extras) {   // independent recurrences of this shape side by side
         const int n = 2 + o.n_more;
-        if (c.ntw != 1 || n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx) return 2;
+        // (32-row groups of the 16-k-step reverse kernel, H > 512, cost 1.9 x a 16-row step: no gain over one after the other)
+        if (n > kMaxSideBySide || n * c.n_groups > kNumXcd * c.gpx || (c.ntw == 2 && c.nkw == 16)) return 2;
         if (ws_bytes < kWsHeaderBytes + kWsCounterBytes + 2 * (size_t)n * c.xslot) return 2;
         p.n_layers = n;
         for (int i = 0; i < o.n_more; ++i) {

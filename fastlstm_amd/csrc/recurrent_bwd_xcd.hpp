@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     // two recurrences in the launch: a stack (HELP == 2), or two independent ones of the same shape side by side
     // (HELP == 0 with n_layers == 2: the two directions of a bidirectional layer; `lower` is then simply the second)
     // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
-    const int n_layers = HELP == 2 ? 2 : (HELP == 0 && NTW == 1 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
+    const int n_layers = HELP == 2 ? 2 : (HELP == 0 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP != 0) {
             if (p.k5_tiles_n > 0) bwd_helper<T, HELP == 2>(p, smem);
@@ -320,7 +320,6 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     // the helper instantiations never see more than two recurrences)
     auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
         if constexpr (HELP != 0) return lower ? a1 : a0;
-        else if constexpr (NTW != 1) return a0;
         else return rec == 0 ? a0 : rec == 1 ? a1 : rec == 2 ? a2 : a3;
     };
     const int u0 = j * HT, b0 = p.b_base + g * BT;   // b_base: first batch row of this launch

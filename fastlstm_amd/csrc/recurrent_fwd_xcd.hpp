@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     // (without helpers n_layers == 2 means two independent recurrences of the same shape side by side: the two
     // directions of a bidirectional layer; nothing links them)
     // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
-    const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : (NTW == 1 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
+    const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : max(1, min(p.n_layers, kMaxSideBySide));
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
             if (p.k1_tiles_n > 0) k1_helper<T>(p, smem);
@@ -292,7 +292,6 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     // the helper instantiations never see more than two layers)
     auto pick = [&](auto a0, auto a1, auto a2, auto a3) {
         if constexpr (HELP) return layer ? a1 : a0;
-        else if constexpr (NTW != 1) return a0;
         else return layer == 0 ? a0 : layer == 1 ? a1 : layer == 2 ? a2 : a3;
     };
     T *ifgo = static_cast<T *>(pick(p.ifgo, p.ifgo2, p.ifgo_more[0], p.ifgo_more[1]));

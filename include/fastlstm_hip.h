@@ -200,8 +200,8 @@ int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_
  * each array belongs to recurrence r): the chunks of a wavefront over stacked layers -- launch k runs layer l's
  * chunk k - l of timesteps for every layer l, a time loop started at out[t0] / cell[t0] continuing the sequence --
  * which spreads the layer loop of fastlstm/lstm.py:685-696 (README.md:94: "doesn't exploit num_layer
- * parallelisation") over the device.  One launch where n x the groups of one recurrence fit the XCDs -- XCD-local
- * kernels with 16-row groups, register-resident kernels with 16- or 32-row groups, and always for H <= 64, whose
+ * parallelisation") over the device.  One launch where n x the groups of one recurrence fit the XCDs -- XCD-local and
+ * register-resident kernels with 16- or 32-row groups, and always for H <= 64, whose
  * workgroups exchange nothing -- (fastlstm_multi_fused), else one recurrence after the other.  ws: fastlstm_multi_workspace_bytes (the exchange
  * slots of n recurrences), zeroed like any recurrent workspace. */
 int fastlstm_fwd_persistent_multi(int n, void *const *ifgo, void *const *out, void *const *cell,
