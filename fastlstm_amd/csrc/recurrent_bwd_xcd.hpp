@@ -303,7 +303,6 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over the layers of the launch
     // two recurrences in the launch: a stack (HELP == 2), or two independent ones of the same shape side by side
     // (HELP == 0 with n_layers == 2: the two directions of a bidirectional layer; `lower` is then simply the second)
-    // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
     const int n_layers = HELP == 2 ? 2 : (HELP == 0 ? max(1, min(p.n_layers, kMaxSideBySide)) : 1);
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP != 0) {

@@ -264,7 +264,6 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_fwd_xcd_kernel(const FwdXcdP
     const int vg = gl * kNumXcd + xcd;          // group index over all layers of the launch
     // (without helpers n_layers == 2 means two independent recurrences of the same shape side by side: the two
     // directions of a bidirectional layer; nothing links them)
-    // (32-row tiles are chosen only when the 16-row groups of ONE recurrence do not fit the device: never several)
     const int n_layers = HELP ? (p.n_layers > 1 ? 2 : 1) : max(1, min(p.n_layers, kMaxSideBySide));
     if (gl >= p.gpx || vg >= p.n_groups * n_layers) {
         if constexpr (HELP) {
