@@ -950,7 +950,7 @@ def _indices_to_device(dev, *tensors):
     return on_dev.split([t.numel() for t in tensors])
 
 
-@functools.lru_cache(maxsize=None)
+@functools.lru_cache(maxsize=4096)
 def _padded_hidden_size(T, B, H, code, device_index):
     """The next hidden size above H (within a quarter, in steps of the MFMA k-step) that the XCD-local or the
     register-resident kernels take, when H itself gets the general kernels; else 0."""
