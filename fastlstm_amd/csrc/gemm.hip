@@ -108,7 +108,9 @@ hipError_t launch_colsum_t(const void *in, void *out, float *part, int R, int C,
 // rows, operands addressable with 32-bit byte offsets.
 bool gemm16_eligible(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km) {
     if (dtype == FASTLSTM_FP32) return false;
-    if (K % 64 != 0 || lda % 8 != 0 || ldb % 8 != 0) return false;
+    // K-major x K-major (the weight gradients, K = T*B rows): any K -- the loop runs to the next multiple of 64 and the
+    // rows past K lie outside both operands' buffer ranges, where loads return zero
+    if ((K % 64 != 0 && !(a_km && b_km)) || lda % 8 != 0 || ldb % 8 != 0) return false;
     // 32-bit byte offsets, with room for the rows a partial tile reaches past the operand
     const size_t a_bytes = (size_t)((a_km ? K : M) + 256) * lda * 2, b_bytes = (size_t)((b_km ? K : N) + 256) * ldb * 2;
     return a_bytes < (1ull << 32) && b_bytes < (1ull << 32);

@@ -509,7 +509,8 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int kb = split * p.k_per_split;
-    gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(p.K, kb + p.k_per_split), smem, acc);
+    const int k_end = (A_KM && B_KM) ? (p.K + 63) / 64 * 64 : p.K;   // (rows past K read as zeros)
+    gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
     if (p.trace) t_epi = (long long)wall_clock64();
     gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, split, smem, acc);
     if (p.trace && threadIdx.x == 0) {   // stamps: start, main loop entered (= start), main loop left, done

@@ -198,7 +198,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
         const GemmParams &q = lo8 ? p.k8_lo : p.k9_lo;
         const int qi = lo8 ? h : h - n8_lo, qtn = lo8 ? p.k8_lo_tiles_n : p.k9_tiles_n;
         const int c = p.k5_chunks - 1 - k;
-        const int kb = c * p.k5_chunk_tiles * 256, ke = min(q.K, kb + p.k5_chunk_tiles * 256);
+        const int kb = c * p.k5_chunk_tiles * 256, ke = min((q.K + 63) / 64 * 64, kb + p.k5_chunk_tiles * 256);   // (rows past K read as zeros)
         helper_wgrad_chunk<T>(q.A, q.B, q.C, q.M, q.N, q.K, q.ldb, (qi / qtn) * 256, (qi % qtn) * 256, kb, ke,
                               reinterpret_cast<f32x4 *>(p.wg_scratch_lo) + (size_t)h * (256 * 256 / 4), k == 0,
                               k + 1 == p.k5_chunks, (FASTLSTM_LDS_PTR unsigned char *)smem);
@@ -216,7 +216,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
         if (threadIdx.x == 0 && k == p.k5_chunks - 1) stamps[3] = (long long)wall_clock64();
 #endif
         if (own) {
-            const int kb = c * p.k5_chunk_tiles * 256, ke = min(wp.K, kb + p.k5_chunk_tiles * 256);
+            const int kb = c * p.k5_chunk_tiles * 256, ke = min((wp.K + 63) / 64 * 64, kb + p.k5_chunk_tiles * 256);   // (rows past K read as zeros)
             if constexpr (STACKED) {
                 helper_wgrad_chunk<T>(wp.A, wp.B, wp.C, wp.M, wp.N, wp.K, wp.ldb, wm0, wn0, kb, ke,
                                       reinterpret_cast<f32x4 *>(p.wg_scratch) + (size_t)h * (256 * 256 / 4), k == 0,

@@ -230,7 +230,8 @@ def test_random_shapes_vs_oracle(oracle, seed):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K", [(1, 4, 3), (130, 260, 70), (257, 123, 515), (512, 1024, 256)])
+@pytest.mark.parametrize("M,N,K", [(1, 4, 3), (130, 260, 70), (257, 123, 515), (512, 1024, 256),
+                                   (700, 1024, 256), (1120, 4096, 1024)])   # T*B no multiple of 64: the tile kernel's weight-gradient loop ends past it
 def test_gemm_stages_vs_matmul(dt, M, N, K):
     """K1 (x.Wx^T + b), K5 (d.Wx) and K8/K9 (d^T.x) against float64 matmul; shapes chosen
     so that T*B = M, 4H = N (K1) etc. hit ragged tiles, unaligned rows and split-K."""
@@ -1056,7 +1057,9 @@ def test_bwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
 @pytest.mark.parametrize("T,B,I,H,dt", [(96, 64, 1024, 1024, torch.float16),    # helpers compute dx inside the launch
                                         (40, 32, 512, 1024, torch.bfloat16),
                                         (24, 48, 256, 512, torch.float16),     # 16 units per workgroup
-                                        (9, 20, 50, 72, torch.float32)])       # general kernels, two launches
+                                        (9, 20, 50, 72, torch.float32),        # general kernels, two launches
+                                        (35, 32, 1024, 1024, torch.float16),   # T*B = 1120: no multiple of 64
+                                        (67, 20, 256, 512, torch.bfloat16)])
 def test_bwd_layer_equals_separate_stages(T, B, I, H, dt):
     """fastlstm_bwd_layer must give the results of fastlstm_bwd_persistent, fastlstm_gemm_dx and
     fastlstm_gemm_wgrad run one after the other, whichever way it schedules the stages: bit-identical
