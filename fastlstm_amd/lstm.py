@@ -54,7 +54,14 @@ def _require_gpu(*tensors):
                 "fastlstm_amd runs on the GPU only (tensor on %s); there is no CPU fallback" % t.device)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """Handle of the current stream of the current device (the raw accessor where this torch has it:
+    torch.cuda.current_stream() costs ~25 us of host time per call, a third of a short forward call)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
