@@ -958,17 +958,20 @@ def _indices_to_device(dev, *tensors):
 
 
 @functools.lru_cache(maxsize=4096)
+def _recurrent_kind(T, B, H, code, device_index):
+    """fastlstm_recurrent_kernel_kind of the forward call for the workspace this module allocates."""
+    lib = _lib.load()
+    device = torch.device("cuda", device_index)
+    with torch.cuda.device(device):
+        plan = _plan(device, B, H, code, False)
+        return lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0))
+
+
+@functools.lru_cache(maxsize=4096)
 def _padded_hidden_size(T, B, H, code, device_index):
     """The next hidden size above H (within a quarter, in steps of the MFMA k-step) that the XCD-local or the
     register-resident kernels take, when H itself gets the general kernels; else 0."""
-    lib = _lib.load()
-    device = torch.device("cuda", device_index)
-
-    def kind(h):
-        with torch.cuda.device(device):
-            plan = _plan(device, B, h, code, False)
-            return lib.fastlstm_recurrent_kernel_kind(T, B, h, code, 0,
-                                                      lib.fastlstm_recurrent_workspace_bytes(plan, T, h, code, 0))
+    kind = lambda h: _recurrent_kind(T, B, h, code, device_index)
     fp32 = code == _DTYPE_CODE[torch.float32]
     if T < 32:   # a few steps do not repay the launches that pad and cut
         return 0
@@ -1348,6 +1351,12 @@ class FastLSTM(nn.Module):
         idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
         H, I = self.hidden_size, self.input_size
         Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx) or H
+        # Where H is padded anyway and stacked layers read it as the K of their input projection: a multiple of 64, which
+        # the MFMA tile kernel takes (2 x (T = 256, B = 32): H = 704 forward + backward 2.19 ms, H = 672 2.32).  (Two
+        # directions make K = 2H; below 512 the projection is too small to matter.)
+        if (Hp != H and self.num_layers > 1 and not self.bidirectional and dt != torch.float32 and Hp % 64 == 32
+                and Hp >= 512 and _recurrent_kind(T, B, Hp + 32, _DTYPE_CODE[dt], idx) in (1, 2)):
+            Hp += 32
         Ip = -(-I // 64) * 64 if dt != torch.float32 and T * B >= 1024 and data.shape[-1] == I else I
         return (Hp, Ip) if (Hp, Ip) != (H, I) else None
 

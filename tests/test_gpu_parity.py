@@ -1246,7 +1246,7 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
 
 
 @pytest.mark.parametrize("kw,T,B,I,H,Hp,Ip,dt", [(dict(bidirectional=True), 32, 24, 50, 100, 112, 50, torch.float32),
-                                                 (dict(), 64, 16, 70, 650, 672, 128, torch.float16),
+                                                 (dict(), 64, 16, 70, 650, 704, 128, torch.float16),   # (stacked layers: a multiple of 64)
                                                  (dict(bidirectional=True), 64, 16, 300, 256, 256, 320, torch.float16),
                                                  (dict(bias=False, batch_first=True), 32, 8, 33, 1150, 1280, 33, torch.bfloat16)])
 def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
