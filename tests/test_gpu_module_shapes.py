@@ -130,3 +130,30 @@ def _check(c, seed):
                                        atol=FP32_TOL * scale, msg=lambda s: "%s %s: %s" % (name, c, s))
         else:
             assert rel_err(got, want) < HALF_TOL, (name, c, rel_err(got, want))
+
+
+@pytest.mark.parametrize("dt,H,scale_x,scale_w", [
+    (torch.float16, 64, 50.0, 1.0), (torch.float16, 1024, 100.0, 1.0), (torch.bfloat16, 2048, 20.0, 2.0),
+    (torch.bfloat16, 300, 60.0, 2.0), (torch.float32, 256, 30.0, 3.0), (torch.float32, 1024, 100.0, 1.0)])
+def test_saturated_gates_stay_finite_and_match_nn_lstm(dt, H, scale_x, scale_w):
+    """Pre-activations of a few hundred: exp() of either sign overflows in the gate formulas, the gates have to
+    come out as exactly 0 / 1 / +-1 all the same, with finite gradients (one kernel family per hidden size)."""
+    torch.manual_seed(0)
+    T, B, I = 40, 16, 64
+    m = FastLSTM(I, H).to("cuda", dt)
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.mul_(scale_w)
+    ref = torch.nn.LSTM(I, H)
+    ref.load_state_dict({k: v.float().cpu() for k, v in m.state_dict().items()})
+    x = (torch.randn(T, B, I) * scale_x).to(dt)
+    xg, xr = x.cuda().requires_grad_(True), x.float().requires_grad_(True)
+    y, (hn, cn) = m(xg)
+    y.float().sum().backward()
+    yr, (hr, cr) = ref(xr)
+    yr.sum().backward()
+    rows = [(y, yr, "y"), (hn, hr, "hn"), (cn, cr, "cn"), (xg.grad, xr.grad, "dx")]
+    rows += [(prm.grad, getattr(ref, n).grad, n) for n, prm in m.named_parameters()]
+    for got, want, name in rows:
+        assert torch.isfinite(got.float()).all(), name
+        assert rel_err(got, want) < (FP32_TOL if dt == torch.float32 else HALF_TOL), (name, rel_err(got, want))
