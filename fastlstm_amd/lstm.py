@@ -973,7 +973,10 @@ def _padded_hidden_size(T, B, H, code, device_index):
     register-resident kernels take, when H itself gets the general kernels; else 0."""
     kind = lambda h: _recurrent_kind(T, B, h, code, device_index)
     fp32 = code == _DTYPE_CODE[torch.float32]
-    if T < 32:   # a few steps do not repay the launches that pad and cut
+    # The launches that pad and cut cost ~0.1 ms forward and ~0.2 ms forward + backward whatever the shape: a few steps
+    # repay them only with many rows and units (T = 16, B = 128, H = 1150 bf16 forward + backward 0.82 ms as it is,
+    # 0.59 ms as 1280; B = 64, H = 650 0.48 against 0.68).
+    if T < 32 and (H <= 64 or T * B * H < (1_200_000 if fp32 else 2_000_000)):
         return 0
     if H <= 64:
         # The general kernels' one-tile form (no exchange between workgroups at all).  In 16 bits it is the fastest

@@ -1248,7 +1248,8 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
 @pytest.mark.parametrize("kw,T,B,I,H,Hp,Ip,dt", [(dict(bidirectional=True), 32, 24, 50, 100, 112, 50, torch.float32),
                                                  (dict(), 64, 16, 70, 650, 704, 128, torch.float16),   # (stacked layers: a multiple of 64)
                                                  (dict(bidirectional=True), 64, 16, 300, 256, 256, 320, torch.float16),
-                                                 (dict(bias=False, batch_first=True), 32, 8, 33, 1150, 1280, 33, torch.bfloat16)])
+                                                 (dict(bias=False, batch_first=True), 32, 8, 33, 1150, 1280, 33, torch.bfloat16),
+                                                 (dict(), 16, 128, 64, 1150, 1280, 64, torch.bfloat16)])   # few steps, many rows
 def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
     """The module pads a hidden size that only the general kernels take to the next one the XCD-local /
     register-resident kernels take (zero weights, biases and initial states for the added units), and a 16-bit
@@ -1268,7 +1269,7 @@ def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I
     # sizes the fast kernels take run as they are; so does H <= 64 (the one-tile form of the general kernels)
     for i_, h_ in ((64, 64), (128, 32), (256, 512), (1024, 2048)):
         assert FastLSTM(i_, h_).to("cuda", torch.float16)._operand_padding(torch.empty(32, 256, i_, device="cuda", dtype=torch.float16)) is None
-    # ... and a few timesteps do not repay the padding
+    # ... and a few timesteps do not repay the padding (unless rows x units are many: the last case)
     assert m._operand_padding(leaves[0][:, :4] if kw.get("batch_first") else leaves[0][:4]) is None
     y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
     yr, (hr, cr) = ref(leaves_r[0], (leaves_r[1], leaves_r[2]))
