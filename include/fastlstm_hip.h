@@ -54,7 +54,11 @@ typedef enum {
  * to other batch tiles.  n_btiles * n_htiles <= num_cus so that every
  * workgroup is resident while its peers spin (the rule of
  * fastlstm/configs.py:29-58); a batch that does not fit is processed in
- * `batch_chunks` sequential launches (fastlstm/kernels.py:514, 663). */
+ * `batch_chunks` sequential launches (fastlstm/kernels.py:514, 663).
+ * The rule counts one launch at a time: two recurrent launches on different
+ * streams of one GPU can each hold a part of the compute units and wait for
+ * the other's missing workgroups until the time-out; callers that use
+ * several streams order the library's calls with an event. */
 typedef struct {
     int num_cus;      /* compute units used for planning */
     int lds_limit;    /* bytes of LDS one workgroup may use */
