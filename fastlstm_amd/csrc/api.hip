@@ -595,7 +595,7 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     const int layers = lower ? 2 : 1;
     if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
     const int n_active = c.n_groups * c.n_ht, n_helpers = kNumXcd * 32 - layers * n_active;
-    if (n_helpers < kNumXcd * 8) return false;
+    if (n_helpers < kNumXcd * (lower ? 6 : 8)) return false;
     const int max_chunks = kMaxChunks;
     const int I = e.I, M = T * B, K = 4 * H;
     if (!gemm16_eligible(dtype, M, I, K, K, I, false, true) || I % 8) return false;
@@ -625,9 +625,17 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     if (lower) {
         // the lower layer runs two chunks behind the upper one: no more than 64 timesteps per chunk
         ct = std::min(ct, std::max(1, 64 * B / 256 / base) * base);
-        // dx, dW_x and dW_h of both layers on the helpers: see plan_k1_helpers (config E: 1.0)
-        const double flop = 2.0 * M * K * (2.0 * I + H) + 2.0 * M * K * ((lower->dx ? 2.0 : 1.0) * lower->I + H);
-        if (flop / (n_helpers * 3.5e9) > 1.25 * T * 3.6e-3) return false;
+        // dx, dW_x and dW_h of both layers on the helpers: see plan_k1_helpers (config E: 1.0).  Where that is too much
+        // for them, both dx alone (the upper one is the lower recurrence's operand and has to be inside): the weight
+        // gradients then follow as launches of their own on the whole device (T = 512, B = 64, I = 256, H = 768 bf16,
+        // two layers: reverse pass 3.6 ms layer by layer).
+        const double dx_flop = 2.0 * M * K * I + (lower->dx ? 2.0 * M * K * lower->I : 0.0);
+        const double flop = dx_flop + 2.0 * M * K * (I + H) + 2.0 * M * K * (lower->I + H);
+        const double budget_ms = 1.25 * T * 3.6e-3;
+        if (flop / (n_helpers * 3.5e9) > budget_ms) {
+            if (dx_flop / (n_helpers * 3.5e9) > budget_ms) return false;
+            wgrad_inside = false;
+        }
     }
     while (cdiv(tiles_m, ct) > max_chunks) ct += base;
     p->n_layers = layers;

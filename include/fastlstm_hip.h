@@ -254,7 +254,8 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
  * workgroups compute dx1 chunk by chunk behind the upper recurrence, the lower recurrence follows
  * dx1 a few chunks behind, and the same workgroups accumulate dWx1, dWh1 and compute dx0; the bias
  * gradients follow as separate launches, and so do the lower layer's weight gradients unless wgrad_ws is
- * large enough to park their tiles between chunks.  ws: fastlstm_stack2_bwd_workspace_bytes, zeroed like
+ * large enough to park their tiles between chunks.  With few idle workgroups (48 to 64 at H = 768 ... 1024
+ * and B = 48 ... 64) they compute dx1 and dx0 only and all four weight gradients follow as launches.  ws: fastlstm_stack2_bwd_workspace_bytes, zeroed like
  * any recurrent workspace; wgrad_ws: at least the larger of the two layers'
  * fastlstm_wgrad_workspace_bytes; with fastlstm_stack2_bwd_wgrad_workspace_bytes (64 MiB at H = I = 1024)
  * the launch takes the lower layer's dWx0, dWh0 too.  Replaces two backward nodes of the layer loop at

@@ -997,6 +997,8 @@ def test_two_layer_module_one_launch_matches_layer_by_layer():
     (3, 24, 256, 1024, torch.float16, True),       # shorter than a chunk
     (30, 64, 256, 1024, torch.float16, False),     # no idle CUs for two layers: one layer after the other
     (9, 20, 50, 72, torch.float32, False),         # general kernels
+    (70, 64, 256, 768, torch.bfloat16, True),      # 64 idle CUs: both dx inside, the weight gradients behind the launch
+    (45, 64, 128, 832, torch.float16, True),       # 48 idle CUs
 ])
 def test_bwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
     """fastlstm_bwd_stack2 must give the results of fastlstm_bwd_layer for the upper layer followed by
