@@ -958,21 +958,26 @@ def _indices_to_device(dev, *tensors):
 
 
 @functools.lru_cache(maxsize=4096)
-def _recurrent_kind(T, B, H, code, device_index):
-    """fastlstm_recurrent_kernel_kind of the forward call for the workspace this module allocates."""
+def _recurrent_kind(T, B, H, code, device_index, backward=False):
+    """fastlstm_recurrent_kernel_kind of the forward (reverse) call for the workspace this module allocates."""
     lib = _lib.load()
     device = torch.device("cuda", device_index)
     with torch.cuda.device(device):
-        plan = _plan(device, B, H, code, False)
-        return lib.fastlstm_recurrent_kernel_kind(T, B, H, code, 0, lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, 0))
+        plan = _plan(device, B, H, code, backward)
+        b = int(backward)
+        return lib.fastlstm_recurrent_kernel_kind(T, B, H, code, b, lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, b))
 
 
 @functools.lru_cache(maxsize=4096)
-def _padded_hidden_size(T, B, H, code, device_index):
+def _padded_hidden_size(T, B, H, code, device_index, training=False):
     """The next hidden size above H (within a quarter, in steps of the MFMA k-step) that the XCD-local or the
-    register-resident kernels take, when H itself gets the general kernels; else 0."""
-    kind = lambda h: _recurrent_kind(T, B, h, code, device_index)
+    register-resident kernels take, when H itself gets the general kernels; else 0.  `training`: a reverse pass
+    follows, whose kernels count too."""
     fp32 = code == _DTYPE_CODE[torch.float32]
+    kind = lambda h: _recurrent_kind(T, B, h, code, device_index)
+    # fp32 with up to 32 rows keeps the general forward kernel at H = 640 ... 1024, but its reverse pass is twice as
+    # fast on the register-resident kernel (T = 256, B = 8, I = 256, forward + backward: H = 576 3.8 ms, H = 640 2.9)
+    fast = lambda h: kind(h) in (1, 2) or (training and fp32 and _recurrent_kind(T, B, h, code, device_index, True) in (1, 2))
     # The launches that pad and cut cost ~0.1 ms forward and ~0.2 ms forward + backward whatever the shape: a few steps
     # repay them only with many rows and units (T = 16, B = 128, H = 1150 bf16 forward + backward 0.82 ms as it is,
     # 0.59 ms as 1280; B = 64, H = 650 0.48 against 0.68).
@@ -989,11 +994,11 @@ def _padded_hidden_size(T, B, H, code, device_index):
         if fp32:
             return 80 if kind(80) == 1 else 0
         return 64 if H < 64 else 0
-    if kind(H) != 0:
+    if kind(H) != 0 or fast(H):
         return 0
     step = 16 if fp32 else 32
     for Hp in range((H // step + 1) * step, H + H // 4 + step + 1, step):
-        if kind(Hp) in (1, 2):
+        if fast(Hp):
             return Hp
     return 0
 
@@ -1353,7 +1358,8 @@ class FastLSTM(nn.Module):
             T, B = (data.shape[1], data.shape[0]) if self.batch_first else (data.shape[0], data.shape[1])
         idx = data.device.index if data.device.index is not None else torch.cuda.current_device()
         H, I = self.hidden_size, self.input_size
-        Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx) or H
+        training = torch.is_grad_enabled() and (data.requires_grad or any(p.requires_grad for p in self.parameters()))
+        Hp = _padded_hidden_size(T, B, H, _DTYPE_CODE[dt], idx, training) or H
         # Where H is padded anyway and stacked layers read it as the K of their input projection: a multiple of 64, which
         # the MFMA tile kernel takes (2 x (T = 256, B = 32): H = 704 forward + backward 2.19 ms, H = 672 2.32).  (Two
         # directions make K = 2H; below 512 the projection is too small to matter.)

@@ -1251,7 +1251,8 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
                                                  (dict(), 64, 16, 70, 650, 704, 128, torch.float16),   # (stacked layers: a multiple of 64)
                                                  (dict(bidirectional=True), 64, 16, 300, 256, 256, 320, torch.float16),
                                                  (dict(bias=False, batch_first=True), 32, 8, 33, 1150, 1280, 33, torch.bfloat16),
-                                                 (dict(), 16, 128, 64, 1150, 1280, 64, torch.bfloat16)])   # few steps, many rows
+                                                 (dict(), 16, 128, 64, 1150, 1280, 64, torch.bfloat16),   # few steps, many rows
+                                                 (dict(), 64, 16, 70, 576, 640, 70, torch.float32)])   # for the reverse pass's sake
 def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
     """The module pads a hidden size that only the general kernels take to the next one the XCD-local /
     register-resident kernels take (zero weights, biases and initial states for the added units), and a 16-bit
