@@ -266,7 +266,7 @@ bool plan_k1_helpers(const XcdCfg &c, const void *x, const void *Wx, const void 
     const int layers = second ? 2 : 1;
     if (layers * c.n_groups > kNumXcd * c.gpx) return false;   // every group needs its CUs on one XCD
     const int n_helpers = kNumXcd * 32 - layers * c.n_groups * c.n_ht;
-    if (n_helpers < kNumXcd * 8) return false;
+    if (n_helpers < kNumXcd * (second ? 6 : 8)) return false;
     const int max_chunks = kMaxChunks;
     const int M = T * B, N = 4 * H;
     if (!gemm16_eligible(dtype, M, N, I, I, I, false, false) || N % 8) return false;

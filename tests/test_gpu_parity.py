@@ -798,6 +798,7 @@ def test_fwd_layer_equals_projection_then_recurrence(T, B, I, H, dt):
     (3, 24, 256, 1024, torch.float16, True),       # shorter than a chunk
     (30, 64, 256, 1024, torch.float16, False),     # 2 x 4 groups leave no idle CUs: one layer after the other
     (9, 20, 50, 72, torch.float32, False),         # general kernels
+    (70, 64, 128, 832, torch.bfloat16, True),      # 48 idle CUs (6 per XCD)
 ])
 def test_fwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
     """fastlstm_fwd_stack2 must give bit-identical results to fastlstm_fwd_layer for the first layer
