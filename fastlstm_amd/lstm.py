@@ -404,6 +404,12 @@ def lstm_persistent_fwd_stack(x, layers, keep_activations=True):
         return _fwd_stack_wavefront(_aligned(x), layers, n, keep_activations)
 
 
+def _pairs_min_hidden(B):
+    """Hidden size from which the reverse pass of three or more stacked layers goes pair by pair (see
+    lstm_persistent_bwd_stack)."""
+    return 576 if B > 32 else 704
+
+
 def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
     """Reverse pass of lstm_persistent_fwd_stack: acts[l] = (out, cell, ifgo), weights[l] = (Wx, Wh), d_states[l] = None
     or (dh_n, dc_n).  [(d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)] per layer; falls back to one layer after the other where
@@ -415,12 +421,13 @@ def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
         lib = _lib.load()
         code = _code(acts[0][2])
         res = [None] * L
-        # From H = 768 on, the reverse pass is faster as the library's two-layer launches from the top down (the GEMMs
-        # inside them) than as one wavefront with the GEMMs in the open, whichever way the forward pass went
-        # (4 x (T = 512, I = H): forward + backward H = 1024, B = 16 6.60 against 7.59 ms, H = 768, B = 16 6.16 / 6.82,
-        # H = 1024, B = 8 6.52 / 7.21; level at H = 512; H = 384 7.68 / 6.90).
+        # From H = 704 on (576 with more than 32 rows), the reverse pass is faster as the library's two-layer launches
+        # from the top down (the GEMMs inside them) than as one wavefront with the GEMMs in the open, whichever way the
+        # forward pass went (4 x (T = 512, I = H): forward + backward H = 1024, B = 16 6.60 against 7.59 ms, H = 768,
+        # B = 16 6.16 / 6.82, H = 1024, B = 8 6.52 / 7.21; level at H = 512; H = 384 7.68 / 6.90; 4 x (T = 512, I = 256,
+        # H = 576): B = 48 6.66 / 9.13, B = 64 7.69 / 9.71, B = 32 6.34 / 6.49).
         plan = _plan(x.device, B, H, code, True)
-        if L >= 3 and H >= 768 and lib.fastlstm_bwd_stack2_fused(
+        if L >= 3 and H >= _pairs_min_hidden(B) and lib.fastlstm_bwd_stack2_fused(
                 T, B, H, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1:
             l = L - 1
             while l >= 1:

@@ -919,6 +919,35 @@ def test_three_and_four_layers_as_a_wavefront(L_, T, B, I, H, dt):
         dh = want[0]
 
 
+@pytest.mark.parametrize("L_,T,B,I,H,dt", [(3, 130, 48, 64, 576, torch.bfloat16),    # a pair and the lowest layer alone
+                                           (4, 70, 16, 128, 768, torch.float16)])   # two pairs
+def test_deep_stack_reverse_pass_pair_by_pair(L_, T, B, I, H, dt):
+    """From a hidden size that depends on the batch, lstm_persistent_bwd_stack runs the library's two-layer reverse
+    launches from the top down instead of a wavefront: against the layer-by-layer ops on the same activations."""
+    lib = _lib.load()
+    code = {torch.float16: 1, torch.bfloat16: 2}[dt]
+    plan = _lib.Plan()
+    _lib.check(lib.fastlstm_plan_device(0, B, H, code, 1, plan), "plan")
+    assert H >= L._pairs_min_hidden(B)
+    assert lib.fastlstm_bwd_stack2_fused(T, B, H, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1
+    gs = [{k: dev(v, dt) for k, v in make_problem(T, B, I if l == 0 else H, H, seed=71 + l + T).items()} for l in range(L_)]
+    keys = ("h0", "c0", "Wx", "bx", "Wh", "bh")
+    acts, xin = [], gs[0]["x"]
+    for g in gs:
+        acts.append(L.lstm_persistent_fwd(xin, *(g[k] for k in keys)))
+        xin = acts[-1][0][1:]
+    res = L.lstm_persistent_bwd_stack(gs[-1]["dout"], gs[0]["x"], acts, [(g["Wx"], g["Wh"]) for g in gs],
+                                      [(g["dh_n"], g["dc_n"]) for g in gs])
+    dh = gs[-1]["dout"]
+    for l in range(L_ - 1, -1, -1):
+        g = gs[l]
+        xin = gs[0]["x"] if l == 0 else acts[l - 1][0][1:]
+        want = L.lstm_persistent_bwd(dh, g["dc_n"].clone(), g["dh_n"].clone(), xin, *acts[l], g["Wx"], g["Wh"])
+        for name, a, b in zip(("d_x", "dh_0", "dc_0", "dWx", "dbx", "dWh", "dbh"), res[l], want):
+            assert rel_err(a, npy(b)) < HALF_TOL, (l, name)
+        dh = want[0]
+
+
 def test_four_layer_module_through_the_wavefront_matches_nn_lstm():
     T, B, I, H, dt = 256, 16, 48, 256, torch.float16
     assert L.stack_wavefront_chunks(4, T, B, H, dt, "cuda") >= 2
