@@ -61,6 +61,12 @@ FORMS = [
     dict(dt=torch.float32, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=1, T=20, B=144, I=64, H=1024),
     dict(dt=torch.float16, kw=dict(bidirectional=True, bias=True, batch_first=False), layers=2, T=40, B=24, I=48, H=48),
     dict(dt=torch.float32, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=2, T=40, B=24, I=48, H=48),
+    # two stacked layers whose reverse launch takes both dx on its few idle workgroups and leaves the weight gradients
+    # to launches of their own; three layers whose reverse pass goes pair by pair; an fp32 hidden size padded for the
+    # reverse pass's sake
+    dict(dt=torch.bfloat16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=2, T=64, B=64, I=128, H=768),
+    dict(dt=torch.bfloat16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=3, T=130, B=48, I=64, H=576),
+    dict(dt=torch.float32, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=1, T=40, B=8, I=64, H=576),
 ]
 
 
