@@ -865,7 +865,7 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
     wgrad_plan(M, H, K, dtype, &tile, &sh, &kps);
     size_t part = std::max(sx > 1 ? (size_t)sx * M * I : 0, sh > 1 ? (size_t)sh * M * H : 0) * sizeof(float);
     size_t cs = (size_t)colsum_chunks(K) * M * sizeof(float);
-    return align_up(cs, 256) + align_up(part, 256) + 256;
+    return std::max(align_up(cs, 256) + align_up(part, 256), wgrad_merged_workspace(dtype, M, I, H, K)) + 256;
 }
 
 int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
@@ -879,6 +879,13 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
     if (ws_bytes < fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype)) return FASTLSTM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int K = T * B, M = 4 * H;
+    {   // both products and the bias gradient as one tile grid, d_ifgo read once
+        int sp, kps;
+        bool merged;
+        if (wgrad_merged_plan(dtype, M, I, H, K, &sp, &kps, &merged))
+            return launch_wgrad_merged(dtype, d_ifgo, x, h, dWx, dWh, db, ws, M, I, H, K, s) == hipSuccess ? FASTLSTM_OK
+                                                                                                            : FASTLSTM_ERR_HIP;
+    }
     const int chunks = colsum_chunks(K);
     float *cs_part = static_cast<float *>(ws);
     float *gemm_part = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) +

@@ -142,6 +142,92 @@ void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool
     }
 }
 
+// ---- both weight gradients + the bias gradient on the tile kernel (gemm16_wgrad_kernel) ------------------------
+// Taken for 16-bit products that the 256 x 256 tile kernel holds.  *merged: both products as one tile grid with
+// one split factor (K = T*B is split so that the tiles of both together fill the device); otherwise each product
+// fills the device on its own and they run as two launches of one round of tiles each, the bias gradient with
+// the first (a second round of tiles starts out of step with its neighbours and shares less in the L2:
+// M = 8192, I = H = 2048, K = 32768: 1.85 ms merged against 2 x 0.86).
+bool wgrad_merged_plan(int dtype, int M, int I, int H, int K, int *splits, int *k_per_split, bool *merged) {
+    if (!gemm16_eligible(dtype, M, I, K, M, I, true, true) || !gemm16_eligible(dtype, M, H, K, M, H, true, true)) return false;
+    if (M < 256 || I < 128 || H < 128) return false;   // thin outputs: the 128 x 128 tiles waste less
+    const int tx = cdiv(M, 256) * cdiv(I, 256), th = cdiv(M, 256) * cdiv(H, 256);
+    *merged = !(tx >= 192 && th >= 192 && tx <= 256 && th <= 256);
+    int sp = 1;
+    if (*merged && tx + th < 192) sp = std::max(1, std::min(cdiv(256, tx + th), K / 512));   // >= 8 k-tiles per split
+    const int kps = cdiv(cdiv(K, sp), 64) * 64;
+    *k_per_split = kps;
+    *splits = cdiv(K, kps);
+    return true;
+}
+
+// workspace: [splits][column tiles][M] for the bias gradient + [splits][M][I] + [splits][M][H] floats with a split
+size_t wgrad_merged_workspace(int dtype, int M, int I, int H, int K) {
+    int sp, kps;
+    bool merged;
+    if (!wgrad_merged_plan(dtype, M, I, H, K, &sp, &kps, &merged)) return 0;
+    const size_t dbp = align_up((size_t)sp * (cdiv(I, 256) + cdiv(H, 256)) * M * sizeof(float), 256);
+    return dbp + (sp > 1 ? (size_t)sp * M * ((size_t)I + H) * sizeof(float) : 0);
+}
+
+template <typename T>
+static hipError_t launch_wgrad_kernel_t(const WgradParams &w, hipStream_t s) {
+    using C = Gemm16Cfg<256, 256, 2, 2, 4, 2>;
+    static bool attr_set = false;
+    auto kern = gemm16_wgrad_kernel<T>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int grid = cdiv(w.x.M, 256) * (w.tiles_nx + cdiv(w.h.N, 256)) * w.x.splits;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, s, w);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_wgrad_merged_t(const WgradParams &w, bool merged, void *db, hipStream_t s) {
+    const int M = w.x.M, I = w.x.N, H = w.h.N, splits = w.x.splits;
+    int db_parts;
+    if (merged) {
+        if (hipError_t e = launch_wgrad_kernel_t<T>(w, s)) return e;
+        db_parts = splits * (w.tiles_nx + cdiv(H, 256));
+    } else {   // the x product with the bias gradient, then the h product alone
+        WgradParams a = w, b = w;
+        a.h.N = 0;
+        b.x = w.h; b.h.N = 0; b.tiles_nx = cdiv(H, 256); b.db_part = nullptr;
+        if (hipError_t e = launch_wgrad_kernel_t<T>(a, s)) return e;
+        if (hipError_t e = launch_wgrad_kernel_t<T>(b, s)) return e;
+        db_parts = splits * w.tiles_nx;
+    }
+    const int ri = splits > 1 ? I : 0, rh = splits > 1 ? H : 0;   // the products need no pass without a split
+    const size_t threads = (size_t)M * ri / 4 + (size_t)M * rh / 4 + M;
+    hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, w.x.Cpart,
+                       static_cast<T *>(w.x.C), w.h.Cpart, static_cast<T *>(w.h.C), w.db_part, static_cast<T *>(db), M, ri, rh,
+                       splits, db_parts);
+    return hipGetLastError();
+}
+
+hipError_t launch_wgrad_merged(int dtype, const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
+                               void *ws, int M, int I, int H, int K, hipStream_t s) {
+    WgradParams w{};
+    int sp, kps;
+    bool merged;
+    if (!wgrad_merged_plan(dtype, M, I, H, K, &sp, &kps, &merged)) return hipErrorInvalidValue;
+    float *db_part = static_cast<float *>(ws);
+    float *part_x = reinterpret_cast<float *>(static_cast<unsigned char *>(ws) +
+                                              align_up((size_t)sp * (cdiv(I, 256) + cdiv(H, 256)) * M * sizeof(float), 256));
+    GemmParams g{};
+    g.A = d_ifgo; g.M = M; g.K = K; g.lda = M; g.splits = sp; g.k_per_split = kps;
+    w.x = g; w.x.B = x; w.x.C = dWx; w.x.N = I; w.x.ldb = I; w.x.ldc = I; w.x.Cpart = part_x;
+    w.h = g; w.h.B = h; w.h.C = dWh; w.h.N = H; w.h.ldb = H; w.h.ldc = H; w.h.Cpart = part_x + (size_t)sp * M * I;
+    w.tiles_nx = cdiv(I, 256);
+    w.db_part = db_part;
+    return dtype == FASTLSTM_FP16 ? launch_wgrad_merged_t<_Float16>(w, merged, db, s)
+                                  : launch_wgrad_merged_t<__bf16>(w, merged, db, s);
+}
+
 static long long *g_trace = nullptr;
 void set_gemm_trace(long long *buf) { g_trace = buf; }
 

@@ -398,9 +398,241 @@ __device__ __forceinline__ void gemm16_mainloop(const GemmParams &p, const int m
     __syncthreads();  // all waves are done reading the stages before the LDS is reused
 }
 
+// LDS reads on LDS byte addresses, as inline assembly (see lds_read_tr16): the wave that uses them waits for
+// them itself (FragSet::landed).
+template <int OFF> __device__ __forceinline__ u32x4 lds_rd128(unsigned addr) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+#else
+    (void)addr;
+#endif
+    return v;
+}
+template <int OFF> __device__ __forceinline__ u32x4 lds_rd_tr16x2(unsigned addr) {
+    u32x2 lo = {0u, 0u}, hi = {0u, 0u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr), "n"(OFF));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(OFF + 2048));
+#else
+    (void)addr;
+#endif
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+}
+
+// The same contraction as gemm16_mainloop for the 256 x 256 x 64 tile with 8 waves (2 x 4) and two LDS
+// stages, scheduled as a ping-pong between the two waves of each SIMD.  Waves 0..3 (the upper half of the
+// C tile) and waves 4..7 (the lower half) run the same sequence of phases one phase apart:
+//     memory phase of k-step j:   read the 12 fragments of the k-step from LDS (and, once per k-tile,
+//                                 request this wave's 8 blocks of the k-tile after next), wait for the
+//                                 fragments
+//     compute phase of k-step j:  32 MFMAs from registers, nothing else
+// with a workgroup barrier between phases, so that on every SIMD one wave issues MFMAs back to back
+// while the other one issues the LDS and vector-memory instructions and absorbs their waits.  (With
+// both waves in the same phase at the same time, as in gemm16_mainloop, the matrix pipe idles at
+// every barrier and behind every queued memory instruction: 1180 -> 1500 TFLOP/s at M = 32768,
+// N = 8192, K = 2048 together with the non-temporal stores of the epilogue.)
+// The LDS-direct loads are inline assembly (dma_block_asm): the kernel's only ones, counted by hand.
+// c + the sum of the 8 elements of a fragment register quad (fp32 accumulate).
+template <typename T> __device__ __forceinline__ float frag_sum(const u32x4 f, float c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (Elem<T>::DT == FASTLSTM_FP16) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const f16x2 one = {(_Float16)1.f, (_Float16)1.f};
+        const f16x8 h = __builtin_bit_cast(f16x8, f);
+        c = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 0, 1), one, c, false);
+        c = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 2, 3), one, c, false);
+        c = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 4, 5), one, c, false);
+        c = __builtin_amdgcn_fdot2(__builtin_shufflevector(h, h, 6, 7), one, c, false);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            c += __builtin_bit_cast(float, f[e] << 16) + __builtin_bit_cast(float, f[e] & 0xffff0000u);
+    }
+#else
+    (void)f;
+#endif
+    return c;
+}
+
+// DB: in the k-tiles with (k-tile index of the whole product) % db_mod == db_rem the waves also sum their A
+// fragments over k: wave column wn adds the lane's 8 elements of fragments 2 wn and 2 wn + 1 to colsum[0],
+// colsum[1] -- this workgroup's share of the column sums of the A operand (the bias gradient of the
+// weight-gradient products), as vector instructions of the memory phase.  The column tiles of a row of C tiles
+// share the A panel, so each takes every db_mod-th k-tile and none of them is slowed down noticeably (all of
+// them in the first column tile: that tile ran 10 % longer and the launch with it).
+template <typename T, bool A_KM, bool B_KM, bool DB = false>
+__device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const int m0, const int n0, const int kb,
+                                                   const int ke, unsigned char *smem, f32x4 (&acc)[8][4],
+                                                   float *colsum = nullptr, const int db_mod = 1, const int db_rem = 0) {
+    constexpr int STAGE = 65536, A_BYTES = 32768;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int q = lane >> 4, r = lane & 15;
+    const int wm = wave >> 2, wn = wave & 3;
+    const int nkt = (ke - kb) / 64;
+    if (nkt <= 0) return;
+    const unsigned lds0 = (unsigned)(size_t)((FASTLSTM_LDS_PTR unsigned char *)smem);
+
+    auto rsrc_of = [](const void *base, unsigned bytes) {
+        const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+        return u32x4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+    };
+    const u32x4 ra = rsrc_of(p.A, (unsigned)((A_KM ? (size_t)p.K : (size_t)p.M) * p.lda * 2));
+    const u32x4 rb = rsrc_of(p.B, (unsigned)((B_KM ? (size_t)p.K : (size_t)p.N) * p.ldb * 2));
+    auto swz = [](int k) { return ((k & 3) << 1) ^ (((k >> 3) & 1) << 3); };   // K-major tiles (see gemm16_mainloop)
+    auto kswz = [](int r16) { return (r16 >> 1) & 7; };                        // K-contiguous tiles
+
+    // global -> LDS: wave w fills the 1 KiB blocks w, w + 8, w + 16, w + 24 of each operand's 32 KiB tile
+    unsigned goff_a, goff_b;
+    if constexpr (!A_KM) {
+        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * 8;
+        goff_a = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * 2);
+    } else {
+        const int P = wave * 64 + lane, k = P / 32, mc = (P % 32) ^ swz(k);
+        goff_a = (unsigned)(((size_t)(kb + k) * p.lda + m0 + mc * 8) * 2);
+    }
+    if constexpr (!B_KM) {
+        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * 8;
+        goff_b = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * 2);
+    } else {
+        const int P = wave * 64 + lane, k = P / 32, nc = (P % 32) ^ swz(k);
+        goff_b = (unsigned)(((size_t)(kb + k) * p.ldb + n0 + nc * 8) * 2);
+    }
+    const unsigned a_istep = (unsigned)(A_KM ? 16 : 64) * p.lda * 2, b_istep = (unsigned)(B_KM ? 16 : 64) * p.ldb * 2;
+    const unsigned a_kstep = A_KM ? 64u * p.lda * 2 : 128u, b_kstep = B_KM ? 64u * p.ldb * 2 : 128u;
+    auto gload = [&](int kt) {
+        const unsigned sa = lds0 + (kt & 1) * STAGE + wave * kFragBytes, sb = sa + A_BYTES;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma_block_asm<false>(ra, sa + i * 8 * kFragBytes, goff_a, kt * a_kstep + i * a_istep);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma_block_asm<false>(rb, sb + i * 8 * kFragBytes, goff_b, kt * b_kstep + i * b_istep);
+    };
+
+    // LDS -> registers.  K-contiguous operand: fragment i of k-step ks at base[ks] + 2048 i.  K-major operand:
+    // the two transposing reads of fragment i at base_i + 16384 ks (+ 2048 for the second one).
+    unsigned a_kc[2], b_kc[2], a_km[8], b_km[4];
+    {
+        const int a = r >> 2, b = r & 3, k = q * 8 + a;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const unsigned c = (unsigned)(r * 128 + (((ks * 4 + q) ^ kswz(r)) * 16));
+            a_kc[ks] = lds0 + wm * 16384 + c;
+            b_kc[ks] = lds0 + A_BYTES + wn * 8192 + c;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            a_km[i] = lds0 + (unsigned)(k * 512 + ((((wm * 8 + i) * 2 + (b >> 1)) ^ swz(k)) * 16) + (b & 1) * 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            b_km[j] = lds0 + A_BYTES + (unsigned)(k * 512 + ((((wn * 4 + j) * 2 + (b >> 1)) ^ swz(k)) * 16) + (b & 1) * 8);
+    }
+    u32x4 fa[8], fb[4];
+    auto read_frags = [&](int kt, auto ks_) {
+        constexpr int ks = decltype(ks_)::value;
+        const unsigned st = (kt & 1) * STAGE;
+        if constexpr (!B_KM) {
+            const unsigned ab = b_kc[ks] + st;
+            fb[0] = lds_rd128<0>(ab); fb[1] = lds_rd128<2048>(ab); fb[2] = lds_rd128<4096>(ab); fb[3] = lds_rd128<6144>(ab);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fb[j] = lds_rd_tr16x2<ks * 16384>(b_km[j] + st);
+        }
+        if constexpr (!A_KM) {
+            const unsigned aa = a_kc[ks] + st;
+            fa[0] = lds_rd128<0>(aa); fa[1] = lds_rd128<2048>(aa); fa[2] = lds_rd128<4096>(aa); fa[3] = lds_rd128<6144>(aa);
+            fa[4] = lds_rd128<8192>(aa); fa[5] = lds_rd128<10240>(aa); fa[6] = lds_rd128<12288>(aa); fa[7] = lds_rd128<14336>(aa);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) fa[i] = lds_rd_tr16x2<ks * 16384>(a_km[i] + st);
+        }
+    };
+    auto landed = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]), "+v"(fa[6]), "+v"(fa[7]),
+                       "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+#endif
+    };
+    int db_cnt = DB ? (kb / 64) % db_mod : 0;   // k-tile index modulo db_mod, counted along
+    bool sum_a = false;
+    auto compute = [&]() {
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i][j] = mfma_kstep<T>(fb[j], fa[i], acc[i][j]);
+        __builtin_amdgcn_s_setprio(0);
+    };
+    // the column sums of the k-step's A fragments, at the end of the memory phase (the other wave of the
+    // SIMD is multiplying meanwhile)
+    auto sum_frags = [&]() {
+        if constexpr (DB) {
+            if (sum_a) {   // the four waves of a row share its 8 A fragments: wave column wn sums fragments 2 wn, 2 wn + 1
+                if (wn == 0) { colsum[0] = frag_sum<T>(fa[0], colsum[0]); colsum[1] = frag_sum<T>(fa[1], colsum[1]); }
+                else if (wn == 1) { colsum[0] = frag_sum<T>(fa[2], colsum[0]); colsum[1] = frag_sum<T>(fa[3], colsum[1]); }
+                else if (wn == 2) { colsum[0] = frag_sum<T>(fa[4], colsum[0]); colsum[1] = frag_sum<T>(fa[5], colsum[1]); }
+                else { colsum[0] = frag_sum<T>(fa[6], colsum[0]); colsum[1] = frag_sum<T>(fa[7], colsum[1]); }
+            }
+        }
+    };
+    auto phase_end = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto loads_landed = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+    };
+
+    // k-tiles 0 and 1 are requested up front; tile kt + 1 (kt >= 1) in the first memory phase of k-tile kt, into
+    // the stage that k-tile kt - 1 left behind the barrier before (both halves have read its last fragments
+    // by then).  A wave waits for its loads of tile kt + 1 at the end of the phase before the one in which the
+    // upper half reads that tile's first fragments: the upper half behind the MFMAs of k-tile kt's second
+    // k-step, the lower half behind that k-step's fragment reads.
+    gload(0);
+    if (nkt > 1) {
+        gload(1);
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+#endif
+    } else {
+        loads_landed();
+    }
+    phase_end();
+    if (wm == 1) phase_end();   // the lower half runs one phase behind
+    for (int kt = 0; kt < nkt; ++kt) {
+        if constexpr (DB) {
+            sum_a = db_cnt == db_rem;
+            if (++db_cnt == db_mod) db_cnt = 0;
+        }
+        read_frags(kt, std::integral_constant<int, 0>{});
+        if (kt >= 1 && kt + 1 < nkt) gload(kt + 1);
+        landed();
+        sum_frags();
+        phase_end();
+        compute();
+        phase_end();
+        read_frags(kt, std::integral_constant<int, 1>{});
+        landed();
+        sum_frags();
+        if (wm == 1) loads_landed();
+        phase_end();
+        compute();
+        if (wm == 0) loads_landed();
+        phase_end();
+    }
+    if (wm == 0) phase_end();
+    __syncthreads();   // every wave has read its last fragments: the LDS is free
+}
+
 // Stores the accumulated tile: fp32 partials of `split` when p.splits > 1, else bias + rounding,
 // staged through LDS and written with 16-byte row-contiguous stores.
-template <typename T, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+// STREAM: the C tile leaves with non-temporal stores.  A stand-alone product writes 128 KiB per workgroup
+// that nothing reads again soon; as ordinary stores those lines displace the operand panels that the
+// workgroups of an XCD share through its L2 (M = 32768, N = 8192, K = 2048: 1240 -> 1500 TFLOP/s).
+template <typename T, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool STREAM = false>
 __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m0, const int n0, const int split,
                                                 unsigned char *smem,
                                                 const f32x4 (&acc)[BM / WVM / 16][BN / WVN / 16]) {
@@ -480,6 +712,26 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
     T *Cg = static_cast<T *>(p.C);
     constexpr int CPR = BN / 8;  // 16-byte chunks per C-tile row
     const bool vec_ok = (p.ldc & 7) == 0;
+    if constexpr ((BM * CPR) % THREADS == 0 && THREADS % CPR == 0) {
+        // a tile inside the matrix: all reads of a thread in flight, then all its stores (the guarded
+        // loop below waits for one LDS read per store)
+        if (vec_ok && m0 + BM <= p.M && n0 + BN <= p.N) {
+            constexpr int IT = BM * CPR / THREADS, RPI = THREADS / CPR;   // iterations; rows per iteration
+            const int ml0 = tid / CPR, nc = tid % CPR;
+            const unsigned char *src = smem + (size_t)ml0 * C::C_LD + nc * 16;
+            T *dst = Cg + (size_t)(m0 + ml0) * p.ldc + n0 + nc * 8;
+            u32x4 v[IT];
+#pragma unroll
+            for (int it = 0; it < IT; ++it) v[it] = *reinterpret_cast<const u32x4 *>(src + (size_t)it * RPI * C::C_LD);
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                u32x4 *d = reinterpret_cast<u32x4 *>(dst + (size_t)it * RPI * p.ldc);
+                if constexpr (STREAM) __builtin_nontemporal_store(v[it], d);
+                else *d = v[it];
+            }
+            return;
+        }
+    }
     for (int c = tid; c < BM * CPR; c += THREADS) {
         const int ml = c / CPR, nc = c % CPR;
         const int m = m0 + ml, n = n0 + nc * 8;
@@ -487,7 +739,8 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
         const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + (size_t)ml * C::C_LD + nc * 16);
         T *dst = Cg + (size_t)m * p.ldc + n;
         if (vec_ok && n + 8 <= p.N) {
-            *reinterpret_cast<u32x4 *>(dst) = v;
+            if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
+            else *reinterpret_cast<u32x4 *>(dst) = v;
         } else {
             const T *tv = reinterpret_cast<const T *>(&v);
             for (int e = 0; e < 8; ++e)
@@ -497,7 +750,9 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
 }
 
 // One BM x BN tile of C (rows m0.., columns n0.., K range of `split`): main loop + epilogue.
-template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
+// ALONE: the tile of a stand-alone GEMM launch (ping-pong main loop where the configuration has one,
+// streaming stores); the tiles that run inside a recurrent launch keep the symmetric loop.
+template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool ALONE = false>
 __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
                                             unsigned char *smem, const int trace_slot) {
     constexpr int TM = BM / WVM / 16, TN = BN / WVN / 16;
@@ -510,9 +765,12 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int kb = split * p.k_per_split;
     const int k_end = (A_KM && B_KM) ? (p.K + 63) / 64 * 64 : p.K;   // (rows past K read as zeros)
-    gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
+    if constexpr (ALONE && BM == 256 && BN == 256 && NS == 2 && WVM == 2 && WVN == 4 && KSPT == 2)
+        gemm16_mainloop_pp<T, A_KM, B_KM>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
+    else
+        gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
     if (p.trace) t_epi = (long long)wall_clock64();
-    gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, split, smem, acc);
+    gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT, ALONE>(p, m0, n0, split, smem, acc);
     if (p.trace && threadIdx.x == 0) {   // stamps: start, main loop entered (= start), main loop left, done
         long long *t = p.trace + (size_t)trace_slot * 4;
         t[0] = t_start; t[1] = t_start; t[2] = t_epi; t[3] = (long long)wall_clock64();
@@ -534,7 +792,91 @@ __global__ __launch_bounds__(64 * WVM * WVN) void gemm16_kernel(const GemmParams
     const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
     const int gsz = min(tiles_m - first_m, GM);
     const int m0 = (first_m + (lin % per_group) % gsz) * BM, n0 = ((lin % per_group) / gsz) * BN;
-    gemm16_tile<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, split, smem, (int)blockIdx.x);
+    gemm16_tile<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT, true>(p, m0, n0, split, smem, (int)blockIdx.x);
+}
+
+// Both weight-gradient products and the bias gradient of a layer in one launch:
+//     dWx[M][I] = A^T . x,   dWh[M][H] = A^T . h,   db[M] = column sums of A        (A = d_ifgo[K][M], K = T*B rows)
+// as one tile grid over [M] x [I | H]: the column tiles of the h product follow those of the x product, so the
+// A panels are shared by both products in the L2 and one split factor fills the device for both.  (h.N == 0:
+// the x product alone.)  Column tile nt of the grid sums the A fragments of the k-tiles congruent to nt modulo
+// the number of column tiles into db_part[split][nt][M] (gemm16_mainloop_pp, DB).  With splits > 1 the
+// products are fp32 partials per split as well; wgrad_reduce_kernel adds everything up in a fixed order.
+struct WgradParams {
+    GemmParams x, h;    // A, M, K, lda, splits, k_per_split agree; C / Cpart / B / N / ldb / ldc per product
+    int tiles_nx;       // column tiles of the x product
+    float *db_part;     // [splits][column tiles][M], or nullptr: no bias gradient
+};
+
+template <typename T> __global__ __launch_bounds__(512) void gemm16_wgrad_kernel(const WgradParams w) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tiles_m = cdiv(w.x.M, 256), tiles_n = w.tiles_nx + cdiv(w.h.N, 256);
+    int bid = blockIdx.x;
+    const int split = bid / (tiles_m * tiles_n);
+    bid -= split * tiles_m * tiles_n;
+    constexpr int GM = 8;
+    const int lin = xcd_major_id(bid, tiles_m * tiles_n);
+    const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    const int m0 = (first_m + (lin % per_group) % gsz) * 256, nt = (lin % per_group) / gsz;
+    const bool second = nt >= w.tiles_nx;
+    GemmParams p = w.x;
+    if (second) {
+        p.B = w.h.B; p.C = w.h.C; p.Cpart = w.h.Cpart;
+        p.N = w.h.N; p.ldb = w.h.ldb; p.ldc = w.h.ldc;
+    }
+    const int n0 = (second ? nt - w.tiles_nx : nt) * 256;
+    f32x4 acc[8][4];
+    float colsum[2] = {0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int kb = split * p.k_per_split, k_end = (p.K + 63) / 64 * 64;   // (rows past K read as zeros)
+    // (no bias gradient wanted: remainder -1 never comes up)
+    gemm16_mainloop_pp<T, true, true, true>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc, colsum, tiles_n,
+                                            w.db_part ? nt : -1);
+    gemm16_epilogue<T, 256, 256, 2, 2, 4, 2, true>(p, m0, n0, split, smem, acc);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (w.db_part) {
+        // lane (q, r) holds the sum over its k-groups for row r of its two fragments: add the four lane groups
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float v = colsum[i];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            const int m = m0 + ((wave >> 2) * 8 + (wave & 3) * 2 + i) * 16 + (lane & 15);
+            if (lane < 16 && m < p.M) w.db_part[((size_t)split * tiles_n + nt) * p.M + m] = v;
+        }
+    }
+}
+
+// Finishes a weight-gradient launch: out = the sum over splits of the fp32 partials, in split order, for dWx
+// (M x I) and dWh (M x H) -- not called for with splits == 1, then I = H = 0 here -- and db (M) = the sum of its
+// db_parts partial sums.  A thread owns four consecutive elements of a matrix (I and H are multiples of 8) or
+// one element of db.
+template <typename T>
+__global__ void wgrad_reduce_kernel(const float *part_x, T *dWx, const float *part_h, T *dWh, const float *part_db, T *db,
+                                    int M, int I, int H, int splits, int db_parts) {
+    const size_t qx = (size_t)M * I / 4, qh = (size_t)M * H / 4;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const float *part;
+    T *out;
+    size_t total;
+    if (i < qx) { part = part_x; out = dWx; total = (size_t)M * I; }
+    else if (i < qx + qh) { i -= qx; part = part_h; out = dWh; total = (size_t)M * H; }
+    else {
+        i -= qx + qh;
+        if (i >= (size_t)M || !db) return;
+        float s = 0.f;
+        for (int k = 0; k < db_parts; ++k) s += part_db[(size_t)k * M + i];
+        db[i] = Elem<T>::from_f32(s);
+        return;
+    }
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < splits; ++k) s += *reinterpret_cast<const f32x4 *>(part + (size_t)k * total + i * 4);
+    T o[4] = {Elem<T>::from_f32(s[0]), Elem<T>::from_f32(s[1]), Elem<T>::from_f32(s[2]), Elem<T>::from_f32(s[3])};
+    *reinterpret_cast<u32x2 *>(out + i * 4) = *reinterpret_cast<u32x2 *>(o);
 }
 
 }  // namespace fastlstm

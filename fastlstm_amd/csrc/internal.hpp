@@ -21,6 +21,12 @@ void set_gemm_trace(long long *buf);
 void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km, bool allow_split,
                int *tile, int *splits);
 hipError_t launch_gemm_tiled(int dtype, const GemmParams &p, bool a_km, bool b_km, int tile, hipStream_t s);
+// dWx[M][I], dWh[M][H], db[M] from d_ifgo[K][M], x[K][I], h[K][H] in one launch (16-bit shapes that
+// wgrad_merged_plan accepts; ws holds wgrad_merged_workspace bytes)
+bool wgrad_merged_plan(int dtype, int M, int I, int H, int K, int *splits, int *k_per_split, bool *merged);
+size_t wgrad_merged_workspace(int dtype, int M, int I, int H, int K);
+hipError_t launch_wgrad_merged(int dtype, const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
+                               void *ws, int M, int I, int H, int K, hipStream_t s);
 
 // one function per element type (separate translation units, compiled in parallel)
 #define FASTLSTM_DECL_REC(SUF)                                                                       \

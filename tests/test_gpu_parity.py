@@ -1080,7 +1080,7 @@ def test_bwd_stack2_equals_two_layer_calls(T, B, I, H, dt, one_launch):
     torch.cuda.synchronize()
     assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
     for k in ref:
-        if k.startswith("dW"):
+        if k.startswith("dW") or k.startswith("db"):   # sums over T*B, in an order that depends on the launch form
             assert rel_err(got[k], ref[k].double().cpu().numpy()) < tol, k
         else:
             assert torch.equal(got[k], ref[k]), k
@@ -1133,9 +1133,9 @@ def test_bwd_layer_equals_separate_stages(T, B, I, H, dt):
         assert lib.fastlstm_ws_status(ws[:64].cpu().numpy().tobytes()) == _lib.OK
         res.append((d_ifgo, dx, dh, dc, db, dWx, dWh))
     for i, (a, b) in enumerate(zip(*res)):
-        if i < 5:
+        if i < 4:
             assert torch.equal(a, b), i
-        else:
+        else:   # db, dWx, dWh: the stand-alone stage sums over T*B in another order (split along K)
             assert rel_err(a, b) < tol, i
 
 
