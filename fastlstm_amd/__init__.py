@@ -1,2 +1,3 @@
 """MI355X-native LSTM forward/backward behind the FastLSTM Python interface."""
-from .lstm import FastLSTM, PersistentLSTMfn, PersistentLSTMStatefn, Wgrad, lstm_persistent_bwd, lstm_persistent_fwd  # noqa: F401
+from .lstm import (FastLSTM, PersistentLSTMfn, PersistentLSTMStatefn, Wgrad, lstm_persistent_bwd,  # noqa: F401
+                   lstm_persistent_fwd, pending_status)

@@ -29,6 +29,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
 def _deps():
     out = [os.path.join(CSRC, f) for f in os.listdir(CSRC)]
     out.append(os.path.join(os.path.dirname(HERE), "include", "fastlstm_hip.h"))
+    out.append(os.path.join(os.path.dirname(HERE), "include", "fastlstm_hip_diag.h"))
     return out
 
 

@@ -97,6 +97,8 @@ void device_info_set_probe(int device, int rr, int *status_host, int *status_dev
         g_device_cache[device].status_host = status_host;
         g_device_cache[device].status_dev = status_dev;
         g_status_words.fetch_add(1);
+    } else if (status_host) {
+        (void)hipHostFree(status_host);   // (a recurrent call has given the device its word already)
     }
 }
 
@@ -144,15 +146,33 @@ void probe_device(int device) {
     device_info_set_probe(device, rr, word, word_dev);
 }
 
-// Behind the launches of a recurrent call: carries the abort flag of its workspace to the device's status word.
-__global__ void collect_status_kernel(const WsHeader *hdr, int *status_word) {
-    if (threadIdx.x == 0 && __hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-        __hip_atomic_store(status_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+// Results of a recurrent call that are overwritten with NaN when its launches ended with the abort flag raised
+// (barrier time-out, workgroup on the wrong XCD): the failing call itself has returned success long before, so the
+// failure has to travel with its data -- a loss, a gradient scaler or an isfinite check trips in the same step.
+struct PoisonList {
+    void *p[8];
+    unsigned n[8];   // elements
+    int count, dtype;
+    void add(void *ptr, size_t elems) {
+        if (ptr && count < 8) { p[count] = ptr; n[count] = (unsigned)std::min<size_t>(elems, 1u << 24); ++count; }
+    }
+};
+
+// Behind the launches of a recurrent call: carries the abort flag of its workspace to the device's status word
+// (if the device has one) and poisons the call's results.
+__global__ void collect_status_kernel(const WsHeader *hdr, int *status_word, const PoisonList pl) {
+    if (!__hip_atomic_load(&hdr->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return;
+    if (threadIdx.x == 0 && status_word) __hip_atomic_store(status_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    for (int k = 0; k < pl.count; ++k)
+        for (unsigned i = threadIdx.x; i < pl.n[k]; i += blockDim.x) {
+            if (pl.dtype == FASTLSTM_FP32) static_cast<unsigned *>(pl.p[k])[i] = 0x7fc00000u;
+            else static_cast<unsigned short *>(pl.p[k])[i] = pl.dtype == FASTLSTM_FP16 ? 0x7e00 : 0x7fc0;
+        }
 }
 
 // The status word of the current device says that an earlier recurrent call failed: report it once.
 int take_pending_status() {
-    if (g_status_words.load() == 0) return FASTLSTM_OK;   // no device was ever planned for: nothing to look at
+    if (g_status_words.load() == 0) return FASTLSTM_OK;   // no device has a status word yet: nothing to look at
     DeviceInfo di;
     if (device_info(-1, &di) != FASTLSTM_OK || !di.status_host) return FASTLSTM_OK;
     if (__atomic_load_n(di.status_host, __ATOMIC_RELAXED) == 0) return FASTLSTM_OK;
@@ -160,13 +180,109 @@ int take_pending_status() {
     return FASTLSTM_ERR_TIMEOUT;
 }
 
+// A caller that never plans (fastlstm_plan_device) still gets a status word: allocated by its first recurrent
+// call outside stream capture (pinned host memory; no device allocation, no synchronisation).
+void ensure_status_word(int device, hipStream_t stream) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return;
+    int *word = nullptr, *word_dev = nullptr;
+    if (hipHostMalloc(reinterpret_cast<void **>(&word), 64, hipHostMallocMapped) != hipSuccess) return;
+    *word = 0;
+    if (hipHostGetDevicePointer(reinterpret_cast<void **>(&word_dev), word, 0) != hipSuccess) {
+        (void)hipHostFree(word);
+        return;
+    }
+    std::lock_guard<std::mutex> lock(g_device_mu);
+    if (device < 0 || device >= 64 || g_device_cache[device].status_host) {
+        (void)hipHostFree(word);   // (another thread was first)
+        return;
+    }
+    g_device_cache[device].status_host = word;
+    g_device_cache[device].status_dev = word_dev;
+    g_status_words.fetch_add(1);
+}
+
+// Recurrent launches of one device run one after the other, whatever streams they are enqueued on.  A
+// persistent launch holds its CUs until its last step; the workgroups of a second one on another stream get
+// the CUs that are left, and where that is not all of a barrier group both launches wait on each other's CUs
+// until the spin limit ends them (4 s).  So the library keeps one event per device: a recurrent entry point
+// records it behind its launches, and the next one on a DIFFERENT stream makes its stream wait for it first
+// (hipStreamWaitEvent: no host synchronisation).  Streams under capture are left alone: a graph orders its own
+// nodes, and an event recorded into a capture could not be waited for outside it.
+struct StreamOrder {
+    hipEvent_t event = nullptr;
+    hipStream_t last = nullptr;
+    bool recorded = false;
+};
+StreamOrder g_order[64];
+std::mutex g_order_mu;
+
+static bool capturing(hipStream_t s) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+}
+
+// At the start of every recurrent entry point: the failure of an earlier call, if one is pending; the wait
+// for the last recurrent call of the device where that one went to another stream.
+int begin_recurrent(void *stream_) {
+    if (int rc = take_pending_status()) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return FASTLSTM_OK;
+    std::lock_guard<std::mutex> lock(g_order_mu);
+    StreamOrder &o = g_order[device];
+    if (!o.recorded || o.last == stream || capturing(stream)) return FASTLSTM_OK;
+    return hipStreamWaitEvent(stream, o.event, 0) == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
+}
+
+// may_create: false for the entry point that must not allocate anything (it records only into an event that a
+// set-up call or an earlier entry point has created)
+static void order_record(int device, hipStream_t stream, bool may_create = true) {
+    if (device < 0 || device >= 64 || capturing(stream)) return;
+    std::lock_guard<std::mutex> lock(g_order_mu);
+    StreamOrder &o = g_order[device];
+    if (!o.event) {
+        if (!may_create) return;
+        if (hipEventCreateWithFlags(&o.event, hipEventDisableTiming) != hipSuccess) {
+            o.event = nullptr;
+            return;
+        }
+    }
+    if (hipEventRecord(o.event, stream) == hipSuccess) {
+        o.last = stream;
+        o.recorded = true;
+    }
+}
+
 // Wraps a recurrent entry point: rc of its launches; on success the status collection is enqueued behind them.
-int finish_recurrent(int rc, void *ws, void *stream) {
+// may_allocate: false for the entry point that must not allocate anything (no status word, no event then, unless a
+// set-up call made them: fastlstm_plan_device, fastlstm_noalloc_scratch_bytes or an earlier entry point).
+int finish_recurrent(int rc, void *ws, void *stream, const PoisonList &poison = PoisonList{}, bool may_allocate = true) {
     if (rc != FASTLSTM_OK) return rc;
     DeviceInfo di;
-    if (device_info(-1, &di) != FASTLSTM_OK || !di.status_dev) return rc;
-    collect_status_kernel<<<1, kWave, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const WsHeader *>(ws), di.status_dev);
-    return hipGetLastError() == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device_info(device, &di) != FASTLSTM_OK) return rc;
+    if (!di.status_dev && may_allocate) {
+        ensure_status_word(device, static_cast<hipStream_t>(stream));
+        (void)device_info(device, &di);
+    }
+    collect_status_kernel<<<1, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const WsHeader *>(ws), di.status_dev, poison);
+    if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
+    order_record(device, static_cast<hipStream_t>(stream), may_allocate);
+    return FASTLSTM_OK;
+}
+
+// the final slab [B*H] of a [T+1][B][H] state history
+static void *last_slab(void *base, int T, int B, int H, int dtype) {
+    return base ? static_cast<unsigned char *>(base) + (size_t)T * B * H * elem_bytes(dtype) : nullptr;
+}
+static PoisonList poison_fwd(int dtype, int T, int B, int H, void *out, void *cell, void *out_b = nullptr, void *cell_b = nullptr) {
+    PoisonList pl{};
+    pl.dtype = dtype;
+    const size_t bh = (size_t)B * H;
+    pl.add(last_slab(out, T, B, H, dtype), bh); pl.add(last_slab(cell, T, B, H, dtype), bh);
+    pl.add(last_slab(out_b, T, B, H, dtype), bh); pl.add(last_slab(cell_b, T, B, H, dtype), bh);
+    return pl;
 }
 
 typedef hipError_t (*FwdLauncher)(const FwdParams &, int, int, int, int, int, hipStream_t, int *);
@@ -608,7 +724,8 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     bool wgrad_inside = true;
     if (!lower) {
         const double per_cu = 3.5e9, rec_ms = T * (c.ntw == 1 ? 3.0e-3 : 5.4e-3);   // flop per ms and CU inside a launch
-        const double dx_flop = 2.0 * M * K * I, wg_flop = 2.0 * M * K * (I + H);
+        // (e.dx null: the caller wants no dx; e.dWx null: no weight gradients)
+        const double dx_flop = e.dx ? 2.0 * M * K * I : 0.0, wg_flop = e.dWx ? 2.0 * M * K * (I + H) : 0.0;
         const int wg_tiles = cdiv(K, 256) * (cdiv(I, 256) + cdiv(H, 256));
         const double tile_ms = cdiv(wg_tiles, n_helpers) * 2.0 * 256 * 256 * M / per_cu;
         const double all_ms = std::max(rec_ms, std::max((dx_flop + wg_flop) / (n_helpers * per_cu), tile_ms));
@@ -616,6 +733,7 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
         const double none_ms = rec_ms + (dx_flop + wg_flop) / (256 * per_cu);
         if (none_ms < std::min(all_ms, dx_ms)) return false;
         wgrad_inside = all_ms <= dx_ms;
+        if ((!wgrad_inside || !e.dWx) && !e.dx) return false;   // nothing left for the helpers
     }
     const int tiles_m = cdiv(M, 256), tiles_n = cdiv(I, 256);
     // a chunk: whole timesteps, about 8 row tiles (a short tail behind the recurrence), at most kMaxChunks chunks
@@ -1041,8 +1159,9 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
 
 int fastlstm_fwd_persistent(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
                             int H, int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
-    return finish_recurrent(fwd_persistent_impl(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream, 1), ws, stream);
+    if (int rc = begin_recurrent(stream)) return rc;
+    return finish_recurrent(fwd_persistent_impl(ifgo, out, cell, Wh, ws, ws_bytes, T, B, H, dtype, stream, 1), ws, stream,
+                            poison_fwd(dtype, T, B, H, out, cell));
 }
 
 // others / n_others: see fwd_persistent_impl (operands in the order of this call's own seven).
@@ -1169,9 +1288,12 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
 int fastlstm_bwd_persistent(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
                             void *d_ifgo, const void *Wh, void *ws, size_t ws_bytes, int T, int B, int H,
                             int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
-    return finish_recurrent(bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream),
-                            ws, stream);
+    if (int rc = begin_recurrent(stream)) return rc;
+    PoisonList pl{};
+    pl.dtype = dtype;
+    pl.add(dh, (size_t)B * H); pl.add(dc, (size_t)B * H); pl.add(d_ifgo, (size_t)4 * H);   // (d_ifgo[0][0]: every product made of it)
+    return finish_recurrent(bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream), ws,
+                            stream, pl);
 }
 
 // n = 2 ... kMaxSideBySide recurrences of one shape (recs[r]: the operand pointers of recurrence r in the order of
@@ -1250,7 +1372,7 @@ static int multi_sequential(bool backward, int n, void *const (*r)[7], void *ws,
 
 int fastlstm_fwd_persistent_multi(int n, void *const *ifgo, void *const *out, void *const *cell, const void *const *Wh, void *ws,
                                   size_t ws_bytes, int T, int B, int H, int dtype, int keep_activations, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     if (!ifgo || !out || !cell || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (n < 1 || n > kMaxSideBySide) return FASTLSTM_ERR_DIM;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
@@ -1267,13 +1389,16 @@ int fastlstm_fwd_persistent_multi(int n, void *const *ifgo, void *const *out, vo
     const int keep = keep_activations ? 1 : 0;
     int rc = try_multi(false, n, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
     if (rc == 1) rc = multi_sequential(false, n, recs, ws, ws_bytes, T, B, H, dtype, stream, keep);
-    return finish_recurrent(rc, ws, stream);
+    PoisonList pl{};
+    pl.dtype = dtype;
+    for (int i = 0; i < n; ++i) { pl.add(last_slab(recs[i][1], T, B, H, dtype), (size_t)B * H); pl.add(last_slab(recs[i][2], T, B, H, dtype), (size_t)B * H); }
+    return finish_recurrent(rc, ws, stream, pl);
 }
 
 int fastlstm_bwd_persistent_multi(int n, const void *const *dout, void *const *dh, void *const *dc, const void *const *ifgo,
                                   const void *const *cell, void *const *d_ifgo, const void *const *Wh, void *ws, size_t ws_bytes,
                                   int T, int B, int H, int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !ws) return FASTLSTM_ERR_NULL;
     if (n < 1 || n > kMaxSideBySide) return FASTLSTM_ERR_DIM;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
@@ -1290,7 +1415,10 @@ int fastlstm_bwd_persistent_multi(int n, const void *const *dout, void *const *d
     if (!aligned16(ws)) return FASTLSTM_ERR_ALIGN;
     int rc = try_multi(true, n, recs, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
     if (rc == 1) rc = multi_sequential(true, n, recs, ws, ws_bytes, T, B, H, dtype, stream, 1);
-    return finish_recurrent(rc, ws, stream);
+    PoisonList pl{};
+    pl.dtype = dtype;
+    for (int i = 0; i < n; ++i) { pl.add(recs[i][1], (size_t)B * H); pl.add(recs[i][5], (size_t)4 * H); }
+    return finish_recurrent(rc, ws, stream, pl);
 }
 
 int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
@@ -1300,7 +1428,7 @@ int fastlstm_pair_fused(int T, int B, int H, int dtype, int backward, size_t ws_
 int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const void *Wh_a, void *ifgo_b, void *out_b,
                                  void *cell_b, const void *Wh_b, void *ws, size_t ws_bytes, int T, int B, int H, int dtype,
                                  int keep_activations, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     if (!ifgo_a || !out_a || !cell_a || !Wh_a || !ifgo_b || !out_b || !cell_b || !Wh_b || !ws) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, H, H)) return rc;
@@ -1313,14 +1441,14 @@ int fastlstm_fwd_persistent_pair(void *ifgo_a, void *out_a, void *cell_a, const 
     for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
     int rc = try_multi(false, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep, false);
     if (rc == 1) rc = multi_sequential(false, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, keep);
-    return finish_recurrent(rc, ws, stream);
+    return finish_recurrent(rc, ws, stream, poison_fwd(dtype, T, B, H, out_a, cell_a, out_b, cell_b));
 }
 
 int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, const void *ifgo_a, const void *cell_a,
                                  void *d_ifgo_a, const void *Wh_a, const void *dout_b, void *dh_b, void *dc_b,
                                  const void *ifgo_b, const void *cell_b, void *d_ifgo_b, const void *Wh_b, void *ws,
                                  size_t ws_bytes, int T, int B, int H, int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     void *const a[7] = {const_cast<void *>(dout_a), dh_a, dc_a, const_cast<void *>(ifgo_a), const_cast<void *>(cell_a), d_ifgo_a,
                         const_cast<void *>(Wh_a)};
     void *const b[7] = {const_cast<void *>(dout_b), dh_b, dc_b, const_cast<void *>(ifgo_b), const_cast<void *>(cell_b), d_ifgo_b,
@@ -1337,7 +1465,10 @@ int fastlstm_bwd_persistent_pair(const void *dout_a, void *dh_a, void *dc_a, con
     for (int i = 0; i < 7; ++i) { recs[0][i] = a[i]; recs[1][i] = b[i]; }
     int rc = try_multi(true, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, 1, false);
     if (rc == 1) rc = multi_sequential(true, 2, recs, ws, ws_bytes, T, B, H, dtype, stream, 1);
-    return finish_recurrent(rc, ws, stream);
+    PoisonList pl{};
+    pl.dtype = dtype;
+    pl.add(dh_a, (size_t)B * H); pl.add(d_ifgo_a, (size_t)4 * H); pl.add(dh_b, (size_t)B * H); pl.add(d_ifgo_b, (size_t)4 * H);
+    return finish_recurrent(rc, ws, stream, pl);
 }
 
 static int fwd_layer_impl(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
@@ -1372,17 +1503,17 @@ static int fwd_layer_impl(const void *x, const void *Wx, const void *bx, const v
 int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
                        void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
                        void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream, 1), ws,
-                            stream);
+                            stream, poison_fwd(dtype, T, B, H, out, cell));
 }
 
 int fastlstm_fwd_layer_infer(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
                              void *out, void *cell, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
                              void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ws, ws_bytes, T, B, I, H, dtype, stream, 0), ws,
-                            stream);
+                            stream, poison_fwd(dtype, T, B, H, out, cell));
 }
 
 // ---- fastlstm_fwd_layer for callers that cannot allocate ---------------------------------------
@@ -1408,14 +1539,29 @@ static int scratch_of_current_device(unsigned char **out) {
     return FASTLSTM_OK;
 }
 
-size_t fastlstm_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+// Also the set-up call of fastlstm_fwd_layer_noalloc for the current device: looks up the array's device address
+// and creates what the failure reporting and the ordering of streams need (a pinned status word, an event), so
+// that the entry point itself -- possibly under stream capture -- neither allocates nor looks anything up.
+size_t fastlstm_noalloc_scratch_bytes(void) {
+    unsigned char *ptr = nullptr;
+    int device = -1;
+    if (scratch_of_current_device(&ptr) == FASTLSTM_OK && hipGetDevice(&device) == hipSuccess) {
+        DeviceInfo di;
+        if (device_info(device, &di) == FASTLSTM_OK && !di.status_dev) ensure_status_word(device, nullptr);
+        std::lock_guard<std::mutex> lock(g_order_mu);
+        if (device >= 0 && device < 64 && !g_order[device].event &&
+            hipEventCreateWithFlags(&g_order[device].event, hipEventDisableTiming) != hipSuccess)
+            g_order[device].event = nullptr;
+    }
+    return kNoAllocScratchBytes;
+}
 
 int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh, void *ifgo,
                                void *out, void *cell, int T, int B, int I, int H, int dtype, void *stream) {
     if (!x || !Wx || !bx || !bh || !Wh || !ifgo || !out || !cell) return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     fastlstm_plan pl;
     if (int rc = plan_device(-1, B, H, dtype, 0, &pl, false)) return rc;
     // the smallest workspace of this shape has to fit; beyond that the call uses as much of the array
@@ -1431,7 +1577,7 @@ int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, co
     zero_words_kernel<<<256, 256, 0, static_cast<hipStream_t>(stream)>>>(reinterpret_cast<unsigned *>(ptr), zero / 4);
     if (hipGetLastError() != hipSuccess) return FASTLSTM_ERR_HIP;
     return finish_recurrent(fwd_layer_impl(x, Wx, bx, bh, Wh, ifgo, out, cell, ptr, use, T, B, I, H, dtype, stream, 1), ptr,
-                            stream);
+                            stream, poison_fwd(dtype, T, B, H, out, cell), false);
 }
 
 size_t fastlstm_stack2_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
@@ -1490,28 +1636,31 @@ int fastlstm_fwd_stack2(const void *x, const void *Wx0, const void *bx0, const v
                         void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1, const void *Wh1,
                         void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T, int B, int I, int H,
                         int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     return finish_recurrent(fwd_stack2_impl(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1,
                                             ws, ws_bytes, T, B, I, H, dtype, stream, 1),
-                            ws, stream);
+                            ws, stream, poison_fwd(dtype, T, B, H, out1, cell1, out0, cell0));
 }
 
 int fastlstm_fwd_stack2_infer(const void *x, const void *Wx0, const void *bx0, const void *bh0, const void *Wh0,
                               void *ifgo0, void *out0, void *cell0, const void *Wx1, const void *bx1, const void *bh1,
                               const void *Wh1, void *ifgo1, void *out1, void *cell1, void *ws, size_t ws_bytes, int T,
                               int B, int I, int H, int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
     return finish_recurrent(fwd_stack2_impl(x, Wx0, bx0, bh0, Wh0, ifgo0, out0, cell0, Wx1, bx1, bh1, Wh1, ifgo1, out1, cell1,
                                             ws, ws_bytes, T, B, I, H, dtype, stream, 0),
-                            ws, stream);
+                            ws, stream, poison_fwd(dtype, T, B, H, out1, cell1, out0, cell0));
 }
 
 static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
                           const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
                           void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
                           int H, int dtype, void *stream) {
-    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !x || !h || !dx || !dWx || !dWh || !db ||
-        !ws || !wgrad_ws)
+    // dx may be null (no gradient of the layer's input is wanted: K5 is skipped), and so may dWx, dWh and db,
+    // all three together (frozen weights: K8, K9 and the bias sum are skipped)
+    const bool want_w = dWx || dWh || db;
+    if (!dout || !dh || !dc || !ifgo || !cell || !d_ifgo || !Wh || !Wx || !x || !h || !ws || !wgrad_ws ||
+        (want_w && (!dWx || !dWh || !db)))
         return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
@@ -1528,7 +1677,7 @@ static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo
     if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     int rc = 1;
-    if (pl.wave_split != 2) {
+    if (pl.wave_split != 2 && (dx || want_w)) {
         const BwdExtras e{Wx, x, h, dx, dWx, dWh, I};
         rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
                          s, &e);
@@ -1544,8 +1693,10 @@ static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo
         if (int r2 = bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
             return r2;
         // (the weight-gradient workspace is free until the next call: scratch for a split along K)
-        if (int r2 = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, wgrad_ws, wgrad_ws_bytes, stream)) return r2;
+        if (dx)
+            if (int r2 = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, wgrad_ws, wgrad_ws_bytes, stream)) return r2;
     }
+    if (!want_w) return FASTLSTM_OK;
     return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
 }
 
@@ -1553,10 +1704,16 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
                        const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
                        void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
                        int H, int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
+    PoisonList pl{};
+    pl.dtype = dtype;
+    if (dtype_ok(dtype) && B > 0 && H > 0 && I > 0) {
+        pl.add(dh, (size_t)B * H); pl.add(dc, (size_t)B * H); pl.add(dx, (size_t)B * I); pl.add(db, (size_t)4 * H);
+        pl.add(dWx, (size_t)I); pl.add(dWh, (size_t)H);
+    }
     return finish_recurrent(bwd_layer_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, Wx, x, h, dx, dWx, dWh, db, ws, ws_bytes,
                                            wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream),
-                            ws, stream);
+                            ws, stream, pl);
 }
 
 size_t fastlstm_stack2_bwd_workspace_bytes(const fastlstm_plan *plan, int T, int H, int dtype) {
@@ -1595,8 +1752,8 @@ static int bwd_stack2_impl(const void *dout, void *dh1, void *dc1, const void *i
                            void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
                            int dtype, void *stream) {
     if (!dout || !dh1 || !dc1 || !ifgo1 || !cell1 || !d_ifgo1 || !Wh1 || !Wx1 || !out1 || !dWx1 || !dWh1 || !db1 || !dx1 ||
-        !dh0 || !dc0 || !ifgo0 || !cell0 || !d_ifgo0 || !Wh0 || !Wx0 || !x || !out0 || !dx0 || !dWx0 || !dWh0 || !db0 ||
-        !ws || !wgrad_ws)
+        !dh0 || !dc0 || !ifgo0 || !cell0 || !d_ifgo0 || !Wh0 || !Wx0 || !x || !out0 || !dWx0 || !dWh0 || !db0 ||
+        !ws || !wgrad_ws)   // (dx0 may be null: no gradient of the stack's input is wanted)
         return FASTLSTM_ERR_NULL;
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
@@ -1653,11 +1810,17 @@ int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo
                         const void *Wx0, const void *x, const void *out0, void *dx0, void *dWx0, void *dWh0, void *db0,
                         void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H,
                         int dtype, void *stream) {
-    if (int rc = take_pending_status()) return rc;
+    if (int rc = begin_recurrent(stream)) return rc;
+    PoisonList pl{};
+    pl.dtype = dtype;
+    if (dtype_ok(dtype) && B > 0 && H > 0 && I > 0) {
+        pl.add(dh1, (size_t)B * H); pl.add(dh0, (size_t)B * H); pl.add(dx0, (size_t)B * I); pl.add(db1, (size_t)4 * H);
+        pl.add(db0, (size_t)4 * H); pl.add(dWx1, (size_t)H); pl.add(dWx0, (size_t)I); pl.add(dx1, (size_t)B * H);
+    }
     return finish_recurrent(bwd_stack2_impl(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, Wx1, out1, dWx1, dWh1, db1, dx1, dh0, dc0,
                                             ifgo0, cell0, d_ifgo0, Wh0, Wx0, x, out0, dx0, dWx0, dWh0, db0, ws, ws_bytes,
                                             wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream),
-                            ws, stream);
+                            ws, stream, pl);
 }
 
 int fastlstm_recurrent_kernel_kind(int T, int B, int H, int dtype, int backward, size_t ws_bytes) {
@@ -1723,6 +1886,7 @@ int fastlstm_device_status(int device, int clear) {
 }
 
 void fastlstm_set_kernel_families(int mask) { fastlstm::g_families.store(mask & 7); }
+int fastlstm_get_kernel_families(void) { return fastlstm::g_families.load(); }
 
 void fastlstm_set_spin_limit(long long ticks) {
     if (ticks > 0) fastlstm::g_spin_limit.store(ticks);

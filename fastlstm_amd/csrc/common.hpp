@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/fastlstm_hip.h"
+#include "../../include/fastlstm_hip_diag.h"
 
 namespace fastlstm {
 

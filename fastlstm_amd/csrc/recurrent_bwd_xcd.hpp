@@ -231,7 +231,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
              i += n_helpers) {
             const int r = i - k * per_chunk;
             const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
-            if (rt >= p.k5_tiles_m) continue;
+            if (rt >= p.k5_tiles_m || !p.k5.C) continue;   // (no dx wanted: the helpers only accumulate weight gradients)
             helper_dx_tile<T>(p.k5.A, p.k5.B, p.k5.C, p.k5.M, p.k5.N, p.k5.K, rt * 256, ct * 256,
                               (FASTLSTM_LDS_PTR unsigned char *)smem);
             if (stacked) {   // the tile's stores acknowledged, this XCD's L2 written back, then counted

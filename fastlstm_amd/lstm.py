@@ -41,6 +41,55 @@ _DTYPE_CODE = {torch.float32: _lib.FP32, torch.float16: _lib.FP16, torch.bfloat1
 CHECK_STATUS = os.environ.get("FASTLSTM_CHECK_STATUS", "0") == "1"
 
 
+# Host-phase profiler ranges (the reference brackets its host phases with torch.cuda.nvtx ranges,
+# fastlstm/lstm.py:32-144, 237-292, 508-516; on ROCm they reach rocprofv3 --marker-trace as roctx ranges).
+# Off unless FASTLSTM_PROFILE_RANGES=1: a range costs a microsecond or two of host time per phase.
+PROFILE_RANGES = os.environ.get("FASTLSTM_PROFILE_RANGES", "0") == "1"
+
+
+class _Range:
+    __slots__ = ("name",)
+
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_push(self.name)
+
+    def __exit__(self, *exc):
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_pop()
+        return False
+
+
+def pending_status(device=None, clear=False):
+    """Status of the recurrent launches enqueued on `device` so far that have already run: 0, or the error code of a
+    launch that ended in a barrier time-out or on the wrong XCD (fastlstm_device_status).  Reads one pinned host
+    word: no synchronisation.  A launch that has not finished yet cannot be reported -- synchronise first to learn
+    about the last call of a program.  clear=True resets the word."""
+    if device is None:
+        idx = torch.cuda.current_device()
+    else:
+        device = torch.device(device)
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+    return _lib.load().fastlstm_device_status(idx, 1 if clear else 0)
+
+
+def _raise_pending(device):
+    """Raises for a failed earlier launch on `device` (and clears the report), before new work is enqueued behind
+    it.  The results of the failed call itself hold NaN (the library poisons them), so a loss computed from them
+    is not finite either."""
+    status = pending_status(device, clear=True)
+    if status != _lib.OK:
+        _lib.check(status, "an earlier fastlstm launch on %s" % (device,))
+
+
+def _raise_pending_before_backward(grad):
+    if grad is not None and grad.is_cuda and not torch.cuda.is_current_stream_capturing():
+        _raise_pending(grad.device)
+
+
 def _code(t):
     if t.dtype not in _DTYPE_CODE:
         raise TypeError("fastlstm_amd supports float32, float16 and bfloat16, got %s" % t.dtype)
@@ -142,16 +191,19 @@ def lstm_persistent_fwd(x, h0, c0, Wx, bx, Wh, bh, version=None, keep_activation
         # be 16-byte aligned for the vector loads of the weight-gradient GEMM
         out = torch.empty((seq_len + 1, batch_size, hidden_size), device=x.device, dtype=x.dtype)
         cell = torch.empty_like(out)
-        plan = _plan(x.device, batch_size, hidden_size, code, False)
-        stream = _stream()
-        ws = _prepared_forward_workspace(plan, seq_len, hidden_size, code, out, cell, h0, c0, stream)
+        with _Range("fastlstm: prepare forward"):
+            plan = _plan(x.device, batch_size, hidden_size, code, False)
+            stream = _stream()
+            ws = _prepared_forward_workspace(plan, seq_len, hidden_size, code, out, cell, h0, c0, stream)
         # input projection + time loop in one call (the library fuses the two where CUs would idle)
         entry = lib.fastlstm_fwd_layer if keep_activations else lib.fastlstm_fwd_layer_infer
-        _lib.check(entry(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
-                         ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws.data_ptr(),
-                         ws.numel(), seq_len, batch_size, input_size, hidden_size, code, stream),
-                   "fastlstm_fwd_layer")
-        _check_ws(ws, "fastlstm_fwd_layer")
+        with _Range("fastlstm: forward layer launch"):
+            _lib.check(entry(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
+                             ifgo.data_ptr(), out.data_ptr(), cell.data_ptr(), ws.data_ptr(),
+                             ws.numel(), seq_len, batch_size, input_size, hidden_size, code, stream),
+                       "fastlstm_fwd_layer")
+        with _Range("fastlstm: status"):
+            _check_ws(ws, "fastlstm_fwd_layer")
     return out, cell, ifgo
 
 
@@ -194,8 +246,18 @@ def multi_runs_in_one_launch(n, T, B, H, dtype, device, backward=False):
         return lib.fastlstm_multi_fused(n, T, B, H, code, int(backward), nb) == 1
 
 
-@functools.lru_cache(maxsize=512)
+def _families():
+    """The kernel families the library may dispatch to (fastlstm_set_kernel_families; all of them unless a test or
+    an experiment switched some off).  Part of every cache key below: their answers depend on it."""
+    return _lib.load().fastlstm_get_kernel_families()
+
+
 def _wavefront_chunks(L, T, B, H, dtype, device, backward):
+    return _wavefront_chunks_cached(L, T, B, H, dtype, device, backward, _families())
+
+
+@functools.lru_cache(maxsize=512)
+def _wavefront_chunks_cached(L, T, B, H, dtype, device, backward, families):
     # chunks of at least 64 timesteps: every launch costs about 50 us besides its steps (launch gaps, the prologue,
     # the small GEMMs in between), which a chunk of 32 steps does not win back (measured: no gain at T = 256 with
     # 8 chunks); whole 16-byte units per timestep, so that every chunk's buffers start on a 16-byte boundary
@@ -303,7 +365,7 @@ def _fwd_stack_wavefront(x, layers, n, keep_activations):
     return bufs
 
 
-def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
+def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n, need_dx=True):
     """Reverse pass of _fwd_stack_wavefront: acts[l] = (out, cell, ifgo), weights[l] = (Wx, Wh), d_states[l] = None or
     (dh_n, dc_n).  Launch k runs chunk n - 1 - (k - u) of layer L - 1 - u for every u side by side; a lower layer's
     dout of a chunk (the dx of the layer above) is a GEMM launch in between; the weight gradients and the lowest
@@ -359,8 +421,10 @@ def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n):
             _ptr_array([pdg[l]]), _ptr_array([pWh[l]]), p(ws), ws.numel(), r, B, H, code, stream), "fastlstm_bwd_persistent_multi")
     for ws in wss:
         _check_ws(ws, "fastlstm_bwd_persistent_multi")
-    dx0 = torch.empty_like(x)
-    _lib.check(lib.fastlstm_gemm_dx(pdg[0], pWx[0], p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
+    dx0 = None
+    if need_dx:   # (else: no gradient of the stack's input is asked for)
+        dx0 = torch.empty_like(x)
+        _lib.check(lib.fastlstm_gemm_dx(pdg[0], pWx[0], p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
     res = []
     for l in range(L):
         xin = x if l == 0 else acts[l - 1][0][1:]
@@ -375,9 +439,10 @@ def _fwd_stack2_wavefront(x, h0a, c0a, Wx0, bx0, Wh0, bh0, h0b, c0b, Wx1, bx1, W
     return out0, cell0, ifgo0, out1, cell1, ifgo1
 
 
-def _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1, n):
+def _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1, n,
+                          need_dx=True):
     r0, r1 = _bwd_stack_wavefront(dh, x, [(out0, cell0, ifgo0), (out1, cell1, ifgo1)], [(Wx0, Wh0), (Wx1, Wh1)],
-                                  [d_state0, d_state1], n)
+                                  [d_state0, d_state1], n, need_dx)
     return r0, r1
 
 
@@ -410,10 +475,10 @@ def _pairs_min_hidden(B):
     return 576 if B > 32 else 704
 
 
-def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
+def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None, need_dx=True):
     """Reverse pass of lstm_persistent_fwd_stack: acts[l] = (out, cell, ifgo), weights[l] = (Wx, Wh), d_states[l] = None
     or (dh_n, dc_n).  [(d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)] per layer; falls back to one layer after the other where
-    the reverse time loops do not fit side by side."""
+    the reverse time loops do not fit side by side.  need_dx=False: the lowest layer's d_x is not computed (None)."""
     L = len(acts)
     d_states = list(d_states) if d_states is not None else [None] * L
     T, B, H = dh.shape
@@ -427,28 +492,33 @@ def lstm_persistent_bwd_stack(dh, x, acts, weights, d_states=None):
         # B = 16 6.16 / 6.82, H = 1024, B = 8 6.52 / 7.21; level at H = 512; H = 384 7.68 / 6.90; 4 x (T = 512, I = 256,
         # H = 576): B = 48 6.66 / 9.13, B = 64 7.69 / 9.71, B = 32 6.34 / 6.49).
         plan = _plan(x.device, B, H, code, True)
-        if L >= 3 and H >= _pairs_min_hidden(B) and lib.fastlstm_bwd_stack2_fused(
-                T, B, H, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1:
+        # (the pairs from the top down: the lowest pair reads the stack's input, whose size need not be H)
+        lowest_I = x.shape[-1] if L % 2 == 0 else H
+        pair_fused = lambda I_: lib.fastlstm_bwd_stack2_fused(
+            T, B, I_, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) == 1
+        if L >= 3 and H >= _pairs_min_hidden(B) and pair_fused(H) and (lowest_I == H or pair_fused(lowest_I)):
             l = L - 1
             while l >= 1:
                 xin = x if l == 1 else acts[l - 2][0][1:]
                 res[l - 1], res[l] = lstm_persistent_bwd_stack2(dh, xin, *acts[l - 1], weights[l - 1][0], weights[l - 1][1],
                                                                 *acts[l], weights[l][0], weights[l][1],
-                                                                d_state0=d_states[l - 1], d_state1=d_states[l])
+                                                                d_state0=d_states[l - 1], d_state1=d_states[l],
+                                                                need_dx=need_dx or l > 1)
                 dh = res[l - 1][0]
                 l -= 2
             L = l + 1   # a lowest layer without a partner follows below
         else:
             n = stack_wavefront_chunks(L, T, B, H, acts[0][2].dtype, x.device, backward=True)
             if n:
-                return _bwd_stack_wavefront(dh, x, acts, weights, d_states, n)
+                return _bwd_stack_wavefront(dh, x, acts, weights, d_states, n, need_dx)
         for l in range(L - 1, -1, -1):
             out, cell, ifgo = acts[l]
             dt = ifgo.dtype
             zeros = lambda: torch.zeros((B, H), device=x.device, dtype=dt)
             dhn, dcn = (zeros(), zeros()) if d_states[l] is None else tuple(d.to(dt).reshape(B, H).clone() for d in d_states[l])
             xin = x if l == 0 else acts[l - 1][0][1:]
-            res[l] = lstm_persistent_bwd(dh, dcn, dhn, xin, out, cell, ifgo, weights[l][0], weights[l][1])
+            res[l] = lstm_persistent_bwd(dh, dcn, dhn, xin, out, cell, ifgo, weights[l][0], weights[l][1],
+                                         need_dx=need_dx or l > 0)
             dh = res[l][0]
         return res
 
@@ -523,11 +593,14 @@ def Wgrad(d_ifgo, x, h):
     return db, db, dWx, dWh
 
 
-def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
+def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh, need_dx=True, need_dw=True):
     """Reverse pass.  dh[T,B,H]: gradient of out[1:]; dc_n, dh_n [B,H]: gradients
     flowing into the last cell / hidden state, overwritten with the gradients of
     the initial state and returned (fastlstm/lstm.py:236-334).
-    Returns (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)."""
+    Returns (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh).  need_dx=False: the product d_ifgo . Wx is
+    skipped and d_x is None (no gradient of the layer's input is asked for: the first layer of most
+    models); need_dw=False: the weight and bias gradients are skipped and None (frozen weights).
+    The reference computes all of them whatever autograd asks for (fastlstm/lstm.py:524-538)."""
     _require_gpu(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh)
     code = _code(ifgo)
     seq_len, batch_size, hidden_size = dh.shape
@@ -539,39 +612,52 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh):
             dh = dh.to(ifgo.dtype)
         dh = _aligned(dh)
         assert dc_n.is_contiguous() and dh_n.is_contiguous()
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_push("fastlstm: prepare backward")
         d_ifgo = torch.empty_like(ifgo)
         plan = _plan(x.device, batch_size, hidden_size, code, True)
         ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
         x, h = _aligned(x.contiguous()), h.contiguous()
-        d_x = torch.empty_like(x)
+        d_x = torch.empty_like(x) if need_dx else None
         G = 4 * hidden_size
-        dWx = torch.empty((G, input_size), device=x.device, dtype=x.dtype)
-        dWh = torch.empty((G, hidden_size), device=x.device, dtype=x.dtype)
-        db = torch.empty((G,), device=x.device, dtype=x.dtype)
+        dWx = dWh = db = None
+        if need_dw:
+            dWx = torch.empty((G, input_size), device=x.device, dtype=x.dtype)
+            dWh = torch.empty((G, hidden_size), device=x.device, dtype=x.dtype)
+            db = torch.empty((G,), device=x.device, dtype=x.dtype)
         wws = torch.empty(lib.fastlstm_wgrad_workspace_bytes(seq_len, batch_size, input_size, hidden_size, code),
                           dtype=torch.uint8, device=x.device)
+        ptr = lambda t: None if t is None else t.data_ptr()   # (a null pointer: that result is not wanted)
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_pop()
         # reverse time loop + dx + weight gradients in one call (the library fuses them where CUs would idle)
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_push("fastlstm: backward layer launch")
         _lib.check(lib.fastlstm_bwd_layer(dh.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
                                           cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), Wx.data_ptr(),
-                                          x.data_ptr(), h.data_ptr(), d_x.data_ptr(), dWx.data_ptr(),
-                                          dWh.data_ptr(), db.data_ptr(), ws.data_ptr(), ws.numel(),
+                                          x.data_ptr(), h.data_ptr(), ptr(d_x), ptr(dWx),
+                                          ptr(dWh), ptr(db), ws.data_ptr(), ws.numel(),
                                           wws.data_ptr(), wws.numel(), seq_len, batch_size, input_size,
                                           hidden_size, code, stream),
                    "fastlstm_bwd_layer")
-        _check_ws(ws, "fastlstm_bwd_layer")
+        if PROFILE_RANGES:
+            torch.cuda.nvtx.range_pop()
+        with _Range("fastlstm: status"):
+            _check_ws(ws, "fastlstm_bwd_layer")
         dbx = dbh = db   # the same tensor twice, as Wgrad returns it (fastlstm/lstm.py:501)
     return d_x, dh_n, dc_n, dWx, dbx, dWh, dbh
 
 
 def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1,
-                               d_state0=None, d_state1=None):
+                               d_state0=None, d_state1=None, need_dx=True):
     """Reverse pass of two stacked layers (suffix 1: upper, 0: lower); dh[T,B,H] is the gradient of
     out1[1:]; d_state0 / d_state1 are optional (dh_n, dc_n) pairs, the gradients flowing into the
     final states of the lower / upper layer (zero when None).  The same results as lstm_persistent_bwd for
     the upper layer followed by lstm_persistent_bwd for the lower layer on the upper layer's d_x;
     one launch for both recurrences where the library can run them side by side.
-    Returns ((d_x, dh_0, dc_0, dWx, dbx, dWh, dbh) of the lower layer, the same of the upper layer)."""
+    Returns ((d_x, dh_0, dc_0, dWx, dbx, dWh, dbh) of the lower layer, the same of the upper layer);
+    need_dx=False: the lower layer's d_x is not computed and None."""
     _require_gpu(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1)
     code = _code(ifgo1)
     T, B, H = dh.shape
@@ -582,7 +668,7 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         n = stack2_wavefront_chunks(T, B, H, ifgo1.dtype, x.device, backward=True)
         if n and lib.fastlstm_bwd_stack2_fused(T, B, I, H, code, lib.fastlstm_stack2_bwd_workspace_bytes(plan, T, H, code)) != 1:
             return _bwd_stack2_wavefront(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1,
-                                         d_state0, d_state1, n)
+                                         d_state0, d_state1, n, need_dx)
         dh = dh.contiguous()
         if dh.dtype != ifgo1.dtype:
             dh = dh.to(ifgo1.dtype)
@@ -593,7 +679,7 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         d_ifgo1, d_ifgo0 = torch.empty_like(ifgo1), torch.empty_like(ifgo0)
         state = lambda d, k: zeros() if d is None else d[k].to(x.dtype).reshape(B, H).clone()
         dh1, dc1, dh0, dc0 = state(d_state1, 0), state(d_state1, 1), state(d_state0, 0), state(d_state0, 1)
-        dx1, dx0 = new(T, B, H), torch.empty_like(x)
+        dx1, dx0 = new(T, B, H), (torch.empty_like(x) if need_dx else None)
         dWx1, dWh1, db1 = new(G, H), new(G, H), new(G)
         dWx0, dWh0, db0 = new(G, I), new(G, H), new(G)
         plan = _plan(x.device, B, H, code, True)
@@ -602,7 +688,7 @@ def lstm_persistent_bwd_stack2(dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1,
         ws[:(n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes))].zero_()
         # (large enough for the one launch to take the lower layer's weight gradients too)
         wws = torch.empty(lib.fastlstm_stack2_bwd_wgrad_workspace_bytes(T, B, I, H, code), dtype=torch.uint8, device=x.device)
-        p = lambda t: t.data_ptr()
+        p = lambda t: None if t is None else t.data_ptr()
         _lib.check(lib.fastlstm_bwd_stack2(
             p(dh), p(dh1), p(dc1), p(ifgo1), p(cell1), p(d_ifgo1), p(Wh1), p(Wx1), p(out1), p(dWx1), p(dWh1), p(db1), p(dx1),
             p(dh0), p(dc0), p(ifgo0), p(cell0), p(d_ifgo0), p(Wh0), p(Wx0), p(x), p(out0), p(dx0), p(dWx0), p(dWh0), p(db0),
@@ -669,11 +755,12 @@ def lstm_persistent_fwd_pair(xa, h0a, c0a, Wxa, bxa, Wha, bha, xb, h0b, c0b, Wxb
 
 
 def lstm_persistent_bwd_pair(dh_a, d_state_a, xa, out_a, cell_a, ifgo_a, Wxa, Wha,
-                             dh_b, d_state_b, xb, out_b, cell_b, ifgo_b, Wxb, Whb):
+                             dh_b, d_state_b, xb, out_b, cell_b, ifgo_b, Wxb, Whb, need_dx=(True, True)):
     """Reverse pass of lstm_persistent_fwd_pair: dh_* [T,B,H] are the gradients of out_*[1:], d_state_* optional
     (dh_n, dc_n) pairs (zero when None).  The two reverse time loops are one launch where the library can run
     them side by side; dx and the weight gradients follow per layer.  The same results as two calls of
-    lstm_persistent_bwd.  Returns two tuples (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh)."""
+    lstm_persistent_bwd.  Returns two tuples (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh); need_dx[k] False: that
+    side's d_x is not computed (None)."""
     _require_gpu(dh_a, dh_b, xa, xb, out_a, cell_a, ifgo_a, Wxa, Wha, out_b, cell_b, ifgo_b, Wxb, Whb)
     code = _code(ifgo_a)
     T, B, H = dh_a.shape
@@ -701,10 +788,13 @@ def lstm_persistent_bwd_pair(dh_a, d_state_a, xa, out_a, cell_a, ifgo_a, Wxa, Wh
             p(ws), ws.numel(), T, B, H, code, stream), "fastlstm_bwd_persistent_pair")
         _check_ws(ws, "fastlstm_bwd_persistent_pair")
         res = []
-        for x, out, d_ifgo, Wx, dhn, dcn in ((xa, out_a, d_ifgo_a, Wxa, dhn_a, dcn_a), (xb, out_b, d_ifgo_b, Wxb, dhn_b, dcn_b)):
+        for x, out, d_ifgo, Wx, dhn, dcn, want in ((xa, out_a, d_ifgo_a, Wxa, dhn_a, dcn_a, need_dx[0]),
+                                                   (xb, out_b, d_ifgo_b, Wxb, dhn_b, dcn_b, need_dx[1])):
             x = _aligned(x.contiguous())
-            d_x = torch.empty_like(x)
-            _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo), p(Wx.contiguous()), p(d_x), T, B, I, H, code, stream), "fastlstm_gemm_dx")
+            d_x = None
+            if want:
+                d_x = torch.empty_like(x)
+                _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo), p(Wx.contiguous()), p(d_x), T, B, I, H, code, stream), "fastlstm_gemm_dx")
             dbx, dbh, dWx, dWh = Wgrad(d_ifgo, x, out)
             res.append((d_x, dhn, dcn, dWx, dbx, dWh, dbh))
     return res[0], res[1]
@@ -739,13 +829,15 @@ class PersistentLSTMfn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh, d_out_cell):
+        _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
         if d_out_cell is None:
             dc_n, dh_n = torch.zeros_like(cell[0]), torch.zeros_like(cell[0])
         else:
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
+        need = ctx.needs_input_grad   # (x, h_0, c_0, Wx, bx, Wh, bh)
         d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(
-            dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh
+            dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh, need_dx=need[0], need_dw=any(need[3:7])
         )
         if ctx.h0_is_nan:
             dh_0 = None
@@ -773,11 +865,14 @@ class PersistentLSTMStatefn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh, dh_n, dc_n):
+        _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
         # the kernel overwrites its state operands with the gradients of the initial state
         dh_n = dh_n.to(cell.dtype).contiguous().clone()
         dc_n = dc_n.to(cell.dtype).contiguous().clone()
-        d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh)
+        need = ctx.needs_input_grad
+        d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh,
+                                                                 need_dx=need[0], need_dw=any(need[3:7]))
         if ctx.no_state:
             dh_0 = dc_0 = None
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
@@ -802,9 +897,12 @@ class PersistentLSTMHistoryfn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh, _):
+        _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
+        need = ctx.needs_input_grad
         d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(
-            dh, torch.zeros_like(cell[0]), torch.zeros_like(cell[0]), x, out, cell, ifgo, Wx, Wh)
+            dh, torch.zeros_like(cell[0]), torch.zeros_like(cell[0]), x, out, cell, ifgo, Wx, Wh,
+            need_dx=need[0], need_dw=any(need[3:7]))
         if ctx.no_state:
             dh_0 = dc_0 = None
         return d_x, dh_0, dc_0, dWx, dbx, dWh, dbh
@@ -834,11 +932,13 @@ class PersistentLSTMPairfn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh_a, dhn_a, dcn_a, dh_b, dhn_b, dcn_b, _ha, _hb):
+        _raise_pending_before_backward(dh_a)   # a failed forward launch is reported before its gradients are computed
         xa, out_a, cell_a, ifgo_a, Wxa, Wha, xb, out_b, cell_b, ifgo_b, Wxb, Whb = ctx.saved_tensors
         pair = lambda h, c: None if h is None and c is None else (
             torch.zeros_like(cell_a[0]) if h is None else h, torch.zeros_like(cell_a[0]) if c is None else c)
         ga, gb = lstm_persistent_bwd_pair(dh_a, pair(dhn_a, dcn_a), xa, out_a, cell_a, ifgo_a, Wxa, Wha,
-                                          dh_b, pair(dhn_b, dcn_b), xb, out_b, cell_b, ifgo_b, Wxb, Whb)
+                                          dh_b, pair(dhn_b, dcn_b), xb, out_b, cell_b, ifgo_b, Wxb, Whb,
+                                          need_dx=(ctx.needs_input_grad[0], ctx.needs_input_grad[7]))
         ga, gb = list(ga), list(gb)
         if ctx.no_state[0]:
             ga[1] = ga[2] = None
@@ -880,6 +980,7 @@ class PersistentLSTMStackfn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh, *d_finals):
+        _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         L = ctx.L
         x, rest = ctx.saved_tensors[0], ctx.saved_tensors[1:]
         acts = [tuple(rest[5 * l:5 * l + 3]) for l in range(L)]
@@ -889,7 +990,7 @@ class PersistentLSTMStackfn(torch.autograd.Function):
         for l in range(L):
             h, c = d_finals[2 * l], d_finals[2 * l + 1]
             d_states.append(None if h is None and c is None else (zero() if h is None else h, zero() if c is None else c))
-        res = lstm_persistent_bwd_stack(dh, x, acts, weights, d_states)
+        res = lstm_persistent_bwd_stack(dh, x, acts, weights, d_states, need_dx=ctx.needs_input_grad[0])
         grads = [res[0][0], None, None]
         for l in range(L):
             _, dh0, dc0, dWx, dbx, dWh, dbh = res[l]
@@ -924,6 +1025,7 @@ class PersistentLSTMStack2fn(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type="cuda")
     def backward(ctx, dh, *d_states):
+        _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1 = ctx.saved_tensors
         d_state0 = d_state1 = None
         if len(d_states) == 4:
@@ -931,7 +1033,8 @@ class PersistentLSTMStack2fn(torch.autograd.Function):
         elif any(d is not None for d in d_states):
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
         (d_x, dh0a, dc0a, dWx0, dbx0, dWh0, dbh0), (_, dh0b, dc0b, dWx1, dbx1, dWh1, dbh1) = lstm_persistent_bwd_stack2(
-            dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1)
+            dh, x, out0, cell0, ifgo0, Wx0, Wh0, out1, cell1, ifgo1, Wx1, Wh1, d_state0, d_state1,
+            need_dx=ctx.needs_input_grad[0])
         if ctx.no_state[0]:
             dh0a = dc0a = None
         if ctx.no_state[1]:
@@ -964,9 +1067,13 @@ def _indices_to_device(dev, *tensors):
     return on_dev.split([t.numel() for t in tensors])
 
 
-@functools.lru_cache(maxsize=4096)
 def _recurrent_kind(T, B, H, code, device_index, backward=False):
     """fastlstm_recurrent_kernel_kind of the forward (reverse) call for the workspace this module allocates."""
+    return _recurrent_kind_cached(T, B, H, code, device_index, backward, _families())
+
+
+@functools.lru_cache(maxsize=4096)
+def _recurrent_kind_cached(T, B, H, code, device_index, backward, families):
     lib = _lib.load()
     device = torch.device("cuda", device_index)
     with torch.cuda.device(device):
@@ -975,8 +1082,12 @@ def _recurrent_kind(T, B, H, code, device_index, backward=False):
         return lib.fastlstm_recurrent_kernel_kind(T, B, H, code, b, lib.fastlstm_recurrent_workspace_bytes(plan, T, H, code, b))
 
 
-@functools.lru_cache(maxsize=4096)
 def _padded_hidden_size(T, B, H, code, device_index, training=False):
+    return _padded_hidden_size_cached(T, B, H, code, device_index, training, _families())
+
+
+@functools.lru_cache(maxsize=4096)
+def _padded_hidden_size_cached(T, B, H, code, device_index, training, families):
     """The next hidden size above H (within a quarter, in steps of the MFMA k-step) that the XCD-local or the
     register-resident kernels take, when H itself gets the general kernels; else 0.  `training`: a reverse pass
     follows, whose kernels count too."""
@@ -1221,6 +1332,9 @@ class FastLSTM(nn.Module):
         if self.version != "persistent":
             # the reference also offers "graph", "naive-pt" and "v1"; this build has one path
             raise ValueError(f"Not Implemnted: {self.version}")
+        data = x.data if isinstance(x, nn.utils.rnn.PackedSequence) else x
+        if data.is_cuda and not torch.cuda.is_current_stream_capturing():
+            _raise_pending(data.device)   # a failed earlier launch is reported before new work goes behind it
         padding = self._operand_padding(x)
         if padding:
             return self._forward_operands_padded(x, h_c_0, *padding)

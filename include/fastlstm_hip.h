@@ -55,10 +55,17 @@ typedef enum {
  * workgroup is resident while its peers spin (the rule of
  * fastlstm/configs.py:29-58); a batch that does not fit is processed in
  * `batch_chunks` sequential launches (fastlstm/kernels.py:514, 663).
- * The rule counts one launch at a time: two recurrent launches on different
- * streams of one GPU can each hold a part of the compute units and wait for
- * the other's missing workgroups until the time-out; callers that use
- * several streams order the library's calls with an event. */
+ * The rule counts one launch at a time.  Two recurrent launches on different
+ * streams of one GPU could each hold a part of the compute units and wait for
+ * the other's missing workgroups until the time-out, so the library orders
+ * them itself: every recurrent entry point records an event (one per device)
+ * behind its launches, and the next recurrent entry point on ANOTHER stream of
+ * that device makes its stream wait for that event first (hipStreamWaitEvent,
+ * no host synchronisation).  Recurrent work of different streams therefore
+ * runs one call after the other on a device.  Not covered: launches recorded
+ * into a graph by stream capture (the library neither records nor waits while
+ * a stream is capturing) -- replaying two such graphs at the same time, or one
+ * next to an eager call, is for the caller to order. */
 typedef struct {
     int num_cus;      /* compute units used for planning */
     int lds_limit;    /* bytes of LDS one workgroup may use */
@@ -130,7 +137,12 @@ int fastlstm_fwd_layer(const void *x, const void *Wx, const void *bx, const void
  * ones).  FASTLSTM_ERR_WORKSPACE if the smallest workspace of the shape (plan.ws_bytes) exceeds the array.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads)
  * race; serialise them.  The XCD-local kernels are only chosen on a device that fastlstm_plan_device has
- * seen (that call probes and may allocate; this one never does). */
+ * seen (that call probes and may allocate; this one never does).  Set-up: call
+ * fastlstm_noalloc_scratch_bytes() once per device, with that device current and outside stream capture,
+ * before the first fastlstm_fwd_layer_noalloc there: it looks up the array's device address and creates
+ * the pinned status word and the event of the failure reporting and stream ordering described above
+ * (without it the entry point still works, looks the address up at its first call -- not a capturable
+ * operation -- and reports no failures until some other call has created the status word). */
 int fastlstm_fwd_layer_noalloc(const void *x, const void *Wx, const void *bx, const void *bh, const void *Wh,
                                void *ifgo, void *out, void *cell, int T, int B, int I, int H, int dtype,
                                void *stream);
@@ -224,7 +236,10 @@ size_t fastlstm_multi_workspace_bytes(const fastlstm_plan *plan, int n, int T, i
  * reverse recurrence leaves CUs without a role, the workgroups on those CUs compute dx and the
  * weight gradients (or dx alone, whichever an estimate of their throughput makes the shorter call) inside
  * the same launch, chunk of timesteps by chunk behind the recurrence; otherwise the stages are launched
- * back to back.  Replaces fastlstm/lstm.py:277-290, 294 and
+ * back to back.  dx may be NULL: no gradient of the layer's input is wanted (autograd's needs_input_grad:
+ * the first layer of most models) and K5 is skipped, inside the launch and outside it; dWx, dWh and db may
+ * be NULL, all three together: the weights are frozen and K6..K9 are skipped.  (The reference computes all
+ * of them whatever autograd asks for, fastlstm/lstm.py:524-538.)  Replaces fastlstm/lstm.py:277-290, 294 and
  * 494-501 together. */
 int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell,
                        void *d_ifgo, const void *Wh, const void *Wx, const void *x, const void *h,
@@ -258,7 +273,8 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
  * and B = 48 ... 64) they compute dx1 and dx0 only and all four weight gradients follow as launches.  ws: fastlstm_stack2_bwd_workspace_bytes, zeroed like
  * any recurrent workspace; wgrad_ws: at least the larger of the two layers'
  * fastlstm_wgrad_workspace_bytes; with fastlstm_stack2_bwd_wgrad_workspace_bytes (64 MiB at H = I = 1024)
- * the launch takes the lower layer's dWx0, dWh0 too.  Replaces two backward nodes of the layer loop at
+ * the launch takes the lower layer's dWx0, dWh0 too.  dx0 may be NULL (no gradient of the stack's input is
+ * wanted: its product is skipped).  Replaces two backward nodes of the layer loop at
  * fastlstm/lstm.py:685-696 (each lstm.py:236-334 + 494-501). */
 int fastlstm_bwd_stack2(const void *dout, void *dh1, void *dc1, const void *ifgo1, const void *cell1,
                         void *d_ifgo1, const void *Wh1, const void *Wx1, const void *out1, void *dWx1,
@@ -298,63 +314,35 @@ int fastlstm_recurrent_rows_per_launch(int T, int B, int H, int dtype, int backw
 int fastlstm_prepare_forward(void *ws, size_t zero_bytes, void *out0, void *cell0, const void *h0, const void *c0,
                              int B, int H, int dtype, void *stream);
 
-/* Diagnostics: which kernel families the recurrent entry points may choose besides the general kernels: bit 0 =
- * the XCD-local kernels, bit 1 = the register-resident kernels of H = 1280 ... 2048, bit 2 = the form of their
- * reverse kernel in which teams of workgroups split the sums over K (default 7: all).  With 0
- * every shape runs the general kernels, which lets a test or a measurement put two families side by side on
- * the same inputs.  Process-wide; no counterpart in the reference. */
-void fastlstm_set_kernel_families(int mask);
-
 /* Reads the status word the recurrent kernels leave at the start of their
  * workspace; `ws_head` points to a HOST copy of the first 64 bytes.
  * 0 = ok, FASTLSTM_ERR_TIMEOUT = a barrier wait gave up (the kernel still ran
  * to completion, its results are invalid). */
 int fastlstm_ws_status(const void *ws_head);
 
-/* Failure reporting without a host synchronisation.  The first fastlstm_plan_device call for a device
- * allocates one pinned, device-visible status word for it.  Every recurrent entry point
- * (fastlstm_fwd_persistent, _fwd_layer[_infer], _fwd_stack2[_infer], _bwd_persistent, _bwd_layer,
- * _bwd_stack2) enqueues, behind its launches, one tiny kernel that sets the word if the call's workspace
- * ended with the abort flag raised (a barrier wait gave up, or a workgroup of an XCD-placed barrier group
- * found itself on another XCD than the one the placement rule assumes).  The NEXT recurrent entry on that
- * device then returns FASTLSTM_ERR_TIMEOUT before launching anything and clears the word: the results
- * of the earlier call are invalid, and the caller learns it at most one call late instead of never.
- * fastlstm_device_status reads the word of `device` (-1: current) at any time: FASTLSTM_OK or
- * FASTLSTM_ERR_TIMEOUT; clear != 0 resets it.  It reflects the calls whose work has completed on the
- * device by now.  No counterpart in the reference (its spin loops are unbounded, fastlstm/kernels.py:546-548). */
+/* Failure reporting without a host synchronisation.  Every device gets one pinned, device-visible status
+ * word: from its first fastlstm_plan_device call, or from its first recurrent entry point outside stream
+ * capture.  Every recurrent entry point (fastlstm_fwd_persistent, _fwd_layer[_infer|_noalloc],
+ * _fwd_stack2[_infer], _fwd/_bwd_persistent_pair, _fwd/_bwd_persistent_multi, _bwd_persistent, _bwd_layer,
+ * _bwd_stack2) enqueues, behind its launches, one tiny kernel that looks at the abort flag of the call's
+ * workspace (a barrier wait gave up, or a workgroup of an XCD-placed barrier group found itself on another
+ * XCD than the placement rule assumes).  If it is raised the kernel
+ *   - sets the device's status word: the NEXT recurrent entry on that device returns FASTLSTM_ERR_TIMEOUT
+ *     before launching anything and clears the word, and fastlstm_device_status reads it at any time;
+ *   - overwrites results of the failed call with NaN -- forward: out[T] and cell[T]; reverse: dh, dc and
+ *     the first row of d_ifgo (fastlstm_bwd_persistent, from which every product made of it inherits),
+ *     or dh, dc, db, the first timestep of dx and the first row of dWx, dWh (fastlstm_bwd_layer,
+ *     _bwd_stack2) -- so that a loss, a gradient scaler or an isfinite check on the results trips in the
+ *     same step, although the failing call itself returned FASTLSTM_OK long before.
+ * What stays unreported: the last call of a program, if nobody looks at its results or at
+ * fastlstm_device_status after synchronising.
+ * fastlstm_device_status reads the word of `device` (-1: current): FASTLSTM_OK or FASTLSTM_ERR_TIMEOUT;
+ * clear != 0 resets it.  It reflects the calls whose work has completed on the device by now.  No
+ * counterpart in the reference (its spin loops are unbounded, fastlstm/kernels.py:546-548). */
 int fastlstm_device_status(int device, int clear);
 
-/* Upper bound, in 100 MHz ticks, a barrier wait may spin before it gives up
- * (default 4e8 = 4 s).  Tests lower it to force the time-out path from the host. */
-void fastlstm_set_spin_limit(long long ticks);
-
-/* Diagnostics: when `buf` (device memory, 32 bytes per workgroup of the largest GEMM grid)
- * is non-NULL the 16-bit GEMM kernels record 4 stamps of the 100 MHz clock per workgroup
- * (start, main loop entered, main loop left, done).  NULL switches it off (default). */
-void fastlstm_set_gemm_trace(void *buf);
-
-/* Diagnostics: when `buf` (zero-filled device memory, 32 bytes per workgroup) is non-NULL the
- * recurrent kernels accumulate, per workgroup and in 100 MHz ticks, four phase times: forward =
- * waiting for peers, operand fetch + MFMA, reduce + gate maths, publish; backward = gate maths,
- * publish + stores, waiting for peers, operand fetch + MFMA + reduce. */
-void fastlstm_set_recurrent_trace(void *buf);
-
-/* Diagnostics: the latency bound of one recurrence step.  Runs `steps` rounds of the links of a timestep
- * that no arithmetic throughput removes, with the recurrent kernels' own barrier and exchange code:
- * mode 0 = the empty barrier (publish + wait), 1 = + every member stores its share of a `rows`-row fp16 h
- * tile into the step's exchange slot (slot t % 2), 2 = + every wave fetches its operand blocks of the step
- * (loads that go past the L1, as in the kernels); 3, 4 (kind 0 only) = the exchange without a barrier:
- * consumers poll the data itself, unwritten values hold an all-ones sentinel, loads bypass the L1 (sc1 /
- * sc0 sc1); the exchange slots of ws (everything from byte 66560 on) must then hold 0xFF bytes.
- * kind 0 = an XCD-local group of `members` <= 32 workgroups (counters in that XCD's L2), kind 1 = a flag
- * group of `members` <= 256 workgroups over all XCDs (device-scope flags).  H <= 2048, a multiple of 32 and of
- * `members`; rows = 16, 32, 48 or 64 batch rows per group.  The caller times the launch (its duration /
- * steps = microseconds per round); ws: zeroed device memory of fastlstm_diag_step_probe_bytes.  No
- * counterpart in the reference. */
-int fastlstm_diag_step_probe(int kind, int mode, int members, int H, int rows, int steps, void *ws,
-                             size_t ws_bytes, void *stream);
-size_t fastlstm_diag_step_probe_bytes(int steps, int H, int rows);
-
+/* (Diagnostics and test hooks -- kernel-family switch, spin limit, clock traces, the step-latency probe --
+ * are declared in fastlstm_hip_diag.h.) */
 const char *fastlstm_strerror(int status);
 const char *fastlstm_version(void);
 

@@ -1,4 +1,4 @@
-"""CPU-side tests: the C ABI loads and exports what include/fastlstm_hip.h declares,
+"""CPU-side tests: the C ABI loads and exports what include/fastlstm_hip.h and fastlstm_hip_diag.h declare,
 argument validation returns error codes before any HIP call, the tiling rule keeps
 its invariants, the barrier/version protocol is deadlock- and hazard-free in a model,
 and the Python module mirrors the reference's interface (fastlstm/lstm.py:586-698)."""
@@ -20,7 +20,11 @@ HAS_GPU = torch.cuda.is_available()
 
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "fastlstm_hip.h")).read()
-    declared = set(re.findall(r"\b(fastlstm_[a-z_0-9]+)\s*\(", header))
+    diag = open(os.path.join(ROOT, "include", "fastlstm_hip_diag.h")).read()
+    product = set(re.findall(r"\b(fastlstm_[a-z_0-9]+)\s*\(", header))
+    # the boundary header carries no process-wide switches and no measurement code
+    assert not any(n.startswith(("fastlstm_set_", "fastlstm_diag_", "fastlstm_get_")) for n in product), product
+    declared = product | set(re.findall(r"\b(fastlstm_[a-z_0-9]+)\s*\(", diag))
     assert {"fastlstm_fwd_persistent", "fastlstm_bwd_persistent", "fastlstm_gemm_ifgo", "fastlstm_gemm_dx",
             "fastlstm_gemm_wgrad", "fastlstm_plan_for", "fastlstm_strerror"} <= declared
     lib = ctypes.CDLL(_lib.LIB_PATH)

@@ -30,15 +30,17 @@ def _buffers(T, B, H, dt, h0, c0):
 # first a shape whose ring fits the static array (XCD-local kernel, projection inside the launch, 5.3 MiB of
 # the array written), then a smaller, ragged one (general kernel, its exchange blocks have padding that must
 # read as zero: the array still holds the first call's data), then the first again
+# ... and a batch of 300 rows at H = 1024, which runs as several launches over ranges of rows that share the array
+# (the barrier counters are cleared in between)
 CASES = [(40, 64, 256, 1024, torch.float16, 1), (12, 20, 48, 160, torch.float16, 2), (9, 33, 70, 300, torch.float32, 3),
-         (40, 64, 256, 1024, torch.float16, 4)]
+         (40, 64, 256, 1024, torch.float16, 4), (24, 300, 128, 1024, torch.float16, 5)]
 
 
 def test_noalloc_forward_equals_forward_with_a_workspace():
     assert torch.cuda.is_available()
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
-    cap = lib.fastlstm_noalloc_scratch_bytes()
+    cap = lib.fastlstm_noalloc_scratch_bytes()   # (also the set-up call: address of the array, status word, event)
     assert cap == 16 << 20
     for T, B, I, H, dt, seed in CASES:
         code = L._DTYPE_CODE[dt]
@@ -53,11 +55,17 @@ def test_noalloc_forward_equals_forward_with_a_workspace():
                                           ifgo_a.data_ptr(), out_a.data_ptr(), cell_a.data_ptr(), ws.data_ptr(), ws.numel(),
                                           T, B, I, H, code, st), "fastlstm_fwd_layer")
         ifgo_b, out_b, cell_b = _buffers(T, B, H, dt, h0, c0)
-        before = torch.cuda.memory_allocated()
+        if B == 300:
+            assert lib.fastlstm_recurrent_rows_per_launch(T, B, H, code, 0, nbytes) > 0   # several launches
+        # the device's own count of free bytes (hipMemGetInfo): it would show a hipMalloc inside the library,
+        # which torch's allocator statistics cannot
+        torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         _lib.check(lib.fastlstm_fwd_layer_noalloc(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), Wh.data_ptr(),
                                                   ifgo_b.data_ptr(), out_b.data_ptr(), cell_b.data_ptr(), T, B, I, H, code,
                                                   st), "fastlstm_fwd_layer_noalloc")
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before
         torch.cuda.synchronize()
         assert lib.fastlstm_device_status(0, 0) == _lib.OK
         assert torch.equal(out_a, out_b), (T, B, I, H)
