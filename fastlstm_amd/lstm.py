@@ -115,9 +115,16 @@ def _stream():
 
 
 def _plan(device, B, H, code, backward):
-    plan = _lib.Plan()
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    _lib.check(_lib.load().fastlstm_plan_device(idx, B, H, code, int(backward), plan), "fastlstm_plan_device")
+    return _plan_cached(idx, B, H, code, int(backward))
+
+
+@functools.lru_cache(maxsize=4096)
+def _plan_cached(idx, B, H, code, backward):
+    """The tiling of a (device, B, H, dtype, direction): a pure function of its arguments (the first call per device
+    also probes the device), kept across calls -- callers only read the struct."""
+    plan = _lib.Plan()
+    _lib.check(_lib.load().fastlstm_plan_device(idx, B, H, code, backward, plan), "fastlstm_plan_device")
     return plan
 
 
@@ -1455,6 +1462,10 @@ class FastLSTM(nn.Module):
             return x, (h_n[0].unsqueeze(0), c_n[0].unsqueeze(0))
         return x, (torch.stack(h_n), torch.stack(c_n))
 
+    # Opt-in (set on an instance or on the class): keep the zero-padded copies of the parameters across inference
+    # calls (see _OperandsPadded._layer_operands for when they are refreshed, and for the case they miss).
+    cache_padded_operands = False
+
     def _operand_padding(self, x):
         """(Hp, Ip): hidden and input size to zero-pad this call to, or None when it runs as it is.
 
@@ -1549,13 +1560,31 @@ class _OperandsPadded:
     def _layer_operands(self, layer, suffix=""):
         if (layer, suffix) not in self._operands:
             H, Hp, D = self._module.hidden_size, self.hidden_size, 2 if self.bidirectional else 1
-            Wx, bx, Wh, bh = self._module._layer_operands(layer, suffix)
+            base = self._module._layer_operands(layer, suffix)
+            Wx, bx, Wh, bh = base
+            # Where no gradient can reach the parameters (inference) and the module opted in
+            # (FastLSTM.cache_padded_operands), the padded copies are kept on the module across calls, stamped with the
+            # identity and the version counter of each parameter: an optimizer step, a load_state_dict or a new
+            # Parameter object makes the stamp differ and the copies are made again.  Off by default: an in-place edit
+            # through `.data` (weight clipping, swapping in averaged weights) bypasses the version counter and would
+            # leave stale copies.  (A training call needs the pads in its autograd graph and makes them per call.)
+            keep = (self.bias and getattr(self._module, "cache_padded_operands", False)
+                    and not (torch.is_grad_enabled() and any(t.requires_grad for t in base)))
+            key = (layer, suffix, Hp, self.input_size)
+            stamp = tuple((id(t), t._version, t.data_ptr(), t.dtype, t.device) for t in base)
+            cache = self._module.__dict__.setdefault("_padded_operand_cache", {})
+            if keep and key in cache and cache[key][0] == stamp:
+                self._operands[(layer, suffix)] = cache[key][1]
+                return cache[key][1]
             p = Hp - H
             if layer == 0:
                 Wx = F.pad(Wx.reshape(4, H, -1), (0, self.input_size - self._module.input_size, 0, p))
             else:
                 Wx = F.pad(Wx.reshape(4, H, D, H), (0, p, 0, 0, 0, p))
-            self._operands[(layer, suffix)] = (
-                Wx.reshape(4 * Hp, -1), F.pad(bx.reshape(4, H), (0, p)).reshape(-1),
-                F.pad(Wh.reshape(4, H, H), (0, p, 0, p)).reshape(4 * Hp, Hp), F.pad(bh.reshape(4, H), (0, p)).reshape(-1))
+            ops = (Wx.reshape(4 * Hp, -1), F.pad(bx.reshape(4, H), (0, p)).reshape(-1),
+                   F.pad(Wh.reshape(4, H, H), (0, p, 0, p)).reshape(4 * Hp, Hp), F.pad(bh.reshape(4, H), (0, p)).reshape(-1))
+            if keep:
+                ops = tuple(t.detach() for t in ops)
+                cache[key] = (stamp, ops)
+            self._operands[(layer, suffix)] = ops
         return self._operands[(layer, suffix)]

@@ -187,3 +187,27 @@ def test_dispatch_caches_follow_the_kernel_family_switch():
     lib.fastlstm_set_kernel_families(7)
     assert L._recurrent_kind(64, 16, 512, code, 0) == 1
     assert L.stack_wavefront_chunks(2, 256, 16, 512, torch.float16, "cuda:0") == chunks
+
+
+def test_padded_operand_cache_is_opt_in_and_follows_the_version_counters():
+    """Inference with a hidden size that runs zero-padded: with cache_padded_operands the padded weights are kept
+    across calls and refreshed when a parameter's version counter moves (an optimizer-style in-place update)."""
+    T, B, I, H, dt = 40, 16, 300, 300, torch.float16
+    m = _module(I, H, 1, dt, 7)
+    x = torch.randn(T, B, I, device="cuda").to(dt)
+    with torch.no_grad():
+        assert m._operand_padding(x) is not None        # this shape is padded
+        y0 = m(x)[0].clone()
+        assert not m.__dict__.get("_padded_operand_cache")    # off by default: nothing kept
+        m.cache_padded_operands = True
+        y1 = m(x)[0].clone()
+        kept = m._padded_operand_cache
+        assert len(kept) == 1 and torch.equal(y0, y1)
+        first = next(iter(kept.values()))[1][0]
+        y2 = m(x)[0].clone()
+        assert next(iter(kept.values()))[1][0] is first and torch.equal(y1, y2)    # reused
+        m.weight_hh_l0.mul_(0.5)                          # bumps the version counter
+        y3 = m(x)[0].clone()
+        assert next(iter(kept.values()))[1][0] is not first
+        m.cache_padded_operands = False
+        assert torch.equal(y3, m(x)[0]) and not torch.equal(y3, y2)
