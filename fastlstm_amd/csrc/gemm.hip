@@ -107,12 +107,13 @@ hipError_t launch_colsum_t(const void *in, void *out, float *part, int R, int C,
 // The 16-bit fast kernel needs: K range of every split a multiple of 64, 16-byte aligned
 // rows, operands addressable with 32-bit byte offsets.
 bool gemm16_eligible(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool b_km) {
-    if (dtype == FASTLSTM_FP32) return false;
+    // (fp32 runs on the 256 x 256 tile only: see gemm_plan)
+    const int es = dtype == FASTLSTM_FP32 ? 4 : 2, epc = 16 / es;
     // K-major x K-major (the weight gradients, K = T*B rows): any K -- the loop runs to the next multiple of 64 and the
     // rows past K lie outside both operands' buffer ranges, where loads return zero
-    if ((K % 64 != 0 && !(a_km && b_km)) || lda % 8 != 0 || ldb % 8 != 0) return false;
+    if ((K % 64 != 0 && !(a_km && b_km)) || lda % epc != 0 || ldb % epc != 0) return false;
     // 32-bit byte offsets, with room for the rows a partial tile reaches past the operand
-    const size_t a_bytes = (size_t)((a_km ? K : M) + 256) * lda * 2, b_bytes = (size_t)((b_km ? K : N) + 256) * ldb * 2;
+    const size_t a_bytes = (size_t)((a_km ? K : M) + 256) * lda * es, b_bytes = (size_t)((b_km ? K : N) + 256) * ldb * es;
     return a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
 }
 
@@ -133,9 +134,18 @@ void gemm_plan(int dtype, int M, int N, int K, int lda, int ldb, bool a_km, bool
     const int max_split = allow_split ? std::max(1, K / 512) : 1;  // >= 8 k-tiles per split
     if (t256 >= 192) {
         *tile = 256;
-    } else if (std::min(cdiv(256, t256), max_split) * t256 >= 192) {
+    } else if (std::min(256 / t256, max_split) * t256 >= 192) {   // (one round of workgroups: the factor rounded down)
         *tile = 256;
-        *splits = std::min(cdiv(256, t256), max_split);
+        *splits = std::min(256 / t256, max_split);
+    } else if (dtype == FASTLSTM_FP32) {
+        // true-fp32 MFMA runs at 1/16 of the 16-bit rate: a product too small to fill the device with 256 x 256 tiles is
+        // left to the generic 128 x 128 kernel (two workgroups per CU), planned as above
+        *tile = 0;
+        const int tiles = cdiv(M, kBM) * cdiv(N, kBN);
+        if (allow_split && tiles < 128) {
+            const int bk = gemm_bk(dtype);
+            *splits = std::max(1, std::min(std::min(cdiv(512, tiles), std::max(1, K / (4 * bk))), 1024));
+        }
     } else {
         *tile = 128;
         if (t128 < 192) *splits = std::max(1, std::min(cdiv(512, t128), max_split));
@@ -154,7 +164,8 @@ bool wgrad_merged_plan(int dtype, int M, int I, int H, int K, int *splits, int *
     const int tx = cdiv(M, 256) * cdiv(I, 256), th = cdiv(M, 256) * cdiv(H, 256);
     *merged = !(tx >= 192 && th >= 192 && tx <= 256 && th <= 256);
     int sp = 1;
-    if (*merged && tx + th < 192) sp = std::max(1, std::min(cdiv(256, tx + th), K / 512));   // >= 8 k-tiles per split
+    // (rounded down: one round of at most 256 workgroups; 60 tiles x 5 splits would be a full round and a sixth of one)
+    if (*merged && tx + th < 192) sp = std::max(1, std::min(256 / (tx + th), K / 512));   // >= 8 k-tiles per split
     const int kps = cdiv(cdiv(K, sp), 64) * 64;
     *k_per_split = kps;
     *splits = cdiv(K, kps);
@@ -224,8 +235,9 @@ hipError_t launch_wgrad_merged(int dtype, const void *d_ifgo, const void *x, con
     w.h = g; w.h.B = h; w.h.C = dWh; w.h.N = H; w.h.ldb = H; w.h.ldc = H; w.h.Cpart = part_x + (size_t)sp * M * I;
     w.tiles_nx = cdiv(I, 256);
     w.db_part = db_part;
-    return dtype == FASTLSTM_FP16 ? launch_wgrad_merged_t<_Float16>(w, merged, db, s)
-                                  : launch_wgrad_merged_t<__bf16>(w, merged, db, s);
+    return dtype == FASTLSTM_FP32 ? launch_wgrad_merged_t<float>(w, merged, db, s)
+           : dtype == FASTLSTM_FP16 ? launch_wgrad_merged_t<_Float16>(w, merged, db, s)
+                                    : launch_wgrad_merged_t<__bf16>(w, merged, db, s);
 }
 
 static long long *g_trace = nullptr;
@@ -238,6 +250,8 @@ hipError_t launch_gemm_tiled(int dtype, const GemmParams &p_in, bool a_km, bool 
     if (tile == ID)                                                                                         \
         return dtype == FASTLSTM_FP16 ? launch_gemm16_dt<_Float16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s) \
                                       : launch_gemm16_dt<__bf16, BM, BN, NS, WVM, WVN, KSPT>(p, a_km, b_km, s);
+    if (tile == 256 && dtype == FASTLSTM_FP32) return launch_gemm16_dt<float, 256, 256, 2, 2, 4, 2>(p, a_km, b_km, s);
+    if (dtype == FASTLSTM_FP32) return launch_gemm(dtype, p, a_km, b_km, s);
     FASTLSTM_TILE_CASE(128, 128, 128, 2, 2, 2, 2)   // 2 workgroups per CU
     FASTLSTM_TILE_CASE(256, 256, 256, 2, 2, 4, 2)   // 8 waves, 128 x 64 per wave, 2 x 64 KiB stages
 #undef FASTLSTM_TILE_CASE

@@ -420,6 +420,22 @@ template <int OFF> __device__ __forceinline__ u32x4 lds_rd_tr16x2(unsigned addr)
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
+// The fp32 fragment of a K-major tile (k-rows of 1 KiB): the lane's 4 consecutive k of one column, four 4-byte reads
+// 1 KiB apart.  (No transposing read exists for 32-bit elements, and none is needed: with true-fp32 MFMA a phase of
+// the loop below is 4096 matrix cycles, next to which 48 such reads per wave do not show.)
+template <int OFF> __device__ __forceinline__ u32x4 lds_rd32x4(unsigned addr) {
+    unsigned e0 = 0u, e1 = 0u, e2 = 0u, e3 = 0u;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(e0) : "v"(addr), "n"(OFF));
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(e1) : "v"(addr), "n"(OFF + 1024));
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(e2) : "v"(addr), "n"(OFF + 2048));
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(e3) : "v"(addr), "n"(OFF + 3072));
+#else
+    (void)addr;
+#endif
+    return u32x4{e0, e1, e2, e3};
+}
+
 // The same contraction as gemm16_mainloop for the 256 x 256 x 64 tile with 8 waves (2 x 4) and two LDS
 // stages, scheduled as a ping-pong between the two waves of each SIMD.  Waves 0..3 (the upper half of the
 // C tile) and waves 4..7 (the lower half) run the same sequence of phases one phase apart:
@@ -433,10 +449,16 @@ template <int OFF> __device__ __forceinline__ u32x4 lds_rd_tr16x2(unsigned addr)
 // every barrier and behind every queued memory instruction: 1180 -> 1500 TFLOP/s at M = 32768,
 // N = 8192, K = 2048 together with the non-temporal stores of the epilogue.)
 // The LDS-direct loads are inline assembly (dma_block_asm): the kernel's only ones, counted by hand.
+// T = float: the same loop on tiles of 128 bytes of K per row, i.e. 32 elements per k-tile in two k-steps of
+// four v_mfma_f32_16x16x4_f32 per fragment pair (true fp32); K-contiguous tiles have the 16-bit layout byte for
+// byte, K-major tiles are 32 k-rows of 1 KiB, unswizzled (lds_rd32x4).
 // c + the sum of the 8 elements of a fragment register quad (fp32 accumulate).
 template <typename T> __device__ __forceinline__ float frag_sum(const u32x4 f, float c) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    if constexpr (Elem<T>::DT == FASTLSTM_FP16) {
+    if constexpr (Elem<T>::DT == FASTLSTM_FP32) {
+        const f32x4 v = __builtin_bit_cast(f32x4, f);
+        c += (v[0] + v[1]) + (v[2] + v[3]);
+    } else if constexpr (Elem<T>::DT == FASTLSTM_FP16) {
         typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
         const f16x2 one = {(_Float16)1.f, (_Float16)1.f};
         const f16x8 h = __builtin_bit_cast(f16x8, f);
@@ -469,7 +491,12 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave >> 2, wn = wave & 3;
-    const int nkt = (ke - kb) / 64;
+    constexpr int ES = sizeof(T), EPC = 16 / ES;    // element size; elements per 16-byte chunk
+    constexpr int BKE = 128 / ES;                     // elements of K per k-tile (rows of 128 bytes)
+    constexpr int KROW = 256 * ES, CPR = KROW / 16;   // K-major tile: bytes and 16-byte chunks per k-row
+    constexpr int KRB = 8 * 64 / CPR;                 // ... k-rows that the 8 waves fill per load step (16 | 8)
+    constexpr bool F32 = ES == 4;
+    const int nkt = (ke - kb) / BKE;
     if (nkt <= 0) return;
     const unsigned lds0 = (unsigned)(size_t)((FASTLSTM_LDS_PTR unsigned char *)smem);
 
@@ -477,29 +504,29 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
         const unsigned long long a = reinterpret_cast<unsigned long long>(base);
         return u32x4{(unsigned)a, (unsigned)(a >> 32) & 0xffffu, bytes, 0x00020000u};
     };
-    const u32x4 ra = rsrc_of(p.A, (unsigned)((A_KM ? (size_t)p.K : (size_t)p.M) * p.lda * 2));
-    const u32x4 rb = rsrc_of(p.B, (unsigned)((B_KM ? (size_t)p.K : (size_t)p.N) * p.ldb * 2));
-    auto swz = [](int k) { return ((k & 3) << 1) ^ (((k >> 3) & 1) << 3); };   // K-major tiles (see gemm16_mainloop)
+    const u32x4 ra = rsrc_of(p.A, (unsigned)((A_KM ? (size_t)p.K : (size_t)p.M) * p.lda * ES));
+    const u32x4 rb = rsrc_of(p.B, (unsigned)((B_KM ? (size_t)p.K : (size_t)p.N) * p.ldb * ES));
+    auto swz = [](int k) { return F32 ? 0 : ((k & 3) << 1) ^ (((k >> 3) & 1) << 3); };   // K-major tiles (see gemm16_mainloop)
     auto kswz = [](int r16) { return (r16 >> 1) & 7; };                        // K-contiguous tiles
 
     // global -> LDS: wave w fills the 1 KiB blocks w, w + 8, w + 16, w + 24 of each operand's 32 KiB tile
     unsigned goff_a, goff_b;
     if constexpr (!A_KM) {
-        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * 8;
-        goff_a = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * 2);
+        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * EPC;
+        goff_a = (unsigned)(((size_t)(m0 + row) * p.lda + kb + k) * ES);
     } else {
-        const int P = wave * 64 + lane, k = P / 32, mc = (P % 32) ^ swz(k);
-        goff_a = (unsigned)(((size_t)(kb + k) * p.lda + m0 + mc * 8) * 2);
+        const int P = wave * 64 + lane, k = P / CPR, mc = (P % CPR) ^ swz(k);
+        goff_a = (unsigned)(((size_t)(kb + k) * p.lda + m0 + mc * EPC) * ES);
     }
     if constexpr (!B_KM) {
-        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * 8;
-        goff_b = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * 2);
+        const int row = wave * 8 + lane / 8, k = ((lane % 8) ^ kswz(row & 15)) * EPC;
+        goff_b = (unsigned)(((size_t)(n0 + row) * p.ldb + kb + k) * ES);
     } else {
-        const int P = wave * 64 + lane, k = P / 32, nc = (P % 32) ^ swz(k);
-        goff_b = (unsigned)(((size_t)(kb + k) * p.ldb + n0 + nc * 8) * 2);
+        const int P = wave * 64 + lane, k = P / CPR, nc = (P % CPR) ^ swz(k);
+        goff_b = (unsigned)(((size_t)(kb + k) * p.ldb + n0 + nc * EPC) * ES);
     }
-    const unsigned a_istep = (unsigned)(A_KM ? 16 : 64) * p.lda * 2, b_istep = (unsigned)(B_KM ? 16 : 64) * p.ldb * 2;
-    const unsigned a_kstep = A_KM ? 64u * p.lda * 2 : 128u, b_kstep = B_KM ? 64u * p.ldb * 2 : 128u;
+    const unsigned a_istep = (unsigned)(A_KM ? KRB : 64) * p.lda * ES, b_istep = (unsigned)(B_KM ? KRB : 64) * p.ldb * ES;
+    const unsigned a_kstep = A_KM ? (unsigned)BKE * p.lda * ES : 128u, b_kstep = B_KM ? (unsigned)BKE * p.ldb * ES : 128u;
     auto gload = [&](int kt) {
         const unsigned sa = lds0 + (kt & 1) * STAGE + wave * kFragBytes, sb = sa + A_BYTES;
 #pragma unroll
@@ -510,7 +537,10 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
 
     // LDS -> registers.  K-contiguous operand: fragment i of k-step ks at base[ks] + 2048 i.  K-major operand:
     // the two transposing reads of fragment i at base_i + 16384 ks (+ 2048 for the second one).
+    // (fp32 K-major operand: fragment i of k-step ks at base + 64 i + 16384 ks, see lds_rd32x4)
     unsigned a_kc[2], b_kc[2], a_km[8], b_km[4];
+    const unsigned a_km32 = lds0 + (unsigned)(q * 4 * KROW + wm * 512 + r * 4);
+    const unsigned b_km32 = lds0 + A_BYTES + (unsigned)(q * 4 * KROW + wn * 256 + r * 4);
     {
         const int a = r >> 2, b = r & 3, k = q * 8 + a;
 #pragma unroll
@@ -533,6 +563,10 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
         if constexpr (!B_KM) {
             const unsigned ab = b_kc[ks] + st;
             fb[0] = lds_rd128<0>(ab); fb[1] = lds_rd128<2048>(ab); fb[2] = lds_rd128<4096>(ab); fb[3] = lds_rd128<6144>(ab);
+        } else if constexpr (F32) {
+            const unsigned ab = b_km32 + st;
+            fb[0] = lds_rd32x4<ks * 16384>(ab); fb[1] = lds_rd32x4<ks * 16384 + 64>(ab);
+            fb[2] = lds_rd32x4<ks * 16384 + 128>(ab); fb[3] = lds_rd32x4<ks * 16384 + 192>(ab);
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) fb[j] = lds_rd_tr16x2<ks * 16384>(b_km[j] + st);
@@ -541,6 +575,12 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
             const unsigned aa = a_kc[ks] + st;
             fa[0] = lds_rd128<0>(aa); fa[1] = lds_rd128<2048>(aa); fa[2] = lds_rd128<4096>(aa); fa[3] = lds_rd128<6144>(aa);
             fa[4] = lds_rd128<8192>(aa); fa[5] = lds_rd128<10240>(aa); fa[6] = lds_rd128<12288>(aa); fa[7] = lds_rd128<14336>(aa);
+        } else if constexpr (F32) {
+            const unsigned aa = a_km32 + st;
+            fa[0] = lds_rd32x4<ks * 16384>(aa); fa[1] = lds_rd32x4<ks * 16384 + 64>(aa);
+            fa[2] = lds_rd32x4<ks * 16384 + 128>(aa); fa[3] = lds_rd32x4<ks * 16384 + 192>(aa);
+            fa[4] = lds_rd32x4<ks * 16384 + 256>(aa); fa[5] = lds_rd32x4<ks * 16384 + 320>(aa);
+            fa[6] = lds_rd32x4<ks * 16384 + 384>(aa); fa[7] = lds_rd32x4<ks * 16384 + 448>(aa);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) fa[i] = lds_rd_tr16x2<ks * 16384>(a_km[i] + st);
@@ -553,7 +593,7 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
                        "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
 #endif
     };
-    int db_cnt = DB ? (kb / 64) % db_mod : 0;   // k-tile index modulo db_mod, counted along
+    int db_cnt = DB ? (kb / BKE) % db_mod : 0;   // k-tile index modulo db_mod, counted along
     bool sum_a = false;
     auto compute = [&]() {
         __builtin_amdgcn_s_setprio(1);
@@ -665,6 +705,38 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
         return;
     }
     const T *bias0 = static_cast<const T *>(p.bias0), *bias1 = static_cast<const T *>(p.bias1);
+    if constexpr (sizeof(T) == 4) {
+        // fp32: a lane's 4 consecutive n are 16 bytes already, and the tile (256 KiB) would not fit the LDS:
+        // stores straight from the accumulators, 64 bytes per row and instruction
+        T *Cg = static_cast<T *>(p.C);
+        const bool vec = (p.ldc & 3) == 0 && (p.N & 3) == 0 && (reinterpret_cast<size_t>(Cg) & 15) == 0;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int nb = n0 + (wn * TN + j) * 16 + q * 4;
+            float b4[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias0)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (nb + e < p.N) b4[e] = bias0[nb + e] + (bias1 ? bias1[nb + e] : 0.f);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int m = m0 + (wm * TM + i) * 16 + r;
+                if (m >= p.M || nb >= p.N) continue;
+                f32x4 v = acc[i][j];
+                v[0] += b4[0]; v[1] += b4[1]; v[2] += b4[2]; v[3] += b4[3];
+                T *dst = Cg + (size_t)m * p.ldc + nb;
+                if (vec && nb + 3 < p.N) {
+                    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst));
+                    else *reinterpret_cast<f32x4 *>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (nb + e < p.N) dst[e] = v[e];
+                }
+            }
+        }
+        return;
+    }
     // the 4 bias elements of every tile column group: one 8-byte load each where the row of
     // biases allows it (all loads in flight together), element loads at a ragged edge
     float bv[TN][4];
@@ -875,8 +947,12 @@ __global__ void wgrad_reduce_kernel(const float *part_x, T *dWx, const float *pa
     }
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
     for (int k = 0; k < splits; ++k) s += *reinterpret_cast<const f32x4 *>(part + (size_t)k * total + i * 4);
-    T o[4] = {Elem<T>::from_f32(s[0]), Elem<T>::from_f32(s[1]), Elem<T>::from_f32(s[2]), Elem<T>::from_f32(s[3])};
-    *reinterpret_cast<u32x2 *>(out + i * 4) = *reinterpret_cast<u32x2 *>(o);
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4 *>(out + i * 4) = s;
+    } else {
+        T o[4] = {Elem<T>::from_f32(s[0]), Elem<T>::from_f32(s[1]), Elem<T>::from_f32(s[2]), Elem<T>::from_f32(s[3])};
+        *reinterpret_cast<u32x2 *>(out + i * 4) = *reinterpret_cast<u32x2 *>(o);
+    }
 }
 
 }  // namespace fastlstm
