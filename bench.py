@@ -299,6 +299,19 @@ def main():
         ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), 2)
         db_fwd, n_fwd = do_bench(step_fwd)
         db_full, n_full = do_bench(step_fwd_bwd)
+        # the reference's stand-alone "bwd" mode (scripts/benchmark.py:79-113): lstm_persistent_bwd of the first layer
+        # on random activations, which its lambda draws inside the timed call; beside it the same call on tensors
+        # drawn beforehand
+        Wx0, Wh0 = model.weight_ih_l0.detach(), model.weight_hh_l0.detach()
+        rnd = lambda *shape: torch.randn(shape, device=dev, dtype=dt)
+
+        def step_bwd_as_reference():
+            return L.lstm_persistent_bwd(rnd(T, B, H), rnd(B, H), rnd(B, H), x, rnd(T + 1, B, H), rnd(T + 1, B, H),
+                                         rnd(T, B, 4 * H), Wx0, Wh0)
+
+        bw_args = (rnd(T, B, H), rnd(B, H), rnd(B, H), x, rnd(T + 1, B, H), rnd(T + 1, B, H), rnd(T, B, 4 * H), Wx0, Wh0)
+        db_bwd_ref, n_bwd_ref = do_bench(step_bwd_as_reference)
+        db_bwd, n_bwd = do_bench(lambda: L.lstm_persistent_bwd(*bw_args))
     value = B * T / (ms * 1e-3)
 
     t_k1 = ev_time(k1)
@@ -427,6 +440,9 @@ def main():
         "fwd_bwd": {"ms": round(ms_full, 4), "bt_per_s": round(B * T / (ms_full * 1e-3), 1)},
         "do_bench": {"fwd_ms": round(db_fwd, 4), "fwd_reps": n_fwd, "fwd_bwd_ms": round(db_full, 4), "fwd_bwd_reps": n_full,
                      "fwd_bt_per_s": round(B * T / (db_fwd * 1e-3), 1), "fwd_bwd_bt_per_s": round(B * T / (db_full * 1e-3), 1),
+                     "bwd_ms": round(db_bwd, 4), "bwd_reps": n_bwd, "bwd_with_randn_inside_ms": round(db_bwd_ref, 4),
+                     "bwd_note": "lstm_persistent_bwd of one layer on random activations (scripts/benchmark.py:79-113); "
+                                 "the reference's lambda draws the six random tensors inside the timed call (second figure)",
                      "protocol": "median; warm-up 40 ms, 160 ms of repetitions, 256 MB buffer cleared before each, one "
                                  "event pair per repetition (the reference's scripts/benchmark.py:118-133)"},
         "roofline": roofline, "kernels": kernels,

@@ -898,6 +898,13 @@ int fastlstm_plan_device(int device, int B, int H, int dtype, int backward, fast
     return plan_device(device, B, H, dtype, backward, plan, true);
 }
 
+// The input projection's output is read back by the time loop that follows it.  Up to half the memory-side cache
+// (256 MiB on this device) it is written with ordinary stores so that the loop, whose step waits for its gate tile,
+// finds it there; a larger one streams out past the caches (GemmParams::keep_c).
+static int gates_stay_cached(size_t rows, int H, int dtype) {
+    return rows * 4 * (size_t)H * elem_bytes(dtype) <= ((size_t)128 << 20) ? 1 : 0;
+}
+
 // K1 on rows [row0, row0 + rows) of x[T*B, I] / ifgo[T*B, 4H]
 static int gemm_ifgo_rows(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, size_t row0,
                           int rows, int I, int H, int dtype, hipStream_t stream) {
@@ -910,6 +917,7 @@ static int gemm_ifgo_rows(const void *x, const void *Wx, const void *bx, const v
     p.M = rows; p.N = 4 * H; p.K = I;
     p.lda = I; p.ldb = I; p.ldc = 4 * H;
     p.splits = 1; p.k_per_split = I;
+    p.keep_c = gates_stay_cached(rows, H, dtype);
     int tile, splits;
     gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, false, false, &tile, &splits);
     return launch_gemm_tiled(dtype, p, false, false, tile, stream) == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
@@ -926,6 +934,7 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
     p.M = T * B; p.N = 4 * H; p.K = I;
     p.lda = I; p.ldb = I; p.ldc = 4 * H;
     p.splits = 1; p.k_per_split = I;
+    p.keep_c = gates_stay_cached(T * B, H, dtype);
     int tile, splits;
     gemm_plan(dtype, p.M, p.N, p.K, p.lda, p.ldb, false, false, false, &tile, &splits);
     return launch_gemm_tiled(dtype, p, false, false, tile, static_cast<hipStream_t>(stream)) == hipSuccess

@@ -25,6 +25,8 @@ struct GemmParams {
     int M, N, K;
     int lda, ldb, ldc;
     int splits, k_per_split;
+    int keep_c;           // 1: C leaves with ordinary stores even from a stand-alone launch (a kernel that reads it next
+                          // finds it in the memory-side cache); 0: non-temporal stores there
     long long *trace;     // optional: 4 clock stamps per workgroup (diagnostics), else nullptr
 };
 

@@ -672,6 +672,9 @@ __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const in
 // STREAM: the C tile leaves with non-temporal stores.  A stand-alone product writes 128 KiB per workgroup
 // that nothing reads again soon; as ordinary stores those lines displace the operand panels that the
 // workgroups of an XCD share through its L2 (M = 32768, N = 8192, K = 2048: 1240 -> 1500 TFLOP/s).
+// p.keep_c switches them off for an output that the next kernel reads back while the memory-side cache
+// still holds it (the gates of a small-H recurrence: T = 1024, B = 256, H = 64, 128 MiB of gates: the
+// time loop that follows runs 0.85 ms after ordinary stores, 1.13 ms after non-temporal ones).
 template <typename T, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool STREAM = false>
 __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m0, const int n0, const int split,
                                                 unsigned char *smem,
@@ -726,7 +729,7 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
                 v[0] += b4[0]; v[1] += b4[1]; v[2] += b4[2]; v[3] += b4[3];
                 T *dst = Cg + (size_t)m * p.ldc + nb;
                 if (vec && nb + 3 < p.N) {
-                    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst));
+                    if (STREAM && !p.keep_c) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst));
                     else *reinterpret_cast<f32x4 *>(dst) = v;
                 } else {
 #pragma unroll
@@ -795,11 +798,13 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
             u32x4 v[IT];
 #pragma unroll
             for (int it = 0; it < IT; ++it) v[it] = *reinterpret_cast<const u32x4 *>(src + (size_t)it * RPI * C::C_LD);
+            if (STREAM && !p.keep_c) {
 #pragma unroll
-            for (int it = 0; it < IT; ++it) {
-                u32x4 *d = reinterpret_cast<u32x4 *>(dst + (size_t)it * RPI * p.ldc);
-                if constexpr (STREAM) __builtin_nontemporal_store(v[it], d);
-                else *d = v[it];
+                for (int it = 0; it < IT; ++it)
+                    __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4 *>(dst + (size_t)it * RPI * p.ldc));
+            } else {
+#pragma unroll
+                for (int it = 0; it < IT; ++it) *reinterpret_cast<u32x4 *>(dst + (size_t)it * RPI * p.ldc) = v[it];
             }
             return;
         }
@@ -811,7 +816,7 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
         const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + (size_t)ml * C::C_LD + nc * 16);
         T *dst = Cg + (size_t)m * p.ldc + n;
         if (vec_ok && n + 8 <= p.N) {
-            if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
+            if (STREAM && !p.keep_c) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
             else *reinterpret_cast<u32x4 *>(dst) = v;
         } else {
             const T *tv = reinterpret_cast<const T *>(&v);
