@@ -74,8 +74,8 @@ def physical_cores():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="B", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-miopen", action="store_true", help="skip the nn.LSTM-on-ROCm leg")
@@ -296,7 +296,7 @@ def main():
     with torch.enable_grad():
         ms = timed(headline, args.steps, args.warmup)
         ms_fwd = ms if mode == "fwd" else timed(step_fwd, args.steps, args.warmup)
-        ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), 2)
+        ms_full = ms if mode == "fwd_bwd" else timed(step_fwd_bwd, max(3, args.steps // 2), max(2, args.warmup // 2))
         db_fwd, n_fwd = do_bench(step_fwd)
         db_full, n_full = do_bench(step_fwd_bwd)
         # the reference's stand-alone "bwd" mode (scripts/benchmark.py:79-113): lstm_persistent_bwd of the first layer
@@ -465,8 +465,8 @@ def main():
                 o, _ = ref(x, (h0, c0))
                 o.sum().backward()
 
-            r_f = timed(ref_fwd, max(3, args.steps // 2), 2)
-            r_b = timed(ref_full, max(3, args.steps // 2), 2)
+            r_f = timed(ref_fwd, max(3, min(20, args.steps // 2)), 2)
+            r_b = timed(ref_full, max(3, min(20, args.steps // 2)), 2)
             res["nn_lstm_rocm"] = {"fwd_ms": round(r_f, 4), "fwd_bwd_ms": round(r_b, 4),
                                    "speedup_fwd": round(r_f / ms_fwd, 3), "speedup_fwd_bwd": round(r_b / ms_full, 3)}
         except Exception as exc:  # MIOpen may not support a configuration

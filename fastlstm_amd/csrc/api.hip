@@ -780,6 +780,7 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
     p->k5.splits = 1; p->k5.k_per_split = K;
     p->k5_tiles_m = tiles_m; p->k5_tiles_n = tiles_n;
     p->k5_chunk_tiles = ct; p->k5_chunk_steps = ct * 256 / B; p->k5_chunks = cdiv(tiles_m, ct);
+    p->k5_tail_by_rec = (!lower && e.dx) ? 1 : 0;
     p->n_active = n_active;
     p->chunk_done = ws_chunk_counters(p->hdr, 0);
     p->wg_tiles = 0;

@@ -166,6 +166,9 @@ bool wgrad_merged_plan(int dtype, int M, int I, int H, int K, int *splits, int *
     int sp = 1;
     // (rounded down: one round of at most 256 workgroups; 60 tiles x 5 splits would be a full round and a sixth of one)
     if (*merged && tx + th < 192) sp = std::max(1, std::min(256 / (tx + th), K / 512));   // >= 8 k-tiles per split
+    // true-fp32 MFMA runs at 1/16 of the 16-bit rate: products that do not fill the device with 256 x 256 tiles stay
+    // with the generic 128 x 128 kernel and its finer split (T*B = 2048, 4H = 1024, I = H = 256: 0.06 against 0.15 ms)
+    if (dtype == FASTLSTM_FP32 && (tx + th) * sp < 192) return false;
     const int kps = cdiv(cdiv(K, sp), 64) * 64;
     *k_per_split = kps;
     *splits = cdiv(K, kps);

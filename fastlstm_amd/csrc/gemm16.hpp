@@ -486,9 +486,11 @@ template <typename T> __device__ __forceinline__ float frag_sum(const u32x4 f, f
 template <typename T, bool A_KM, bool B_KM, bool DB = false>
 __device__ __forceinline__ void gemm16_mainloop_pp(const GemmParams &p, const int m0, const int n0, const int kb,
                                                    const int ke, unsigned char *smem, f32x4 (&acc)[8][4],
-                                                   float *colsum = nullptr, const int db_mod = 1, const int db_rem = 0) {
+                                                   float *colsum = nullptr, const int db_mod = 1, const int db_rem = 0,
+                                                   const int tid_salt = 0) {
     constexpr int STAGE = 65536, A_BYTES = 32768;
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // (tid_salt: an opaque zero from a caller inside a loop, see gemm16_mainloop)
+    const int tid = threadIdx.x + tid_salt, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = lane >> 4, r = lane & 15;
     const int wm = wave >> 2, wn = wave & 3;
     constexpr int ES = sizeof(T), EPC = 16 / ES;    // element size; elements per 16-byte chunk
@@ -827,9 +829,10 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
 }
 
 // One BM x BN tile of C (rows m0.., columns n0.., K range of `split`): main loop + epilogue.
-// ALONE: the tile of a stand-alone GEMM launch (ping-pong main loop where the configuration has one,
-// streaming stores); the tiles that run inside a recurrent launch keep the symmetric loop.
-template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool ALONE = false>
+// ALONE: the tile of a stand-alone GEMM launch (streaming stores); PP: the ping-pong main loop where the
+// configuration has one.
+template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool ALONE = false,
+          bool PP = ALONE>
 __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
                                             unsigned char *smem, const int trace_slot) {
     constexpr int TM = BM / WVM / 16, TN = BN / WVN / 16;
@@ -842,7 +845,7 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int kb = split * p.k_per_split;
     const int k_end = (A_KM && B_KM) ? (p.K + 63) / 64 * 64 : p.K;   // (rows past K read as zeros)
-    if constexpr (ALONE && BM == 256 && BN == 256 && NS == 2 && WVM == 2 && WVN == 4 && KSPT == 2)
+    if constexpr (PP && BM == 256 && BN == 256 && NS == 2 && WVM == 2 && WVN == 4 && KSPT == 2)
         gemm16_mainloop_pp<T, A_KM, B_KM>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
     else
         gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);

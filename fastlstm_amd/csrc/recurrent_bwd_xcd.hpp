@@ -38,6 +38,9 @@ struct BwdXcdParams {
     // recurrence has finished a chunk of k5_chunk_steps timesteps (k5_chunk_tiles row tiles);
     // chunk_done[c] counts the recurrence workgroups (n_active) whose part of chunk c is in memory.
     GemmParams k5;      // M = T*B, N = I, K = 4H, A = d_ifgo, B = Wx (K-major), C = dx
+    int k5_tail_by_rec; // 1: the dx tiles of the chunk that completes last (timesteps 0 ..) are computed by the recurrence
+                        // workgroups once their time loop has ended, not by the helpers, which still owe that chunk's
+                        // share of their weight-gradient tiles (single-layer launches)
     int k5_tiles_m, k5_tiles_n;
     int k5_chunk_tiles, k5_chunk_steps, k5_chunks;
     // In-kernel weight gradients (wg_tiles > 0): dWx = d_ifgo^T . x and dWh = d_ifgo^T . h, 256 x 256
@@ -77,6 +80,10 @@ struct BwdXcdParams {
     unsigned char *partials;   // lstm_bwd_wide_split_kernel: the teams' partial sums (see there)
 };
 
+#ifndef FASTLSTM_HELPER_PP
+#define FASTLSTM_HELPER_PP true   // the GEMM tiles inside the recurrent launches use the ping-pong main loop
+#endif
+
 // One 256 x 256 tile of dx = d_ifgo . Wx as a real function call.  The caller keeps the 128
 // accumulator registers of its weight-gradient tile across the call: the calling convention saves
 // and restores them around it (once per dx tile), where inlining would spill inside the GEMM
@@ -91,7 +98,7 @@ __device__ __attribute__((noinline)) void helper_dx_tile(const void *A, const vo
     g.lda = g.K; g.ldb = g.N; g.ldc = g.N;
     g.splits = 1; g.k_per_split = g.K;
     unsigned char *smem = (unsigned char *)(FASTLSTM_LDS_PTR unsigned char *)(size_t)(unsigned)uniform_int((int)(size_t)lds);
-    gemm16_tile<T, false, true, 256, 256, 2, 2, 4, 2>(g, uniform_int(m0), uniform_int(n0), 0, smem, 0);
+    gemm16_tile<T, false, true, 256, 256, 2, 2, 4, 2, false, FASTLSTM_HELPER_PP>(g, uniform_int(m0), uniform_int(n0), 0, smem, 0);
     __syncthreads();   // the LDS is reused by the caller
 }
 
@@ -118,7 +125,8 @@ __device__ __attribute__((noinline)) void helper_wgrad_chunk(const void *A, cons
 #pragma unroll
         for (int j = 0; j < TN; ++j)
             acc[i][j] = uniform_int(first) ? f32x4{0.f, 0.f, 0.f, 0.f} : park[(i * TN + j) * (kWave * 8)];
-    gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(g, m0, n0, uniform_int(kb), uniform_int(ke), smem, acc);
+    if constexpr (FASTLSTM_HELPER_PP) gemm16_mainloop_pp<T, true, true>(g, m0, n0, uniform_int(kb), uniform_int(ke), smem, acc);
+    else gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(g, m0, n0, uniform_int(kb), uniform_int(ke), smem, acc);
     if (uniform_int(last)) {
         gemm16_epilogue<T, 256, 256, 2, WVM, WVN, 2>(g, m0, n0, 0, smem, acc);
         __syncthreads();
@@ -224,6 +232,8 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
             } else {
                 int salt = 0;
                 asm volatile("" : "+v"(salt));   // opaque zero: see gemm16_mainloop
+                // (the symmetric loop: the ping-pong loop, inlined here with the accumulators live across the
+                // calls around it, spills them inside its k loop)
                 gemm16_mainloop<T, true, true, 256, 256, 2, WVM, WVN, 2>(wp, wm0, wn0, kb, ke, smem, acc, salt);
             }
         }
@@ -232,6 +242,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
             const int r = i - k * per_chunk;
             const int rt = c * p.k5_chunk_tiles + r / p.k5_tiles_n, ct = r % p.k5_tiles_n;
             if (rt >= p.k5_tiles_m || !p.k5.C) continue;   // (no dx wanted: the helpers only accumulate weight gradients)
+            if (!stacked && c == 0 && p.k5_tail_by_rec) continue;   // the recurrence workgroups take these
             helper_dx_tile<T>(p.k5.A, p.k5.B, p.k5.C, p.k5.M, p.k5.N, p.k5.K, rt * 256, ct * 256,
                               (FASTLSTM_LDS_PTR unsigned char *)smem);
             if (stacked) {   // the tile's stores acknowledged, this XCD's L2 written back, then counted
@@ -262,7 +273,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
         const bool w8 = w < n8;
         const GemmParams &q = w8 ? p.k8 : p.k9;
         const int qi = w8 ? w : w - n8, qtn = w8 ? p.k8_tiles_n : p.k9_tiles_n;
-        gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
+        gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2, false, FASTLSTM_HELPER_PP>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
         __syncthreads();
     }
     if (stacked)
@@ -270,7 +281,7 @@ __device__ __forceinline__ void bwd_helper(const BwdXcdParams &p, unsigned char 
             const bool w8 = w < n8_lo;
             const GemmParams &q = w8 ? p.k8_lo : p.k9_lo;
             const int qi = w8 ? w : w - n8_lo, qtn = w8 ? p.k8_lo_tiles_n : p.k9_tiles_n;
-            gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
+            gemm16_tile<T, true, true, 256, 256, 2, WVM, WVN, 2, false, FASTLSTM_HELPER_PP>(q, (qi / qtn) * 256, (qi % qtn) * 256, 0, smem, 0);
             __syncthreads();
         }
 }
@@ -662,6 +673,22 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             dh_state[off_h[m]] = E::from_f32(dh_rec[m]);
             dc_state_buf[off_h[m]] = E::from_f32(dc_state[m]);
         }
+    if constexpr (HELP == 1) {
+        // The time loop is over and this CU would idle while the helpers finish: the dx tiles of the last chunk
+        // (complete once every recurrence workgroup has counted it, just above) are dealt to the recurrence
+        // workgroups, one 256 x 256 tile each as far as they go.
+        if (k5_live && p.k5.C && p.k5_tail_by_rec) {
+            if (wave == 0) wait_versions<100>(p.chunk_done, 1, p.n_active, p.hdr, p.spin_limit, -1, 0);
+            __syncthreads();
+            const int per = min(p.k5_chunk_tiles, p.k5_tiles_m) * p.k5_tiles_n;
+            for (int i = g * p.n_ht + j; i < per; i += p.n_active)
+                helper_dx_tile<T>(p.k5.A, p.k5.B, p.k5.C, p.k5.M, p.k5.N, p.k5.K, (i / p.k5_tiles_n) * 256, (i % p.k5_tiles_n) * 256,
+                                  (FASTLSTM_LDS_PTR unsigned char *)smem);
+        }
+    }
+#ifdef FASTLSTM_BWD_STAMPS
+    if (tid == 0) stamps[3] = (long long)wall_clock64();
+#endif
 }
 
 }  // namespace fastlstm

@@ -216,8 +216,9 @@ __device__ __forceinline__ void k1_helper(const FwdXcdParams &p, unsigned char *
         }
         int rt, ct;
         tile_of(second ? i1 : i0, &rt, &ct);
-        if (second) gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1b, rt * 256, ct * 256, 0, smem, 0);
-        else gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2>(p.k1, rt * 256, ct * 256, 0, smem, 0);
+        // (the ping-pong main loop, ordinary stores: the time loop reads these gates within a chunk or two)
+        if (second) gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2, false, true>(p.k1b, rt * 256, ct * 256, 0, smem, 0);
+        else gemm16_tile<T, false, false, 256, 256, 2, 2, 4, 2, false, true>(p.k1, rt * 256, ct * 256, 0, smem, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // every wave's part of the tile is in the L2 (and the LDS may be reused)
         if (threadIdx.x == 0)
