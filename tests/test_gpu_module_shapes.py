@@ -6,8 +6,7 @@ Every case draws its shape and options from its seed: sequence length, batch, in
 state_grads, dtype.  The module chooses among its forms by shape (general / XCD-local / register-resident
 kernels, pairs of layers in one launch, wavefronts of chunked launches, both directions side by side,
 zero-padded sizes, packed batches cut at row ranges); whichever it takes, outputs, final states and every
-gradient have to match nn.LSTM: fp32 rtol = atol = 1e-4 (atol scaled by the reference's magnitude for
-gradients), 16-bit <= 2e-2 of the reference's max-norm (reference evaluated with the rounded weights
+gradient have to match nn.LSTM: fp32 rtol = atol = 1e-4 element by element, 16-bit <= 2e-2 of the reference's max-norm (reference evaluated with the rounded weights
 and inputs)."""
 import random
 
@@ -86,7 +85,11 @@ def _check(c, seed):
     D = 2 if kw["bidirectional"] else 1
     torch.manual_seed(seed)
     m = FastLSTM(I, H, num_layers=layers, state_grads=c["state_grads"], **kw)
-    ref = torch.nn.LSTM(I, H, num_layers=layers, **kw)
+    # reference: nn.LSTM on the CPU; for the fp32 cases in float64, so that the element-wise 1e-4 bound measures this
+    # build's error alone (a bias gradient is a sum over T*B terms of mixed sign: two fp32 evaluations of an element
+    # near zero can differ by more than 1e-4 of it while each is well inside 1e-4 of the exact value)
+    rdt = torch.float64 if dt == torch.float32 else torch.float32
+    ref = torch.nn.LSTM(I, H, num_layers=layers, **kw).to(rdt)
     with torch.no_grad():
         for n, prm in m.named_parameters():
             prm.copy_(prm.to(dt).float())
@@ -98,28 +101,28 @@ def _check(c, seed):
     wh, wc = rnd(layers * D, B, H), rnd(layers * D, B, H)
     state = (lambda *ts: tuple(ts)) if c["states"] else (lambda *ts: None)
     leaves = [t.cuda().to(dt).requires_grad_(True) for t in (h0, c0)]
-    leaves_r = [t.clone().requires_grad_(True) for t in (h0, c0)]
+    leaves_r = [t.clone().to(rdt).requires_grad_(True) for t in (h0, c0)]
     if c["packed"]:
         lengths = [int(v) for v in torch.randint(1, T + 1, (B,), generator=g)]
         seqs = [rnd(n, I) for n in lengths]
         xs = [s.cuda().to(dt).requires_grad_(True) for s in seqs]
-        xr = [s.clone().requires_grad_(True) for s in seqs]
+        xr = [s.clone().to(rdt).requires_grad_(True) for s in seqs]
         y, (hn, cn) = m(pack_sequence(xs, enforce_sorted=False), state(*leaves))
         yr, (hr, cr) = ref(pack_sequence(xr, enforce_sorted=False), state(*leaves_r))
         assert torch.equal(y.batch_sizes, yr.batch_sizes)
         y, yr = y.data, yr.data
     else:
         x = rnd(B, T, I) if kw["batch_first"] else rnd(T, B, I)
-        xs, xr = [x.cuda().to(dt).requires_grad_(True)], [x.clone().requires_grad_(True)]
+        xs, xr = [x.cuda().to(dt).requires_grad_(True)], [x.clone().to(rdt).requires_grad_(True)]
         y, (hn, cn) = m(xs[0], state(*leaves))
         yr, (hr, cr) = ref(xr[0], state(*leaves_r))
     assert y.shape == yr.shape and hn.shape == hr.shape and cn.shape == cr.shape, c
     wy = rnd(*yr.shape)
-    loss, loss_r = (y.float() * wy.cuda()).sum(), (yr * wy).sum()
+    loss, loss_r = (y.float() * wy.cuda()).sum(), (yr * wy.to(rdt)).sum()
     if c["state_grads"] or c["packed"]:   # final states that carry a gradient
-        loss, loss_r = loss + (hn.float() * wh.cuda()).sum(), loss_r + (hr * wh).sum()
+        loss, loss_r = loss + (hn.float() * wh.cuda()).sum(), loss_r + (hr * wh.to(rdt)).sum()
     if c["state_grads"] and not c["packed"]:
-        loss, loss_r = loss + (cn.float() * wc.cuda()).sum(), loss_r + (cr * wc).sum()
+        loss, loss_r = loss + (cn.float() * wc.cuda()).sum(), loss_r + (cr * wc.to(rdt)).sum()
     loss.backward()
     loss_r.backward()
     rows = [(y, yr, "y"), (hn, hr, "hn"), (cn, cr, "cn")]
@@ -131,9 +134,8 @@ def _check(c, seed):
     for got, want, name in rows:
         assert got is not None and got.shape == want.shape, (name, c)
         if dt == torch.float32:
-            scale = max(1.0, float(want.detach().abs().max()))
             torch.testing.assert_close(got.detach().cpu().double(), want.detach().double(), rtol=FP32_TOL,
-                                       atol=FP32_TOL * scale, msg=lambda s: "%s %s: %s" % (name, c, s))
+                                       atol=FP32_TOL, msg=lambda s: "%s %s: %s" % (name, c, s))
         else:
             assert rel_err(got, want) < HALF_TOL, (name, c, rel_err(got, want))
 
