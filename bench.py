@@ -246,7 +246,10 @@ def main():
         zero_ws(ws_b, plan_b); dh_n.zero_(); dc_n.zero_()
 
     def k5():
-        _lib.check(lib.fastlstm_gemm_dx(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, stream), "k5")
+        # (with the weight-gradient workspace as scratch, as fastlstm_bwd_layer calls it: a dx with few output
+        # tiles is split along K)
+        _lib.check(lib.fastlstm_gemm_dx_split(d_ifgo.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code,
+                                              ws_w.data_ptr(), ws_w.numel(), stream), "k5")
 
     def k89():
         _lib.check(lib.fastlstm_gemm_wgrad(d_ifgo.data_ptr(), x.data_ptr(), out.data_ptr(), dWx.data_ptr(),

@@ -59,6 +59,7 @@ SIGNATURES = {
     "fastlstm_bwd_layer": (_i, [_vp] * 15 + [_sz, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_bwd_persistent": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "fastlstm_gemm_dx": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "fastlstm_gemm_dx_split": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "fastlstm_gemm_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "fastlstm_diag_step_probe": (_i, [_i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),

@@ -976,6 +976,15 @@ int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B,
     return gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, nullptr, 0, stream);
 }
 
+int fastlstm_gemm_dx_split(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
+                           void *scratch, size_t scratch_bytes, void *stream) {
+    if (!d_ifgo || !Wx || !dx) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(d_ifgo) || !aligned16(Wx) || !aligned16(dx) || !aligned16(scratch)) return FASTLSTM_ERR_ALIGN;
+    return gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, scratch_bytes ? scratch : nullptr, scratch_bytes, stream);
+}
+
 // tile and split-K factor of a weight-gradient product C[M,N] = A^T.B with reduction length K
 static void wgrad_plan(int M, int N, int K, int dtype, int *tile, int *splits, int *k_per_split) {
     gemm_plan(dtype, M, N, K, M, N, true, true, true, tile, splits);

@@ -251,6 +251,13 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
 int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H,
                      int dtype, void *stream);
 
+/* The same product with device scratch memory (any size; fp32 partial sums): a dx with too few output tiles
+ * to fill the device (T*B*I small against 4H) is split along K where `scratch` holds the partials, else
+ * computed as fastlstm_gemm_dx does.  fastlstm_bwd_layer splits the same way into its weight-gradient
+ * workspace.  Replaces fastlstm/lstm.py:294. */
+int fastlstm_gemm_dx_split(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H,
+                           int dtype, void *scratch, size_t scratch_bytes, void *stream);
+
 /* K6-K9 -- dWx[4H,I] = d_ifgo^T . x,  dWh[4H,H] = d_ifgo^T . h[0..T-1],
  * db[4H] = column sums of d_ifgo; no transposed copy of d_ifgo is made.
  * h: [T+1,B,H] (only slots 0..T-1 are read).  ws: fastlstm_wgrad_workspace_bytes.

@@ -266,6 +266,11 @@ def test_gemm_stages_vs_matmul(dt, M, N, K):
     _lib.check(lib.fastlstm_gemm_dx(d.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, st), "k5")
     want = d.double().view(B, -1) @ Wx.double()
     within(dx.reshape(B, I), want, tol)
+    scratch = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")   # ... split along K where that fills the device
+    dx.zero_()
+    _lib.check(lib.fastlstm_gemm_dx_split(d.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code,
+                                          scratch.data_ptr(), scratch.numel(), st), "k5 split")
+    within(dx.reshape(B, I), want, tol)
     h = torch.randn(T + 1, B, H, generator=g).to(dt).cuda()
     dbx, dbh, dWx, dWh = L.Wgrad(d, x, h)
     assert dbx is dbh
