@@ -681,6 +681,7 @@ struct BwdExtras {
     const void *Wx, *x, *h;
     void *dx, *dWx, *dWh;
     int I;
+    float *db_part = nullptr;   // [ceil(B / 16)][4H] floats: where the launch may leave the bias gradient's partial sums
 };
 
 // In-kernel dx (and, where the shapes suit the 16-bit tile kernel, dWx and dWh) by the workgroups
@@ -699,6 +700,7 @@ struct LowerLayer {
     size_t scratch_bytes;
     const void *x, *h;      // the lower layer's input and its out (for its weight gradients; may be null)
     void *dWx, *dWh;
+    float *db_part = nullptr;   // as BwdExtras::db_part, for the lower layer
     const void *dout = nullptr;   // two independent recurrences side by side (no extras): the second one's dout
 };
 
@@ -819,6 +821,12 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
             }
         }
     }
+    // the bias gradient of a layer whose weight gradients are part of the launch: summed by its recurrence workgroups
+    p->db_lds_off = (c.lds + 15) / 16 * 16;
+    const int ipt = cdiv(16 * c.mt * 16 * c.ntw, kWave * 8);   // (unit, row) items per thread of the reverse kernel
+    const bool slots_fit = p->db_lds_off + ipt * kWave * 8 * 16 <= Gemm16Cfg<256, 256, 2, 2, 4, 2>::LDS_BYTES;
+    p->db_part = (*wgrad_fused && slots_fit) ? e.db_part : nullptr;
+    p->db_part_lo = (lower && lower_wgrad_fused && *lower_wgrad_fused && slots_fit) ? lower->db_part : nullptr;
     return true;
 }
 
@@ -828,7 +836,10 @@ bool plan_bwd_helpers(const XcdCfg &c, const void *d_ifgo, const BwdExtras &e, i
 int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo, const void *Wh,
                 unsigned char *wsb, size_t ws_bytes, int T, int B, int H, int dtype, hipStream_t stream,
                 const BwdExtras *extras = nullptr, const LowerLayer *lower = nullptr, bool dry_run = false,
-                bool *lower_wgrad_fused = nullptr, const LaunchOpts &o = LaunchOpts()) {
+                bool *lower_wgrad_fused = nullptr, const LaunchOpts &o = LaunchOpts(), int *db_done = nullptr) {
+    // *db_done: bit 0 / bit 1 set when the launch leaves the bias gradient's partial sums of the (upper) layer / the
+    // lower layer in extras->db_part / lower->db_part
+    if (db_done) *db_done = 0;
     XcdCfg c;
     const int copies = (lower && !extras) ? 2 + o.n_more : 1;   // independent recurrences side by side
     if (!select_xcd(T, B, H, dtype, true, ws_bytes, &c, o.rows, copies)) return copies > 1 ? 2 : 1;
@@ -867,6 +878,7 @@ int try_bwd_xcd(const void *dout, void *dh, void *dc, const void *ifgo, const vo
         if (occ < 1) return 2;
         if (dry_run) return wgrad_fused ? FASTLSTM_OK : 3;
         if (hl(p, c.mt, c.nkw, c.ntw, kNumXcd * 32, lds, stream, nullptr) != hipSuccess) return FASTLSTM_ERR_HIP;
+        if (db_done) *db_done = (p.db_part ? 1 : 0) | (p.db_part_lo ? 2 : 0);
         return wgrad_fused ? FASTLSTM_OK : 3;
     }
     BwdXcdLauncher launch = dtype == FASTLSTM_FP32 ? launch_bwd_xcd_f32
@@ -1671,6 +1683,9 @@ int fastlstm_fwd_stack2_infer(const void *x, const void *Wx0, const void *bx0, c
                             ws, stream, poison_fwd(dtype, T, B, H, out1, cell1, out0, cell0));
 }
 
+// bytes of the partial sums that a reverse launch leaves of a layer's bias gradient (BwdXcdParams::db_part)
+static size_t db_part_bytes(int B, int H) { return align_up((size_t)cdiv(B, 16) * 4 * H * sizeof(float), 256); }
+
 static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo, const void *cell, void *d_ifgo,
                           const void *Wh, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
                           void *db, void *ws, size_t ws_bytes, void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I,
@@ -1696,14 +1711,22 @@ static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo
     if (int rc = plan_device(-1, B, H, dtype, 1, &pl, false)) return rc;
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     int rc = 1;
+    int db_done = 0;
     if (pl.wave_split != 2 && (dx || want_w)) {
-        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I};
+        // (the weight-gradient workspace is not used by a launch that has the weight gradients inside: it takes the
+        // partial sums of the bias gradient)
+        float *db_part = want_w && db_part_bytes(B, H) <= wgrad_ws_bytes ? static_cast<float *>(wgrad_ws) : nullptr;
+        const BwdExtras e{Wx, x, h, dx, dWx, dWh, I, db_part};
         rc = try_bwd_xcd(dout, dh, dc, ifgo, cell, d_ifgo, Wh, static_cast<unsigned char *>(ws), ws_bytes, T, B, H, dtype,
-                         s, &e);
+                         s, &e, nullptr, false, nullptr, LaunchOpts(), &db_done);
         if (rc < 0) return rc;
     }
-    if (rc == 0) {   // everything but the bias gradient was part of the launch
-        const int chunks = colsum_chunks(T * B);
+    if (rc == 0) {   // everything was part of the launch but the last step of the bias gradient ...
+        if (db_done & 1)
+            return launch_colsum_final(dtype, static_cast<float *>(wgrad_ws), db, 4 * H, cdiv(B, 16), s) == hipSuccess
+                       ? FASTLSTM_OK
+                       : FASTLSTM_ERR_HIP;
+        const int chunks = colsum_chunks(T * B);   // ... or all of it
         return launch_colsum(dtype, d_ifgo, db, static_cast<float *>(wgrad_ws), T * B, 4 * H, chunks, s) == hipSuccess
                    ? FASTLSTM_OK
                    : FASTLSTM_ERR_HIP;
@@ -1750,7 +1773,8 @@ size_t fastlstm_stack2_bwd_wgrad_workspace_bytes(int T, int B, int I, int H, int
     const size_t tile_bytes = (size_t)256 * 256 * sizeof(float);
     const int rows = cdiv(4 * H, 256), helpers = kNumXcd * 32;
     const size_t upper = std::min(rows * 2 * cdiv(H, 256), helpers), lower = std::min(rows * (cdiv(I, 256) + cdiv(H, 256)), helpers);
-    return std::max(need, (upper + lower) * tile_bytes);
+    // ... and the partial sums of both layers' bias gradients behind them
+    return std::max(need, (upper + lower) * tile_bytes) + 2 * db_part_bytes(B, H) + 256;
 }
 
 int fastlstm_bwd_stack2_fused(int T, int B, int I, int H, int dtype, size_t ws_bytes) {
@@ -1789,26 +1813,40 @@ static int bwd_stack2_impl(const void *dout, void *dh1, void *dc1, const void *i
     // the upper layer's input is the lower layer's h: x1 = out0[1:]
     const void *x1 = static_cast<const unsigned char *>(out0) + (size_t)B * H * elem_bytes(dtype);
     if (pl.wave_split != 2) {
-        const BwdExtras e{Wx1, x1, out1, dx1, dWx1, dWh1, H};
-        const LowerLayer lower{dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, dx0, I, wgrad_ws, wgrad_ws_bytes, x, out0, dWx0, dWh0};
+        // the end of the weight-gradient workspace takes the two layers' partial sums of the bias gradients, the
+        // parked weight-gradient tiles come before them
+        const size_t dbb = db_part_bytes(B, H);
+        const bool db_room = wgrad_ws_bytes >= need + 2 * dbb;
+        const size_t park_bytes = db_room ? (wgrad_ws_bytes - 2 * dbb) / 256 * 256 : wgrad_ws_bytes;
+        float *dbp1 = db_room ? reinterpret_cast<float *>(static_cast<unsigned char *>(wgrad_ws) + park_bytes) : nullptr;
+        float *dbp0 = db_room ? reinterpret_cast<float *>(static_cast<unsigned char *>(wgrad_ws) + park_bytes + dbb) : nullptr;
+        const BwdExtras e{Wx1, x1, out1, dx1, dWx1, dWh1, H, dbp1};
+        const LowerLayer lower{dh0, dc0, ifgo0, cell0, d_ifgo0, Wh0, Wx0, dx0, I, wgrad_ws, park_bytes, x, out0, dWx0, dWh0, dbp0};
         bool lower_wgrad_done = false;
+        int db_done = 0;
         const int rc = try_bwd_xcd(dout, dh1, dc1, ifgo1, cell1, d_ifgo1, Wh1, static_cast<unsigned char *>(ws), ws_bytes, T, B,
-                                   H, dtype, s, &e, &lower, false, &lower_wgrad_done);
+                                   H, dtype, s, &e, &lower, false, &lower_wgrad_done, LaunchOpts(), &db_done);
         if (rc < 0) return rc;
         if (rc == 0) {   // both recurrences, both dx and the upper weight gradients were one launch
-            const int chunks = colsum_chunks(T * B);
-            if (launch_colsum(dtype, d_ifgo1, db1, static_cast<float *>(wgrad_ws), T * B, 4 * H, chunks, s) != hipSuccess)
+            if (db_done & 1) {
+                if (launch_colsum_final(dtype, dbp1, db1, 4 * H, cdiv(B, 16), s) != hipSuccess) return FASTLSTM_ERR_HIP;
+            } else if (launch_colsum(dtype, d_ifgo1, db1, static_cast<float *>(wgrad_ws), T * B, 4 * H, colsum_chunks(T * B), s) !=
+                       hipSuccess) {
                 return FASTLSTM_ERR_HIP;
+            }
         } else if (rc == 3) {   // ... but for the upper weight gradients (T*B not a multiple of the GEMM k-tile)
             if (int r2 = fastlstm_gemm_wgrad(d_ifgo1, x1, out1, dWx1, dWh1, db1, wgrad_ws, wgrad_ws_bytes, T, B, H, H, dtype,
                                              stream))
                 return r2;
         }
-        if ((rc == 0 || rc == 3) && lower_wgrad_done)   // only the lower layer's bias gradient is left
+        if ((rc == 0 || rc == 3) && lower_wgrad_done) {   // only the lower layer's bias gradient is left
+            if (db_done & 2)
+                return launch_colsum_final(dtype, dbp0, db0, 4 * H, cdiv(B, 16), s) == hipSuccess ? FASTLSTM_OK : FASTLSTM_ERR_HIP;
             return launch_colsum(dtype, d_ifgo0, db0, static_cast<float *>(wgrad_ws), T * B, 4 * H, colsum_chunks(T * B), s) ==
                            hipSuccess
                        ? FASTLSTM_OK
                        : FASTLSTM_ERR_HIP;
+        }
         if (rc == 0 || rc == 3)
             return fastlstm_gemm_wgrad(d_ifgo0, x, out0, dWx0, dWh0, db0, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);
     }

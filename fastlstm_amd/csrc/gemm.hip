@@ -278,6 +278,15 @@ hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int 
     }
 }
 
+// the second stage alone: out[C] = the sum over `chunks` rows of part[chunks][C]
+hipError_t launch_colsum_final(int dtype, const float *part, void *out, int C, int chunks, hipStream_t s) {
+    const dim3 grid(cdiv(C, kColsumFinalCols)), block(256);
+    if (dtype == FASTLSTM_FP32) hipLaunchKernelGGL(colsum_final_kernel<float>, grid, block, 0, s, part, static_cast<float *>(out), C, chunks);
+    else if (dtype == FASTLSTM_FP16) hipLaunchKernelGGL(colsum_final_kernel<_Float16>, grid, block, 0, s, part, static_cast<_Float16 *>(out), C, chunks);
+    else hipLaunchKernelGGL(colsum_final_kernel<__bf16>, grid, block, 0, s, part, static_cast<__bf16 *>(out), C, chunks);
+    return hipGetLastError();
+}
+
 int gemm_bk(int dtype) { return dtype == FASTLSTM_FP32 ? GemmTile<float>::BK : GemmTile<_Float16>::BK; }
 
 }  // namespace fastlstm

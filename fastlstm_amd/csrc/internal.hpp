@@ -13,6 +13,7 @@ struct FwdXcdParams;
 struct BwdXcdParams;
 
 hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hipStream_t s);
+hipError_t launch_colsum_final(int dtype, const float *part, void *out, int C, int chunks, hipStream_t s);
 hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
                          hipStream_t s);
 int gemm_bk(int dtype);

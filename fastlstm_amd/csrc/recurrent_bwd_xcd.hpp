@@ -38,6 +38,13 @@ struct BwdXcdParams {
     // recurrence has finished a chunk of k5_chunk_steps timesteps (k5_chunk_tiles row tiles);
     // chunk_done[c] counts the recurrence workgroups (n_active) whose part of chunk c is in memory.
     GemmParams k5;      // M = T*B, N = I, K = 4H, A = d_ifgo, B = Wx (K-major), C = dx
+    // Bias gradient inside the launch (HELP instantiations, db_part != nullptr): every recurrence workgroup sums the
+    // d_ifgo values it produces over all timesteps -- thread-private fp32 slots in LDS, updated behind the publish of
+    // each step, while the workgroup waits for its peers anyway -- and writes the sums of its 16-row batch tiles to
+    // db_part[batch tile][4H] at the end; a small kernel adds the batch tiles up.  The separate column-sum pass
+    // over d_ifgo (one more read of T*B*4H elements) is not needed then.
+    float *db_part, *db_part_lo;   // [ceil(B / 16)][4H] each; _lo: the lower layer of a stacked launch
+    int db_lds_off;                // byte offset of the slots in the workgroup's LDS (behind the recurrence's own use)
     int k5_tail_by_rec; // 1: the dx tiles of the chunk that completes last (timesteps 0 ..) are computed by the recurrence
                         // workgroups once their time loop has ended, not by the helpers, which still owe that chunk's
                         // share of their weight-gradient tiles (single-layer launches)
@@ -357,6 +364,12 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
     const T *Wh = static_cast<const T *>(pick(p.Wh, p.Wh_lo, p.Wh_more[0], p.Wh_more[1]));
     T *dh_state = static_cast<T *>(pick(p.dh, p.dh_lo, p.dh_more[0], p.dh_more[1]));
     T *dc_state_buf = static_cast<T *>(pick(p.dc, p.dc_lo, p.dc_more[0], p.dc_more[1]));
+    float *db_part = nullptr;
+    if constexpr (HELP != 0) db_part = lower ? p.db_part_lo : p.db_part;
+    f32x4 *db_slots = reinterpret_cast<f32x4 *>(smem + p.db_lds_off) + tid;   // slot of item m: db_slots[m * NTHR]
+    if (db_part)
+#pragma unroll
+        for (int m = 0; m < IPT; ++m) db_slots[m * NTHR] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // ---- prologue: this wave's fragments of Wh[:, units]^T, gathered from global memory ----
     // fragment (unit tile a, k-step ks): lane (q, r) holds row r = unit u0 + 16a + r and
@@ -545,6 +558,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
         if (follows && wave == 0 && t >= DIST && (t - DIST) % p.k5_chunk_steps == p.k5_chunk_steps - 1) wait_dout(t - DIST);
 
         // ---- point-wise gate backward for this thread's items --------------------------
+        u32x2 d_kept[IPT];   // the items' four stored gate gradients, for the bias sums behind the publish
 #pragma unroll
         for (int m = 0; m < IPT; ++m) {
             T st_d[4];
@@ -576,6 +590,7 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
 #pragma unroll
                 for (int gt = 0; gt < 4; ++gt) st_d[gt] = E::from_f32(0.f);
             }
+            if constexpr (HELP != 0 && E::BYTES == 2) d_kept[m] = *reinterpret_cast<u32x2 *>(st_d);
             // exchange copy: 4 consecutive k = (unit, gate 0..3).  16-bit types: lanes l and l+16
             // own units u and u+1 of the same batch row; the even-unit lane writes both (16 bytes)
             if constexpr (E::BYTES == 2) {
@@ -598,6 +613,17 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             __hip_atomic_fetch_add(grp_counters + tid * kXcdCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         tile_to_global(t);
         if (s + DIST < T_) fetch_tiles(t - DIST, gpre[PAR], cpre[PAR], dpre[PAR]);
+        if constexpr (HELP != 0 && E::BYTES == 2) {
+            if (db_part) {   // (the rounded values, as they were stored: db is the column sum of d_ifgo)
+#pragma unroll
+                for (int m = 0; m < IPT; ++m) {
+                    const T *dv = reinterpret_cast<const T *>(&d_kept[m]);
+                    f32x4 a = db_slots[m * NTHR];
+                    a[0] += E::to_f32(dv[0]); a[1] += E::to_f32(dv[1]); a[2] += E::to_f32(dv[2]); a[3] += E::to_f32(dv[3]);
+                    db_slots[m * NTHR] = a;
+                }
+            }
+        }
 
         if (wave == 0) wait_counter(my_counter, p.n_ht * (s + 1), p.hdr, p.spin_limit, vg, s);
         __syncthreads();
@@ -673,6 +699,24 @@ __global__ __launch_bounds__(kWave * NWV) void lstm_bwd_xcd_kernel(const BwdXcdP
             dh_state[off_h[m]] = E::from_f32(dh_rec[m]);
             dc_state_buf[off_h[m]] = E::from_f32(dc_state[m]);
         }
+    if constexpr (HELP != 0) {
+        if (db_part) {   // sums over the 16 rows of a batch tile (16 neighbouring lanes), one lane writes the four gates
+#pragma unroll
+            for (int m = 0; m < IPT; ++m) {
+                f32x4 a = db_slots[m * NTHR];
+#pragma unroll
+                for (int d = 1; d < 16; d <<= 1) {
+                    a[0] += __shfl_xor(a[0], d); a[1] += __shfl_xor(a[1], d);
+                    a[2] += __shfl_xor(a[2], d); a[3] += __shfl_xor(a[3], d);
+                }
+                const int it = tid + NTHR * m, rest = it >> 4, ul = rest % HT, nt = rest / HT;
+                if ((it & 15) == 0 && nt < NT && b0 + nt * 16 < B) {
+                    float *dst = db_part + (size_t)((b0 + nt * 16) >> 4) * 4 * H + u0 + ul;
+                    dst[0] = a[0]; dst[H] = a[1]; dst[2 * (size_t)H] = a[2]; dst[3 * (size_t)H] = a[3];
+                }
+            }
+        }
+    }
     if constexpr (HELP == 1) {
         // The time loop is over and this CU would idle while the helpers finish: the dx tiles of the last chunk
         // (complete once every recurrence workgroup has counted it, just above) are dealt to the recurrence
