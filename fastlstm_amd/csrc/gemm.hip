@@ -44,7 +44,9 @@ hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const int grid = cdiv(p.M, BM) * cdiv(p.N, BN) * p.splits;
+    // the 256 x 256 configuration (one workgroup per CU) walks through a longer tile list with one workgroup per CU
+    const int tiles = cdiv(p.M, BM) * cdiv(p.N, BN) * p.splits;
+    const int grid = (BM == 256 && BN == 256) ? std::min(tiles, kNumXcd * 32) : tiles;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

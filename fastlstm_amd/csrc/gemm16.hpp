@@ -828,12 +828,80 @@ __device__ __forceinline__ void gemm16_epilogue(const GemmParams &p, const int m
     }
 }
 
+// The C tile of an interior 256 x 256 tile (16-bit types, no split) straight from the accumulators: no LDS
+// staging, no barrier, and nothing waits for the stores -- a persistent workgroup goes on to its next tile
+// while they drain.  Lane (q, r) holds C[row r][4q .. 4q+3] of each 16 x 16 tile.  Two neighbouring tiles swap
+// halves between the lane groups q and q ^ 1 (v_permlane16_swap), which leaves every lane with 8 consecutive
+// columns (16 bytes) of one of them; the two 64-byte packets of a row then trade places between rows r and
+// r ^ 8 (DPP), so that one store instruction writes 8 rows x 128 bytes: whole cache lines.
+// Same values as gemm16_epilogue (bias added in fp32, one rounding).
+template <typename T>
+__device__ __forceinline__ void gemm16_epilogue_direct(const GemmParams &p, const int m0, const int n0,
+                                                       const f32x4 (&acc)[8][4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r = lane & 15, wm = wave >> 2, wn = wave & 3;
+    const T *bias0 = static_cast<const T *>(p.bias0), *bias1 = static_cast<const T *>(p.bias1);
+    float bv[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        u32x2 raw0 = {0u, 0u}, raw1 = {0u, 0u};
+        const int n = n0 + (wn * 4 + j) * 16 + q * 4;
+        if (bias0) raw0 = *reinterpret_cast<const u32x2 *>(bias0 + n);
+        if (bias0 && bias1) raw1 = *reinterpret_cast<const u32x2 *>(bias1 + n);
+        const T *t0 = reinterpret_cast<const T *>(&raw0), *t1 = reinterpret_cast<const T *>(&raw1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bv[j][e] = Elem<T>::to_f32(t0[e]) + Elem<T>::to_f32(t1[e]);
+    }
+    const __amdgpu_buffer_rsrc_t rc =
+        __builtin_amdgcn_make_buffer_rsrc(p.C, 0, (unsigned)((size_t)p.M * p.ldc * sizeof(T)), 0x00020000);
+    const bool hi = r >= 8;
+    const unsigned colb = (unsigned)(n0 + wn * 64 + (hi ? 32 : 0) + (q & 1) * 16 + (q >> 1) * 8);
+    const int aux = p.keep_c ? 0 : 2;   // 2: non-temporal
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        u32x4 pkt[2];
+#pragma unroll
+        for (int jp = 0; jp < 2; ++jp) {
+            const f32x4 v0 = acc[i][2 * jp], v1 = acc[i][2 * jp + 1];
+            T pk0[4] = {Elem<T>::from_f32(v0[0] + bv[2 * jp][0]), Elem<T>::from_f32(v0[1] + bv[2 * jp][1]),
+                        Elem<T>::from_f32(v0[2] + bv[2 * jp][2]), Elem<T>::from_f32(v0[3] + bv[2 * jp][3])};
+            T pk1[4] = {Elem<T>::from_f32(v1[0] + bv[2 * jp + 1][0]), Elem<T>::from_f32(v1[1] + bv[2 * jp + 1][1]),
+                        Elem<T>::from_f32(v1[2] + bv[2 * jp + 1][2]), Elem<T>::from_f32(v1[3] + bv[2 * jp + 1][3])};
+            const u32x2 a = *reinterpret_cast<u32x2 *>(pk0), b = *reinterpret_cast<u32x2 *>(pk1);
+            // lane group q: tile 2 jp + (q & 1), columns 8 (q >> 1) .. + 7
+            const u32x2 s0 = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+            const u32x2 s1 = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+            pkt[jp] = u32x4{s0[0], s1[0], s0[1], s1[1]};
+        }
+        // rows r < 8 keep their columns 0 .. 31 and take those of row r + 8; rows r >= 8 keep their columns 32 .. 63
+        // and take those of row r - 8
+        const u32x4 snd = hi ? pkt[0] : pkt[1];
+        u32x4 rcv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) rcv[e] = (unsigned)__builtin_amdgcn_update_dpp(0, (int)snd[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+        const u32x4 first = hi ? rcv : pkt[0], second = hi ? pkt[1] : rcv;   // rows (r & 7) and (r & 7) + 8 of the 16
+        const unsigned row0 = (unsigned)(m0 + (wm * 8 + i) * 16 + (r & 7));
+        const unsigned off = (row0 * (unsigned)p.ldc + colb) * (unsigned)sizeof(T);
+        if (aux) {
+            __builtin_amdgcn_raw_buffer_store_b128(first, rc, off, 0, 2);
+            __builtin_amdgcn_raw_buffer_store_b128(second, rc, off + 8u * (unsigned)p.ldc * (unsigned)sizeof(T), 0, 2);
+        } else {
+            __builtin_amdgcn_raw_buffer_store_b128(first, rc, off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(second, rc, off + 8u * (unsigned)p.ldc * (unsigned)sizeof(T), 0, 0);
+        }
+    }
+#else
+    (void)p; (void)m0; (void)n0; (void)acc;
+#endif
+}
+
 // One BM x BN tile of C (rows m0.., columns n0.., K range of `split`): main loop + epilogue.
 // ALONE: the tile of a stand-alone GEMM launch (streaming stores); PP: the ping-pong main loop where the
 // configuration has one.
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT, bool ALONE = false,
           bool PP = ALONE>
-__device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
+__device__ __forceinline__ bool gemm16_tile(const GemmParams &p, const int m0, const int n0, const int split,
                                             unsigned char *smem, const int trace_slot) {
     constexpr int TM = BM / WVM / 16, TN = BN / WVN / 16;
     long long t_start = 0, t_epi = 0;
@@ -850,29 +918,52 @@ __device__ __forceinline__ void gemm16_tile(const GemmParams &p, const int m0, c
     else
         gemm16_mainloop<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc);
     if (p.trace) t_epi = (long long)wall_clock64();
-    gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT, ALONE>(p, m0, n0, split, smem, acc);
+    bool lds_used = true;   // (by the epilogue: a caller that goes on to another tile has to wait for its readers)
+    if constexpr (ALONE && sizeof(T) == 2 && BM == 256 && BN == 256 && WVM == 2 && WVN == 4) {
+        // the whole tile inside C, rows that take 16-byte stores, biases that take 8-byte loads (or none)
+        const bool direct = p.splits == 1 && m0 + BM <= p.M && n0 + BN <= p.N && (p.ldc & 7) == 0 &&
+                            (reinterpret_cast<size_t>(p.C) & 15) == 0 && (size_t)p.M * p.ldc * sizeof(T) < ((size_t)1 << 32) &&
+                            ((reinterpret_cast<size_t>(p.bias0) | reinterpret_cast<size_t>(p.bias1)) & 7) == 0;
+        if (direct) {
+            gemm16_epilogue_direct<T>(p, m0, n0, acc);
+            lds_used = false;
+        } else {
+            gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT, ALONE>(p, m0, n0, split, smem, acc);
+        }
+    } else {
+        gemm16_epilogue<T, BM, BN, NS, WVM, WVN, KSPT, ALONE>(p, m0, n0, split, smem, acc);
+        lds_used = !(sizeof(T) == 4 || p.splits > 1);   // (those store from the accumulators)
+    }
     if (p.trace && threadIdx.x == 0) {   // stamps: start, main loop entered (= start), main loop left, done
         long long *t = p.trace + (size_t)trace_slot * 4;
         t[0] = t_start; t[1] = t_start; t[2] = t_epi; t[3] = (long long)wall_clock64();
     }
+    return lds_used;
 }
 
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
 __global__ __launch_bounds__(64 * WVM * WVN) void gemm16_kernel(const GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tiles_n = cdiv(p.N, BN), tiles_m = cdiv(p.M, BM);
-    int bid = blockIdx.x;
-    const int split = bid / (tiles_m * tiles_n);
-    bid -= split * tiles_m * tiles_n;
-    // Tile order: every XCD gets a contiguous range of a grouped order in which 8 x 8 blocks
-    // of C tiles are consecutive, so the ~64 workgroups an XCD runs at a time re-use each
-    // other's A and B tiles out of that XCD's L2.
-    constexpr int GM = 8;
-    const int lin = xcd_major_id(bid, tiles_m * tiles_n);
-    const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
-    const int gsz = min(tiles_m - first_m, GM);
-    const int m0 = (first_m + (lin % per_group) % gsz) * BM, n0 = ((lin % per_group) / gsz) * BN;
-    gemm16_tile<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT, true>(p, m0, n0, split, smem, (int)blockIdx.x);
+    const int total = tiles_m * tiles_n * p.splits;
+    // A launch with more tiles than the device has CUs is a grid of one workgroup per CU that walks through the
+    // tile list (tile b, b + gridDim.x, ...: the tiles that a one-tile-per-workgroup launch would run together
+    // still do, on the same XCDs): a workgroup starts its next tile while the stores of the last one drain.
+    for (int b = blockIdx.x; b < total; b += gridDim.x) {
+        int bid = b;
+        const int split = bid / (tiles_m * tiles_n);
+        bid -= split * tiles_m * tiles_n;
+        // Tile order: every XCD gets a contiguous range of a grouped order in which 8 x 8 blocks
+        // of C tiles are consecutive, so the ~64 workgroups an XCD runs at a time re-use each
+        // other's A and B tiles out of that XCD's L2.
+        constexpr int GM = 8;
+        const int lin = xcd_major_id(bid, tiles_m * tiles_n);
+        const int per_group = GM * tiles_n, first_m = (lin / per_group) * GM;
+        const int gsz = min(tiles_m - first_m, GM);
+        const int m0 = (first_m + (lin % per_group) % gsz) * BM, n0 = ((lin % per_group) / gsz) * BN;
+        const bool lds_used = gemm16_tile<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT, true>(p, m0, n0, split, smem, b);
+        if (lds_used && b + (int)gridDim.x < total) __syncthreads();   // the staged C tile was read: the stages are free
+    }
 }
 
 // Both weight-gradient products and the bias gradient of a layer in one launch:
@@ -916,7 +1007,15 @@ template <typename T> __global__ __launch_bounds__(512) void gemm16_wgrad_kernel
     // (no bias gradient wanted: remainder -1 never comes up)
     gemm16_mainloop_pp<T, true, true, true>(p, m0, n0, kb, min(k_end, kb + p.k_per_split), smem, acc, colsum, tiles_n,
                                             w.db_part ? nt : -1);
-    gemm16_epilogue<T, 256, 256, 2, 2, 4, 2, true>(p, m0, n0, split, smem, acc);
+    bool direct = false;
+    if constexpr (sizeof(T) == 2)
+        direct = p.splits == 1 && m0 + 256 <= p.M && n0 + 256 <= p.N && (p.ldc & 7) == 0 &&
+                 (reinterpret_cast<size_t>(p.C) & 15) == 0 && (size_t)p.M * p.ldc * sizeof(T) < ((size_t)1 << 32);
+    if (direct) {
+        if constexpr (sizeof(T) == 2) gemm16_epilogue_direct<T>(p, m0, n0, acc);   // (no biases in these products)
+    } else {
+        gemm16_epilogue<T, 256, 256, 2, 2, 4, 2, true>(p, m0, n0, split, smem, acc);
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (w.db_part) {
         // lane (q, r) holds the sum over its k-groups for row r of its two fragments: add the four lane groups
