@@ -603,12 +603,14 @@ def Wgrad(d_ifgo, x, h):
 def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh, need_dx=True, need_dw=True):
     """Reverse pass.  dh[T,B,H]: gradient of out[1:]; dc_n, dh_n [B,H]: gradients
     flowing into the last cell / hidden state, overwritten with the gradients of
-    the initial state and returned (fastlstm/lstm.py:236-334).
+    the initial state and returned (fastlstm/lstm.py:236-334).  dc_n = dh_n = None: no gradient flows
+    into the final state (the buffers are made here and zeroed by the launch that clears the workspace).
     Returns (d_x, dh_0, dc_0, dWx, dbx, dWh, dbh).  need_dx=False: the product d_ifgo . Wx is
     skipped and d_x is None (no gradient of the layer's input is asked for: the first layer of most
     models); need_dw=False: the weight and bias gradients are skipped and None (frozen weights).
     The reference computes all of them whatever autograd asks for (fastlstm/lstm.py:524-538)."""
-    _require_gpu(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh)
+    no_state_grad = dc_n is None and dh_n is None
+    _require_gpu(dh, x, h, cell, ifgo, Wx, Wh, *(() if no_state_grad else (dc_n, dh_n)))
     code = _code(ifgo)
     seq_len, batch_size, hidden_size = dh.shape
     input_size = Wx.shape[1]
@@ -618,13 +620,21 @@ def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh, need_dx=True, 
         if dh.dtype != ifgo.dtype:
             dh = dh.to(ifgo.dtype)
         dh = _aligned(dh)
-        assert dc_n.is_contiguous() and dh_n.is_contiguous()
         if PROFILE_RANGES:
             torch.cuda.nvtx.range_push("fastlstm: prepare backward")
         d_ifgo = torch.empty_like(ifgo)
         plan = _plan(x.device, batch_size, hidden_size, code, True)
-        ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         stream = _stream()
+        if no_state_grad:   # one launch: workspace cleared, both state gradients zero
+            dc_n, dh_n = torch.empty_like(cell[0]), torch.empty_like(cell[0])
+            n = lib.fastlstm_recurrent_workspace_bytes(plan, seq_len, hidden_size, code, 1)
+            ws = torch.empty(n, dtype=torch.uint8, device=x.device)
+            _lib.check(lib.fastlstm_prepare_forward(ws.data_ptr(), n if plan.ring_needs_zero else min(n, plan.ws_zero_bytes),
+                                                    dh_n.data_ptr(), dc_n.data_ptr(), None, None, batch_size, hidden_size,
+                                                    code, stream), "fastlstm_prepare_forward")
+        else:
+            assert dc_n.is_contiguous() and dh_n.is_contiguous()
+            ws = _workspace(plan, seq_len, hidden_size, code, True, x.device)
         x, h = _aligned(x.contiguous()), h.contiguous()
         d_x = torch.empty_like(x) if need_dx else None
         G = 4 * hidden_size
@@ -838,13 +848,12 @@ class PersistentLSTMfn(torch.autograd.Function):
     def backward(ctx, dh, d_out_cell):
         _raise_pending_before_backward(dh)   # a failed forward launch is reported before its gradients are computed
         x, out, cell, ifgo, Wx, Wh = ctx.saved_tensors
-        if d_out_cell is None:
-            dc_n, dh_n = torch.zeros_like(cell[0]), torch.zeros_like(cell[0])
-        else:
+        if d_out_cell is not None:
             raise ValueError("Not implemented")  # fastlstm/lstm.py:528-531
         need = ctx.needs_input_grad   # (x, h_0, c_0, Wx, bx, Wh, bh)
+        # (no gradient into the final state: the reference passes two zeros_like, fastlstm/lstm.py:524-527)
         d_x, dh_0, dc_0, dWx, dbx, dWh, dbh = lstm_persistent_bwd(
-            dh, dc_n, dh_n, x, out, cell, ifgo, Wx, Wh, need_dx=need[0], need_dw=any(need[3:7])
+            dh, None, None, x, out, cell, ifgo, Wx, Wh, need_dx=need[0], need_dw=any(need[3:7])
         )
         if ctx.h0_is_nan:
             dh_0 = None

@@ -317,7 +317,9 @@ int fastlstm_recurrent_rows_per_launch(int T, int B, int H, int dtype, int backw
  * `zero_bytes` bytes of the workspace (a multiple of 4; see fastlstm_recurrent_workspace_bytes for how many a
  * call needs zeroed) and writes the initial state into slot 0 of out and cell: h0, c0 ([B,H] each, dense), or
  * zeros when both are NULL.  Replaces `out[0] = h_0; cell[0] = c_0` / the zero initialisation of
- * fastlstm/lstm.py:84-90.  A fill kernel, not a memset: the call can be captured into a graph. */
+ * fastlstm/lstm.py:84-90.  A fill kernel, not a memset: the call can be captured into a graph.
+ * The same launch gets a reverse call ready: its workspace, and dh / dc ([B,H] each) in the place of out / cell
+ * (zeros when no gradient flows into the final state: the two zeros_like of fastlstm/lstm.py:524-527). */
 int fastlstm_prepare_forward(void *ws, size_t zero_bytes, void *out0, void *cell0, const void *h0, const void *c0,
                              int B, int H, int dtype, void *stream);
 
