@@ -348,6 +348,18 @@ def main():
         "gemm_wgrad_frac_of_mfma_peak": round(gw / (t_k89 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
         "bwd_layer_ms": round(t_lb, 4),
     })
+    # the same three stages with the tile kernel in its earlier form (one tile per workgroup, symmetric main loop,
+    # LDS-staged ordinary stores, weight gradients as two products + a column-sum pass), same operands, same process:
+    # box-to-box variation is larger than several of the steps in between
+    if dname != "fp32":
+        try:
+            lib.fastlstm_set_gemm_baseline(1)
+            tb1, tb5, tb89 = ev_time(k1, reps=5), ev_time(k5, reps=5), ev_time(k89, reps=5)
+        finally:
+            lib.fastlstm_set_gemm_baseline(0)
+        kernels["gemm_earlier_form_ms"] = {"ifgo": round(tb1, 4), "dx": round(tb5, 4), "wgrad": round(tb89, 4)}
+        kernels["gemm_gain_over_earlier_form"] = {"ifgo": round(tb1 / t_k1, 3), "dx": round(tb5 / t_k5, 3),
+                                                  "wgrad": round(tb89 / t_k89, 3)}
     # yardstick for the three GEMM stages: the vendor library (torch.matmul = hipBLASLt / rocBLAS) on the same
     # operands and shapes, timed the same way; not part of any measured step
     if dname != "f32":

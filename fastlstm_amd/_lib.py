@@ -69,6 +69,7 @@ SIGNATURES = {
     "fastlstm_prepare_forward": (_i, [_vp, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "fastlstm_set_spin_limit": (None, [ctypes.c_longlong]),
     "fastlstm_set_kernel_families": (None, [_i]),
+    "fastlstm_set_gemm_baseline": (None, [_i]),
     "fastlstm_get_kernel_families": (_i, []),
     "fastlstm_set_gemm_trace": (None, [_vp]),
     "fastlstm_set_recurrent_trace": (None, [_vp]),

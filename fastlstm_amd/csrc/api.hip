@@ -1031,7 +1031,7 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
     {   // both products and the bias gradient as one tile grid, d_ifgo read once
         int sp, kps;
         bool merged;
-        if (wgrad_merged_plan(dtype, M, I, H, K, &sp, &kps, &merged))
+        if (!gemm_baseline() && wgrad_merged_plan(dtype, M, I, H, K, &sp, &kps, &merged))
             return launch_wgrad_merged(dtype, d_ifgo, x, h, dWx, dWh, db, ws, M, I, H, K, s) == hipSuccess ? FASTLSTM_OK
                                                                                                             : FASTLSTM_ERR_HIP;
     }
@@ -1942,6 +1942,7 @@ int fastlstm_device_status(int device, int clear) {
     return FASTLSTM_ERR_TIMEOUT;
 }
 
+void fastlstm_set_gemm_baseline(int on) { fastlstm::set_gemm_baseline(on); }
 void fastlstm_set_kernel_families(int mask) { fastlstm::g_families.store(mask & 7); }
 int fastlstm_get_kernel_families(void) { return fastlstm::g_families.load(); }
 

@@ -1,6 +1,7 @@
 // Host launchers for the MFMA GEMM stages (K1, K5, K8, K9) and the db column sum.
 #include "gemm.hpp"
 #include "gemm16.hpp"
+#include <atomic>
 #include "internal.hpp"
 
 namespace fastlstm {
@@ -33,11 +34,33 @@ hipError_t launch_gemm_t(const GemmParams &p, hipStream_t stream) {
     return e;
 }
 
+std::atomic<int> g_gemm_baseline{0};   // diagnostics: 1 = stand-alone 16-bit 256 x 256 launches run gemm16_onetile_kernel
+
+// one 256 x 256 tile per workgroup (gemm16_onetile_kernel); with splits > 1 the caller reduces the partials
+template <typename T, bool A_KM, bool B_KM> static hipError_t launch_onetile_t(const GemmParams &p, hipStream_t stream) {
+    using C = Gemm16Cfg<256, 256, 2, 2, 4, 2>;
+    static bool attr_set = false;
+    auto kern = gemm16_onetile_kernel<T, A_KM, B_KM>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(cdiv(p.M, 256) * cdiv(p.N, 256) * p.splits), dim3(C::THREADS), C::LDS_BYTES, stream, p);
+    return hipGetLastError();
+}
+
 template <typename T, bool A_KM, bool B_KM, int BM, int BN, int NS, int WVM, int WVN, int KSPT>
 hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
     using C = Gemm16Cfg<BM, BN, NS, WVM, WVN, KSPT>;
     static bool attr_set = false;
+    const bool baseline = BM == 256 && BN == 256 && sizeof(T) == 2 && g_gemm_baseline.load() != 0;
     auto kern = gemm16_kernel<T, A_KM, B_KM, BM, BN, NS, WVM, WVN, KSPT>;
+    if constexpr (BM == 256 && BN == 256 && sizeof(T) == 2) {
+        if (baseline)
+            if (hipError_t e = launch_onetile_t<T, A_KM, B_KM>(p, stream)) return e;
+    }
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
@@ -47,7 +70,7 @@ hipError_t launch_gemm16_t(const GemmParams &p, hipStream_t stream) {
     // the 256 x 256 configuration (one workgroup per CU) walks through a longer tile list with one workgroup per CU
     const int tiles = cdiv(p.M, BM) * cdiv(p.N, BN) * p.splits;
     const int grid = (BM == 256 && BN == 256) ? std::min(tiles, kNumXcd * 32) : tiles;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, stream, p);
+    if (!baseline) hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.splits > 1) {
@@ -214,7 +237,11 @@ static hipError_t launch_wgrad_merged_t(const WgradParams &w, bool merged, void 
         a.h.N = 0;
         b.x = w.h; b.h.N = 0; b.tiles_nx = cdiv(H, 256); b.db_part = nullptr;
         if (hipError_t e = launch_wgrad_kernel_t<T>(a, s)) return e;
-        if (hipError_t e = launch_wgrad_kernel_t<T>(b, s)) return e;
+        if constexpr (sizeof(T) == 2) {   // one round of tiles, both operands K-major: the symmetric loop (gemm16_onetile_kernel)
+            if (hipError_t e = launch_onetile_t<T, true, true>(w.h, s)) return e;
+        } else {
+            if (hipError_t e = launch_wgrad_kernel_t<T>(b, s)) return e;
+        }
         db_parts = splits * w.tiles_nx;
     }
     const int ri = splits > 1 ? I : 0, rh = splits > 1 ? H : 0;   // the products need no pass without a split
@@ -244,6 +271,9 @@ hipError_t launch_wgrad_merged(int dtype, const void *d_ifgo, const void *x, con
            : dtype == FASTLSTM_FP16 ? launch_wgrad_merged_t<_Float16>(w, merged, db, s)
                                     : launch_wgrad_merged_t<__bf16>(w, merged, db, s);
 }
+
+void set_gemm_baseline(int on) { g_gemm_baseline.store(on ? 1 : 0); }
+int gemm_baseline() { return g_gemm_baseline.load(); }
 
 static long long *g_trace = nullptr;
 void set_gemm_trace(long long *buf) { g_trace = buf; }

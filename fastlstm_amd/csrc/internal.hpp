@@ -13,6 +13,9 @@ struct FwdXcdParams;
 struct BwdXcdParams;
 
 hipError_t launch_gemm(int dtype, const GemmParams &p, bool a_km, bool b_km, hipStream_t s);
+// diagnostics: the stand-alone 16-bit tile launches in their earlier form (gemm16_onetile_kernel)
+void set_gemm_baseline(int on);
+int gemm_baseline();
 hipError_t launch_colsum_final(int dtype, const float *part, void *out, int C, int chunks, hipStream_t s);
 hipError_t launch_colsum(int dtype, const void *in, void *out, float *part, int R, int C, int chunks,
                          hipStream_t s);

@@ -21,6 +21,13 @@ extern "C" {
 void fastlstm_set_kernel_families(int mask);
 int fastlstm_get_kernel_families(void);
 
+/* Measurement: with `on` != 0 the stand-alone 16-bit GEMM launches (fastlstm_gemm_ifgo, _dx, _wgrad) run the tile
+ * kernel in its earlier form -- one tile per workgroup, symmetric main loop, C staged through LDS and written with
+ * ordinary stores, the weight gradients as two products followed by a column-sum pass -- so that a benchmark can
+ * time both forms on the same operands in one process (the results agree to rounding; bench.py reports both).
+ * Process-wide, default 0; no counterpart in the reference. */
+void fastlstm_set_gemm_baseline(int on);
+
 /* Upper bound, in 100 MHz ticks, a barrier wait may spin before it gives up
  * (default 4e8 = 4 s).  Tests lower it to force the time-out path from the host. */
 void fastlstm_set_spin_limit(long long ticks);

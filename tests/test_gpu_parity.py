@@ -289,6 +289,39 @@ def test_gemm_stages_vs_matmul(dt, M, N, K):
     within(dbx, d2.sum(0), tol)
 
 
+def test_gemm_earlier_form_switch_agrees():
+    """fastlstm_set_gemm_baseline(1): the stand-alone products in the tile kernel's earlier form (what bench.py times
+    beside the current one) -- same results to rounding, and the switch goes back."""
+    lib = _lib.load()
+    dt, code = torch.float16, RM[torch.float16]
+    T, B, I, H = 4, 320, 512, 256
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, B, I, generator=g).to(dt).cuda()
+    Wx = (torch.randn(4 * H, I, generator=g) * 0.1).to(dt).cuda()
+    bx, bh = torch.randn(4 * H, generator=g).to(dt).cuda(), torch.randn(4 * H, generator=g).to(dt).cuda()
+    d = torch.randn(T, B, 4 * H, generator=g).to(dt).cuda()
+    h = torch.randn(T + 1, B, H, generator=g).to(dt).cuda()
+    st = torch.cuda.current_stream().cuda_stream
+    res = []
+    try:
+        for on in (0, 1):
+            lib.fastlstm_set_gemm_baseline(on)
+            ifgo = torch.empty(T, B, 4 * H, dtype=dt, device="cuda")
+            dx = torch.empty(T, B, I, dtype=dt, device="cuda")
+            _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), ifgo.data_ptr(),
+                                              T, B, I, H, code, st), "k1")
+            _lib.check(lib.fastlstm_gemm_dx(d.data_ptr(), Wx.data_ptr(), dx.data_ptr(), T, B, I, H, code, st), "k5")
+            res.append((ifgo, dx) + tuple(L.Wgrad(d, x, h)[1:]))
+    finally:
+        lib.fastlstm_set_gemm_baseline(0)
+    torch.cuda.synchronize()
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])   # same products in the same order
+    for a, b in zip(res[0][2:], res[1][2:]):
+        within(a, b.double(), HALF_TOL)
+    want = x.double().view(T * B, I) @ Wx.double().T + bx.double() + bh.double()
+    within(res[1][0].reshape(T * B, -1), want, HALF_TOL)
+
+
 def test_gpu_matches_golden_vectors():
     z = np.load(os.path.join(ROOT, "tests", "golden", "lstm_golden.npz"))
     for name in ("tiny", "ragged", "nostate", "onestep"):
