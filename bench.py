@@ -256,6 +256,11 @@ def main():
                                            dWh_.data_ptr(), db.data_ptr(), ws_w.data_ptr(), ws_w.numel(), T, B, I, H,
                                            code, stream), "wgrad")
 
+    def k589():   # K5 + K8 + K9 + db in one call: one pass over d_ifgo for a narrow layer (workload D), the two stages otherwise
+        _lib.check(lib.fastlstm_gemm_dx_wgrad(d_ifgo.data_ptr(), Wx.data_ptr(), x.data_ptr(), out.data_ptr(), dx.data_ptr(),
+                                              dWx.data_ptr(), dWh_.data_ptr(), db.data_ptr(), ws_w.data_ptr(), ws_w.numel(),
+                                              T, B, I, H, code, stream), "dx + wgrad")
+
     def layer_bwd():   # what lstm_persistent_bwd calls: recurrence + dx + dWx + dWh + db, fused where CUs would idle
         _lib.check(lib.fastlstm_bwd_layer(dout.data_ptr(), dh_n.data_ptr(), dc_n.data_ptr(), ifgo.data_ptr(),
                                           cell.data_ptr(), d_ifgo.data_ptr(), Wh.data_ptr(), Wx.data_ptr(),
@@ -333,6 +338,7 @@ def main():
     t_rb = ev_time(rec_bwd, reps=5, pre=rec_bwd_pre)
     t_k5 = ev_time(k5, reps=5)
     t_k89 = ev_time(k89, reps=5)
+    t_k589 = ev_time(k589, reps=5)
     t_lb = ev_time(layer_bwd, reps=5, pre=rec_bwd_pre)
     torch.cuda.synchronize()
     _lib.check(lib.fastlstm_ws_status(ws_b[:64].cpu().numpy().tobytes()), "backward barrier status")
@@ -346,6 +352,7 @@ def main():
         "gemm_wgrad_ms": round(t_k89, 4),
         "gemm_wgrad_tflops": round(gw / (t_k89 * 1e-3) / 1e12, 2),
         "gemm_wgrad_frac_of_mfma_peak": round(gw / (t_k89 * 1e-3) / 1e12 / PEAK_TFLOPS[dname], 4),
+        "gemm_dx_wgrad_ms": round(t_k589, 4),
         "bwd_layer_ms": round(t_lb, 4),
     })
     # the same three stages with the tile kernel in its earlier form (one tile per workgroup, symmetric main loop,

@@ -62,6 +62,7 @@ SIGNATURES = {
     "fastlstm_gemm_dx_split": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "fastlstm_gemm_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "fastlstm_gemm_dx_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _vp]),
     "fastlstm_diag_step_probe": (_i, [_i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "fastlstm_diag_step_probe_bytes": (_sz, [_i, _i, _i]),
     "fastlstm_ws_status": (_i, [_vp]),

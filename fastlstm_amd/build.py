@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(LIBDIR, "libfastlstm_hip.so")
-SOURCES = ["api.hip", "gemm.hip", "diag.hip", "recurrent_stream.hip", "plan.cpp", "recurrent_f32.hip", "recurrent_f16.hip", "recurrent_bf16.hip",
+SOURCES = ["api.hip", "gemm.hip", "gemm_small.hip", "diag.hip", "recurrent_stream.hip", "plan.cpp", "recurrent_f32.hip", "recurrent_f16.hip", "recurrent_bf16.hip",
            "recurrent_wreg_f32.hip", "recurrent_wreg_f16.hip", "recurrent_wreg_bf16.hip",
            "recurrent_xcd_f32.hip", "recurrent_xcd_f16.hip", "recurrent_xcd_bf16.hip",
            "recurrent_wsplit_f16.hip", "recurrent_wsplit_bf16.hip"]

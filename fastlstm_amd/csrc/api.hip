@@ -1014,7 +1014,8 @@ size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype) {
     wgrad_plan(M, H, K, dtype, &tile, &sh, &kps);
     size_t part = std::max(sx > 1 ? (size_t)sx * M * I : 0, sh > 1 ? (size_t)sh * M * H : 0) * sizeof(float);
     size_t cs = (size_t)colsum_chunks(K) * M * sizeof(float);
-    return std::max(align_up(cs, 256) + align_up(part, 256), wgrad_merged_workspace(dtype, M, I, H, K)) + 256;
+    const size_t small = small_bwd_eligible(dtype, K, I, H) ? small_bwd_workspace(K, I, H) : 0;
+    return std::max(std::max(align_up(cs, 256) + align_up(part, 256), wgrad_merged_workspace(dtype, M, I, H, K)), small) + 256;
 }
 
 int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
@@ -1028,6 +1029,9 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
     if (ws_bytes < fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype)) return FASTLSTM_ERR_WORKSPACE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int K = T * B, M = 4 * H;
+    if (!gemm_baseline() && small_bwd_eligible(dtype, K, I, H))   // narrow layer: one streaming pass (gemm_small.hpp)
+        return launch_small_bwd(dtype, d_ifgo, nullptr, x, h, nullptr, dWx, dWh, db, ws, K, I, H, s) == hipSuccess ? FASTLSTM_OK
+                                                                                                                  : FASTLSTM_ERR_HIP;
     {   // both products and the bias gradient as one tile grid, d_ifgo read once
         int sp, kps;
         bool merged;
@@ -1052,6 +1056,38 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
         if (launch_gemm_tiled(dtype, p, true, true, tile, s) != hipSuccess) return FASTLSTM_ERR_HIP;
     }
     return FASTLSTM_OK;
+}
+
+// K5, K8, K9 and the bias gradient behind a reverse recurrence: one pass over d_ifgo for a narrow 16-bit layer
+// (gemm_small.hpp), else the two stages one after the other.  dx may be null, and so may dWx, dWh, db (all three).
+static int gemm_dx_wgrad_impl(const void *d_ifgo, const void *Wx, const void *x, const void *h, void *dx, void *dWx,
+                              void *dWh, void *db, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype,
+                              void *stream) {
+    const bool want_w = dWx != nullptr;
+    if (!dx && !want_w) return FASTLSTM_OK;
+    if (small_bwd_eligible(dtype, T * B, I, H) && (!want_w || ws_bytes >= small_bwd_workspace(T * B, I, H)))
+        return launch_small_bwd(dtype, d_ifgo, Wx, x, h, dx, dWx, dWh, db, ws, T * B, I, H, static_cast<hipStream_t>(stream)) ==
+                       hipSuccess
+                   ? FASTLSTM_OK
+                   : FASTLSTM_ERR_HIP;
+    // (the weight-gradient workspace is free until the weight gradients start: scratch for a split along K)
+    if (dx)
+        if (int rc = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, ws, ws_bytes, stream)) return rc;
+    if (!want_w) return FASTLSTM_OK;
+    return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, ws, ws_bytes, T, B, I, H, dtype, stream);
+}
+
+int fastlstm_gemm_dx_wgrad(const void *d_ifgo, const void *Wx, const void *x, const void *h, void *dx, void *dWx, void *dWh,
+                           void *db, void *ws, size_t ws_bytes, int T, int B, int I, int H, int dtype, void *stream) {
+    const bool want_w = dWx || dWh || db;
+    if (!d_ifgo || !Wx || !x || !h || !ws || (want_w && (!dWx || !dWh || !db))) return FASTLSTM_ERR_NULL;
+    if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
+    if (int rc = check_dims(T, B, I, H)) return rc;
+    if (!aligned16(d_ifgo) || !aligned16(Wx) || !aligned16(x) || !aligned16(h) || !aligned16(dx) || !aligned16(dWx) ||
+        !aligned16(dWh) || !aligned16(ws))
+        return FASTLSTM_ERR_ALIGN;
+    if (ws_bytes < fastlstm_wgrad_workspace_bytes(T, B, I, H, dtype)) return FASTLSTM_ERR_WORKSPACE;
+    return gemm_dx_wgrad_impl(d_ifgo, Wx, x, h, dx, dWx, dWh, db, ws, ws_bytes, T, B, I, H, dtype, stream);
 }
 
 // keep: see LaunchOpts
@@ -1734,9 +1770,8 @@ static int bwd_layer_impl(const void *dout, void *dh, void *dc, const void *ifgo
     if (rc != 3) {   // nothing was launched: recurrence, then dx
         if (int r2 = bwd_persistent_impl(dout, dh, dc, ifgo, cell, d_ifgo, Wh, ws, ws_bytes, T, B, H, dtype, stream))
             return r2;
-        // (the weight-gradient workspace is free until the next call: scratch for a split along K)
-        if (dx)
-            if (int r2 = gemm_dx_impl(d_ifgo, Wx, dx, T, B, I, H, dtype, wgrad_ws, wgrad_ws_bytes, stream)) return r2;
+        return gemm_dx_wgrad_impl(d_ifgo, Wx, x, h, dx, want_w ? dWx : nullptr, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H,
+                                  dtype, stream);
     }
     if (!want_w) return FASTLSTM_OK;
     return fastlstm_gemm_wgrad(d_ifgo, x, h, dWx, dWh, db, wgrad_ws, wgrad_ws_bytes, T, B, I, H, dtype, stream);

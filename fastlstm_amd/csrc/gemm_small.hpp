@@ -1,0 +1,264 @@
+// The reverse pass's three products and the bias gradient for a narrow layer, in ONE pass over d_ifgo:
+//     dx[R][I]  = d_ifgo . Wx                    (K5)
+//     dWx[G][I] = d_ifgo^T . x,  dWh[G][H] = d_ifgo^T . h,  db[G] = column sums of d_ifgo      (K8, K9, db)
+// for G = 4H <= 256, I <= 64, H <= 64 (multiples of 16), 16-bit elements, R = T*B rows.  With rows this short
+// every product is bound by the memory traffic of d_ifgo (a row of d_ifgo is 4 to 8 times as wide as the rows
+// of x, h and dx together), and as four launches d_ifgo is read four times.  Here a workgroup takes blocks of
+// 64 rows: it brings the block of d_ifgo (<= 32 KiB) and the matching blocks of x and h into LDS ONCE and uses
+// it for all of them:
+//     K-major (transposing reads, k = row)  -> dW tiles: wave w owns G tiles 2w, 2w + 1 x all column tiles, the
+//                                              accumulators stay in registers over all blocks of the workgroup;
+//                                              the bias gradient is one more column tile against a fragment of ones
+//     row-major (k = gate column)           -> the block's 64 x I tile of dx against W_x fragments held in registers
+// The partial weight gradients of the workgroups (fp32) are added up in a fixed order by small_bwd_reduce_kernel.
+// Loads are LDS-direct, two stages: the next block is in flight while this one is multiplied.
+#pragma once
+#include "gemm16.hpp"
+
+namespace fastlstm {
+
+struct SmallBwdParams {
+    const void *d_ifgo, *Wx, *x, *h;   // [R][G], [G][I], [R][I], [R][H]
+    void *dx;                          // [R][I], or nullptr: not wanted
+    float *part;                       // [workers][G * (I + H + 1)] fp32: dWx | dWh | db of each worker; nullptr: not wanted
+    int R, G, I, H;
+};
+
+constexpr int kSmallRows = 64;                                   // rows of a block
+constexpr int kSmallDBytes = kSmallRows * 512, kSmallXBytes = kSmallRows * 128;
+constexpr int kSmallStage = kSmallDBytes + 2 * kSmallXBytes;     // d_ifgo | x | h blocks
+constexpr int kSmallLdsBytes = 2 * kSmallStage;
+
+// two transposing reads OFF2 bytes apart (4 k-rows), see lds_rd_tr16x2
+template <int OFF2> __device__ __forceinline__ u32x4 lds_rd_tr16_pair(unsigned addr) {
+    u32x2 lo = {0u, 0u}, hi = {0u, 0u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(OFF2));
+#else
+    (void)addr;
+#endif
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+}
+
+template <int N> __device__ __forceinline__ void small_frags_landed(u32x4 (&f)[N]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+#else
+    (void)f;
+#endif
+}
+
+// Worker `worker` of `n_workers` takes blocks worker, worker + n_workers, ... (counted from the last rows down when
+// `from_end`: the order in which a reverse recurrence produces them).  gate(first_row, rows) is called before a
+// block's loads are requested; a caller that runs next to the producer of d_ifgo waits there.  512 threads,
+// kSmallLdsBytes of LDS at smem; ends behind a workgroup barrier.
+template <typename T, typename Gate>
+__device__ __forceinline__ void small_bwd_pass(const SmallBwdParams &p, unsigned char *smem, const int worker,
+                                               const int n_workers, const bool from_end, Gate gate) {
+    static_assert(sizeof(T) == 2, "16-bit element types");
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int q = lane >> 4, r = lane & 15, a = r >> 2, b = r & 3;
+    const unsigned lds0 = (unsigned)(size_t)((FASTLSTM_LDS_PTR unsigned char *)smem);
+    const bool want_w = p.part != nullptr, want_dx = p.dx != nullptr;
+    const int G = p.G, I = p.I, H = p.H, R = p.R;
+    const int nblk = (R + kSmallRows - 1) / kSmallRows;
+
+    auto rsrc_of = [](const void *base, unsigned bytes) {
+        const unsigned long long ad = reinterpret_cast<unsigned long long>(base);
+        return u32x4{(unsigned)ad, (unsigned)(ad >> 32) & 0xffffu, bytes, 0x00020000u};
+    };
+    const u32x4 rd = rsrc_of(p.d_ifgo, (unsigned)((size_t)R * G * 2)), rx = rsrc_of(p.x, (unsigned)((size_t)R * I * 2));
+    const u32x4 rh = rsrc_of(p.h, (unsigned)((size_t)R * H * 2)), rw = rsrc_of(p.Wx, (unsigned)((size_t)G * I * 2));
+    // XOR swizzles of the 16-byte chunk index of a row, as functions of the row: the rows that the lanes of one
+    // transposing read touch (k, k + 1, k + 2, k + 3 and the same eight rows on) land in different banks.
+    // Rows of 512 bytes (d_ifgo) and rows of 128 bytes (x, h, W_x).
+    auto swzd = [](int k) { return ((k & 3) << 1) ^ (((k >> 3) & 1) << 3); };
+    auto swzx = [](int k) { return (((k >> 1) & 1) | (((k >> 3) & 1) << 1)) << 1; };
+    constexpr unsigned kOut = 0xfffffff0u;   // an offset outside every operand: the load returns zeros
+
+    // ---- global -> LDS.  One wave instruction fills 1 KiB: lane l the 16 bytes at 16 l.  d_ifgo: 32 blocks of two
+    // rows each, wave w fills blocks w, w + 8, w + 16, w + 24 (rows 2w + 16j + l / 32); x, h: 8 blocks of 8 rows, one per wave.
+    const int d_row = 2 * wave + (lane >> 5), d_c = (lane & 31) ^ swzd(d_row);
+    const int x_row = 8 * wave + (lane >> 3), x_c = (lane & 7) ^ swzx(x_row);
+    const bool d_ok = d_c * 8 < G, x_ok = x_c * 8 < I, h_ok = x_c * 8 < H;
+    auto issue = [&](int row0, int stage) {
+        const unsigned sd = lds0 + stage * kSmallStage + wave * kFragBytes;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned off = (unsigned)(((size_t)(row0 + d_row + 16 * j) * G + d_c * 8) * 2);
+            dma_block_asm<false>(rd, sd + j * 8 * kFragBytes, d_ok ? off : kOut, 0u);
+        }
+        const unsigned sx = lds0 + stage * kSmallStage + kSmallDBytes + wave * kFragBytes;
+        if (want_w) {
+            const unsigned offx = (unsigned)(((size_t)(row0 + x_row) * I + x_c * 8) * 2);
+            const unsigned offh = (unsigned)(((size_t)(row0 + x_row) * H + x_c * 8) * 2);
+            dma_block_asm<false>(rx, sx, x_ok ? offx : kOut, 0u);
+            dma_block_asm<false>(rh, sx + kSmallXBytes, h_ok ? offh : kOut, 0u);
+        }
+    };
+    auto loads_landed = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+        __syncthreads();
+    };
+
+    // ---- fragment addresses.  Transposing reads: lane (a, b) of a 16-lane group addresses 4 consecutive columns
+    // (8 bytes) of row k = 8q + a; the second read takes rows k + 4 (same swizzle).
+    const int k0 = q * 8 + a;   // + 32 ks
+    auto tr_d = [&](unsigned stage_base, int gt, int ks) {
+        const int k = ks * 32 + k0;
+        return lds_rd_tr16_pair<4 * 512>(stage_base + (unsigned)(k * 512 + (((gt * 2 + (b >> 1)) ^ swzd(k)) * 16) + (b & 1) * 8));
+    };
+    auto tr_x = [&](unsigned base, int ct, int ks) {
+        const int k = ks * 32 + k0;
+        return lds_rd_tr16_pair<4 * 128>(base + (unsigned)(k * 128 + (((ct * 2 + (b >> 1)) ^ swzx(k)) * 16) + (b & 1) * 8));
+    };
+
+    // ---- W_x as MFMA fragments in registers (dx): through LDS once, in the layout of an x block of 256 rows
+    const int rt = wave & 3, ct0 = 2 * (wave >> 2);   // dx: row tile and first of two column tiles of this wave
+    u32x4 wx[2][8];
+    if (want_dx) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int g = 8 * (wave + 8 * j) + (lane >> 3);
+            const unsigned off = (unsigned)(((size_t)g * I + x_c * 8) * 2);   // (g >= G: outside the operand)
+            dma_block_asm<false>(rw, lds0 + (wave + 8 * j) * kFragBytes, x_ok ? off : kOut, 0u);
+        }
+        loads_landed();
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) wx[c][ks] = tr_x(lds0, ct0 + c, ks);
+            small_frags_landed(wx[c]);
+        }
+        __syncthreads();
+    }
+
+    f32x4 accx[2][4], acch[2][4], accb[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        accb[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) accx[t][c] = acch[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    u32x4 ones;
+    if constexpr (Elem<T>::DT == FASTLSTM_FP16) ones = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+    else ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    const int gt0 = 2 * wave;
+    const bool g_on[2] = {gt0 * 16 < G, (gt0 + 1) * 16 < G};
+    const int nxt = I / 16, nht = H / 16;
+
+    auto row0_of = [&](int blk) { return (from_end ? nblk - 1 - blk : blk) * kSmallRows; };
+    int blk = worker;
+    if (blk < nblk) {
+        gate(row0_of(blk), kSmallRows);
+        issue(row0_of(blk), 0);
+    }
+    for (int n = 0; blk < nblk; blk += n_workers, ++n) {
+        const int stage = n & 1, row0 = row0_of(blk);
+        loads_landed();   // this block is in LDS; every wave is done with the other stage
+        if (blk + n_workers < nblk) {
+            gate(row0_of(blk + n_workers), kSmallRows);
+            issue(row0_of(blk + n_workers), stage ^ 1);
+        }
+        const unsigned sd = lds0 + stage * kSmallStage, sx = sd + kSmallDBytes, sh = sx + kSmallXBytes;
+        if (want_w && g_on[0]) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                u32x4 f[10];   // d^T fragments of the two G tiles, x and h fragments of the column tiles
+                f[0] = tr_d(sd, gt0, ks);
+                f[1] = tr_d(sd, gt0 + 1, ks);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    f[2 + c] = tr_x(sx, c, ks);
+                    f[6 + c] = tr_x(sh, c, ks);
+                }
+                small_frags_landed(f);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if (!g_on[t]) continue;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        if (c < nxt) accx[t][c] = mfma_kstep<T>(f[2 + c], f[t], accx[t][c]);
+                        if (c < nht) acch[t][c] = mfma_kstep<T>(f[6 + c], f[t], acch[t][c]);
+                    }
+                    accb[t] = mfma_kstep<T>(ones, f[t], accb[t]);
+                }
+            }
+        }
+        if (want_dx && ct0 < nxt) {
+            u32x4 f[8];   // rows rt*16 + r of the block, all of G
+            const int row = rt * 16 + r;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) f[ks] = lds_rd128<0>(sd + (unsigned)(row * 512 + (((ks * 4 + q) ^ swzd(row)) * 16)));
+            small_frags_landed(f);
+            f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                if (ks * 32 >= G) continue;
+                acc[0] = mfma_kstep<T>(wx[0][ks], f[ks], acc[0]);
+                acc[1] = mfma_kstep<T>(wx[1][ks], f[ks], acc[1]);
+            }
+            // lane (q, r): dx[row0 + 16 rt + r][16 (ct0 + c) + 4q .. + 3]
+            if (row0 + row < R) {
+                T *dst = static_cast<T *>(p.dx) + (size_t)(row0 + row) * I + ct0 * 16 + 4 * q;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    if (ct0 + c >= nxt) continue;
+                    typedef T tx4 __attribute__((ext_vector_type(4)));
+                    const tx4 v = {Elem<T>::from_f32(acc[c][0]), Elem<T>::from_f32(acc[c][1]), Elem<T>::from_f32(acc[c][2]),
+                                   Elem<T>::from_f32(acc[c][3])};
+                    *reinterpret_cast<tx4 *>(dst + c * 16) = v;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (want_w) {
+        // lane (q, r): dW[16 (gt0 + t) + r][16 c + 4q .. + 3]
+        float *part = p.part + (size_t)worker * G * (I + H + 1);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (!g_on[t]) continue;
+            const int g = (gt0 + t) * 16 + r;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (c < nxt) *reinterpret_cast<f32x4 *>(part + (size_t)g * I + c * 16 + 4 * q) = accx[t][c];
+                if (c < nht) *reinterpret_cast<f32x4 *>(part + (size_t)G * I + (size_t)g * H + c * 16 + 4 * q) = acch[t][c];
+            }
+            if (q == 0) part[(size_t)G * (I + H) + g] = accb[t][0];
+        }
+    }
+}
+
+template <typename T> __global__ __launch_bounds__(512) void small_bwd_kernel(const SmallBwdParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    small_bwd_pass<T>(p, smem, (int)blockIdx.x, (int)gridDim.x, false, [](int, int) {});
+}
+
+// dWx | dWh | db = the sum over the workers' partial sums, in worker order.  A thread block takes 32 groups of four
+// consecutive sums; its 8 x 32 threads add every eighth worker each and then the eight slices in order.
+template <typename T>
+__global__ __launch_bounds__(256) void small_bwd_reduce_kernel(const float *part, T *dWx, T *dWh, T *db, int G, int I, int H,
+                                                               int workers) {
+    __shared__ f32x4 sm[8][32];
+    const int S = G * (I + H + 1), quad = blockIdx.x * 32 + (threadIdx.x & 31), sl = threadIdx.x >> 5;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    if (quad * 4 < S)
+        for (int w = sl; w < workers; w += 8) s += *reinterpret_cast<const f32x4 *>(part + (size_t)w * S + quad * 4);
+    sm[sl][threadIdx.x & 31] = s;
+    __syncthreads();
+    if (sl != 0 || quad * 4 >= S) return;
+#pragma unroll
+    for (int i = 1; i < 8; ++i) s += sm[i][threadIdx.x & 31];
+    const int e = quad * 4;
+    T *out = e < G * I ? dWx + e : e < G * (I + H) ? dWh + (e - G * I) : db + (e - G * (I + H));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = Elem<T>::from_f32(s[i]);
+}
+
+}  // namespace fastlstm

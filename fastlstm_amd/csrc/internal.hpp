@@ -31,6 +31,12 @@ bool wgrad_merged_plan(int dtype, int M, int I, int H, int K, int *splits, int *
 size_t wgrad_merged_workspace(int dtype, int M, int I, int H, int K);
 hipError_t launch_wgrad_merged(int dtype, const void *d_ifgo, const void *x, const void *h, void *dWx, void *dWh, void *db,
                                void *ws, int M, int I, int H, int K, hipStream_t s);
+// K5, K8, K9 and the bias gradient of a narrow 16-bit layer in one pass over d_ifgo (gemm_small.hpp); dx may be null,
+// and so may dWx, dWh, db (all three); ws: small_bwd_workspace bytes
+bool small_bwd_eligible(int dtype, int R, int I, int H);
+size_t small_bwd_workspace(int R, int I, int H);
+hipError_t launch_small_bwd(int dtype, const void *d_ifgo, const void *Wx, const void *x, const void *h, void *dx, void *dWx,
+                            void *dWh, void *db, void *ws, int R, int I, int H, hipStream_t s);
 
 // one function per element type (separate translation units, compiled in parallel)
 #define FASTLSTM_DECL_REC(SUF)                                                                       \

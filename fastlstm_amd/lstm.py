@@ -428,14 +428,12 @@ def _bwd_stack_wavefront(dh, x, acts, weights, d_states, n, need_dx=True):
             _ptr_array([pdg[l]]), _ptr_array([pWh[l]]), p(ws), ws.numel(), r, B, H, code, stream), "fastlstm_bwd_persistent_multi")
     for ws in wss:
         _check_ws(ws, "fastlstm_bwd_persistent_multi")
-    dx0 = None
-    if need_dx:   # (else: no gradient of the stack's input is asked for)
-        dx0 = torch.empty_like(x)
-        _lib.check(lib.fastlstm_gemm_dx(pdg[0], pWx[0], p(dx0), T, B, I, H, code, stream), "fastlstm_gemm_dx")
     res = []
     for l in range(L):
-        xin = x if l == 0 else acts[l - 1][0][1:]
-        db, _, dWx, dWh = Wgrad(d_ifgo[l], xin, acts[l][0])
+        if l == 0:   # (need_dx false: no gradient of the stack's input is asked for)
+            dx0, db, _, dWx, dWh = DxWgrad(d_ifgo[0], Wxc[0], x, acts[0][0], need_dx)
+        else:
+            db, _, dWx, dWh = Wgrad(d_ifgo[l], acts[l - 1][0][1:], acts[l][0])
         res.append((dx0 if l == 0 else douts[l - 1], dhs[l], dcs[l], dWx, db, dWh, db))
     return res
 
@@ -598,6 +596,30 @@ def Wgrad(d_ifgo, x, h):
                                            dWh.data_ptr(), db.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I,
                                            H, code, _stream()), "fastlstm_gemm_wgrad")
     return db, db, dWx, dWh
+
+
+def DxWgrad(d_ifgo, Wx, x, h, need_dx=True):
+    """(d_x | None, dbx, dbh, dWx, dWh): the input gradient d_ifgo . Wx (fastlstm/lstm.py:294) and Wgrad
+    (fastlstm/lstm.py:494-501) in one library call -- one pass over d_ifgo for a narrow layer, the two stages
+    otherwise."""
+    _require_gpu(d_ifgo, x, h, Wx)
+    code = _code(d_ifgo)
+    T, B, G = d_ifgo.shape
+    H, I = G // 4, x.shape[-1]
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        d_ifgo, x, h, Wx = _aligned(d_ifgo.contiguous()), _aligned(x.contiguous()), _aligned(h.contiguous()), _aligned(Wx.contiguous())
+        d_x = torch.empty_like(x) if need_dx else None
+        dWx = torch.empty((G, I), device=x.device, dtype=x.dtype)
+        dWh = torch.empty((G, H), device=x.device, dtype=x.dtype)
+        db = torch.empty((G,), device=x.device, dtype=x.dtype)
+        nbytes = lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        _lib.check(lib.fastlstm_gemm_dx_wgrad(d_ifgo.data_ptr(), Wx.data_ptr(), x.data_ptr(), h.data_ptr(),
+                                              d_x.data_ptr() if need_dx else None, dWx.data_ptr(), dWh.data_ptr(),
+                                              db.data_ptr(), ws.data_ptr(), ws.numel(), T, B, I, H, code, _stream()),
+                   "fastlstm_gemm_dx_wgrad")
+    return d_x, db, db, dWx, dWh
 
 
 def lstm_persistent_bwd(dh, dc_n, dh_n, x, h, cell, ifgo, Wx, Wh, need_dx=True, need_dw=True):
@@ -807,12 +829,7 @@ def lstm_persistent_bwd_pair(dh_a, d_state_a, xa, out_a, cell_a, ifgo_a, Wxa, Wh
         res = []
         for x, out, d_ifgo, Wx, dhn, dcn, want in ((xa, out_a, d_ifgo_a, Wxa, dhn_a, dcn_a, need_dx[0]),
                                                    (xb, out_b, d_ifgo_b, Wxb, dhn_b, dcn_b, need_dx[1])):
-            x = _aligned(x.contiguous())
-            d_x = None
-            if want:
-                d_x = torch.empty_like(x)
-                _lib.check(lib.fastlstm_gemm_dx(p(d_ifgo), p(Wx.contiguous()), p(d_x), T, B, I, H, code, stream), "fastlstm_gemm_dx")
-            dbx, dbh, dWx, dWh = Wgrad(d_ifgo, x, out)
+            d_x, dbx, dbh, dWx, dWh = DxWgrad(d_ifgo, Wx, x, out, want)
             res.append((d_x, dhn, dcn, dWx, dbx, dWh, dbh))
     return res[0], res[1]
 

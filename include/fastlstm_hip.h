@@ -267,6 +267,17 @@ int fastlstm_gemm_wgrad(const void *d_ifgo, const void *x, const void *h, void *
                         int dtype, void *stream);
 size_t fastlstm_wgrad_workspace_bytes(int T, int B, int I, int H, int dtype);
 
+/* K5 and K6-K9 in one call: dx, dWx, dWh, db as fastlstm_gemm_dx_split and fastlstm_gemm_wgrad compute them
+ * (dW to the rounding of a different summation order).  For a narrow layer (fp16 / bf16, H <= 64 and
+ * I <= 64 in multiples of 16, T*B >= 256) the four results come from ONE pass over d_ifgo -- every
+ * product of such a layer is bound by the traffic of d_ifgo, which separate launches read four times;
+ * other shapes run the two stages one after the other.  fastlstm_bwd_layer does the same behind a
+ * recurrence that leaves no CUs idle for these products.  dx may be NULL, and so may dWx, dWh and db (all
+ * three together).  ws: fastlstm_wgrad_workspace_bytes.  Replaces fastlstm/lstm.py:294 and 494-501. */
+int fastlstm_gemm_dx_wgrad(const void *d_ifgo, const void *Wx, const void *x, const void *h, void *dx,
+                           void *dWx, void *dWh, void *db, void *ws, size_t ws_bytes, int T, int B,
+                           int I, int H, int dtype, void *stream);
+
 /* The reverse pass of two stacked layers in one call (suffix 1: upper layer, 0: lower layer; the
  * upper layer's input is out0[1:]).  The same results as fastlstm_bwd_layer for the upper layer
  * followed by fastlstm_bwd_layer for the lower layer with dout = dx1 (dW to the rounding of a

@@ -289,6 +289,55 @@ def test_gemm_stages_vs_matmul(dt, M, N, K):
     within(dbx, d2.sum(0), tol)
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,B,I,H", [(64, 64, 64, 64),      # whole blocks, every tile in use
+                                     (100, 33, 32, 48),     # last block ragged (3300 rows), unused G, I and H tiles
+                                     (30, 20, 16, 16),      # one G tile per wave pair, one column tile
+                                     (256, 256, 64, 64),    # more blocks than workgroups: accumulators carried over blocks
+                                     (9, 20, 64, 64),       # fewer rows than the one-pass form takes
+                                     (40, 40, 80, 64),      # I too wide for it
+                                     (40, 40, 64, 128)])    # H too wide for it
+@pytest.mark.parametrize("want", ["all", "dx", "dw"])
+def test_gemm_dx_wgrad_vs_matmul(dt, T, B, I, H, want):
+    """fastlstm_gemm_dx_wgrad (one pass over d_ifgo for narrow 16-bit layers, the two stages otherwise) against float64
+    matmul, with either half of the results not asked for; what is not asked for stays untouched."""
+    if want != "all" and (T, B) not in ((100, 33), (40, 40)):
+        pytest.skip("the partial forms on one shape per path")
+    lib = _lib.load()
+    code, tol = RM[dt], (FP32_TOL if dt == torch.float32 else HALF_TOL)
+    g = torch.Generator().manual_seed(T * 7 + B * 5 + I * 3 + H)
+    d = (torch.randn(T, B, 4 * H, generator=g) * 0.5).to(dt).cuda()
+    x = torch.randn(T, B, I, generator=g).to(dt).cuda()
+    h = (torch.rand(T + 1, B, H, generator=g) * 2 - 1).to(dt).cuda()
+    Wx = (torch.randn(4 * H, I, generator=g) * 0.2).to(dt).cuda()
+    nb = lib.fastlstm_wgrad_workspace_bytes(T, B, I, H, code)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    mark = 12345.0
+    dx = torch.full((T, B, I), mark, dtype=dt, device="cuda")
+    dWx, dWh, db = (torch.full(sh, mark, dtype=dt, device="cuda") for sh in ((4 * H, I), (4 * H, H), (4 * H,)))
+    w_dx, w_dw = want in ("all", "dx"), want in ("all", "dw")
+    _lib.check(lib.fastlstm_gemm_dx_wgrad(d.data_ptr(), Wx.data_ptr(), x.data_ptr(), h.data_ptr(), dx.data_ptr() if w_dx else None,
+                                          dWx.data_ptr() if w_dw else None, dWh.data_ptr() if w_dw else None,
+                                          db.data_ptr() if w_dw else None, ws.data_ptr(), nb, T, B, I, H, code,
+                                          torch.cuda.current_stream().cuda_stream), "fastlstm_gemm_dx_wgrad")
+    D = d.double().view(T * B, -1)
+    if w_dx:
+        within(dx.view(T * B, I), D @ Wx.double(), tol)
+    else:
+        assert bool((dx == mark).all())
+    if w_dw:
+        within(dWx, D.T @ x.double().view(T * B, I), tol)
+        within(dWh, D.T @ h[:T].double().reshape(T * B, H), tol)
+        within(db, D.sum(0), tol)
+    else:
+        assert all(bool((t == mark).all()) for t in (dWx, dWh, db))
+    if w_dx and w_dw:   # the host wrapper, same call
+        got = L.DxWgrad(d, Wx, x, h)
+        assert got[1] is got[2]
+        for a, b_ in zip((got[0], got[1], got[3], got[4]), (dx, db, dWx, dWh)):
+            assert torch.equal(a, b_)
+
+
 def test_gemm_earlier_form_switch_agrees():
     """fastlstm_set_gemm_baseline(1): the stand-alone products in the tile kernel's earlier form (what bench.py times
     beside the current one) -- same results to rounding, and the switch goes back."""
