@@ -62,19 +62,28 @@ struct FwdParams {
 // memory and LDS (the gates of the step after next in, the results of the last step out).  In one wave the
 // two jobs queue behind each other in a step that is one chain of dependent latencies; side by side they
 // overlap (H = 64, B = 256, fp16: 1.00 -> 0.78 us per step; the reverse kernel 1.10 -> 0.98).
-template <int SPLIT, bool VIO> constexpr int fwd_threads() { return (SPLIT == 2 && VIO) ? 2 * kThreads : kThreads; }
+// CW (that form only): the number of computing waves, 4 or 8, each with MT of the workgroup's CW * MT row tiles;
+// the four tile-moving waves come behind them.  What is left of such a step is mostly the gate arithmetic -- five
+// exponentials and five reciprocals per cell at a quarter of the vector rate, ~290 cycles per cell and lane, 1160 of
+// the step's 1870 cycles on each SIMD -- which more waves do not shorten (the same 4 SIMDs issue it); 8 waves of 2
+// cells per lane overlap the rest of the chain better where no activations are stored (inference), and only there.
+template <int SPLIT, bool VIO, int CW = 4> constexpr int fwd_threads() {
+    return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
+}
 
-template <typename T, int MT, int NTW, int SPLIT, bool VIO, int NKW = 0>
-__global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persistent_kernel(const FwdParams p) {
+template <typename T, int MT, int NTW, int SPLIT, bool VIO, int NKW = 0, int CW = 4>
+__global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_persistent_kernel(const FwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
-    constexpr bool IOW = SPLIT == 2 && VIO;   // tile-moving waves 4..7 beside the computing waves 0..3
+    constexpr bool IOW = SPLIT == 2 && VIO;   // tile-moving waves CW..CW+3 behind the computing waves 0..CW-1
+    static_assert(CW == 4 || (IOW && CW == 8), "8 computing waves: the one-tile form with tile I/O");
+    constexpr int CT = CW * kWave;            // threads of the computing waves
     constexpr bool ACC = (E::DT == FASTLSTM_FP32);
-    constexpr int MTT = SPLIT == 2 ? 4 * MT : MT;    // m-tiles per workgroup
+    constexpr int MTT = SPLIT == 2 ? CW * MT : MT;    // m-tiles per workgroup
     constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;   // n-tiles per workgroup
     constexpr int P = SPLIT == 0 ? 4 : 1;            // partial sums per output tile
     constexpr int TILES = MTT * NT;
-    constexpr int IPT = (TILES + 3) / 4;             // (tile, lane) items per thread
+    constexpr int IPT = (TILES + CW - 1) / CW;       // (tile, lane) items per thread
     constexpr int HT = 4 * MTT, BT = 16 * NT;
     constexpr int CH = 8 / NTW;                      // k-steps fetched per batch of loads
     constexpr bool WREG = NKW > 0;
@@ -82,8 +91,8 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
-    const bool cw = !IOW || tid < kThreads;              // a computing wave
-    const int wave = IOW ? (tid >> 6) & 3 : tid >> 6;    // (a tile-moving wave mirrors the set-up of wave - 4 and never uses it)
+    const bool cw = !IOW || tid < CT;                    // a computing wave
+    const int wave = IOW ? (tid >> 6) & (CW - 1) : tid >> 6;   // (a tile-moving wave mirrors the set-up of a computing wave and never uses it)
     const int q = lane >> 4, n = lane & 15;
     const int KS = p.KS, H = p.H, B = p.B, T_ = p.T;
     const bool keep = p.keep != 0;   // training: gate pre-activations and every cell state are stored
@@ -132,7 +141,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
     // (one hidden tile per workgroup: by the four waves that do nothing else)
     constexpr int IOT = IOW ? kThreads : kThreads - kWave;
     constexpr int GPT = (GPIECES + IOT - 1) / IOT, SPT = (SPIECES + IOT - 1) / IOT;
-    const int io_tid = IOW ? tid - kThreads : tid - kWave;   // < 0: not an I/O thread
+    const int io_tid = IOW ? tid - CT : tid - kWave;   // < 0: not an I/O thread
     constexpr int TILE_BYTES = BT * GROW + 2 * BT * SROW;   // gates tile + h tile + c tile
     static_assert(!VIO || VEC_OK, "tile I/O needs 16-byte gate segments");
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KS * kFragBytes);  // SYNC: 1 set, else 2 (step parity)
@@ -166,7 +175,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
         const int chunks_per_row = KS * 4;  // 16-byte chunks along K
         const int total = MTT * 16 * chunks_per_row;
         const bool vec = (H % E::EPL) == 0;
-        for (int idx = tid; cw && idx < total; idx += kThreads) {
+        for (int idx = tid; cw && idx < total; idx += CT) {
             const int row = idx / chunks_per_row, kc = idx % chunks_per_row;
             const int mt = row >> 4, r = row & 15;
             // row r of an m-tile is gate r % 4 of the tile's unit r / 4.  One hidden tile per workgroup:
@@ -191,7 +200,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO>())) void lstm_fwd_persiste
         }
         if (tid < kWave) reinterpret_cast<u32x4 *>(Wl + zero_off)[tid] = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!SYNC) {
-            for (int idx = tid; cw && idx < 2 * KS * kWave; idx += kThreads)
+            for (int idx = tid; cw && idx < 2 * KS * kWave; idx += CT)
                 reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
         }
     }
