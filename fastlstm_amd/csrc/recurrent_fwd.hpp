@@ -63,10 +63,10 @@ struct FwdParams {
 // two jobs queue behind each other in a step that is one chain of dependent latencies; side by side they
 // overlap (H = 64, B = 256, fp16: 1.00 -> 0.78 us per step; the reverse kernel 1.10 -> 0.98).
 // CW (that form only): the number of computing waves, 4 or 8, each with MT of the workgroup's CW * MT row tiles;
-// the four tile-moving waves come behind them.  What is left of such a step is mostly the gate arithmetic -- five
-// exponentials and five reciprocals per cell at a quarter of the vector rate, ~290 cycles per cell and lane, 1160 of
-// the step's 1870 cycles on each SIMD -- which more waves do not shorten (the same 4 SIMDs issue it); 8 waves of 2
-// cells per lane overlap the rest of the chain better where no activations are stored (inference), and only there.
+// the four tile-moving waves come behind them.  Eight waves of 2 cells per lane instead of four waves of 4 shorten
+// the step only where no activations are stored (inference: 0.755 -> 0.695 us per step at 64 units); with the
+// stores it is 2.5 % slower -- the gate arithmetic is issued by the same 4 SIMDs either way, and the LDS
+// instructions double -- so the host takes CW = 8 for inference alone.
 template <int SPLIT, bool VIO, int CW = 4> constexpr int fwd_threads() {
     return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
 }
