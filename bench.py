@@ -290,12 +290,13 @@ def main():
             elif args.stage == "bwd_layer":
                 rec_bwd_pre()
                 layer_bwd()
-            else:   # gemms: K1, K5, K8 + K9 (+ db) as stand-alone launches
+            else:   # gemms: K1, K5, K8 + K9 (+ db) as stand-alone launches, then K5 + K8 + K9 + db as one call
                 rec_bwd_pre()
                 rec_bwd()            # a real d_ifgo
                 k1()
                 k5()
                 k89()
+                k589()               # K5 + K8 + K9 + db in one call
             cal_dst.copy_(cal_src)
         torch.cuda.synchronize()
         return

@@ -248,8 +248,16 @@ __global__ __launch_bounds__(256) void small_bwd_reduce_kernel(const float *part
     __shared__ f32x4 sm[8][32];
     const int S = G * (I + H + 1), quad = blockIdx.x * 32 + (threadIdx.x & 31), sl = threadIdx.x >> 5;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
-    if (quad * 4 < S)
-        for (int w = sl; w < workers; w += 8) s += *reinterpret_cast<const f32x4 *>(part + (size_t)w * S + quad * 4);
+    if (quad * 4 < S) {
+        const float *src = part + (size_t)sl * S + quad * 4;
+        int w = sl;
+        for (; w + 24 < workers; w += 32, src += (size_t)32 * S) {   // four loads in flight per thread
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + (size_t)8 * S);
+            const f32x4 c = *reinterpret_cast<const f32x4 *>(src + (size_t)16 * S), d = *reinterpret_cast<const f32x4 *>(src + (size_t)24 * S);
+            s += a; s += b; s += c; s += d;
+        }
+        for (; w < workers; w += 8, src += (size_t)8 * S) s += *reinterpret_cast<const f32x4 *>(src);
+    }
     sm[sl][threadIdx.x & 31] = s;
     __syncthreads();
     if (sl != 0 || quad * 4 >= S) return;
