@@ -959,6 +959,12 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
 // split along K so that it fills the device; without one it is a single pass.
 static int gemm_dx_impl(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H, int dtype,
                         void *scratch, size_t scratch_bytes, void *stream) {
+    // a narrow layer: the streaming pass of gemm_small.hpp with dx alone (T*B = 262144, I = H = 64: 0.057 -> 0.03 ms)
+    if (!gemm_baseline() && small_bwd_eligible(dtype, T * B, I, H))
+        return launch_small_bwd(dtype, d_ifgo, Wx, nullptr, nullptr, dx, nullptr, nullptr, nullptr, nullptr, T * B, I, H,
+                                static_cast<hipStream_t>(stream)) == hipSuccess
+                   ? FASTLSTM_OK
+                   : FASTLSTM_ERR_HIP;
     GemmParams p{};
     p.A = d_ifgo; p.B = Wx; p.C = dx;
     p.M = T * B; p.N = I; p.K = 4 * H;

@@ -247,7 +247,8 @@ int fastlstm_bwd_layer(const void *dout, void *dh, void *dc, const void *ifgo, c
                        void *wgrad_ws, size_t wgrad_ws_bytes, int T, int B, int I, int H, int dtype,
                        void *stream);
 
-/* K5 -- dx[T*B,I] = d_ifgo[T*B,4H] . Wx[4H,I].   Replaces fastlstm/lstm.py:294. */
+/* K5 -- dx[T*B,I] = d_ifgo[T*B,4H] . Wx[4H,I].   Replaces fastlstm/lstm.py:294.  (A narrow 16-bit layer, see
+ * fastlstm_gemm_dx_wgrad: the streaming pass of that call with dx alone.) */
 int fastlstm_gemm_dx(const void *d_ifgo, const void *Wx, void *dx, int T, int B, int I, int H,
                      int dtype, void *stream);
 

@@ -323,6 +323,10 @@ def test_gemm_dx_wgrad_vs_matmul(dt, T, B, I, H, want):
     D = d.double().view(T * B, -1)
     if w_dx:
         within(dx.view(T * B, I), D @ Wx.double(), tol)
+        dx2 = torch.full_like(dx, mark)   # K5 by its own entry point (a narrow layer: the same streaming pass, dx alone)
+        _lib.check(lib.fastlstm_gemm_dx(d.data_ptr(), Wx.data_ptr(), dx2.data_ptr(), T, B, I, H, code,
+                                        torch.cuda.current_stream().cuda_stream), "fastlstm_gemm_dx")
+        within(dx2.view(T * B, I), D @ Wx.double(), tol)
     else:
         assert bool((dx == mark).all())
     if w_dw:
