@@ -922,6 +922,13 @@ static int gates_stay_cached(size_t rows, int H, int dtype) {
 static int gemm_ifgo_rows(const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, size_t row0,
                           int rows, int I, int H, int dtype, hipStream_t stream) {
     const size_t s = elem_bytes(dtype);
+    // a narrow layer whose I the tile kernel does not take (no whole k-tile of 64): the streaming form of gemm_small.hpp
+    // (T*B = 262144, I = H = 32: 0.062 ms on the generic kernel, 0.021 here; at I = 64 the tile kernel is the faster one)
+    if (!gemm_baseline() && I % 64 != 0 && small_bwd_eligible(dtype, rows, I, H))
+        return launch_small_k1(dtype, static_cast<const unsigned char *>(x) + row0 * I * s, Wx, bx, bh,
+                               static_cast<unsigned char *>(ifgo) + row0 * 4 * H * s, rows, I, H, stream) == hipSuccess
+                   ? FASTLSTM_OK
+                   : FASTLSTM_ERR_HIP;
     GemmParams p{};
     p.A = static_cast<const unsigned char *>(x) + row0 * I * s;
     p.B = Wx;
@@ -942,6 +949,10 @@ int fastlstm_gemm_ifgo(const void *x, const void *Wx, const void *bx, const void
     if (!dtype_ok(dtype)) return FASTLSTM_ERR_DTYPE;
     if (int rc = check_dims(T, B, I, H)) return rc;
     if (!aligned16(x) || !aligned16(Wx) || !aligned16(ifgo)) return FASTLSTM_ERR_ALIGN;
+    if (!gemm_baseline() && I % 64 != 0 && small_bwd_eligible(dtype, T * B, I, H))   // (see gemm_ifgo_rows)
+        return launch_small_k1(dtype, x, Wx, bx, bh, ifgo, T * B, I, H, static_cast<hipStream_t>(stream)) == hipSuccess
+                   ? FASTLSTM_OK
+                   : FASTLSTM_ERR_HIP;
     GemmParams p{};
     p.A = x; p.B = Wx; p.C = ifgo; p.bias0 = bx; p.bias1 = bh;
     p.M = T * B; p.N = 4 * H; p.K = I;

@@ -49,4 +49,25 @@ hipError_t launch_small_bwd(int dtype, const void *d_ifgo, const void *Wx, const
     return dtype == FASTLSTM_FP16 ? launch_small_bwd_t<_Float16>(p, dWx, dWh, db, s) : launch_small_bwd_t<__bf16>(p, dWx, dWh, db, s);
 }
 
+// K1 of a narrow layer (small_k1_kernel): rows [0, R) of x[R][I] -> ifgo[R][4H]; the shapes of small_bwd_eligible
+hipError_t launch_small_k1(int dtype, const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int R, int I,
+                           int H, hipStream_t s) {
+    SmallK1Params p{};
+    p.x = x; p.Wx = Wx; p.bx = bx; p.bh = bh; p.ifgo = ifgo;
+    p.R = R; p.G = 4 * H; p.I = I;
+    const int grid = std::min(cdiv(R, kSmallRows), 2 * kNumXcd * 32);   // two workgroups per CU (68 KiB of LDS each)
+    auto launch = [&](auto kern) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   kSmallK1LdsBytes))
+                return e;
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kSmallK1LdsBytes, s, p);
+        return hipGetLastError();
+    };
+    return dtype == FASTLSTM_FP16 ? launch(small_k1_kernel<_Float16>) : launch(small_k1_kernel<__bf16>);
+}
+
 }  // namespace fastlstm

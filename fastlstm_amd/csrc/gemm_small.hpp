@@ -269,4 +269,125 @@ __global__ __launch_bounds__(256) void small_bwd_reduce_kernel(const float *part
     for (int i = 0; i < 4; ++i) out[i] = Elem<T>::from_f32(s[i]);
 }
 
+// K1 of a narrow layer: ifgo[R][G] = x[R][I] . Wx[G][I]^T + bx + bh for G = 4H <= 256, I <= 64 (multiples of 16),
+// 16-bit elements -- a product that writes four to sixteen times what it reads and is bound by that write stream
+// (~3 TB/s on this device).  The host takes it where I is no multiple of 64, which the tile kernel needs; where both
+// apply the tile kernel is 10-30 % faster.
+// Both operands are K-contiguous, so the MFMA fragments are 16-byte global loads (no LDS on the way in): a wave keeps
+// the W_x fragments of its two G tiles and the bias sums in registers for the whole launch and streams blocks of 64
+// rows of x, the next block's fragments in flight while this one is multiplied.  The results are the bits of the
+// tile kernel (gemm16_kernel: the same two k-steps in the same order, bias added in fp32 before rounding); they
+// leave through one of two LDS tiles as whole rows, 16 bytes per lane, with ordinary stores -- the time loop reads
+// them next and finds them in the memory-side cache.
+struct SmallK1Params {
+    const void *x, *Wx, *bx, *bh;   // [R][I], [G][I], [G], [G]
+    void *ifgo;                     // [R][G]
+    int R, G, I;
+};
+constexpr int kSmallK1Row = 512 + 32;                      // bytes of a staged row (bank spread)
+constexpr int kSmallK1LdsBytes = 2 * kSmallRows * kSmallK1Row;
+
+template <typename T> __global__ __launch_bounds__(512) void small_k1_kernel(const SmallK1Params p) {
+    static_assert(sizeof(T) == 2, "16-bit element types");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q = lane >> 4, r = lane & 15;
+    const int G = p.G, I = p.I, R = p.R;
+    const int nblk = (R + kSmallRows - 1) / kSmallRows;
+    const T *Wx = static_cast<const T *>(p.Wx), *bx = static_cast<const T *>(p.bx), *bh = static_cast<const T *>(p.bh);
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    // x and ifgo through buffer descriptors: a row past R reads as zeros and its stores are dropped, so every
+    // load and store below is unconditional and the compiler's counted waits leave the stores of a block in flight
+    // while the next block's fragments are awaited
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.x), 0, (unsigned)((size_t)R * I * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(p.ifgo, 0, (unsigned)((size_t)R * G * 2), 0x00020000);
+    constexpr unsigned kOut = 0xfffffff0u;
+
+    // this wave's two G tiles: fragments of W_x (lane (q, r): row 16 gt + r, k = 32 ks + 8q ..) and the bias sums of
+    // the lane's four output columns 16 gt + 4q ..
+    u32x4 wf[2][2];
+    float bv[2][4];
+    bool g_on[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int gt = 2 * wave + t, g = gt * 16 + r;
+        g_on[t] = gt * 16 < G;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int k = ks * 32 + 8 * q;
+            wf[t][ks] = (g < G && k < I) ? *reinterpret_cast<const u32x4 *>(Wx + (size_t)g * I + k) : zero;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int gc = gt * 16 + 4 * q + e;
+            bv[t][e] = gc < G ? Elem<T>::to_f32(bx[gc]) + Elem<T>::to_f32(bh[gc]) : 0.f;
+        }
+    }
+    // fragments of a block of x: lane (q, r): row 16 rt + r of the block, k = 32 ks + 8q .. (k past I: zeros)
+    unsigned xoff[4][2];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int k = ks * 32 + 8 * q;
+            xoff[rt][ks] = k < I ? (unsigned)(((rt * 16 + r) * I + k) * 2) : kOut;
+        }
+    u32x4 xf[4][2];
+    auto load_x = [&](int blk) {
+        const unsigned base = (unsigned)((size_t)blk * kSmallRows * I * 2);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+                xf[rt][ks] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[rt][ks] == kOut ? kOut : xoff[rt][ks] + base, 0, 0));
+    };
+    // stores: 16-byte chunk c = tid + 512 j of the staged block -> row c / (G / 8), columns 8 (c % (G / 8)) ..
+    const int cpr = G / 8;
+    unsigned so_lds[4], so_glb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = tid + 512 * j, row = c / cpr, cc = c - row * cpr;
+        const bool ok = c < kSmallRows * cpr;
+        so_lds[j] = ok ? (unsigned)(row * kSmallK1Row + cc * 16) : 0u;
+        so_glb[j] = ok ? (unsigned)((row * G + cc * 8) * 2) : kOut;
+    }
+    int blk = blockIdx.x;
+    if (blk < nblk) load_x(blk);
+    // (four stores outside the operand, which the hardware drops: the loop is then entered with the same sequence of
+    // vector-memory operations in flight as it is re-entered with -- 8 loads, 4 stores -- and the compiler's counted
+    // wait for the fragments leaves the 4 stores of the last block in flight instead of draining everything)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) __builtin_amdgcn_raw_buffer_store_b128(zero, ro, kOut, 0, 0);
+    for (int n = 0; blk < nblk; blk += gridDim.x, ++n) {
+        unsigned char *st = smem + (n & 1) * kSmallRows * kSmallK1Row;
+        f32x4 acc[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                acc[t][rt] = mfma_kstep<T>(wf[t][0], xf[rt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                acc[t][rt] = mfma_kstep<T>(wf[t][1], xf[rt][1], acc[t][rt]);
+            }
+        load_x(blk + gridDim.x);   // in flight behind the staging and the stores (past the last block: zeros, unused)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (!g_on[t]) continue;
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                // lane (q, r): ifgo[row 16 rt + r][16 gt + 4q .. + 3]
+                typedef T tx4 __attribute__((ext_vector_type(4)));
+                const tx4 v = {Elem<T>::from_f32(acc[t][rt][0] + bv[t][0]), Elem<T>::from_f32(acc[t][rt][1] + bv[t][1]),
+                               Elem<T>::from_f32(acc[t][rt][2] + bv[t][2]), Elem<T>::from_f32(acc[t][rt][3] + bv[t][3])};
+                *reinterpret_cast<tx4 *>(st + (rt * 16 + r) * kSmallK1Row + ((2 * wave + t) * 16 + 4 * q) * 2) = v;
+            }
+        }
+        __syncthreads();   // the block is staged (and every wave is done reading the other tile: two barriers ago)
+        const unsigned base = (unsigned)((size_t)blk * kSmallRows * G * 2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(st + so_lds[j]), ro,
+                                                   so_glb[j] == kOut ? kOut : so_glb[j] + base, 0, 0);
+    }
+}
+
 }  // namespace fastlstm

@@ -38,6 +38,9 @@ size_t small_bwd_workspace(int R, int I, int H);
 hipError_t launch_small_bwd(int dtype, const void *d_ifgo, const void *Wx, const void *x, const void *h, void *dx, void *dWx,
                             void *dWh, void *db, void *ws, int R, int I, int H, hipStream_t s);
 
+hipError_t launch_small_k1(int dtype, const void *x, const void *Wx, const void *bx, const void *bh, void *ifgo, int R, int I,
+                           int H, hipStream_t s);
+
 // one function per element type (separate translation units, compiled in parallel)
 #define FASTLSTM_DECL_REC(SUF)                                                                       \
     hipError_t launch_fwd_##SUF(const FwdParams &p, int ht, int bt, int split, int grid, int lds,   \

@@ -321,6 +321,12 @@ def test_gemm_dx_wgrad_vs_matmul(dt, T, B, I, H, want):
                                           db.data_ptr() if w_dw else None, ws.data_ptr(), nb, T, B, I, H, code,
                                           torch.cuda.current_stream().cuda_stream), "fastlstm_gemm_dx_wgrad")
     D = d.double().view(T * B, -1)
+    if want == "all":   # K1 on the same shape (I no multiple of 64 and a narrow layer: the streaming form)
+        bx, bh = torch.randn(4 * H, generator=g).to(dt).cuda(), torch.randn(4 * H, generator=g).to(dt).cuda()
+        ifgo = torch.full((T, B, 4 * H), mark, dtype=dt, device="cuda")
+        _lib.check(lib.fastlstm_gemm_ifgo(x.data_ptr(), Wx.data_ptr(), bx.data_ptr(), bh.data_ptr(), ifgo.data_ptr(), T, B, I, H,
+                                          code, torch.cuda.current_stream().cuda_stream), "fastlstm_gemm_ifgo")
+        within(ifgo.view(T * B, -1), x.double().view(T * B, I) @ Wx.double().T + bx.double() + bh.double(), tol)
     if w_dx:
         within(dx.view(T * B, I), D @ Wx.double(), tol)
         dx2 = torch.full_like(dx, mark)   # K5 by its own entry point (a narrow layer: the same streaming pass, dx alone)
