@@ -339,11 +339,118 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
     };
     auto prefetch = [&](int t, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
+        if constexpr (IOW) return;   // (the tile-moving waves have a loop of their own, below)
         if (t < T_) {
             if constexpr (VIO) fetch_tile(t, gpre[u]);
             else fetch_pre(t, pre[u]);
         }
     };
+    // ---- the tile-moving waves of the one-tile form: their own time loop --------------------------------
+    // Every vector-memory instruction of this loop is unconditional -- a piece that does not exist, a row past
+    // the batch, a timestep past the end, a store that is not wanted get an offset outside the buffer
+    // descriptor (loads return zeros, stores are dropped) -- and four steps are unrolled without a branch
+    // between them.  The compiler can then count: its s_waitcnt vmcnt(N) in front of "tile t + 1 into LDS"
+    // names exactly the loads of that tile and leaves the 12 younger operations -- the stores of the last two
+    // steps, the tiles of steps t + 2 and t + 3 -- in flight.  With conditional stores and loads in between
+    // (and the roles of the waves decided by a branch around them) it could only wait for everything: every
+    // step then paid the round trip of the loads it had just requested four steps ahead, and of its stores
+    // (T = 1024, B = 256, H = 64: 0.78 -> FIXME us per step).
+    if constexpr (IOW) {
+        if (!cw) {
+            constexpr unsigned kOut = 0xfffffff0u;
+            constexpr int EPC = 16 / E::BYTES;
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            unsigned gv[GPT], gvs[GPT], sv[SPT];   // byte offsets inside ifgo[t] (loads / stores) and out[t]; kOut: none
+            int gl[GPT], sl[SPT];                  // byte offsets inside the LDS tiles; -1: no such piece
+#pragma unroll
+            for (int i = 0; i < GPT; ++i) {
+                const int pc = io_tid + IOT * i;
+                const int row = pc / (4 * PPSEG), rem = pc % (4 * PPSEG), seg = rem / PPSEG, k = rem % PPSEG;
+                const bool ok = pc < GPIECES && b0 + row < B;
+                gv[i] = ok ? (unsigned)((((size_t)(b0 + row) * 4 + seg) * H + u0 + k * EPC) * E::BYTES) : kOut;
+                gvs[i] = keep ? gv[i] : kOut;
+                gl[i] = ok ? row * GROW + seg * GSEG + k * 16 : -1;
+            }
+#pragma unroll
+            for (int i = 0; i < SPT; ++i) {
+                const int pc = io_tid + IOT * i;
+                const int row = pc / PPSEG, k = pc % PPSEG;
+                const bool ok = pc < SPIECES && b0 + row < B;
+                sv[i] = ok ? (unsigned)(((size_t)(b0 + row) * H + u0 + k * EPC) * E::BYTES) : kOut;
+                sl[i] = ok ? row * SROW + k * 16 : -1;
+            }
+            const unsigned g_bytes = (unsigned)(B4H * E::BYTES), s_bytes = (unsigned)(BH * E::BYTES);
+            auto rsrc_g = [&](int t) {   // ifgo[t]; past the last timestep: an empty buffer
+                return __builtin_amdgcn_make_buffer_rsrc(ifgo + (size_t)min(t, T_ - 1) * B4H, 0, t < T_ ? g_bytes : 0u, 0x00020000);
+            };
+            u32x4 ring[PD][GPT];
+            auto load_tile = [&](int t, auto uc) __attribute__((always_inline)) {
+                constexpr int u = decltype(uc)::value;
+                const __amdgpu_buffer_rsrc_t rg = rsrc_g(t);
+#pragma unroll
+                for (int i = 0; i < GPT; ++i) ring[u][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rg, gv[i], 0, 0));
+            };
+            auto dropped_stores = [&](unsigned group) __attribute__((always_inline)) {   // as many as a step issues
+                const __amdgpu_buffer_rsrc_t rg = rsrc_g(0);   // (each at an offset of its own, or the compiler keeps one of them)
+#pragma unroll
+                for (int i = 0; i < GPT + 2 * SPT; ++i)
+                    __builtin_amdgcn_raw_buffer_store_b128(zero, rg, kOut - 16u * (group * (GPT + 2 * SPT) + i), 0, 0);
+            };
+            auto to_lds = [&](auto uc, unsigned char *gt) __attribute__((always_inline)) {
+                constexpr int u = decltype(uc)::value;
+#pragma unroll
+                for (int i = 0; i < GPT; ++i)
+                    if (gl[i] >= 0) *reinterpret_cast<u32x4 *>(gt + gl[i]) = ring[u][i];
+            };
+            auto to_global = [&](int t, const unsigned char *gt) __attribute__((always_inline)) {
+                const unsigned char *sth = gt + BT * GROW, *stc = sth + BT * SROW;
+                const __amdgpu_buffer_rsrc_t rg = rsrc_g(t);
+                const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(out + (size_t)(t + 1) * BH, 0, s_bytes, 0x00020000);
+                const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(cell + (size_t)(t + 1) * BH, 0, s_bytes, 0x00020000);
+                const bool cell_wanted = keep || t + 1 == T_;
+#pragma unroll
+                for (int i = 0; i < GPT; ++i)
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(gt + max(gl[i], 0)), rg, gvs[i], 0, 0);
+#pragma unroll
+                for (int i = 0; i < SPT; ++i) {
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(sth + max(sl[i], 0)), rh, sv[i], 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(stc + max(sl[i], 0)), rc,
+                                                           cell_wanted ? sv[i] : kOut, 0, 0);
+                }
+            };
+            // step t: tile t + 1 (ring entry (u + 1) % PD) into the other tile set before the barrier, this step's
+            // results out of this one behind it, tile t + PD requested into the entry that tile t left
+            auto io_step = [&](int t, auto uc) __attribute__((always_inline)) {
+                constexpr int u = decltype(uc)::value;
+                to_lds(std::integral_constant<int, (u + 1) % PD>{}, tiles + ((t + 1) & 1) * TILE_BYTES);
+                __syncthreads();
+                to_global(t, tiles + (t & 1) * TILE_BYTES);
+                load_tile(t + PD, uc);
+            };
+            static_assert(PD == 4, "four steps per pass of the loop");
+            // (the loop is entered with what every later pass finds in flight: between the tiles, as many stores as a step issues)
+            load_tile(0, std::integral_constant<int, 0>{});
+            dropped_stores(0);
+            load_tile(1, std::integral_constant<int, 1>{});
+            dropped_stores(1);
+            load_tile(2, std::integral_constant<int, 2>{});
+            dropped_stores(2);
+            load_tile(3, std::integral_constant<int, 3>{});
+            to_lds(std::integral_constant<int, 0>{}, tiles);
+            __syncthreads();
+            int t0 = 0;
+            for (; t0 + PD <= T_; t0 += PD) {
+                io_step(t0, std::integral_constant<int, 0>{});
+                io_step(t0 + 1, std::integral_constant<int, 1>{});
+                io_step(t0 + 2, std::integral_constant<int, 2>{});
+                io_step(t0 + 3, std::integral_constant<int, 3>{});
+            }
+            if (t0 < T_) io_step(t0, std::integral_constant<int, 0>{});
+            if (t0 + 1 < T_) io_step(t0 + 1, std::integral_constant<int, 1>{});
+            if (t0 + 2 < T_) io_step(t0 + 2, std::integral_constant<int, 2>{});
+            return;
+        }
+    }
     prefetch(0, std::integral_constant<int, 0>{});
     prefetch(1, std::integral_constant<int, 1>{});
     if constexpr (PD > 2) {
@@ -352,10 +459,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
     }
 
     int slot_r = 0;  // ring slot that holds h_{t-1}
-    if constexpr (SPLIT == 2 && VIO) {   // the gates tile of step 0 (every later one is moved a step ahead)
-        tile_to_lds(gpre[0], tiles);
-        __syncthreads();
-    }
+    if constexpr (IOW) __syncthreads();   // the gates tile of step 0 is in LDS (every later one is moved a step ahead)
     // One timestep; u = t % PD selects the prefetch ring entry at compile time.
     auto step = [&](const int t, auto uc) __attribute__((always_inline)) {
         constexpr int u = decltype(uc)::value;
@@ -452,13 +556,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
             }   // computing waves
             // tile-moving waves (with tile I/O; without it nobody): the next step's gates into the other
             // tile set before the barrier, this step's results out of this one behind it
-            if constexpr (VIO) {
-                if (t + 1 < T_) tile_to_lds(gpre[(u + 1) % PD], tiles + ((t + 1) & 1) * TILE_BYTES);
-                __syncthreads();
-                tiles_to_global(t, gt);
-            } else {
-                __syncthreads();
-            }
+            __syncthreads();   // (with tile I/O: the tile-moving waves meet it in their own loop)
             prefetch(t + PD, uc);
             slot_r = slot_w;
             return;
