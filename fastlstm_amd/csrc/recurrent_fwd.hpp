@@ -354,7 +354,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
     // steps, the tiles of steps t + 2 and t + 3 -- in flight.  With conditional stores and loads in between
     // (and the roles of the waves decided by a branch around them) it could only wait for everything: every
     // step then paid the round trip of the loads it had just requested four steps ahead, and of its stores
-    // (T = 1024, B = 256, H = 64: 0.78 -> FIXME us per step).
+    // (T = 1024, B = 256, H = 64: 0.78 -> 0.63 us per step).
     if constexpr (IOW) {
         if (!cw) {
             constexpr unsigned kOut = 0xfffffff0u;
