@@ -55,26 +55,35 @@ struct BwdParams {
 // SPLIT 2: barrier-free small-H form, wave w owns unit tile w (up to 64 units), one n-tile.
 // VIO: the workgroup's tiles of ifgo[t], cell[t], dout[t] and d_ifgo[t] move between global memory
 // and LDS in 16-byte pieces (waves 1..3) instead of element by element; see the forward kernel.
-// SPLIT 2 with tile I/O runs 8 waves, as the forward kernel does: waves 0..3 compute, waves 4..7 move the tiles.
-template <int SPLIT, bool VIO> constexpr int bwd_threads() { return (SPLIT == 2 && VIO) ? 2 * kThreads : kThreads; }
+// SPLIT 2 with tile I/O runs CW computing waves and four that move the tiles, as the forward kernel does.  CW = 8:
+// the waves 2w and 2w + 1 both multiply unit tile w (8 MFMAs each, on different SIMDs) and each takes two of the
+// four units that a lane's accumulator holds: half the gate arithmetic per wave, two waves per SIMD that overlap
+// each other's latencies.
+template <int SPLIT, bool VIO, int CW = 4> constexpr int bwd_threads() {
+    return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
+}
 
-template <typename T, int NTW, int SPLIT, bool VIO>
-__global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persistent_kernel(const BwdParams p) {
+template <typename T, int NTW, int SPLIT, bool VIO, int CW = 4>
+__global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_persistent_kernel(const BwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
-    constexpr bool IOW = SPLIT == 2 && VIO;   // tile-moving waves 4..7 beside the computing waves 0..3
+    constexpr bool IOW = SPLIT == 2 && VIO;   // tile-moving waves CW..CW+3 behind the computing waves 0..CW-1
+    static_assert(CW == 4 || (IOW && CW == 8), "8 computing waves: the one-tile form with tile I/O");
+    constexpr int CT = CW * kWave;            // threads of the computing waves
+    constexpr int UPL = 16 / CW;              // SPLIT 2: units of a lane (of the four its accumulator holds)
     constexpr bool ACC = (E::DT == FASTLSTM_FP32);
     constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;
     constexpr int P = SPLIT == 0 ? 4 : 1;
     constexpr int MTB = SPLIT == 2 ? 4 : 1;          // unit tiles (16 rows each) per workgroup
-    constexpr int IPT = SPLIT == 2 ? 4 : NT;         // (unit, batch row) items per thread, upper bound
+    constexpr int IPT = SPLIT == 2 ? UPL : NT;       // (unit, batch row) items per thread, upper bound
     constexpr int BT = 16 * NT;
     constexpr int CH = 16 / NTW;                     // k-steps fetched per batch of loads (2 batches in flight)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
-    const bool cw = !IOW || tid < kThreads;              // a computing wave
-    const int wave = IOW ? (tid >> 6) & 3 : tid >> 6;    // (a tile-moving wave mirrors the set-up of wave - 4 and never uses it)
+    const bool cw = !IOW || tid < CT;                    // a computing wave
+    const int wave = IOW ? (tid >> 6) & (CW - 1) : tid >> 6;   // (a tile-moving wave mirrors the set-up of a computing wave and never uses it)
+    const int ut = CW == 8 ? wave >> 1 : wave, mh = CW == 8 ? (wave & 1) : 0;   // SPLIT 2: the wave's unit tile, and which units of it
     const int KSB = p.KSB, H = p.H, B = p.B, T_ = p.T;
     const int HT = SYNC ? p.ht : 16 * MTB;           // unit slots per workgroup
     const int RPT = SYNC ? p.ht : 16;                // weight rows stored per unit tile
@@ -120,7 +129,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
     const int PPSEG = GSEG / 16;            // 16-byte pieces per segment (>= 1 when VIO)
     const int TILE_BYTES = BT * GROW + 2 * BT * SROW;
     unsigned char *tiles = xl + (SYNC ? 0 : 2 * (size_t)KSB * kFragBytes);   // SYNC: 1 set, else 2 (step parity)
-    const int io_tid = IOW ? tid - kThreads : tid - kWave;   // < 0: not an I/O thread
+    const int io_tid = IOW ? tid - CT : tid - kWave;   // < 0: not an I/O thread
 
     const T *dout = static_cast<const T *>(pick(p.dout, p.dout_x[0], p.dout_x[1], p.dout_x[2]));
     const T *ifgo = static_cast<const T *>(pick(p.ifgo, p.ifgo_x[0], p.ifgo_x[1], p.ifgo_x[2]));
@@ -134,7 +143,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
     {
         const int Kpad = KSB * E::KSTEP;
         const int total = Kpad * HT;
-        for (int idx = tid; cw && idx < total; idx += kThreads) {
+        for (int idx = tid; cw && idx < total; idx += CT) {
             const int ul = idx % HT, k = idx / HT;
             const int uk = k >> 2, gate = k & 3;
             T v = E::from_f32(0.f);
@@ -148,7 +157,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
         }
         if (tid < kWave) reinterpret_cast<u32x4 *>(Wl + zero_off)[tid] = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!SYNC) {
-            for (int idx = tid; cw && idx < 2 * KSB * kWave; idx += kThreads)
+            for (int idx = tid; cw && idx < 2 * KSB * kWave; idx += CT)
                 reinterpret_cast<u32x4 *>(xl)[idx] = u32x4{0u, 0u, 0u, 0u};
         }
     }
@@ -161,8 +170,8 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
         const int q_ = lane >> 4, r_ = lane & 15;
 #pragma unroll
         for (int ks = 0; ks < KSB2; ++ks) {
-            const bool ok = ks < KSB && wave < n_utiles;
-            const unsigned char *wp = ok ? Wl + ((((size_t)wave * KSB + ks) * 4 + q_) * RPT + (r_ % RPT)) * 16
+            const bool ok = ks < KSB && ut < n_utiles;
+            const unsigned char *wp = ok ? Wl + ((((size_t)ut * KSB + ks) * 4 + q_) * RPT + (r_ % RPT)) * 16
                                          : Wl + zero_off + lane * 16;
             wb2[ks] = *reinterpret_cast<const u32x4 *>(wp);
         }
@@ -177,11 +186,11 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
     const size_t BH = (size_t)B * H, B4H = (size_t)B * 4 * H;
 #pragma unroll
     for (int m = 0; m < IPT; ++m) {
-        // SPLIT 2: the item is element m of the lane's own accumulator -- unit 4 * (lane / 16) + m of the
-        // wave's unit tile, batch row lane % 16 -- so the product of a step lands where it is used
+        // SPLIT 2: the item is element mh * UPL + m of the lane's own accumulator -- that unit of 4 * (lane / 16) .. + 3
+        // of the wave's unit tile, batch row lane % 16 -- so the product of a step lands where it is used
         const int it = tid + kThreads * m;
         const int n = SPLIT == 2 ? (lane & 15) : (it & 15), rest = it >> 4;
-        const int ul = SPLIT == 2 ? wave * 16 + (lane >> 4) * 4 + m : rest % HT, nt = SPLIT == 2 ? 0 : rest / HT;
+        const int ul = SPLIT == 2 ? ut * 16 + (lane >> 4) * 4 + mh * UPL + m : rest % HT, nt = SPLIT == 2 ? 0 : rest / HT;
         const int unit = u0 + ul, b = b0 + nt * 16 + n;
         valid[m] = nt < NT && unit < H && b < B;
         // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
@@ -374,9 +383,9 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
     }
 
     int slot = 0;  // ring slot of this step's d_ifgo
-    // One hidden tile per workgroup: the lane's four units of the current step's tile rows (4 gates,
+    // One hidden tile per workgroup: the lane's UPL units of the current step's tile rows (4 gates,
     // c_{t-1}, dout), read a step ahead
-    using NxV = typename VecBytes<4 * E::BYTES>::type;
+    using NxV = typename VecBytes<(SPLIT == 2 ? UPL : 4) * E::BYTES>::type;
     NxV nx[6];
     auto load_items = [&](const unsigned char *gt_) __attribute__((always_inline)) {
 #pragma unroll
@@ -404,18 +413,17 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
             // slots of the exchange copy, and the product comes back in the lane's own accumulator (nothing
             // is reduced).  One workgroup barrier per step: behind it the exchange copy, the d_ifgo tile
             // and the next step's input tiles are all in LDS.
-            using V = typename VecBytes<4 * E::BYTES>::type;
-            constexpr int un_ = (u + 1) % PD;
+            using V = typename VecBytes<UPL * E::BYTES>::type;
             if (cw) {
-            T xg[4][4], xc[4], xd[4], st_d[4][4];
+            T xg[4][UPL], xc[UPL], xd[UPL], st_d[UPL][4];
             if constexpr (VIO) {   // read behind the previous step's barrier (or in the prologue)
 #pragma unroll
-                for (int gg = 0; gg < 4; ++gg) __builtin_memcpy(xg[gg], &nx[gg], 4 * E::BYTES);
-                __builtin_memcpy(xc, &nx[4], 4 * E::BYTES);
-                __builtin_memcpy(xd, &nx[5], 4 * E::BYTES);
+                for (int gg = 0; gg < 4; ++gg) __builtin_memcpy(xg[gg], &nx[gg], UPL * E::BYTES);
+                __builtin_memcpy(xc, &nx[4], UPL * E::BYTES);
+                __builtin_memcpy(xd, &nx[5], UPL * E::BYTES);
             } else {
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
+                for (int m = 0; m < UPL; ++m) {
 #pragma unroll
                     for (int gg = 0; gg < 4; ++gg) xg[gg][m] = pre[u][m][gg];
                     xc[m] = c0r[u][m];
@@ -423,7 +431,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
                 }
             }
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
+            for (int m = 0; m < UPL; ++m) {
                 const float si = sigmoidf_<ACC>(E::to_f32(xg[0][m]));
                 const float sf = sigmoidf_<ACC>(E::to_f32(xg[1][m]));
                 const float tg = tanhf_<ACC>(E::to_f32(xg[2][m]));
@@ -448,7 +456,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
             // type, one of fp32); slots past 4H do not exist in the blocks and are left alone
             if constexpr (E::BYTES == 2) {
 #pragma unroll
-                for (int m = 0; m < 4; m += 2)
+                for (int m = 0; m < UPL; m += 2)
                     if (valid[m]) {
                         u32x4 v;
                         __builtin_memcpy(&v, st_d[m], 16);
@@ -456,7 +464,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
                     }
             } else {
 #pragma unroll
-                for (int m = 0; m < 4; ++m)
+                for (int m = 0; m < UPL; ++m)
                     if (valid[m]) {
                         u32x4 v;
                         __builtin_memcpy(&v, st_d[m], 16);
@@ -466,16 +474,16 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
             if constexpr (VIO) {
 #pragma unroll
                 for (int gg = 0; gg < 4; ++gg) {
-                    T pk[4];
+                    T pk[UPL];
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) pk[m] = st_d[m][gg];
+                    for (int m = 0; m < UPL; ++m) pk[m] = st_d[m][gg];
                     V v;
                     __builtin_memcpy(&v, pk, sizeof(V));
                     *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = v;
                 }
             } else {
 #pragma unroll
-                for (int m = 0; m < 4; ++m)
+                for (int m = 0; m < UPL; ++m)
                     if (valid[m]) {
                         T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
                         dst[0] = st_d[m][0];
@@ -503,7 +511,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO>())) void lstm_bwd_persiste
 #pragma unroll
             for (int ks = 0; ks < KSB2; ++ks) acc = mfma_kstep<T>(wb2[ks], bq[ks], acc);
 #pragma unroll
-            for (int m = 0; m < 4; ++m) dh_rec[m] = acc[m];
+            for (int m = 0; m < UPL; ++m) dh_rec[m] = (CW == 8 && mh) ? acc[UPL + m] : acc[m];
             return;
         }
         // ---- point-wise gate backward for this thread's items --------------------------

@@ -64,9 +64,8 @@ struct FwdParams {
 // overlap (H = 64, B = 256, fp16: 1.00 -> 0.78 us per step; the reverse kernel 1.10 -> 0.98).
 // CW (that form only): the number of computing waves, 4 or 8, each with MT of the workgroup's CW * MT row tiles;
 // the four tile-moving waves come behind them.  Eight waves of 2 cells per lane instead of four waves of 4 shorten
-// the step only where no activations are stored (inference: 0.755 -> 0.695 us per step at 64 units); with the
-// stores it is 2.5 % slower -- the gate arithmetic is issued by the same 4 SIMDs either way, and the LDS
-// instructions double -- so the host takes CW = 8 for inference alone.
+// the step of 64 units by 11 % (two waves per SIMD overlap each other's LDS and MFMA latencies; it showed only
+// once the tile-moving waves had stopped being the bound, see their loop below).
 template <int SPLIT, bool VIO, int CW = 4> constexpr int fwd_threads() {
     return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
 }
