@@ -48,7 +48,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain
 # copy of known size.  Counters cannot be read from inside this process: the figures are copied from the
 # committed summaries named here (made by `rocprofv3 --pmc ... -- python3 bench.py --stage fwd_layer`).
-TRAFFIC = {"B": (1411.3e6, "profiles/recurrence_lds_l2_B.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
+TRAFFIC = {"B": (1411.1e6, "profiles/recurrence_lds_l2_B.md"), "D": (336.1e6, "profiles/fwd_recurrence_D_pmc.md")}
 
 
 def physical_cores():
