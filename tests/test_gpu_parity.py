@@ -115,6 +115,10 @@ STAGE_CASES = [
     (9, 12, 128, 213, torch.float32),     # the reference's unit-test shape (test_lstm.py:46-69)
     (5, 33, 70, 300, torch.float32),
     (6, 20, 64, 64, torch.float16),       # config D's hidden size
+    (1, 16, 32, 64, torch.float16),       # one-tile form, tile-moving waves' loop: a single step (nothing but its remainder path)
+    (3, 33, 16, 32, torch.bfloat16),      # ... fewer steps than one pass of the unrolled loop, a ragged last batch tile
+    (13, 50, 64, 16, torch.float16),      # ... three passes and a remainder of one, 16 units (one row tile per workgroup)
+    (9, 16, 64, 64, torch.float32),       # ... fp32 pieces (two per row segment)
     (6, 20, 40, 72, torch.float16),       # H % 8 == 0 but not a tile multiple
     (5, 7, 30, 100, torch.bfloat16),      # H % 8 != 0: unaligned rows in every kernel
     (4, 64, 256, 1024, torch.float16),    # config B tiles
