@@ -58,7 +58,7 @@ struct FwdParams {
 // NKW > 0 (SPLIT 0 only): every wave keeps its share of the W_h slice -- MT x NKW operand
 // fragments, k-steps wave, wave+4, ... -- in registers instead of re-reading it from LDS every
 // timestep (the LDS reads of a 128 KiB slice alone take ~0.4 us per step).  Needs KS <= 4*NKW.
-// SPLIT 2 with tile I/O runs 8 waves: waves 0..3 compute, waves 4..7 only move the tiles between global
+// SPLIT 2 with tile I/O runs CW computing waves and four more that only move the tiles between global
 // memory and LDS (the gates of the step after next in, the results of the last step out).  In one wave the
 // two jobs queue behind each other in a step that is one chain of dependent latencies; side by side they
 // overlap (H = 64, B = 256, fp16: 1.00 -> 0.78 us per step; the reverse kernel 1.10 -> 0.98).
