@@ -1115,6 +1115,26 @@ int fastlstm_gemm_dx_wgrad(const void *d_ifgo, const void *Wx, const void *x, co
 // keep: see LaunchOpts
 // others / n_others: further independent recurrences of this shape (operands in the order ifgo, out, cell, Wh) that
 // share every launch -- only where the plan is the one-tile form (wave_split 2: no exchange between workgroups).
+// The one-tile kernels of 64 hidden units (no exchange between workgroups) are bound by the vector ALU of their CU:
+// a step of 16 rows x 64 units is 1024 cells of 10 exp / rcp at a quarter of the rate and ~35 other instructions
+// each, on one CU, while the others idle.  Rows per workgroup 16 -> 8 -> 4 spreads the cells over 2 x / 4 x the CUs
+// (the MFMAs still produce 16 columns; the lanes of the columns that do not exist take over cells of the lane's other
+// row tiles, so a lane computes one cell per step, not two or four).  T = 1024, B = 256, I = H = 64, fp16, forward /
+// reverse us per step: 16 rows 0.556 / 0.82, 8 rows 0.401 / 0.593, 4 rows 0.339 / 0.458.
+// Returns the factor (0: 16 rows, 2, 4) for `n_rec` recurrences of B rows side by side in one launch.
+static int one_tile_row_split(int B, int n_rec, int num_cus) {
+    if ((long long)n_rec * cdiv(B, 4) <= num_cus) return 4;
+    if ((long long)n_rec * cdiv(B, 8) <= num_cus) return 2;
+    return 0;
+}
+
+// coalesced tile I/O of the general kernels needs complete, 16-byte aligned row segments and room in LDS
+static bool fwd_tile_io(const fastlstm_plan &pl, int H, int dtype, int *tile_bytes) {
+    const int s = elem_bytes(dtype), gseg = pl.ht * s;
+    *tile_bytes = (pl.bt * (4 * gseg + 16) + 2 * pl.bt * (gseg + 16)) * (pl.wave_split != 2 ? 1 : 2);
+    return gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && pl.lds_bytes + *tile_bytes <= pl.lds_limit;
+}
+
 static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
                                int H, int dtype, void *stream, int keep, void *const (*others)[7] = nullptr,
                                int n_others = 0) {
@@ -1128,6 +1148,10 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     if (ws_bytes < pl.ws_bytes) return FASTLSTM_ERR_WORKSPACE;
     const bool sync = pl.wave_split != 2;
     if (n_others && (sync || n_others > 3)) return FASTLSTM_ERR_DIM;
+    // 64 units per workgroup: batch tiles of 4 or 8 rows where that many workgroups still find a CU each
+    int tile_bytes = 0;
+    const bool tile_io = fwd_tile_io(pl, H, dtype, &tile_bytes);
+    const int rs = (!sync && tile_io && pl.ht == 64 && pl.bt == 16) ? one_tile_row_split(B, 1 + n_others, pl.num_cus) : 0;
     const int kstep = dtype == FASTLSTM_FP32 ? 16 : 32;
     unsigned char *wsb = static_cast<unsigned char *>(ws);
     if (pl.wave_split == 3) {   // W_h does not fit on chip: pack it once, then stream it every step
@@ -1208,32 +1232,35 @@ static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh
     for (int i = 0; i < n_others; ++i) {
         p.ifgo_x[i] = others[i][0]; p.out_x[i] = others[i][1]; p.cell_x[i] = others[i][2]; p.Wh_x[i] = others[i][3];
     }
-    const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, false);
-    // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
     int lds_bytes = pl.lds_bytes;
     {
-        const int s = elem_bytes(dtype), gseg = pl.ht * s;
-        const int tile_bytes = (pl.bt * (4 * gseg + 16) + 2 * pl.bt * (gseg + 16)) * (sync ? 1 : 2);
-        p.vec_io = (gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && lds_bytes + tile_bytes <= pl.lds_limit) ? 1 : 0;
+        p.vec_io = tile_io ? 1 : 0;
         if (p.vec_io) lds_bytes += tile_bytes;
 #ifdef FASTLSTM_TIMELINE
         lds_bytes += 4096;   // room for the diagnostic time stamps of the kernel
 #endif
     }
+    int bt = pl.bt, n_btiles = pl.n_btiles;
+    if (rs) {
+        p.rs = rs;
+        bt = 16 / rs;
+        n_btiles = cdiv(B, bt);
+    }
+    const int n_bt_total = cdiv(B, bt);
     // K-split kernels keep the slice in registers when a wave's share is at most 32 fragments
     if (pl.wave_split == 0) {
         const int nkw = cdiv(p.KS, 4) <= 4 ? 4 : (cdiv(p.KS, 4) <= 8 ? 8 : 0);
         if (nkw && (pl.ht / 4) * nkw <= 32) p.w_regs = nkw;
     }
     FwdLauncher launch = fwd_launcher(dtype);
-    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
-        const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += n_btiles) {
+        const int n_bt = std::min(n_btiles, n_bt_total - bt0);
         p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;  // exchange-slot stride is sized for a full launch
-        p.b_base = bt0 * pl.bt;
+        p.b_base = bt0 * bt;
         p.n_bt_launch = n_bt;
         const int grid = p.n_rec * n_bt * pl.n_htiles;
         int occ = 0;
@@ -1344,7 +1371,6 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
         p.dout_x[i] = others[i][0]; p.dh_x[i] = others[i][1]; p.dc_x[i] = others[i][2]; p.ifgo_x[i] = others[i][3];
         p.cell_x[i] = others[i][4]; p.d_ifgo_x[i] = others[i][5]; p.Wh_x[i] = others[i][6];
     }
-    const int n_bt_total = cdiv(B, pl.bt);
     const size_t flags_bytes = recurrent_flags_bytes(pl.n_btiles, pl.n_htiles);
     const size_t slot_bytes = recurrent_slot_bytes(H, dtype, pl.bt, pl.n_btiles, true);
     // coalesced tile I/O needs complete, 16-byte aligned row segments and room in LDS
@@ -1355,13 +1381,21 @@ static int bwd_persistent_impl(const void *dout, void *dh, void *dc, const void 
         p.vec_io = (gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && lds_bytes + tile_bytes <= pl.lds_limit) ? 1 : 0;
         if (p.vec_io) lds_bytes += tile_bytes;
     }
+    // 64 units per workgroup: batch tiles of 4 or 8 rows where that many workgroups still find a CU each
+    int bt = pl.bt, n_btiles = pl.n_btiles;
+    if (!sync && p.vec_io && pl.ht == 64 && pl.bt == 16) {
+        p.rs = one_tile_row_split(B, 1 + n_others, pl.num_cus);
+        bt = 16 / std::max(p.rs, 1);
+        n_btiles = cdiv(B, bt);
+    }
+    const int n_bt_total = cdiv(B, bt);
     BwdLauncher launch = bwd_launcher(dtype);
-    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += pl.n_btiles) {
-        const int n_bt = std::min(pl.n_btiles, n_bt_total - bt0);
+    for (int c = 0, bt0 = 0; bt0 < n_bt_total; ++c, bt0 += n_btiles) {
+        const int n_bt = std::min(n_btiles, n_bt_total - bt0);
         p.flags = reinterpret_cast<int *>(wsb + kWsHeaderBytes + kWsCounterBytes + (size_t)c * flags_bytes);
         p.xbuf = wsb + pl.ws_zero_bytes + (size_t)c * 2 * slot_bytes;
         p.n_bt = pl.n_btiles;
-        p.b_base = bt0 * pl.bt;
+        p.b_base = bt0 * bt;
         p.n_bt_launch = n_bt;
         const int grid = p.n_rec * n_bt * pl.n_htiles;
         int occ = 0;

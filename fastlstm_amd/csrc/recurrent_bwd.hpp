@@ -47,6 +47,7 @@ struct BwdParams {
     long long *trace;   // optional diagnostics: 4 accumulated phase times per workgroup, else nullptr
     // SPLIT 2 only: n_rec > 1 independent recurrences of this shape share the launch (see FwdParams)
     int n_rec, n_bt_launch;
+    int rs;             // 2, 4: batch tiles of 16 / rs rows (RS instantiation; b_base and n_bt_launch count in those), else 0
     const void *dout_x[3], *ifgo_x[3], *cell_x[3], *Wh_x[3];
     void *dh_x[3], *dc_x[3], *d_ifgo_x[3];
 };
@@ -63,7 +64,12 @@ template <int SPLIT, bool VIO, int CW = 4> constexpr int bwd_threads() {
     return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
 }
 
-template <typename T, int NTW, int SPLIT, bool VIO, int CW = 4>
+// RS = 2 (with CW = 8) or 4 (with CW = 4): batch tiles of 16 / RS rows -- RS times the workgroups -- and ONE cell
+// per lane instead of two or four: the lanes of the columns that do not exist take over the lane's other units
+// through DPP rotations of the accumulator within the row of 16 lanes (the operand rows that do not exist are
+// zeros).  See the forward kernel: the step of the 16-row form is bound by the vector ALU (T = 1024, B = 256, fp16:
+// 0.82 us per step with 16 rows, 0.593 with 8, 0.458 with 4).
+template <typename T, int NTW, int SPLIT, bool VIO, int CW = 4, int RS = 1>
 __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_persistent_kernel(const BwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
@@ -75,8 +81,11 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
     constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;
     constexpr int P = SPLIT == 0 ? 4 : 1;
     constexpr int MTB = SPLIT == 2 ? 4 : 1;          // unit tiles (16 rows each) per workgroup
-    constexpr int IPT = SPLIT == 2 ? UPL : NT;       // (unit, batch row) items per thread, upper bound
-    constexpr int BT = 16 * NT;
+    static_assert(RS == 1 || (IOW && NTW == 1 && ((RS == 2 && CW == 8) || (RS == 4 && CW == 4))),
+                  "batch tiles of 16 / RS rows: the one-tile form, RS units per lane folded into one cell");
+    constexpr int NI = RS > 1 ? 1 : UPL;             // SPLIT 2: cells per lane
+    constexpr int IPT = SPLIT == 2 ? NI : NT;        // (unit, batch row) items per thread, upper bound
+    constexpr int BT = 16 * NT / RS;
     constexpr int CH = 16 / NTW;                     // k-steps fetched per batch of loads (2 batches in flight)
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -189,8 +198,11 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
         // SPLIT 2: the item is element mh * UPL + m of the lane's own accumulator -- that unit of 4 * (lane / 16) .. + 3
         // of the wave's unit tile, batch row lane % 16 -- so the product of a step lands where it is used
         const int it = tid + kThreads * m;
-        const int n = SPLIT == 2 ? (lane & 15) : (it & 15), rest = it >> 4;
-        const int ul = SPLIT == 2 ? ut * 16 + (lane >> 4) * 4 + mh * UPL + m : rest % HT, nt = SPLIT == 2 ? 0 : rest / HT;
+        // (RS 2, 4: row lane % (16 / RS), and of the wave's RS units per lane group the one that lane % 16 / (16 / RS) names)
+        const int n = RS > 1 ? (lane & 15) % (16 / RS) : SPLIT == 2 ? (lane & 15) : (it & 15), rest = it >> 4;
+        const int ul = RS > 1 ? ut * 16 + (lane >> 4) * 4 + mh * UPL + (lane & 15) / (16 / RS)
+                              : SPLIT == 2 ? ut * 16 + (lane >> 4) * 4 + mh * UPL + m : rest % HT;
+        const int nt = SPLIT == 2 ? 0 : rest / HT;
         const int unit = u0 + ul, b = b0 + nt * 16 + n;
         valid[m] = nt < NT && unit < H && b < B;
         // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
@@ -385,7 +397,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
     int slot = 0;  // ring slot of this step's d_ifgo
     // One hidden tile per workgroup: the lane's UPL units of the current step's tile rows (4 gates,
     // c_{t-1}, dout), read a step ahead
-    using NxV = typename VecBytes<(SPLIT == 2 ? UPL : 4) * E::BYTES>::type;
+    using NxV = typename VecBytes<(SPLIT == 2 ? NI : 4) * E::BYTES>::type;
     NxV nx[6];
     auto load_items = [&](const unsigned char *gt_) __attribute__((always_inline)) {
 #pragma unroll
@@ -413,17 +425,17 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
             // slots of the exchange copy, and the product comes back in the lane's own accumulator (nothing
             // is reduced).  One workgroup barrier per step: behind it the exchange copy, the d_ifgo tile
             // and the next step's input tiles are all in LDS.
-            using V = typename VecBytes<UPL * E::BYTES>::type;
+            using V = typename VecBytes<NI * E::BYTES>::type;
             if (cw) {
-            T xg[4][UPL], xc[UPL], xd[UPL], st_d[UPL][4];
+            T xg[4][NI], xc[NI], xd[NI], st_d[NI][4];
             if constexpr (VIO) {   // read behind the previous step's barrier (or in the prologue)
 #pragma unroll
-                for (int gg = 0; gg < 4; ++gg) __builtin_memcpy(xg[gg], &nx[gg], UPL * E::BYTES);
-                __builtin_memcpy(xc, &nx[4], UPL * E::BYTES);
-                __builtin_memcpy(xd, &nx[5], UPL * E::BYTES);
+                for (int gg = 0; gg < 4; ++gg) __builtin_memcpy(xg[gg], &nx[gg], NI * E::BYTES);
+                __builtin_memcpy(xc, &nx[4], NI * E::BYTES);
+                __builtin_memcpy(xd, &nx[5], NI * E::BYTES);
             } else {
 #pragma unroll
-                for (int m = 0; m < UPL; ++m) {
+                for (int m = 0; m < NI; ++m) {
 #pragma unroll
                     for (int gg = 0; gg < 4; ++gg) xg[gg][m] = pre[u][m][gg];
                     xc[m] = c0r[u][m];
@@ -431,7 +443,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
                 }
             }
 #pragma unroll
-            for (int m = 0; m < UPL; ++m) {
+            for (int m = 0; m < NI; ++m) {
                 const float si = sigmoidf_<ACC>(E::to_f32(xg[0][m]));
                 const float sf = sigmoidf_<ACC>(E::to_f32(xg[1][m]));
                 const float tg = tanhf_<ACC>(E::to_f32(xg[2][m]));
@@ -454,9 +466,15 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
             }
             // exchange copy: k = 4 * unit + gate, whole 16-byte operand slots (two units of a 16-bit
             // type, one of fp32); slots past 4H do not exist in the blocks and are left alone
-            if constexpr (E::BYTES == 2) {
+            if constexpr (RS > 1 && E::BYTES == 2) {   // one unit: half an operand slot
+                if (valid[0]) {
+                    u32x2 v;
+                    __builtin_memcpy(&v, st_d[0], 8);
+                    xch.store8(xw + xoff[0], v);
+                }
+            } else if constexpr (E::BYTES == 2) {
 #pragma unroll
-                for (int m = 0; m < UPL; m += 2)
+                for (int m = 0; m < NI; m += 2)
                     if (valid[m]) {
                         u32x4 v;
                         __builtin_memcpy(&v, st_d[m], 16);
@@ -464,7 +482,7 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
                     }
             } else {
 #pragma unroll
-                for (int m = 0; m < UPL; ++m)
+                for (int m = 0; m < NI; ++m)
                     if (valid[m]) {
                         u32x4 v;
                         __builtin_memcpy(&v, st_d[m], 16);
@@ -474,16 +492,16 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
             if constexpr (VIO) {
 #pragma unroll
                 for (int gg = 0; gg < 4; ++gg) {
-                    T pk[UPL];
+                    T pk[NI];
 #pragma unroll
-                    for (int m = 0; m < UPL; ++m) pk[m] = st_d[m][gg];
+                    for (int m = 0; m < NI; ++m) pk[m] = st_d[m][gg];
                     V v;
                     __builtin_memcpy(&v, pk, sizeof(V));
                     *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = v;
                 }
             } else {
 #pragma unroll
-                for (int m = 0; m < UPL; ++m)
+                for (int m = 0; m < NI; ++m)
                     if (valid[m]) {
                         T *dst = d_ifgo + (size_t)t * B4H + off_p[m];
                         dst[0] = st_d[m][0];
@@ -510,8 +528,17 @@ __global__ __launch_bounds__((bwd_threads<SPLIT, VIO, CW>())) void lstm_bwd_pers
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < KSB2; ++ks) acc = mfma_kstep<T>(wb2[ks], bq[ks], acc);
+            if constexpr (RS == 2) {
+                // (scalars, not elements of the vector inside the builtin: see the forward kernel)
+                const float a0 = acc[0], a1 = acc[1], a2 = acc[2], a3 = acc[3];
+                dh_rec[0] = fold_upper_half(mh ? a2 : a0, mh ? a3 : a1);
+            } else if constexpr (RS == 4) {
+                const float a0 = acc[0], a1 = acc[1], a2 = acc[2], a3 = acc[3];
+                dh_rec[0] = fold_quarters(a0, a1, a2, a3);
+            } else {
 #pragma unroll
-            for (int m = 0; m < UPL; ++m) dh_rec[m] = (CW == 8 && mh) ? acc[UPL + m] : acc[m];
+                for (int m = 0; m < UPL; ++m) dh_rec[m] = (CW == 8 && mh) ? acc[UPL + m] : acc[m];
+            }
             return;
         }
         // ---- point-wise gate backward for this thread's items --------------------------

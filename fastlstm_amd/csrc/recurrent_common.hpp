@@ -82,6 +82,18 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
     }
 }
 
+// lanes 0..7 of every row of 16 lanes keep lo, lanes 8..15 take hi of the lane 8 below (row_ror:8 into banks 2 and 3)
+__device__ __forceinline__ float fold_upper_half(float lo, float hi) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, lo), __builtin_bit_cast(int, hi), 0x128, 0xf, 0xc, false));
+}
+// lanes 4j .. 4j + 3 of every row of 16 lanes take v_j of the lane 4j below (row_ror:4j into bank j)
+__device__ __forceinline__ float fold_quarters(float v0, float v1, float v2, float v3) {
+    int r = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v0), __builtin_bit_cast(int, v1), 0x124, 0xf, 0x2, false);
+    r = __builtin_amdgcn_update_dpp(r, __builtin_bit_cast(int, v2), 0x128, 0xf, 0x4, false);
+    r = __builtin_amdgcn_update_dpp(r, __builtin_bit_cast(int, v3), 0x12c, 0xf, 0x8, false);
+    return __builtin_bit_cast(float, r);
+}
+
 // A value that is the same in all lanes, moved to scalar registers (the compiler cannot always tell).
 __device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }
 template <typename P> __device__ __forceinline__ P *uniform_ptr(P *ptr) {

@@ -48,6 +48,7 @@ struct FwdParams {
     // SPLIT 2 only (no exchange between workgroups): n_rec > 1 independent recurrences of this shape share the launch,
     // recurrence r on the workgroups r * n_bt_launch ...; operands of recurrences 1 ... in the arrays
     int n_rec, n_bt_launch;
+    int rs;            // 2, 4: batch tiles of 16 / rs rows (RS instantiation; b_base and n_bt_launch count in those), else 0
     void *ifgo_x[3], *out_x[3], *cell_x[3];
     const void *Wh_x[3];
 };
@@ -70,7 +71,15 @@ template <int SPLIT, bool VIO, int CW = 4> constexpr int fwd_threads() {
     return (SPLIT == 2 && VIO) ? (CW + 4) * kWave : kThreads;
 }
 
-template <typename T, int MT, int NTW, int SPLIT, bool VIO, int NKW = 0, int CW = 4>
+// RS = 2 (8 computing waves of 2 row tiles) or 4 (4 computing waves of 4 row tiles), 64 units: a workgroup takes
+// 16 / RS batch rows, i.e. the batch spreads over RS times the CUs.  The MFMAs still produce 16 columns (the operand
+// rows that do not exist are zeros); the RS accumulator tiles of a lane are folded into one -- the lanes of the
+// columns that do not exist take the columns 0 .. 16 / RS - 1 of the lane's other tiles through DPP rotations
+// within the row of 16 lanes -- so that every lane computes ONE cell per step instead of two or four.  The step of
+// the 16-row kernel is bound by the vector ALU, not by a latency: per wave and step 20 exp / rcp at a quarter of the
+// rate and 70 other instructions for two cells, two such waves per SIMD, is 1200 of the step's 1170 cycles
+// (T = 1024, B = 256, fp16: 0.556 us per step with 16 rows, 0.401 with 8, 0.339 with 4).
+template <typename T, int MT, int NTW, int SPLIT, bool VIO, int NKW = 0, int CW = 4, int RS = 1>
 __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_persistent_kernel(const FwdParams p) {
     using E = Elem<T>;
     constexpr bool SYNC = SPLIT != 2;
@@ -82,8 +91,10 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
     constexpr int NT = SPLIT == 1 ? 4 * NTW : NTW;   // n-tiles per workgroup
     constexpr int P = SPLIT == 0 ? 4 : 1;            // partial sums per output tile
     constexpr int TILES = MTT * NT;
-    constexpr int IPT = (TILES + CW - 1) / CW;       // (tile, lane) items per thread
-    constexpr int HT = 4 * MTT, BT = 16 * NT;
+    static_assert(RS == 1 || (IOW && NTW == 1 && ((RS == 2 && CW == 8 && MT == 2) || (RS == 4 && CW == 4 && MT == 4))),
+                  "batch tiles of 16 / RS rows: RS row tiles per wave, folded into one cell per lane");
+    constexpr int IPT = RS > 1 ? 1 : (TILES + CW - 1) / CW;   // (tile, lane) items per thread
+    constexpr int HT = 4 * MTT, BT = 16 * NT / RS;
     constexpr int CH = 8 / NTW;                      // k-steps fetched per batch of loads
     constexpr bool WREG = NKW > 0;
     static_assert(!WREG || SPLIT == 0, "register-resident weights: K-split kernels only");
@@ -243,15 +254,18 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
         // SPLIT 2: the item is the lane's own accumulator of the wave's m-tile m (see the weight rows above)
         const int tl = SPLIT == 2 ? wave * MT + m : wave + 4 * m;
         const int mt = tl / NT, nt = tl % NT;
-        const int ul = SPLIT == 2 ? wave * 4 * MT + q * MT + m : mt * 4 + q;   // unit inside the hidden tile
-        const int unit = u0 + ul, b = b0 + nt * 16 + n;
+        // (RS 2, 4: the lane's one item is row n % (16 / RS) of the wave's row tile n / (16 / RS))
+        const int ul = RS > 1 ? wave * 4 * MT + q * MT + n / (16 / RS)
+                              : SPLIT == 2 ? wave * 4 * MT + q * MT + m : mt * 4 + q;   // unit inside the hidden tile
+        const int row = RS > 1 ? n % (16 / RS) : nt * 16 + n;
+        const int unit = u0 + ul, b = b0 + row;
         valid[m] = (tl < TILES) && unit < H && b < B;
         // invalid items point at the tile's first element: their loads stay in bounds, nothing is stored
         off_h[m] = valid[m] ? (size_t)b * H + unit : (size_t)b0 * H + u0;
         off_p[m] = valid[m] ? (size_t)b * 4 * H + unit : (size_t)b0 * 4 * H + u0;
-        xoff[m] = nt * KS * kFragBytes + frag_offset<T>(n, unit);
-        goff[m] = (nt * 16 + n) * GROW + ul * E::BYTES;
-        soff[m] = (nt * 16 + n) * SROW + ul * E::BYTES;
+        xoff[m] = RS > 1 ? frag_offset<T>(row, unit) : nt * KS * kFragBytes + frag_offset<T>(n, unit);
+        goff[m] = row * GROW + ul * E::BYTES;
+        soff[m] = row * SROW + ul * E::BYTES;
         c_state[m] = valid[m] ? E::to_f32(cell[off_h[m]]) : 0.f;
     }
 
@@ -426,27 +440,19 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
                 to_global(t, tiles + (t & 1) * TILE_BYTES);
                 load_tile(t + PD, uc);
             };
-            static_assert(PD == 4, "four steps per pass of the loop");
             // (the loop is entered with what every later pass finds in flight: between the tiles, as many stores as a step issues)
-            load_tile(0, std::integral_constant<int, 0>{});
-            dropped_stores(0);
-            load_tile(1, std::integral_constant<int, 1>{});
-            dropped_stores(1);
-            load_tile(2, std::integral_constant<int, 2>{});
-            dropped_stores(2);
-            load_tile(3, std::integral_constant<int, 3>{});
+            static_for<0, PD>([&](auto uc) __attribute__((always_inline)) {
+                load_tile(decltype(uc)::value, uc);
+                if constexpr (decltype(uc)::value + 1 < PD) dropped_stores(decltype(uc)::value);
+            });
             to_lds(std::integral_constant<int, 0>{}, tiles);
             __syncthreads();
             int t0 = 0;
-            for (; t0 + PD <= T_; t0 += PD) {
-                io_step(t0, std::integral_constant<int, 0>{});
-                io_step(t0 + 1, std::integral_constant<int, 1>{});
-                io_step(t0 + 2, std::integral_constant<int, 2>{});
-                io_step(t0 + 3, std::integral_constant<int, 3>{});
-            }
-            if (t0 < T_) io_step(t0, std::integral_constant<int, 0>{});
-            if (t0 + 1 < T_) io_step(t0 + 1, std::integral_constant<int, 1>{});
-            if (t0 + 2 < T_) io_step(t0 + 2, std::integral_constant<int, 2>{});
+            for (; t0 + PD <= T_; t0 += PD)
+                static_for<0, PD>([&](auto uc) __attribute__((always_inline)) { io_step(t0 + decltype(uc)::value, uc); });
+            static_for<0, PD - 1>([&](auto uc) __attribute__((always_inline)) {
+                if (t0 + decltype(uc)::value < T_) io_step(t0 + decltype(uc)::value, uc);
+            });
             return;
         }
     }
@@ -470,7 +476,8 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
             // nothing but h_t crosses waves; the lane moves its MT consecutive units of every tile row
             // with one LDS access.  One workgroup barrier per step: behind it h_t (operand blocks), this
             // step's result tiles and the next step's gates tile are all in LDS.
-            using V = typename VecBytes<MT * E::BYTES>::type;
+            constexpr int NI = RS > 1 ? 1 : MT;   // cells per lane
+            using V = typename VecBytes<NI * E::BYTES>::type;
             const unsigned xb = (unsigned)slot_r * xslot, xn = (unsigned)slot_w * xslot;
             if (cw) {
             f32x4 acc[MT];
@@ -492,18 +499,35 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
 #pragma unroll
                     for (int a = 0; a < MT; ++a) acc[a] = mfma_kstep<T>(w2[a][ks], bq[ks], acc[a]);
             }
-            T x4[4][MT], st_p[IPT][4], st_h[IPT], st_c[IPT];
+            if constexpr (RS == 2) {
+                // lanes 8..15 of every row of 16: columns 0..7 of the second tile (row_ror:8 into banks 2 and 3)
+                // (element by element on scalars: written as a loop over the vectors' elements, the compiler emitted
+                // the first element's move four times)
+                const float lo0 = acc[0][0], lo1 = acc[0][1], lo2 = acc[0][2], lo3 = acc[0][3];
+                const float hi0 = acc[1][0], hi1 = acc[1][1], hi2 = acc[1][2], hi3 = acc[1][3];
+                acc[0] = f32x4{fold_upper_half(lo0, hi0), fold_upper_half(lo1, hi1), fold_upper_half(lo2, hi2), fold_upper_half(lo3, hi3)};
+            }
+            if constexpr (RS == 4) {   // lanes 4j .. 4j + 3: columns 0..3 of the wave's tile j
+                float f[4][4];
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    f[a][0] = acc[a][0]; f[a][1] = acc[a][1]; f[a][2] = acc[a][2]; f[a][3] = acc[a][3];
+                }
+                acc[0] = f32x4{fold_quarters(f[0][0], f[1][0], f[2][0], f[3][0]), fold_quarters(f[0][1], f[1][1], f[2][1], f[3][1]),
+                               fold_quarters(f[0][2], f[1][2], f[2][2], f[3][2]), fold_quarters(f[0][3], f[1][3], f[2][3], f[3][3])};
+            }
+            T x4[4][NI], st_p[IPT][4], st_h[IPT], st_c[IPT];
 #pragma unroll
             for (int gg = 0; gg < 4; ++gg) {
                 if constexpr (VIO) {
                     __builtin_memcpy(x4[gg], &xv[gg], sizeof(V));
                 } else {
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) x4[gg][m] = pre[u][m][gg];
+                    for (int m = 0; m < NI; ++m) x4[gg][m] = pre[u][m][gg];
                 }
             }
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
+            for (int m = 0; m < NI; ++m) {
                 const float pi = E::to_f32(x4[0][m]) + acc[m][0];
                 const float pf = E::to_f32(x4[1][m]) + acc[m][1];
                 const float pg = E::to_f32(x4[2][m]) + acc[m][2];
@@ -527,9 +551,9 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
             if constexpr (VIO) {
 #pragma unroll
                 for (int gg = 0; gg < 4; ++gg) {
-                    T pk[MT];
+                    T pk[NI];
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) pk[m] = st_p[m][gg];
+                    for (int m = 0; m < NI; ++m) pk[m] = st_p[m][gg];
                     V vp;
                     __builtin_memcpy(&vp, pk, sizeof(V));
                     *reinterpret_cast<V *>(gt + goff[0] + gg * GSEG) = vp;
@@ -538,7 +562,7 @@ __global__ __launch_bounds__((fwd_threads<SPLIT, VIO, CW>())) void lstm_fwd_pers
                 *reinterpret_cast<V *>(gt + BT * GROW + BT * SROW + soff[0]) = vc;
             } else {
 #pragma unroll
-                for (int m = 0; m < MT; ++m) {
+                for (int m = 0; m < NI; ++m) {
                     if (valid[m]) {
                         if (keep) {
                             T *dst = ifgo + (size_t)t * B4H + off_p[m];

@@ -114,11 +114,13 @@ STAGE_CASES = [
     (7, 5, 11, 13, torch.float32),        # tiny, everything ragged, barrier-free form
     (9, 12, 128, 213, torch.float32),     # the reference's unit-test shape (test_lstm.py:46-69)
     (5, 33, 70, 300, torch.float32),
-    (6, 20, 64, 64, torch.float16),       # config D's hidden size
+    (6, 20, 64, 64, torch.float16),       # config D's hidden size: batch tiles of 4 rows, one cell per lane
     (1, 16, 32, 64, torch.float16),       # one-tile form, tile-moving waves' loop: a single step (nothing but its remainder path)
     (3, 33, 16, 32, torch.bfloat16),      # ... fewer steps than one pass of the unrolled loop, a ragged last batch tile
     (13, 50, 64, 16, torch.float16),      # ... three passes and a remainder of one, 16 units (one row tile per workgroup)
     (9, 16, 64, 64, torch.float32),       # ... fp32 pieces (two per row segment)
+    (3, 1100, 32, 64, torch.float16),     # ... 64 units with more rows than CUs x 4: batch tiles of 8 rows (the last one ragged)
+    (2, 2100, 16, 64, torch.bfloat16),    # ... and more than CUs x 8: batch tiles of 16 rows
     (6, 20, 40, 72, torch.float16),       # H % 8 == 0 but not a tile multiple
     (5, 7, 30, 100, torch.bfloat16),      # H % 8 != 0: unaligned rows in every kernel
     (4, 64, 256, 1024, torch.float16),    # config B tiles
@@ -773,6 +775,7 @@ PAIR_CASES = [
     (3, 24, 64, 1024, torch.float32, True),       # ... fp32
     (3, 64, 64, 2048, torch.float16, False),      # 64-row groups: one after the other
     (6, 200, 48, 64, torch.float16, True),        # one hidden tile per workgroup: both recurrences' workgroups in one grid
+    (3, 600, 32, 64, torch.bfloat16, True),       # ... of 8-row batch tiles (2 x 150 of 4 rows are more than the CUs)
     (5, 33, 16, 32, torch.float32, True),
 ]
 
@@ -877,7 +880,13 @@ def test_xcd_local_kernels_agree_with_general_kernels_and_oracle(oracle, T, B, H
 @pytest.mark.parametrize("T,B,I,H,dt", [(96, 64, 1024, 1024, torch.float16),    # helpers compute K1 inside the launch
                                         (40, 32, 512, 1024, torch.bfloat16),   # same, 8 timesteps per row tile
                                         (12, 40, 96, 512, torch.float16),      # 4-wave kernel: two launches
-                                        (9, 20, 50, 72, torch.float32)])       # general kernels
+                                        (9, 20, 50, 72, torch.float32),        # general kernels
+                                        (40, 48, 64, 64, torch.float16),       # 64 units, one tile: batch tiles of 4 rows
+                                        (131, 100, 48, 64, torch.bfloat16),    # ... a ragged batch tile
+                                        (1, 16, 8, 64, torch.float16),         # ... one step
+                                        (7, 1100, 32, 64, torch.bfloat16),     # ... batch tiles of 8 rows, T % 4 = 3
+                                        (6, 2100, 40, 64, torch.float16),      # ... batch tiles of 16 rows, T % 4 = 2
+                                        (5, 20, 64, 32, torch.float16)])       # 32 units
 def test_fwd_layer_equals_projection_then_recurrence(T, B, I, H, dt):
     """fastlstm_fwd_layer must give bit-identical results to fastlstm_gemm_ifgo followed by
     fastlstm_fwd_persistent, whichever way it schedules the two stages."""
