@@ -410,6 +410,8 @@ def main():
         # one hidden tile per workgroup (H <= 64): no exchange between CUs at all; the kernel streams the
         # gate tiles through (read + write-back) and writes out / cell -- priced against HBM
         sz = 2 if dname != "fp32" else 4
+        # (64 units: batch tiles of 4 or 8 rows where that many workgroups find a CU each, as the library decides)
+        rows_wg = 16 if H != 64 else (4 if -(-B // 4) <= plan_f.num_cus else 8 if -(-B // 8) <= plan_f.num_cus else 16)
         nbytes = sz * (2.0 * T * B * 4 * H + 2.0 * T * B * H + 4.0 * H * H)
         ach = nbytes / (t_rec * 1e-3) / 1e9
         roofline = {"kernel": "lstm_fwd_persistent_kernel<SPLIT=2> (one hidden tile per workgroup)", "bound": "hbm",
@@ -417,8 +419,8 @@ def main():
                     "traffic": traffic, "traffic_source": traffic_src,
                     "algorithmic": "s*(2*T*B*4H + 2*T*B*H + 4H*H) bytes per launch = %.1f MB" % (nbytes / 1e6),
                     "launch_ms": round(t_rec, 4),
-                    "note": "latency-bound, not HBM-bound: %d independent workgroups (16 batch rows each) walk through "
-                            "T sequential steps; us/step is in kernels.recurrent_fwd_us_per_step" % plan_f.n_btiles}
+                    "note": "latency-bound, not HBM-bound: %d independent workgroups (%d batch rows each) walk through "
+                            "T sequential steps; us/step is in kernels.recurrent_fwd_us_per_step" % (-(-B // rows_wg), rows_wg)}
     elif dname != "fp32" and H % 32 == 0 and H <= 2048:
         # ---- the latency floor of a step, measured with the recurrence's own barrier and exchange code ----
         # (fastlstm_diag_step_probe: 16-bit h tiles; one group is timed alone on an otherwise idle device)
