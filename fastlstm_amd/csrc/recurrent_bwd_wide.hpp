@@ -27,7 +27,7 @@ constexpr int kWideRing = 12;   // LDS blocks (1 KiB) per wave for operand block
 template <typename T, int NKW, int NT>
 __global__ __launch_bounds__(kWave * 8) void lstm_bwd_wide_kernel(const BwdXcdParams p) {
     using E = Elem<T>;
-    constexpr bool ACC = E::BYTES == 4;                // fp32: library exp and IEEE division in the gates
+    constexpr bool ACC = E::BYTES == 4;                // fp32: refined reciprocal in the gates
     constexpr int NWV = 8, NTHR = kWave * NWV;
     constexpr int HT = 16, BT = 16 * NT;
     constexpr int IPT = (HT * BT + NTHR - 1) / NTHR;   // (unit, batch row) items per thread

@@ -34,7 +34,7 @@ namespace fastlstm {
 template <typename T, int NKW, int NT>
 __global__ __launch_bounds__(kWave * 8) void lstm_fwd_wide_kernel(const FwdXcdParams p) {
     using E = Elem<T>;
-    constexpr bool ACC = E::BYTES == 4;                      // fp32: library exp and IEEE division in the gates
+    constexpr bool ACC = E::BYTES == 4;                      // fp32: refined reciprocal in the gates
     constexpr int NWV = 8, NTHR = kWave * NWV;
     constexpr int MT = 4, TILES = MT * NT;                   // unit tiles, batch tiles of 16 rows
     constexpr int IPT = (TILES + NWV - 1) / NWV;             // (tile, lane) items per thread
