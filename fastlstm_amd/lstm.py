@@ -1136,14 +1136,18 @@ def _padded_hidden_size_cached(T, B, H, code, device_index, training, families):
         return 0
     if H <= 64:
         # The general kernels' one-tile form (no exchange between workgroups at all).  In 16 bits it is the fastest
-        # there is at H = 64 (T = 1024, B = 256, I = H = 64 forward + backward 2.1 ms as it is, 3.4 ms as H = 96), and
-        # at 16 and 32, but sizes in between lose the 16-byte tile moves (T = 256, B = 64, forward / forward +
-        # backward: H = 48 0.91 / 1.83 ms, H = 64 0.25 / 0.58).  In fp32 it is bound by the true-fp32 MFMA rate and the
-        # XCD-local kernels win from H = 80 on (H = 64 0.73 / 1.57, H = 48 1.34 / 2.73, as H = 80 0.60 / 1.22).
-        if H <= 16 or H == 32:
-            return 0
+        # there is at H = 64 (T = 1024, B = 256, I = H = 64 forward + backward 0.93 ms as it is, 3.4 ms as H = 96):
+        # its 64-unit kernels spread the batch over tiles of 4 rows and move whole tiles in both directions, which the
+        # narrower forms do not (T = 1024, B = 256, inference forward / forward + backward of a training step with its
+        # loss: H = 32 as it is 0.50 / 3.20 ms, H = 16 0.42 / 2.12, H = 64 0.42 / 1.18).  In fp32 it is bound by the
+        # true-fp32 MFMA rate and the XCD-local kernels win from H = 80 on (H = 64 0.73 / 1.57, H = 48 1.34 / 2.73, as
+        # H = 80 0.60 / 1.22).
         if fp32:
+            if H <= 16 or H == 32:
+                return 0
             return 80 if kind(80) == 1 else 0
+        if H <= 16 and not training:
+            return 0
         return 64 if H < 64 else 0
     if kind(H) != 0 or fast(H):
         return 0

@@ -1411,7 +1411,9 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
                                                  (dict(bidirectional=True), 64, 16, 300, 256, 256, 320, torch.float16),
                                                  (dict(bias=False, batch_first=True), 32, 8, 33, 1150, 1280, 33, torch.bfloat16),
                                                  (dict(), 16, 128, 64, 1150, 1280, 64, torch.bfloat16),   # few steps, many rows
-                                                 (dict(), 64, 16, 70, 576, 640, 70, torch.float32)])   # for the reverse pass's sake
+                                                 (dict(), 64, 16, 70, 576, 640, 70, torch.float32),    # for the reverse pass's sake
+                                                 (dict(), 64, 40, 20, 32, 64, 64, torch.float16),      # narrow layers: as 64 units
+                                                 (dict(bidirectional=True), 40, 30, 16, 16, 64, 64, torch.bfloat16)])
 def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
     """The module pads a hidden size that only the general kernels take to the next one the XCD-local /
     register-resident kernels take (zero weights, biases and initial states for the added units), and a 16-bit
@@ -1428,9 +1430,11 @@ def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I
     leaves = [t.cuda().to(dt).requires_grad_(True) for t in (x, h0, c0)]
     leaves_r = [t.clone().requires_grad_(True) for t in (x, h0, c0)]
     assert m._operand_padding(leaves[0]) == (Hp, Ip)
-    # sizes the fast kernels take run as they are; so does H <= 64 (the one-tile form of the general kernels)
-    for i_, h_ in ((64, 64), (128, 32), (256, 512), (1024, 2048)):
+    # sizes the fast kernels take run as they are, H = 64 (the one-tile form of the general kernels) among them;
+    # narrower 16-bit layers run as 64 units
+    for i_, h_ in ((64, 64), (256, 512), (1024, 2048)):
         assert FastLSTM(i_, h_).to("cuda", torch.float16)._operand_padding(torch.empty(32, 256, i_, device="cuda", dtype=torch.float16)) is None
+    assert FastLSTM(128, 32).to("cuda", torch.float16)._operand_padding(torch.empty(32, 256, 128, device="cuda", dtype=torch.float16)) == (64, 128)
     # ... and a few timesteps do not repay the padding (unless rows x units are many: the last case)
     assert m._operand_padding(leaves[0][:, :4] if kw.get("batch_first") else leaves[0][:4]) is None
     y, (hn, cn) = m(leaves[0], (leaves[1], leaves[2]))
