@@ -1139,16 +1139,16 @@ def _padded_hidden_size_cached(T, B, H, code, device_index, training, families):
         # there is at H = 64 (T = 1024, B = 256, I = H = 64 forward + backward 0.93 ms as it is, 3.4 ms as H = 96):
         # its 64-unit kernels spread the batch over tiles of 4 rows and move whole tiles in both directions, which the
         # narrower forms do not (T = 1024, B = 256, inference forward / forward + backward of a training step with its
-        # loss: H = 32 as it is 0.50 / 3.20 ms, H = 16 0.42 / 2.12, H = 64 0.42 / 1.18).  In fp32 it is bound by the
-        # true-fp32 MFMA rate and the XCD-local kernels win from H = 80 on (H = 64 0.73 / 1.57, H = 48 1.34 / 2.73, as
-        # H = 80 0.60 / 1.22).
-        if fp32:
-            if H <= 16 or H == 32:
-                return 0
-            return 80 if kind(80) == 1 else 0
-        if H <= 16 and not training:
+        # loss: H = 32 as it is 0.50 / 3.20 ms, H = 16 0.42 / 2.12, H = 64 0.42 / 1.18).  The same holds in fp32 since
+        # the 4-row tiles spread its true-fp32 MFMAs over four times the CUs (T = 256, B = 64: H = 64 as it is 0.36 /
+        # 0.86 ms, as H = 80 on the XCD-local kernels 0.57 / 1.21; H = 48 as it is 0.74 / 2.40, as 64 0.45 / 0.98), except
+        # that up to 16 units nothing gains (H = 16 0.18 / 1.03 as it is, 0.45 / 0.99 as 64) and up to 32 only a
+        # training step does (H = 32 0.28 / 1.16 as it is, 0.45 / 0.98 as 64).
+        if H == 64 or H <= (16 if fp32 or not training else 0):
             return 0
-        return 64 if H < 64 else 0
+        if fp32 and H <= 32 and not training:
+            return 0
+        return 64
     if kind(H) != 0 or fast(H):
         return 0
     step = 16 if fp32 else 32

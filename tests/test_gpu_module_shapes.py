@@ -50,7 +50,7 @@ def draw(seed):
 # Shapes at which the dispatch changes form: both directions side by side with a larger unit tile; two stacked
 # layers in one launch at a small batch (chunks of 64 timesteps); reverse launches that keep all, only dx, or none
 # of their GEMMs inside; row ranges of 32-row groups; a remainder of rows behind full fp32 register-resident
-# launches; small hidden sizes that run as 64 / 80.
+# launches; small hidden sizes that run as 64 units.
 FORMS = [
     dict(dt=torch.float16, kw=dict(bidirectional=True, bias=True, batch_first=False), layers=1, T=64, B=128, I=256, H=256),
     dict(dt=torch.float16, kw=dict(bidirectional=False, bias=True, batch_first=False), layers=2, T=256, B=16, I=1024, H=1024),
