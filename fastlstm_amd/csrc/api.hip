@@ -1112,9 +1112,6 @@ int fastlstm_gemm_dx_wgrad(const void *d_ifgo, const void *Wx, const void *x, co
     return gemm_dx_wgrad_impl(d_ifgo, Wx, x, h, dx, dWx, dWh, db, ws, ws_bytes, T, B, I, H, dtype, stream);
 }
 
-// keep: see LaunchOpts
-// others / n_others: further independent recurrences of this shape (operands in the order ifgo, out, cell, Wh) that
-// share every launch -- only where the plan is the one-tile form (wave_split 2: no exchange between workgroups).
 // The one-tile kernels of 64 hidden units (no exchange between workgroups) are bound by the vector ALU of their CU:
 // a step of 16 rows x 64 units is 1024 cells of 10 exp / rcp at a quarter of the rate and ~35 other instructions
 // each, on one CU, while the others idle.  Rows per workgroup 16 -> 8 -> 4 spreads the cells over 2 x / 4 x the CUs
@@ -1135,6 +1132,9 @@ static bool fwd_tile_io(const fastlstm_plan &pl, int H, int dtype, int *tile_byt
     return gseg >= 16 && (H * s) % 16 == 0 && H % pl.ht == 0 && pl.lds_bytes + *tile_bytes <= pl.lds_limit;
 }
 
+// keep: see LaunchOpts
+// others / n_others: further independent recurrences of this shape (operands in the order ifgo, out, cell, Wh) that
+// share every launch -- only where the plan is the one-tile form (wave_split 2: no exchange between workgroups).
 static int fwd_persistent_impl(void *ifgo, void *out, void *cell, const void *Wh, void *ws, size_t ws_bytes, int T, int B,
                                int H, int dtype, void *stream, int keep, void *const (*others)[7] = nullptr,
                                int n_others = 0) {
