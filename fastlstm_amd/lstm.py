@@ -1529,6 +1529,8 @@ class FastLSTM(nn.Module):
                 and Hp >= 512 and _recurrent_kind(T, B, Hp + 32, _DTYPE_CODE[dt], idx) in (1, 2)):
             Hp += 32
         Ip = -(-I // 64) * 64 if dt != torch.float32 and T * B >= 1024 and data.shape[-1] == I else I
+        if Hp <= 64 and I <= 64 and I % 16 == 0:   # a narrow layer's streaming products take any multiple of 16
+            Ip = I
         return (Hp, Ip) if (Hp, Ip) != (H, I) else None
 
     def _forward_operands_padded(self, x, h_c_0, Hp, Ip):

@@ -1413,7 +1413,7 @@ def test_packed_sequence_vs_nn_lstm(kw, lengths):
                                                  (dict(), 16, 128, 64, 1150, 1280, 64, torch.bfloat16),   # few steps, many rows
                                                  (dict(), 64, 16, 70, 576, 640, 70, torch.float32),    # for the reverse pass's sake
                                                  (dict(), 64, 40, 20, 32, 64, 64, torch.float16),      # narrow layers: as 64 units
-                                                 (dict(bidirectional=True), 40, 30, 16, 16, 64, 64, torch.bfloat16)])
+                                                 (dict(bidirectional=True), 40, 30, 16, 16, 64, 16, torch.bfloat16)])   # (an input size the streaming products take)
 def test_hidden_and_input_sizes_off_the_fast_kernels_run_zero_padded(kw, T, B, I, H, Hp, Ip, dt):
     """The module pads a hidden size that only the general kernels take to the next one the XCD-local /
     register-resident kernels take (zero weights, biases and initial states for the added units), and a 16-bit
